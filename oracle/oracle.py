@@ -1,0 +1,213 @@
+"""ctypes front end of the CPU oracle.  TEST INFRASTRUCTURE ONLY.
+
+Only the test suite, the smoke check and the benchmark's CPU-baseline leg import
+this module; the shipped package never does.  Each wrapper names the reference
+lines its C counterpart in ``fg_oracle.c`` follows.
+
+Two kinds of checker live here:
+
+* ``spmm_csr_x86`` / ``spmm_dds_x86`` / ``sddmm_x86`` / ``csr_to_dds`` /
+  ``partition_coo_2d`` -- the C restatement of the reference's x86 loop nests
+  and host partitioners (fp32, reference summation order).
+* ``spmm_f64`` / ``sddmm_f64`` / ``sddmm_multihead_f64`` -- float64 closed
+  forms through scipy / numpy library routines, the neutral truth both the C
+  restatement and the HIP kernels are compared with.
+
+``sddmm_multihead`` is PARITY UNPINNED by the reference (it has no multi-head
+op); see the header of ``fg_oracle.c``.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import scipy.sparse
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libfg_oracle.so")
+_lib = None
+
+_i32p = ctypes.POINTER(ctypes.c_int32)
+_u32p = ctypes.POINTER(ctypes.c_uint32)
+_f32p = ctypes.POINTER(ctypes.c_float)
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+
+def build(force=False):
+    """Compile ``fg_oracle.c`` with the Makefile beside it."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-C", _HERE, "libfg_oracle.so"])
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        L.orc_max_threads.restype = _int
+        L.orc_spmm_csr_x86.argtypes = [_i64, _i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int]
+        L.orc_spmm_csr_rowwise.argtypes = [_i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int]
+        L.orc_spmm_dds_x86.argtypes = [_i64, _i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int]
+        L.orc_sddmm_x86.argtypes = [_i64, _i64, _i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int, _int]
+        L.orc_sddmm_multihead.argtypes = [_i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int]
+        L.orc_csr_to_dds.argtypes = [_i64, _i64, _i32p, _i32p, _u32p, _int, _i32p, _i32p, _u32p]
+        L.orc_partition_coo_2d.argtypes = [_i64, _i64, _i64, _i32p, _i32p, _int, _int, _i32p, _i32p, _i32p]
+        _lib = L
+    return _lib
+
+
+def max_threads():
+    return int(lib().orc_max_threads())
+
+
+def _c(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+def _p(a, ptype):
+    return a.ctypes.data_as(ptype)
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise RuntimeError("oracle %s failed with code %d" % (what, rc))
+
+
+def spmm_csr_x86(indptr, indices, vals, x, num_feat_partitions=1, nthreads=1):
+    """python/featgraph/op/vanilla_spmm.py:6-62 + schedule :65-80."""
+    indptr = _c(indptr, np.int32); indices = _c(indices, np.int32)
+    vals = _c(vals, np.float32); x = _c(x, np.float32)
+    n_dst = indptr.shape[0] - 1
+    n_src, F = x.shape
+    out = np.empty((n_dst, F), dtype=np.float32)
+    _check(lib().orc_spmm_csr_x86(n_dst, n_src, F, _p(indptr, _i32p), _p(indices, _i32p),
+                                  _p(vals, _f32p), _p(x, _f32p), _p(out, _f32p),
+                                  num_feat_partitions, nthreads), "spmm_csr_x86")
+    return out
+
+
+def spmm_csr_rowwise(indptr, indices, vals, x, nthreads=1):
+    """python/featgraph/op/vanilla_spmm.py:83-125 (math of the CUDA compute)."""
+    indptr = _c(indptr, np.int32); indices = _c(indices, np.int32)
+    vals = _c(vals, np.float32); x = _c(x, np.float32)
+    n_dst = indptr.shape[0] - 1
+    F = x.shape[1]
+    out = np.empty((n_dst, F), dtype=np.float32)
+    _check(lib().orc_spmm_csr_rowwise(n_dst, F, _p(indptr, _i32p), _p(indices, _i32p),
+                                      _p(vals, _f32p), _p(x, _f32p), _p(out, _f32p), nthreads),
+           "spmm_csr_rowwise")
+    return out
+
+
+def spmm_dds_x86(s1_pos, s1_idx, vals, x, n_dst, num_col_partitions,
+                 num_feat_partitions=1, nthreads=1):
+    """python/featgraph/op/vanilla_spmm.py:149-224 + schedule :227-246."""
+    s1_pos = _c(s1_pos, np.int32); s1_idx = _c(s1_idx, np.int32)
+    vals = _c(vals, np.float32); x = _c(x, np.float32)
+    n_src, F = x.shape
+    assert s1_pos.shape[0] == num_col_partitions * (n_dst + 1)
+    out = np.empty((n_dst, F), dtype=np.float32)
+    _check(lib().orc_spmm_dds_x86(n_dst, n_src, F, num_col_partitions, _p(s1_pos, _i32p),
+                                  _p(s1_idx, _i32p), _p(vals, _f32p), _p(x, _f32p),
+                                  _p(out, _f32p), num_feat_partitions, nthreads), "spmm_dds_x86")
+    return out
+
+
+def sddmm_x86(row, col, src, dst, num_feat_partitions=1, parallel_edges=False, nthreads=1):
+    """python/featgraph/op/vanilla_sddmm.py:6-63 + schedule :66-74.
+
+    ``src`` is gathered with ``col`` and ``dst`` with ``row`` (:47)."""
+    row = _c(row, np.int32); col = _c(col, np.int32)
+    src = _c(src, np.float32); dst = _c(dst, np.float32)
+    E = row.shape[0]
+    F = src.shape[1]
+    assert dst.shape[1] == F and col.shape[0] == E
+    out = np.empty((E,), dtype=np.float32)
+    _check(lib().orc_sddmm_x86(E, src.shape[0], dst.shape[0], F, _p(row, _i32p), _p(col, _i32p),
+                               _p(src, _f32p), _p(dst, _f32p), _p(out, _f32p),
+                               num_feat_partitions, int(bool(parallel_edges)), nthreads), "sddmm_x86")
+    return out
+
+
+def sddmm_multihead(row, col, src, dst, nthreads=1):
+    """Closed form Out[e,h] = <Src[col[e],h,:], Dst[row[e],h,:]>; not in the reference."""
+    row = _c(row, np.int32); col = _c(col, np.int32)
+    src = _c(src, np.float32); dst = _c(dst, np.float32)
+    E = row.shape[0]
+    _, H, D = src.shape
+    assert dst.shape[1:] == (H, D)
+    out = np.empty((E, H), dtype=np.float32)
+    _check(lib().orc_sddmm_multihead(E, H, D, _p(row, _i32p), _p(col, _i32p), _p(src, _f32p),
+                                     _p(dst, _f32p), _p(out, _f32p), nthreads), "sddmm_multihead")
+    return out
+
+
+def csr_to_dds(adj_csr, num_col_partitions):
+    """python/featgraph/util/adj_partitioning.py:7-57.  Returns (s1_pos, s1_idx, vals)."""
+    assert adj_csr.format == "csr"
+    n_rows, n_cols = adj_csr.shape
+    indptr = _c(adj_csr.indptr, np.int32); indices = _c(adj_csr.indices, np.int32)
+    data = np.ascontiguousarray(adj_csr.data)
+    assert data.dtype.itemsize == 4, "values are moved as 32-bit words"
+    s1_pos = np.zeros(num_col_partitions * (n_rows + 1), dtype=np.int32)
+    s1_idx = np.zeros(indices.shape, dtype=np.int32)
+    vals = np.zeros(data.shape, dtype=data.dtype)
+    _check(lib().orc_csr_to_dds(n_rows, n_cols, _p(indptr, _i32p), _p(indices, _i32p),
+                                _p(data.view(np.uint32), _u32p), num_col_partitions,
+                                _p(s1_pos, _i32p), _p(s1_idx, _i32p),
+                                _p(vals.view(np.uint32), _u32p)), "csr_to_dds")
+    return s1_pos, s1_idx, vals
+
+
+def partition_coo_2d(adj_coo, num_row_partitions, num_col_partitions):
+    """python/featgraph/util/adj_partitioning.py:60-128.
+
+    Returns (edge_ids 1-based, rows, cols) in partitioned order; does not touch
+    the caller's matrix (the reference overwrites ``.data``, :92)."""
+    assert adj_coo.format == "coo"
+    n_rows, n_cols = adj_coo.shape
+    row = _c(adj_coo.row, np.int32); col = _c(adj_coo.col, np.int32)
+    nnz = row.shape[0]
+    eid = np.zeros(nnz, dtype=np.int32)
+    orow = np.zeros(nnz, dtype=np.int32)
+    ocol = np.zeros(nnz, dtype=np.int32)
+    _check(lib().orc_partition_coo_2d(n_rows, n_cols, nnz, _p(row, _i32p), _p(col, _i32p),
+                                      num_row_partitions, num_col_partitions,
+                                      _p(eid, _i32p), _p(orow, _i32p), _p(ocol, _i32p)),
+           "partition_coo_2d")
+    return eid, orow, ocol
+
+
+# ---- float64 closed forms through library routines ---------------------------------
+
+def spmm_f64(adj_csr, x):
+    """A.dot(X) in float64 -- the reference's own check (tests/test_module_spmm.py:29)
+    at higher precision."""
+    a = scipy.sparse.csr_matrix(adj_csr).astype(np.float64)
+    return np.asarray(a.dot(np.asarray(x, dtype=np.float64)))
+
+
+def sddmm_f64(row, col, src, dst, chunk=1 << 20):
+    """(src[col] * dst[row]).sum(-1) in float64 (tests/test_module_sddmm.py:34-36)."""
+    row = np.asarray(row); col = np.asarray(col)
+    out = np.empty(row.shape[0], dtype=np.float64)
+    for s in range(0, row.shape[0], chunk):
+        e = slice(s, s + chunk)
+        out[e] = np.einsum("ef,ef->e", src[col[e]].astype(np.float64),
+                           dst[row[e]].astype(np.float64))
+    return out
+
+
+def sddmm_multihead_f64(row, col, src, dst, chunk=1 << 18):
+    """einsum('ehd,ehd->eh', src[col], dst[row]) in float64."""
+    row = np.asarray(row); col = np.asarray(col)
+    out = np.empty((row.shape[0], src.shape[1]), dtype=np.float64)
+    for s in range(0, row.shape[0], chunk):
+        e = slice(s, s + chunk)
+        out[e] = np.einsum("ehd,ehd->eh", src[col[e]].astype(np.float64),
+                           dst[row[e]].astype(np.float64))
+    return out

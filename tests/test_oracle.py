@@ -1,0 +1,256 @@
+"""Pins the CPU oracle before anything is compared with it (CPU only).
+
+Each oracle function is checked against something it does not share code with:
+the reference's stored vectors, scipy/numpy library routines (the reference's
+own checks), exact special cases and brute force on tiny inputs.
+"""
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "util_5x5.json")
+
+
+def _golden():
+    with open(GOLDEN) as f:
+        g = json.load(f)
+    coo = sp.coo_matrix((np.array(g["data"], dtype="int32"), (g["row"], g["col"])),
+                        shape=tuple(g["shape"]), dtype="int32")
+    return g, coo
+
+
+def _rand_csr(rng, n_rows, n_cols, density, dtype="float32"):
+    a = sp.random(n_rows, n_cols, density=density, format="csr", random_state=rng,
+                  data_rvs=lambda k: rng.random(k)).astype(dtype)
+    a.sort_indices()
+    return a
+
+
+# ---- partitioners: stored vectors ---------------------------------------------------
+
+def test_dds_golden(oracle):
+    g, coo = _golden()
+    s1_pos, s1_idx, vals = oracle.csr_to_dds(coo.tocsr(), g["dds_num_col_partitions"])
+    assert vals.tolist() == g["dds_vals"]
+    assert s1_idx.tolist() == g["dds_s1_idx"]
+    assert s1_pos.tolist() == g["dds_s1_pos"]
+    assert s1_pos.dtype == np.int32 and s1_idx.dtype == np.int32
+
+
+def test_partition_2d_golden(oracle):
+    g, coo = _golden()
+    data_before = coo.data.copy()
+    eid, row, col = oracle.partition_coo_2d(coo, g["part2d_num_row_partitions"],
+                                            g["part2d_num_col_partitions"])
+    assert eid.tolist() == g["part2d_edge_id_list"]
+    # global ids of the permuted edges are the original edges' ids
+    assert row.tolist() == [g["row"][i - 1] for i in eid]
+    assert col.tolist() == [g["col"][i - 1] for i in eid]
+    assert (coo.data == data_before).all()
+
+
+# ---- partitioners: scipy sub-matrix slicing on random matrices ------------------------
+
+def _dds_by_slicing(a, P):
+    """Column slices through scipy's own sub-matrix routine."""
+    n_rows, n_cols = a.shape
+    c = -(-n_cols // P)
+    pos, idx, vals, counter = [], [], [], 0
+    for p in range(P):
+        sub = a[:, p * c:] if p == P - 1 else a[:, p * c:(p + 1) * c]
+        pos.append(sub.indptr + counter); idx.append(sub.indices); vals.append(sub.data)
+        counter += sub.nnz
+    return np.concatenate(pos), np.concatenate(idx), np.concatenate(vals)
+
+
+@pytest.mark.parametrize("shape,P", [((127, 255), 4), ((127, 255), 1), ((64, 7), 3),
+                                     ((5, 40), 7), ((33, 33), 33), ((9, 4), 6)])
+def test_dds_vs_scipy_slicing(oracle, shape, P):
+    rng = np.random.default_rng(11)
+    a = _rand_csr(rng, shape[0], shape[1], 0.15)
+    s1_pos, s1_idx, vals = oracle.csr_to_dds(a, P)
+    epos, eidx, evals = _dds_by_slicing(a, P)
+    np.testing.assert_array_equal(s1_pos, epos)
+    np.testing.assert_array_equal(s1_idx, eidx)
+    np.testing.assert_array_equal(vals, evals)
+
+
+def _part2d_by_slicing(coo, R, C):
+    n_rows, n_cols = coo.shape
+    ids = sp.coo_matrix((np.arange(1, coo.nnz + 1, dtype="int32"), (coo.row, coo.col)),
+                        shape=coo.shape).tocsr()
+    rp, cp = -(-n_rows // R), -(-n_cols // C)
+    eid, rows, cols = [], [], []
+    for r in range(R):
+        for c in range(C):
+            rs = slice(r * rp, None if r == R - 1 else (r + 1) * rp)
+            cs = slice(c * cp, None if c == C - 1 else (c + 1) * cp)
+            blk = ids[rs, cs].tocoo()
+            eid.append(blk.data); rows.append(blk.row + r * rp); cols.append(blk.col + c * cp)
+    return np.concatenate(eid), np.concatenate(rows), np.concatenate(cols)
+
+
+@pytest.mark.parametrize("shape,R,C", [((127, 255), 4, 4), ((127, 255), 1, 1), ((127, 255), 3, 5),
+                                       ((20, 9), 7, 2), ((6, 6), 6, 6), ((5, 5), 4, 4)])
+def test_partition_2d_vs_scipy_slicing(oracle, shape, R, C):
+    rng = np.random.default_rng(5)
+    coo = _rand_csr(rng, shape[0], shape[1], 0.2).tocoo()
+    perm = rng.permutation(coo.nnz)            # arbitrary stored COO order
+    coo = sp.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+    eid, row, col = oracle.partition_coo_2d(coo, R, C)
+    e2, r2, c2 = _part2d_by_slicing(coo, R, C)
+    np.testing.assert_array_equal(eid, e2)
+    np.testing.assert_array_equal(row, r2)
+    np.testing.assert_array_equal(col, c2)
+    # argsort of the ids is the inverse permutation (module/sddmm.py:49)
+    mapping = np.argsort(eid)
+    np.testing.assert_array_equal(row[mapping], coo.row)
+    np.testing.assert_array_equal(col[mapping], coo.col)
+
+
+def test_partitioners_bruteforce_tiny(oracle):
+    """Every pattern on a 3x3 grid (512 matrices), every partition count up to 4."""
+    cells = [(r, c) for r in range(3) for c in range(3)]
+    for mask in range(1, 512):
+        rc = [cells[i] for i in range(9) if mask >> i & 1]
+        row = np.array([r for r, _ in rc], dtype="int32"); col = np.array([c for _, c in rc], dtype="int32")
+        data = np.arange(1, len(rc) + 1, dtype="int32")
+        coo = sp.coo_matrix((data, (row, col)), shape=(3, 3))
+        csr = coo.tocsr()
+        for P in (1, 2, 3, 4):
+            s1_pos, s1_idx, vals = oracle.csr_to_dds(csr, P)
+            c = -(-3 // P)
+            d2 = 4
+            assert s1_pos[-1] == len(rc)
+            got = set()
+            for p in range(P):
+                pos = s1_pos[p * d2:(p + 1) * d2]
+                assert (np.diff(pos) >= 0).all()
+                for r in range(3):
+                    for e in range(pos[r], pos[r + 1]):
+                        got.add((r, int(s1_idx[e]) + p * c, int(vals[e])))
+            assert got == {(r, c_, int(csr[r, c_])) for r, c_ in rc}
+        for R, C in itertools.product((1, 2, 3), (1, 2, 3)):
+            eid, orow, ocol = oracle.partition_coo_2d(coo, R, C)
+            assert sorted(eid.tolist()) == list(range(1, len(rc) + 1))
+            rp, cp = -(-3 // R), -(-3 // C)
+            keys = [(orow[i] // rp, ocol[i] // cp, orow[i], ocol[i]) for i in range(len(rc))]
+            assert keys == sorted(keys)
+            assert [rc[i - 1] for i in eid] == list(zip(orow.tolist(), ocol.tolist()))
+
+
+def test_partition_2d_rejects_duplicates(oracle):
+    coo = sp.coo_matrix((np.ones(3, dtype="int32"), ([0, 0, 1], [1, 1, 0])), shape=(2, 2))
+    with pytest.raises(RuntimeError):
+        oracle.partition_coo_2d(coo, 2, 2)
+
+
+# ---- SpMM restatements --------------------------------------------------------------
+
+@pytest.mark.parametrize("T,P", [(1, 1), (4, 1), (1, 4), (4, 4), (128, 7)])
+def test_spmm_reference_shape(oracle, T, P):
+    """The reference's case: 127x255, density 0.1, F=128, csr.dot, rtol=atol=1e-4
+    (tests/test_module_spmm.py:16-34, :63)."""
+    rng = np.random.default_rng(0)
+    a = _rand_csr(rng, 127, 255, 0.1)
+    x = rng.random((255, 128)).astype("float32")
+    expect = a.dot(x)
+    if P == 1:
+        out = oracle.spmm_csr_x86(a.indptr, a.indices, a.data, x, T, nthreads=2)
+    else:
+        s1_pos, s1_idx, vals = oracle.csr_to_dds(a, P)
+        out = oracle.spmm_dds_x86(s1_pos, s1_idx, vals, x, 127, P, T, nthreads=2)
+    np.testing.assert_allclose(out, expect, rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(out, oracle.spmm_f64(a, x), rtol=1e-4, atol=1e-5)
+
+
+def test_spmm_bit_invariance_and_special_cases(oracle):
+    rng = np.random.default_rng(1)
+    a = _rand_csr(rng, 200, 150, 0.05).tolil()
+    a[[0, 17, 199], :] = 0                      # rows without any edge
+    a = a.tocsr().astype("float32")
+    a.eliminate_zeros()
+    x = rng.standard_normal((150, 64)).astype("float32")
+    base = oracle.spmm_csr_x86(a.indptr, a.indices, a.data, x, 1)
+    for T in (2, 4, 16, 64):
+        # feature tiling leaves each output element's summation order unchanged
+        assert np.array_equal(base, oracle.spmm_csr_x86(a.indptr, a.indices, a.data, x, T, nthreads=3))
+    assert np.array_equal(base, oracle.spmm_csr_rowwise(a.indptr, a.indices, a.data, x, nthreads=2))
+    # one column partition == CSR
+    s1_pos, s1_idx, vals = oracle.csr_to_dds(a, 1)
+    assert np.array_equal(base, oracle.spmm_dds_x86(s1_pos, s1_idx, vals, x, 200, 1, 4))
+    # empty rows are exact zeros
+    empty = np.diff(a.indptr) == 0
+    assert empty.any() and (base[empty] == 0).all()
+    # identity adjacency copies X bit-exactly; a transposed operand would fail the shape
+    eye = sp.identity(150, dtype="float32", format="csr")
+    assert np.array_equal(oracle.spmm_csr_x86(eye.indptr, eye.indices, eye.data, x, 4), x)
+    # a permutation matrix gathers rows: pins indices[] -> X row (not column) indexing
+    perm = rng.permutation(150)
+    pm = sp.csr_matrix((np.ones(150, "float32"), perm, np.arange(151)), shape=(150, 150))
+    assert np.array_equal(oracle.spmm_csr_rowwise(pm.indptr, pm.indices, pm.data, x), x[perm])
+    # linear in the edge weights
+    twice = oracle.spmm_csr_x86(a.indptr, a.indices, 2 * a.data, x, 1)
+    assert np.array_equal(twice, 2 * base)
+
+
+def test_spmm_rejects_bad_feature_partition(oracle):
+    a = sp.identity(4, dtype="float32", format="csr")
+    with pytest.raises(RuntimeError):
+        oracle.spmm_csr_x86(a.indptr, a.indices, a.data, np.ones((4, 6), "float32"), 4)
+
+
+# ---- SDDMM restatements -------------------------------------------------------------
+
+@pytest.mark.parametrize("T,par", [(1, False), (4, False), (4, True), (128, False)])
+def test_sddmm_reference_shape(oracle, T, par):
+    """127x255, density 0.1, F=128; Src is (num_cols, F) gathered by col, Dst is
+    (num_rows, F) gathered by row (tests/test_module_sddmm.py:18-19, :34-37)."""
+    rng = np.random.default_rng(2)
+    coo = _rand_csr(rng, 127, 255, 0.1).tocoo()
+    src = rng.random((255, 128)).astype("float32")
+    dst = rng.random((127, 128)).astype("float32")
+    expect = (src[coo.col] * dst[coo.row]).sum(axis=-1)
+    out = oracle.sddmm_x86(coo.row, coo.col, src, dst, T, parallel_edges=par, nthreads=3)
+    np.testing.assert_allclose(out, expect, rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(out, oracle.sddmm_f64(coo.row, coo.col, src, dst), rtol=1e-4, atol=1e-5)
+
+
+def test_sddmm_invariants(oracle):
+    rng = np.random.default_rng(3)
+    coo = _rand_csr(rng, 90, 90, 0.1).tocoo()
+    src = rng.standard_normal((90, 32)).astype("float32")
+    dst = rng.standard_normal((90, 32)).astype("float32")
+    base = oracle.sddmm_x86(coo.row, coo.col, src, dst)
+    for T in (2, 8, 32):
+        assert np.array_equal(base, oracle.sddmm_x86(coo.row, coo.col, src, dst, T))
+    assert np.array_equal(base, oracle.sddmm_x86(coo.row, coo.col, src, dst, 1, True, 4))
+    # swapping (Src, col) with (Dst, row) is the same product
+    assert np.array_equal(base, oracle.sddmm_x86(coo.col, coo.row, dst, src))
+    # one-hot operands pick single entries: pins which index gathers which operand
+    n = 6
+    row = np.array([0, 1, 5], "int32"); col = np.array([2, 2, 4], "int32")
+    s = np.zeros((n, n), "float32"); d = np.zeros((n, n), "float32")
+    s[np.arange(n), np.arange(n)] = np.arange(1, n + 1)      # src[c] = (c+1) e_c
+    d[:] = 1.0
+    assert oracle.sddmm_x86(row, col, s, d).tolist() == [3.0, 3.0, 5.0]
+
+
+def test_multihead_closed_form(oracle):
+    rng = np.random.default_rng(4)
+    coo = _rand_csr(rng, 80, 120, 0.1).tocoo()
+    for H, D in ((1, 32), (4, 32), (8, 64), (3, 5)):
+        src = rng.standard_normal((120, H, D)).astype("float32")
+        dst = rng.standard_normal((80, H, D)).astype("float32")
+        out = oracle.sddmm_multihead(coo.row, coo.col, src, dst, nthreads=2)
+        expect = np.einsum("ehd,ehd->eh", src[coo.col].astype("f8"), dst[coo.row].astype("f8"))
+        np.testing.assert_allclose(out, expect, rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(oracle.sddmm_multihead_f64(coo.row, coo.col, src, dst), expect)
+        flat = oracle.sddmm_x86(coo.row, coo.col, src.reshape(120, -1), dst.reshape(80, -1))
+        np.testing.assert_allclose(out.sum(1), flat, rtol=1e-4, atol=1e-4)
+        if H == 1:
+            assert np.array_equal(out[:, 0], flat)
