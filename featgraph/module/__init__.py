@@ -1,0 +1,3 @@
+from featgraph_amd.module import (VanillaSpMMhip, VanillaSpMMx86, VanillaSpMMcuda,
+                                  VanillaSDDMMhip, VanillaSDDMMx86, VanillaSDDMMcuda,
+                                  MultiHeadSDDMMhip, placeholder)

@@ -1,0 +1,60 @@
+// Shared internals of libfeatgraph_hip.so: error reporting and the plan layout.
+#pragma once
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <vector>
+
+#include "../../include/featgraph_hip.h"
+
+namespace fg {
+
+// Records a message for fg_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define FG_HIP_TRY(expr)                                                              \
+    do {                                                                              \
+        hipError_t _e = (expr);                                                       \
+        if (_e != hipSuccess)                                                         \
+            return ::fg::fail(FG_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(_e)); \
+    } while (0)
+
+// One unit of wavefront work: `len` consecutive stored elements starting at `start`,
+// all belonging to output row `row`.  slot < 0: the wavefront owns the whole row
+// segment and writes the row itself.  slot >= 0: the row segment is longer than the
+// split threshold; this piece's sum goes to partial[slot] and a second kernel adds
+// the pieces.
+struct Item {
+    int32_t start;
+    int32_t len;
+    int32_t row;
+    int32_t slot;
+};
+
+// A row segment that was split: pieces partial[slot0 .. slot0 + n_pieces) add up to it.
+struct Fixup {
+    int32_t row;
+    int32_t slot0;
+    int32_t n_pieces;
+    int32_t pad;
+};
+
+}  // namespace fg
+
+struct fg_spmm_plan {
+    int64_t n_dst = 0, n_src = 0, nnz = 0;
+    int num_col_partitions = 1;
+    int split_threshold = 0;
+    int device = 0;
+    // per partition: [item_begin, item_end) and [fixup_begin, fixup_end)
+    std::vector<int64_t> item_off, fixup_off;
+    int64_t n_items = 0, n_fixups = 0, n_slots = 0, max_slots_in_partition = 0;
+    fg::Item *items_dev = nullptr;
+    fg::Fixup *fixups_dev = nullptr;
+    // partial sums of split rows; grown on demand to max_slots_in_partition * F floats
+    mutable float *partial_dev = nullptr;
+    mutable size_t partial_floats = 0;
+    // statistics for fg_spmm_plan_describe
+    int64_t max_len = 0, n_empty = 0, n_split_rows = 0;
+};

@@ -1,0 +1,124 @@
+// Load-balance plan of one adjacency: the list of per-wavefront work items that both the
+// SpMM kernels and the CSR-order SDDMM kernel walk.  Built on the host from the position
+// array, kept on the device.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+#include <string>
+
+#include "fg_common.h"
+
+using fg::fail;
+using fg::Fixup;
+using fg::Item;
+
+namespace {
+constexpr int kDefaultSplit = 1024;   // elements per wavefront piece of a long row
+}
+
+extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_src, int P,
+                                   const fg_plan_opts *opts, fg_spmm_plan **plan_out) {
+    if (!plan_out) return fail(FG_ERR_ARG, "fg_spmm_plan_create: plan_out is null");
+    *plan_out = nullptr;
+    if (!pos || n_dst < 0 || n_src < 0) return fail(FG_ERR_ARG, "fg_spmm_plan_create: bad argument");
+    if (P < 1) return fail(FG_ERR_ARG, "num_col_partitions should be larger than or equal to 1");
+    if (n_dst >= INT32_MAX || n_src >= INT32_MAX) return fail(FG_ERR_SHAPE, "vertex count does not fit int32");
+    int split = (opts && opts->split_threshold > 0) ? opts->split_threshold : kDefaultSplit;
+    const int64_t d2 = n_dst + 1;
+
+    // structure check: one non-decreasing run of positions across all partitions
+    int64_t prev = 0;
+    for (int p = 0; p < P; ++p)
+        for (int64_t r = 0; r <= n_dst; ++r) {
+            const int64_t v = pos[p * d2 + r];
+            if ((p == 0 && r == 0 && v != 0) || v < prev || (r == 0 && v != prev))
+                return fail(FG_ERR_GRAPH, "position array is not a monotone run at partition %d row %lld",
+                            p, (long long)r);
+            prev = v;
+        }
+
+    auto *pl = new fg_spmm_plan();
+    pl->n_dst = n_dst; pl->n_src = n_src; pl->nnz = prev;
+    pl->num_col_partitions = P; pl->split_threshold = split;
+    std::vector<Item> items;
+    std::vector<Fixup> fixups;
+    items.reserve((size_t)(n_dst + n_dst / 8 + 16));
+    pl->item_off.push_back(0);
+    pl->fixup_off.push_back(0);
+    for (int p = 0; p < P; ++p) {
+        int32_t slot = 0;
+        for (int64_t r = 0; r < n_dst; ++r) {
+            const int32_t start = pos[p * d2 + r];
+            const int32_t len = pos[p * d2 + r + 1] - start;
+            pl->max_len = std::max<int64_t>(pl->max_len, len);
+            if (len == 0) {
+                if (p == 0) { items.push_back({start, 0, (int32_t)r, -1}); pl->n_empty++; }
+                continue;                      // later partitions only add: nothing to do
+            }
+            if (len <= split) { items.push_back({start, len, (int32_t)r, -1}); continue; }
+            const int32_t pieces = (len + split - 1) / split;
+            // equal pieces, rounded up to whole 64-element staging rounds
+            const int32_t piece_len = (((len + pieces - 1) / pieces) + 63) / 64 * 64;
+            int32_t made = 0;
+            for (int32_t s = 0; s < len; s += piece_len, ++made)
+                items.push_back({start + s, std::min(piece_len, len - s), (int32_t)r, slot + made});
+            fixups.push_back({(int32_t)r, slot, made, 0});
+            slot += made;
+            pl->n_split_rows++;
+        }
+        pl->item_off.push_back((int64_t)items.size());
+        pl->fixup_off.push_back((int64_t)fixups.size());
+        pl->n_slots += slot;
+        pl->max_slots_in_partition = std::max<int64_t>(pl->max_slots_in_partition, slot);
+    }
+    pl->n_items = (int64_t)items.size();
+    pl->n_fixups = (int64_t)fixups.size();
+
+    hipError_t e = hipGetDevice(&pl->device);
+    if (e == hipSuccess && pl->n_items) e = hipMalloc((void **)&pl->items_dev, sizeof(Item) * items.size());
+    if (e == hipSuccess && pl->n_items)
+        e = hipMemcpy(pl->items_dev, items.data(), sizeof(Item) * items.size(), hipMemcpyHostToDevice);
+    if (e == hipSuccess && pl->n_fixups) e = hipMalloc((void **)&pl->fixups_dev, sizeof(Fixup) * fixups.size());
+    if (e == hipSuccess && pl->n_fixups)
+        e = hipMemcpy(pl->fixups_dev, fixups.data(), sizeof(Fixup) * fixups.size(), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        fg_spmm_plan_destroy(pl);
+        return fail(FG_ERR_HIP, "fg_spmm_plan_create: %s", hipGetErrorString(e));
+    }
+    *plan_out = pl;
+    return FG_OK;
+}
+
+extern "C" void fg_spmm_plan_destroy(fg_spmm_plan *pl) {
+    if (!pl) return;
+    if (pl->items_dev) (void)hipFree(pl->items_dev);
+    if (pl->fixups_dev) (void)hipFree(pl->fixups_dev);
+    if (pl->partial_dev) (void)hipFree(pl->partial_dev);
+    delete pl;
+}
+
+namespace fg {
+// Declared in fg_spmm.hip: text of the launch the SpMM entry points would use.
+std::string spmm_launch_text(const fg_spmm_plan *plan, int F, int num_feat_partitions);
+}
+
+extern "C" int fg_spmm_plan_describe(const fg_spmm_plan *pl, int F, int T, char *buf, size_t buf_len) {
+    if (!pl || !buf || buf_len == 0) return fail(FG_ERR_ARG, "fg_spmm_plan_describe: bad argument");
+    char head[640];
+    snprintf(head, sizeof(head),
+             "featgraph-hip plan (gfx950)\n"
+             "  adjacency        : %lld dst x %lld src, nnz %lld, %d source-column partition(s)\n"
+             "  work items       : %lld (one wavefront each; 4 per workgroup)\n"
+             "  split threshold  : %d elements; %lld row segment(s) split into %lld piece(s)\n"
+             "  longest segment  : %lld elements; %lld empty row(s)\n",
+             (long long)pl->n_dst, (long long)pl->n_src, (long long)pl->nnz, pl->num_col_partitions,
+             (long long)pl->n_items, pl->split_threshold, (long long)pl->n_split_rows,
+             (long long)pl->n_slots, (long long)pl->max_len, (long long)pl->n_empty);
+    std::string s = head;
+    if (F > 0) s += fg::spmm_launch_text(pl, F, T);
+    const size_t n = std::min(s.size(), buf_len - 1);
+    memcpy(buf, s.data(), n);
+    buf[n] = 0;
+    return (int)n;
+}

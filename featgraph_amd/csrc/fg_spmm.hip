@@ -1,0 +1,327 @@
+// CSR / DDS SpMM for gfx950: out[v, :] = sum_e vals[e] * X[indices[e], :].
+//
+// One wavefront per plan item (a short row, or a piece of a long row).  The feature axis is
+// spread over lanes in vectors of V floats: a group of L lanes covers V*L*K consecutive
+// floats of one source row with K coalesced vector loads, and the 64/L groups of the
+// wavefront take different elements of the row at the same time.  Column ids and weights
+// are staged 64 at a time in LDS by one coalesced load per array and read back as
+// broadcasts, so no lane re-reads them from global memory.  Wide rows are cut into feature
+// tiles; the tile index is the fastest-varying part of the workgroup id, so consecutive
+// workgroups (which the dispatcher deals round-robin to the 8 XCDs) work on the same
+// elements but different feature tiles, and every XCD's L2 holds only its tiles' slice of X.
+#include <hip/hip_runtime.h>
+
+#include <string>
+
+#include "fg_common.h"
+
+using fg::fail;
+using fg::Fixup;
+using fg::Item;
+
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = 64 * kWavesPerBlock;
+
+template <int V> struct Vec;
+template <> struct Vec<4> { using type = float4; };
+template <> struct Vec<1> { using type = float; };
+
+__device__ __forceinline__ float4 vzero(float4) { return make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ __forceinline__ float vzero(float) { return 0.f; }
+__device__ __forceinline__ void vfma(float4 &a, float w, const float4 &x) {
+    a.x += w * x.x; a.y += w * x.y; a.z += w * x.z; a.w += w * x.w;
+}
+__device__ __forceinline__ void vfma(float &a, float w, const float &x) { a += w * x; }
+__device__ __forceinline__ void vadd(float4 &a, const float4 &b) { a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w; }
+__device__ __forceinline__ void vadd(float &a, const float &b) { a += b; }
+__device__ __forceinline__ float4 vshfl_xor(const float4 &a, int off) {
+    return make_float4(__shfl_xor(a.x, off), __shfl_xor(a.y, off), __shfl_xor(a.z, off), __shfl_xor(a.w, off));
+}
+__device__ __forceinline__ float vshfl_xor(const float &a, int off) { return __shfl_xor(a, off); }
+
+// Orders this wavefront's LDS writes before its later LDS reads (and the reverse); the
+// staging buffers are private to one wavefront, so no workgroup barrier is involved.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+struct SpmmArgs {
+    const Item *items;
+    int64_t n_items;
+    const int32_t *indices;
+    const float *vals;
+    const float *x;        // already offset to the partition's first source row
+    float *out;
+    float *partial;
+    int F;                 // row stride of x / out in floats
+    int tile_w;            // floats per requested feature tile (F / num_feat_partitions)
+    int sub_per_tile;      // kernel tiles (V*L*K floats each) per requested tile
+    int n_ftiles;          // num_feat_partitions * sub_per_tile
+    int accumulate;        // add to out instead of overwriting it
+};
+
+// V: floats per lane per load; L: lanes per source row; K: loads per lane per source row;
+// FULL: every lane's columns are inside the tile (no masking needed).
+template <int V, int L, int K, bool FULL>
+__global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
+    using vec = typename Vec<V>::type;
+    constexpr int G = 64 / L;              // elements processed per step
+    constexpr int FT = V * L * K;          // floats per kernel tile
+    constexpr int U = (K >= 2) ? 4 : 8;    // steps whose loads are issued back to back
+    __shared__ int32_t s_idx[kWavesPerBlock][64];
+    __shared__ float s_val[kWavesPerBlock][64];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int tile = (int)(blockIdx.x % (unsigned)a.n_ftiles);
+    const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_ftiles) * kWavesPerBlock + wave;
+    if (item_id >= a.n_items) return;      // uniform per wavefront; no workgroup barriers below
+    const Item it = a.items[item_id];
+    const int g = lane / L, li = lane % L;
+
+    const int rt = tile / a.sub_per_tile, st = tile % a.sub_per_tile;
+    const int f_end = (rt + 1) * a.tile_w;
+    const int f_lo = rt * a.tile_w + st * FT + li * V;      // first column of this lane, k = 0
+    bool on[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
+
+    vec acc[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
+    const float *xb = a.x + f_lo;
+    const int64_t F = a.F;
+
+    for (int32_t base = 0; base < it.len; base += 64) {
+        const int n = min(64, it.len - base);
+        int32_t ci = 0;
+        float cw = 0.f;
+        if (lane < n) {
+            ci = a.indices[it.start + base + lane];
+            cw = a.vals[it.start + base + lane];
+        }
+        wave_lds_sync();                   // earlier reads of the staging rows are done
+        s_idx[wave][lane] = ci;
+        s_val[wave][lane] = cw;
+        wave_lds_sync();
+
+        const int nfull = n / G;           // steps in which every group has an element
+        int s = 0;
+        for (; s + U <= nfull; s += U) {
+            int32_t c[U];
+            float w[U];
+            vec xv[U][K];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                c[u] = s_idx[wave][(s + u) * G + g];
+                w[u] = s_val[wave][(s + u) * G + g];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    if (on[k]) xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)c[u] * F + k * L * V);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    if (on[k]) vfma(acc[k], w[u], xv[u][k]);
+        }
+        for (; s < nfull; ++s) {
+            const int32_t c = s_idx[wave][s * G + g];
+            const float w = s_val[wave][s * G + g];
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (on[k]) vfma(acc[k], w, *reinterpret_cast<const vec *>(xb + (int64_t)c * F + k * L * V));
+        }
+        if (G > 1 && nfull * G + g < n) {  // last, partly filled step
+            const int32_t c = s_idx[wave][nfull * G + g];
+            const float w = s_val[wave][nfull * G + g];
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (on[k]) vfma(acc[k], w, *reinterpret_cast<const vec *>(xb + (int64_t)c * F + k * L * V));
+        }
+    }
+
+    // add the groups' sums; group 0 ends up with the row's sum
+#pragma unroll
+    for (int off = L; off < 64; off <<= 1)
+#pragma unroll
+        for (int k = 0; k < K; ++k) vadd(acc[k], vshfl_xor(acc[k], off));
+
+    if (g == 0) {
+        float *dst = (it.slot < 0 ? a.out + (int64_t)it.row * F : a.partial + (int64_t)it.slot * F) + f_lo;
+        const bool add = a.accumulate && it.slot < 0;
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            if (on[k]) {
+                vec *p = reinterpret_cast<vec *>(dst + k * L * V);
+                vec r = acc[k];
+                if (add) vadd(r, *p);
+                *p = r;
+            }
+    }
+}
+
+// out[row, :] (+)= sum of the row's pieces, in piece order.  One lane per V columns.
+template <int V>
+__global__ __launch_bounds__(256) void spmm_fixup_kernel(const Fixup *fixups, int64_t n_fixups,
+                                                         const float *partial, float *out, int F,
+                                                         int accumulate) {
+    using vec = typename Vec<V>::type;
+    const int per_row = F / V;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_fixups * per_row) return;
+    const Fixup fx = fixups[t / per_row];
+    const int f = (int)(t % per_row) * V;
+    vec sum = *reinterpret_cast<const vec *>(partial + (int64_t)fx.slot0 * F + f);
+    for (int p = 1; p < fx.n_pieces; ++p)
+        vadd(sum, *reinterpret_cast<const vec *>(partial + (int64_t)(fx.slot0 + p) * F + f));
+    vec *o = reinterpret_cast<vec *>(out + (int64_t)fx.row * F + f);
+    if (accumulate) vadd(sum, *o);
+    *o = sum;
+}
+
+struct SpmmConfig {
+    int V, L, K;
+    int tile_w, sub_per_tile, n_ftiles;
+    bool full;
+};
+
+int pow2_ceil(int v) { int p = 1; while (p < v) p <<= 1; return p; }
+
+// Picks vector width, lanes per row and loads per lane for feature length F cut into T
+// requested tiles (T == 0: one tile).  `aligned16`: x and out are 16-byte aligned.
+int choose_config(int F, int T, bool aligned16, SpmmConfig *c) {
+    if (F < 1) return fail(FG_ERR_SHAPE, "feature length must be positive, got %d", F);
+    if (T < 0) return fail(FG_ERR_ARG, "num_feat_partitions must be >= 0, got %d", T);
+    if (T == 0) T = 1;
+    if (F % T != 0) return fail(FG_ERR_SHAPE, "feature length %d is not divisible by num_feat_partitions %d", F, T);
+    const int Fp = F / T;
+    c->V = (aligned16 && F % 4 == 0 && Fp % 4 == 0) ? 4 : 1;
+    const int lanes = Fp / c->V;
+    if (lanes <= 64) { c->L = pow2_ceil(lanes) < 4 ? 4 : pow2_ceil(lanes); c->K = 1; }
+    else { c->L = 64; c->K = (lanes >= 256 && c->V == 1) ? 4 : 2; }
+    const int ft = c->V * c->L * c->K;
+    c->tile_w = Fp;
+    c->sub_per_tile = (Fp + ft - 1) / ft;
+    c->n_ftiles = T * c->sub_per_tile;
+    c->full = (Fp % ft == 0);
+    return FG_OK;
+}
+
+template <int V, int L, int K>
+void launch_vlk(bool full, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+    if (full) hipLaunchKernelGGL((spmm_items_kernel<V, L, K, true>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, false>), grid, dim3(kBlock), 0, st, a);
+}
+
+template <int V>
+int launch_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+    if (c.K == 1) {
+        switch (c.L) {
+            case 4: launch_vlk<V, 4, 1>(c.full, grid, st, a); return FG_OK;
+            case 8: launch_vlk<V, 8, 1>(c.full, grid, st, a); return FG_OK;
+            case 16: launch_vlk<V, 16, 1>(c.full, grid, st, a); return FG_OK;
+            case 32: launch_vlk<V, 32, 1>(c.full, grid, st, a); return FG_OK;
+            case 64: launch_vlk<V, 64, 1>(c.full, grid, st, a); return FG_OK;
+        }
+    } else if (c.L == 64 && c.K == 2) { launch_vlk<V, 64, 2>(c.full, grid, st, a); return FG_OK; }
+    else if (c.L == 64 && c.K == 4) { launch_vlk<V, 64, 4>(c.full, grid, st, a); return FG_OK; }
+    return fail(FG_ERR_SHAPE, "no SpMM kernel for V=%d L=%d K=%d", V, c.L, c.K);
+}
+
+int ensure_partial(const fg_spmm_plan *pl, int F) {
+    const size_t need = (size_t)pl->max_slots_in_partition * (size_t)F;
+    if (need <= pl->partial_floats) return FG_OK;
+    if (pl->partial_dev) FG_HIP_TRY(hipFree(pl->partial_dev));
+    pl->partial_dev = nullptr; pl->partial_floats = 0;
+    FG_HIP_TRY(hipMalloc((void **)&pl->partial_dev, need * sizeof(float)));
+    pl->partial_floats = need;
+    return FG_OK;
+}
+
+int spmm_run(const fg_spmm_plan *pl, const int32_t *idx, const float *vals, const float *x,
+             float *out, int F, int T, void *stream) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (pl->n_dst == 0) return FG_OK;
+    if (!out || (pl->nnz > 0 && (!idx || !vals || !x))) return fail(FG_ERR_ARG, "null device pointer");
+    const bool aligned16 = (((uintptr_t)x | (uintptr_t)out) & 15) == 0;
+    SpmmConfig c;
+    int rc = choose_config(F, T, aligned16, &c);
+    if (rc != FG_OK) return rc;
+    if ((rc = ensure_partial(pl, F)) != FG_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const int P = pl->num_col_partitions;
+    const int64_t width = (pl->n_src + P - 1) / P;
+    for (int p = 0; p < P; ++p) {
+        const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
+        if (i1 > i0) {
+            SpmmArgs a;
+            a.items = pl->items_dev + i0; a.n_items = i1 - i0;
+            a.indices = idx; a.vals = vals;
+            a.x = x + (int64_t)p * width * F;
+            a.out = out; a.partial = pl->partial_dev;
+            a.F = F; a.tile_w = c.tile_w; a.sub_per_tile = c.sub_per_tile; a.n_ftiles = c.n_ftiles;
+            a.accumulate = p > 0;
+            const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * c.n_ftiles;
+            if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
+            rc = (c.V == 4) ? launch_v<4>(c, dim3((unsigned)blocks), st, a) : launch_v<1>(c, dim3((unsigned)blocks), st, a);
+            if (rc != FG_OK) return rc;
+        }
+        const int64_t x0 = pl->fixup_off[p], x1 = pl->fixup_off[p + 1];
+        if (x1 > x0) {
+            const int fv = (aligned16 && F % 4 == 0) ? 4 : 1;
+            const int64_t threads = (x1 - x0) * (F / fv);
+            const unsigned blocks = (unsigned)((threads + 255) / 256);
+            if (fv == 4)
+                hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, pl->fixups_dev + x0,
+                                   x1 - x0, pl->partial_dev, out, F, (int)(p > 0));
+            else
+                hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, pl->fixups_dev + x0,
+                                   x1 - x0, pl->partial_dev, out, F, (int)(p > 0));
+        }
+    }
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
+}
+
+}  // namespace
+
+namespace fg {
+std::string spmm_launch_text(const fg_spmm_plan *pl, int F, int T) {
+    SpmmConfig c;
+    if (choose_config(F, T, true, &c) != FG_OK) return std::string("  launch           : ") + fg_last_error() + "\n";
+    char b[512];
+    const int64_t per_part = pl->item_off.size() > 1 ? pl->item_off[1] - pl->item_off[0] : 0;
+    snprintf(b, sizeof(b),
+             "  feature length   : %d, %d requested tile(s) of %d, %d kernel tile(s) of %d floats\n"
+             "  kernel           : spmm_items_kernel<V=%d, L=%d, K=%d, FULL=%d>; %d element(s) per step\n"
+             "  launch           : %d pass(es); first pass grid %lld x block %d; fixup rows %lld\n",
+             F, c.n_ftiles / c.sub_per_tile, c.tile_w, c.n_ftiles, c.V * c.L * c.K, c.V, c.L, c.K,
+             (int)c.full, 64 / c.L, pl->num_col_partitions,
+             (long long)(((per_part + kWavesPerBlock - 1) / kWavesPerBlock) * c.n_ftiles), kBlock,
+             (long long)pl->n_fixups);
+    return b;
+}
+}  // namespace fg
+
+extern "C" int fg_spmm_csr_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev,
+                               const int32_t *indices_dev, const float *vals_dev, const float *x_dev,
+                               float *out_dev, int F, int num_feat_partitions, void *stream) {
+    (void)indptr_dev;   // row boundaries live in the plan's items
+    if (plan && plan->num_col_partitions != 1)
+        return fail(FG_ERR_ARG, "fg_spmm_csr_f32 needs a plan with one column partition; use fg_spmm_dds_f32");
+    return spmm_run(plan, indices_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
+}
+
+extern "C" int fg_spmm_dds_f32(const fg_spmm_plan *plan, const int32_t *s1_pos_dev,
+                               const int32_t *s1_idx_dev, const float *vals_dev, const float *x_dev,
+                               float *out_dev, int F, int num_feat_partitions, void *stream) {
+    (void)s1_pos_dev;
+    return spmm_run(plan, s1_idx_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
+}

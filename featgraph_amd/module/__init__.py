@@ -1,0 +1,3 @@
+from .spmm import VanillaSpMMhip, VanillaSpMMx86, VanillaSpMMcuda
+from .sddmm import VanillaSDDMMhip, VanillaSDDMMx86, VanillaSDDMMcuda, MultiHeadSDDMMhip
+from .common import placeholder

@@ -1,0 +1,80 @@
+"""Pieces shared by the SpMM and SDDMM module classes."""
+import numpy as np
+import torch
+
+from .. import _lib
+
+
+class placeholder(object):
+    """Shape/dtype record of a dense input, standing where the reference's callers pass
+    ``te.placeholder(shape)`` to ``build`` (tests/test_module_spmm.py:18-19)."""
+
+    def __init__(self, shape, dtype="float32", name="placeholder"):
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = str(dtype)
+        self.name = name
+        if self.dtype != "float32":
+            raise ValueError("only float32 features are supported, got %s" % self.dtype)
+
+    def __repr__(self):
+        return "placeholder(%s, shape=%s, dtype=%s)" % (self.name, self.shape, self.dtype)
+
+
+def device():
+    """The GPU every module object lives on.  Fails loudly without one: there is no CPU path."""
+    if not torch.cuda.is_available():
+        raise RuntimeError("featgraph_amd needs a ROCm GPU (gfx950); torch.cuda.is_available() is False")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def to_device_i32(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(dev)
+
+
+def to_device_f32(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(dev)
+
+
+def stream_ptr():
+    import ctypes
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def check_inputs(tensors, placeholders, dev):
+    if len(tensors) != len(placeholders):
+        raise ValueError("expected %d input array(s), got %d" % (len(placeholders), len(tensors)))
+    for t, ph in zip(tensors, placeholders):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError("inputs must be torch tensors on the module's device, got %s" % type(t))
+        if t.device != dev:
+            raise ValueError("input is on %s, the module lives on %s" % (t.device, dev))
+        if t.dtype != torch.float32:
+            raise ValueError("input dtype must be float32, got %s" % t.dtype)
+        if tuple(t.shape) != ph.shape:
+            raise ValueError("input shape %s does not match the built shape %s" % (tuple(t.shape), ph.shape))
+        if not t.is_contiguous():
+            raise ValueError("inputs must be contiguous (row-major)")
+
+
+def timed_mean_seconds(fn, num_runs):
+    """Mean seconds of `num_runs` back-to-back launches between two events on the current
+    stream, after one untimed call (the protocol of Module.time_evaluator(number=num_runs)
+    used at python/featgraph/module/spmm.py:179-186, plus a warm-up)."""
+    assert num_runs >= 1
+    fn()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(num_runs):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) * 1e-3 / num_runs
+
+
+def take_args(args, allowed, what):
+    """Mirrors the reference's ``**args`` unpacking: an unknown key is a TypeError."""
+    for k in args:
+        if k not in allowed:
+            raise TypeError("%s got an unexpected keyword argument '%s'" % (what, k))
+    return dict(args)

@@ -1,0 +1,263 @@
+"""SDDMM module classes: the build()/run() surface of the reference's
+python/featgraph/module/sddmm.py, executing hand-written gfx950 kernels."""
+import ctypes
+
+import numpy as np
+import torch
+
+from .. import _lib
+from ..util import util_partition_adj_coo_2d
+from . import common
+
+
+class SDDMMbase(object):
+    """The base class for SDDMM-like computation kernels (python/featgraph/module/sddmm.py:11-165)."""
+
+    def __init__(self, adj_scipy, num_row_partitions=1, num_col_partitions=1):
+        """Doing 2D graph partitioning during init.
+
+        Parameters
+        ----------
+        adj_scipy : scipy.sparse.coo_matrix or scipy.sparse.csr_matrix
+            The input scipy sparse matrix (only its structure is used)
+
+        num_row_partitions : int
+            Number of partitions along the row dimension
+
+        num_col_partitions : int
+            Number of partitions along the col dimension (honoured; the reference overwrites
+            it with num_row_partitions, python/featgraph/module/sddmm.py:37)
+        """
+        if adj_scipy.format != 'coo':
+            adj_scipy_coo = adj_scipy.tocoo()
+        else:
+            adj_scipy_coo = adj_scipy
+        self._num_rows = adj_scipy_coo.shape[0]
+        self._num_cols = adj_scipy_coo.shape[1]
+        assert num_row_partitions >= 1, "num_row_partitions should be larger than or equal to 1"
+        assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
+        self._num_row_partitions = num_row_partitions
+        self._num_col_partitions = num_col_partitions
+        self._target = None
+        self._ctx = None
+        self._register()
+        # 2D graph partitioning
+        if self._num_row_partitions > 1 or self._num_col_partitions > 1:
+            edge_id_list, adj_row_indices, adj_col_indices = self._preprocess_adj(
+                adj_scipy_coo, self._num_row_partitions, self._num_col_partitions)
+            self._edge_mapping = np.argsort(edge_id_list)
+        else:
+            adj_row_indices = np.ascontiguousarray(adj_scipy_coo.row, dtype=np.int32)
+            adj_col_indices = np.ascontiguousarray(adj_scipy_coo.col, dtype=np.int32)
+            self._edge_mapping = None
+        nnz = adj_row_indices.shape[0]
+        if nnz:
+            if adj_row_indices.min() < 0 or adj_row_indices.max() >= self._num_rows or \
+                    adj_col_indices.min() < 0 or adj_col_indices.max() >= self._num_cols:
+                raise ValueError("edge endpoints outside the %d x %d matrix" % (self._num_rows, self._num_cols))
+        self._adj_row_indices = adj_row_indices
+        self._adj_col_indices = adj_col_indices
+        self._adj_row_indices_dev = common.to_device_i32(adj_row_indices, self._ctx)
+        self._adj_col_indices_dev = common.to_device_i32(adj_col_indices, self._ctx)
+        # Stored order with non-decreasing row ids is CSR order: row pieces from the SpMM plan
+        # then replace the per-edge row array and dst rows are fetched once per piece.
+        self._plan = ctypes.c_void_p()
+        self._adj_indptr_dev = None
+        self._row_sorted = bool(nnz == 0 or (np.diff(adj_row_indices) >= 0).all())
+        if self._row_sorted:
+            counts = np.bincount(adj_row_indices, minlength=self._num_rows) if nnz else np.zeros(self._num_rows, np.int64)
+            indptr = np.zeros(self._num_rows + 1, dtype=np.int32)
+            np.cumsum(counts, out=indptr[1:])
+            self._adj_indptr_dev = common.to_device_i32(indptr, self._ctx)
+            with torch.cuda.device(self._ctx):
+                _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(indptr), self._num_rows, self._num_cols,
+                                                          1, None, ctypes.byref(self._plan)))
+        # To be updated in self.build
+        self._func = None
+        self._placeholders = None
+        self._heads = 1
+        self._head_len = None
+        self._use_csr = False
+        self._notes = []
+        self.out_tvm = None
+
+    def __del__(self):
+        plan = getattr(self, "_plan", None)
+        if plan is not None and plan.value:
+            try:
+                _lib.lib().fg_spmm_plan_destroy(plan)
+            except Exception:
+                pass
+            self._plan = None
+
+    def _preprocess_adj(self, adj_scipy_coo, num_row_partitions=1, num_col_partitions=1):
+        return util_partition_adj_coo_2d(adj_scipy_coo, num_row_partitions, num_col_partitions)
+
+    def _register(self):
+        raise NotImplementedError("Please register target and ctx.")
+
+    def _feature_shape(self, src_ph, dst_ph):
+        """(H, D) from the two placeholders; vanilla SDDMM takes 2-D inputs."""
+        if len(src_ph.shape) != 2 or len(dst_ph.shape) != 2:
+            raise ValueError("SrcFeat / DstFeat must be 2-D, got %s and %s" % (src_ph.shape, dst_ph.shape))
+        return 1, src_ph.shape[1]
+
+    def _resolve(self, input_placeholders, compute_args, schedule_args):
+        compute_args = common.take_args(compute_args, self._compute_keys, "compute_func")
+        schedule_args = common.take_args(schedule_args, self._schedule_keys, "schedule_func")
+        if len(input_placeholders) != 2:
+            raise ValueError("SDDMM takes two dense inputs (SrcFeat, DstFeat), got %d" % len(input_placeholders))
+        src_ph, dst_ph = input_placeholders
+        assert src_ph.shape[1:] == dst_ph.shape[1:], "dimension mismatch"
+        if src_ph.shape[0] != self._num_cols or dst_ph.shape[0] != self._num_rows:
+            raise ValueError("SrcFeat must have num_cols=%d rows and DstFeat num_rows=%d rows, got %s and %s"
+                             % (self._num_cols, self._num_rows, src_ph.shape, dst_ph.shape))
+        H, D = self._feature_shape(src_ph, dst_ph)
+        notes = []
+        T = compute_args.get('num_feat_partitions', 1) or 1
+        Ts = schedule_args.get('num_feat_partitions', T) or 1
+        for t in (T, Ts):
+            if t < 1 or (H * D) % t != 0:
+                raise ValueError("feat_len %d is not divisible by num_feat_partitions %d" % (H * D, t))
+        if T != 1 or Ts != 1:
+            notes.append("num_feat_partitions accepted; an edge's dot product is reduced inside one "
+                         "wavefront, so the feature axis is not tiled across workgroups")
+        blocks = schedule_args.get('num_cuda_blocks')
+        if blocks is not None:
+            # same bound as schedule_vanilla_sddmm_cuda_tree_reduce (vanilla_sddmm.py:82-83)
+            assert blocks <= self._adj_row_indices.shape[0], \
+                "num_cuda_blocks must be smaller than num_edges, which is {}.".format(self._adj_row_indices.shape[0])
+            notes.append("num_cuda_blocks has no counterpart: the grid follows the edge count")
+        order = schedule_args.get('order', 'auto')
+        if order not in ('auto', 'csr', 'coo'):
+            raise ValueError("order must be 'auto', 'csr' or 'coo'")
+        if order == 'csr' and not self._row_sorted:
+            raise ValueError("order='csr' needs stored edges with non-decreasing row ids")
+        use_csr = self._row_sorted and order != 'coo'
+        return [src_ph, dst_ph], H, D, use_csr, notes
+
+    def build(self, input_placeholders, compute_args, schedule_args):
+        """Fix the feature shape and kernel variant, allocate the output once.
+
+        Parameters
+        ----------
+        input_placeholders : list of placeholder
+            [SrcFeat (num_cols, feat_len), DstFeat (num_rows, feat_len)]
+
+        compute_args : dict
+            {'num_feat_partitions': T} is accepted (see lower_to_ir for what it maps to)
+
+        schedule_args : dict
+            'num_feat_partitions', 'num_cuda_blocks' (reference keys) and 'order' in
+            {'auto', 'csr', 'coo'}: which kernel walks the stored edges
+        """
+        phs, H, D, use_csr, notes = self._resolve(input_placeholders, compute_args, schedule_args)
+        self._placeholders = phs
+        self._heads, self._head_len, self._use_csr, self._notes = H, D, use_csr, notes
+        self._func = _lib.lib().fg_sddmm_csr_f32 if use_csr else _lib.lib().fg_sddmm_coo_f32
+        nnz = self._adj_row_indices.shape[0]
+        oshape = (nnz,) if self._out_1d else (nnz, H)
+        self.out_tvm = torch.zeros(oshape, dtype=torch.float32, device=self._ctx)
+
+    def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
+        """Return a text description of the launch. This can be useful for debug."""
+        _, H, D, use_csr, notes = self._resolve(input_placeholders, compute_args, schedule_args)
+        nnz = self._adj_row_indices.shape[0]
+        text = "featgraph-hip SDDMM (gfx950)\n"
+        text += "  adjacency        : %d x %d, %d stored edges, %d x %d partition blocks\n" % (
+            self._num_rows, self._num_cols, nnz, self._num_row_partitions, self._num_col_partitions)
+        text += "  features         : %d head(s) x %d floats\n" % (H, D)
+        text += "  kernel           : %s\n" % ("sddmm_csr_kernel over row pieces (dst row held in registers)"
+                                               if use_csr else "sddmm_coo_kernel, 256 stored edges per wavefront")
+        for n in notes:
+            text += "  note             : %s\n" % n
+        return text
+
+    def _launch(self, src_feat, dst_feat):
+        s = common.stream_ptr()
+        if self._use_csr:
+            _lib.check(self._func(self._plan, _lib.dev_ptr(self._adj_indptr_dev), _lib.dev_ptr(self._adj_col_indices_dev),
+                                  _lib.dev_ptr(src_feat), _lib.dev_ptr(dst_feat), _lib.dev_ptr(self.out_tvm),
+                                  self._heads, self._head_len, s))
+        else:
+            _lib.check(self._func(_lib.dev_ptr(self._adj_row_indices_dev), _lib.dev_ptr(self._adj_col_indices_dev),
+                                  self._adj_row_indices.shape[0], _lib.dev_ptr(src_feat), _lib.dev_ptr(dst_feat),
+                                  _lib.dev_ptr(self.out_tvm), self._heads, self._head_len, s))
+
+    def run(self, input_tvm_ndarrays):
+        """Run the built func with the given inputs [SrcFeat, DstFeat] (float32 torch tensors on
+        the module's device).  Returns self.out_tvm, one value per stored edge (and head), in the
+        stored (possibly partitioned) edge order; enqueued on torch's current stream."""
+        if self._func is None:
+            raise RuntimeError("call build() before run()")
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        self._launch(input_tvm_ndarrays[0], input_tvm_ndarrays[1])
+        return self.out_tvm
+
+    def measure_average_time(self, input_tvm_ndarrays, num_runs):
+        """Average run time in seconds over `num_runs` back-to-back launches."""
+        if self._func is None:
+            raise RuntimeError("call build() before measure_average_time()")
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        s, d = input_tvm_ndarrays
+        return common.timed_mean_seconds(lambda: self._launch(s, d), num_runs)
+
+    @property
+    def edge_mapping(self):
+        assert self._target != 'cuda', "no graph partitioning on cuda, no edge_mapping"
+        assert self._num_row_partitions > 1 or self._num_col_partitions > 1, \
+            "no graph partitioning, no edge_mapping"
+        return self._edge_mapping
+
+    @property
+    def ctx(self):
+        return self._ctx
+
+    @property
+    def target(self):
+        return self._target
+
+
+class VanillaSDDMMhip(SDDMMbase):
+    """Edge-wise dot product on gfx950, optionally over a 2-D partitioned edge order."""
+    _compute_keys = ('num_feat_partitions',)
+    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order')
+    _out_1d = True
+
+    def __init__(self, adj_scipy, num_row_partitions=1, num_col_partitions=1):
+        super(VanillaSDDMMhip, self).__init__(adj_scipy, num_row_partitions, num_col_partitions)
+
+    def _register(self):
+        self._target = 'rocm'
+        self._ctx = common.device()
+
+
+class VanillaSDDMMx86(VanillaSDDMMhip):
+    """Constructor and knobs of the reference's VanillaSDDMMx86
+    (python/featgraph/module/sddmm.py:168-176); the partitioned traversal runs on the GPU."""
+    _schedule_keys = ('num_feat_partitions', 'order')
+
+
+class VanillaSDDMMcuda(VanillaSDDMMhip):
+    """Constructor and knobs of the reference's VanillaSDDMMcuda
+    (python/featgraph/module/sddmm.py:179-187): no partitioning, hence no edge_mapping."""
+    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order')
+
+    def __init__(self, adj_scipy):
+        super(VanillaSDDMMcuda, self).__init__(adj_scipy, num_row_partitions=1, num_col_partitions=1)
+
+    @property
+    def edge_mapping(self):
+        raise AssertionError("no graph partitioning on cuda, no edge_mapping")
+
+
+class MultiHeadSDDMMhip(VanillaSDDMMhip):
+    """Per-edge, per-head dot products: SrcFeat (num_cols, H, D), DstFeat (num_rows, H, D),
+    output (num_edges, H).  Not present in the reference; H == 1 equals VanillaSDDMM."""
+    _out_1d = False
+
+    def _feature_shape(self, src_ph, dst_ph):
+        if len(src_ph.shape) != 3 or len(dst_ph.shape) != 3:
+            raise ValueError("multi-head SrcFeat / DstFeat must be 3-D [n, H, D], got %s and %s"
+                             % (src_ph.shape, dst_ph.shape))
+        return src_ph.shape[1], src_ph.shape[2]

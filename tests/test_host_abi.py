@@ -1,0 +1,152 @@
+"""CPU-only tests of the shipped library's host side: the C ABI loads and exports what the
+header declares, the host partitioners are bit-exact with the oracle and the reference's
+stored vectors, structural checks reject bad graphs, the generator is deterministic, and the
+operator classes refuse to run without a GPU instead of falling back."""
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def fg():
+    from featgraph_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from featgraph_amd import build
+        build.build(verbose=False)
+    _lib.lib()
+    return _lib
+
+
+def test_header_symbols_exported(fg):
+    text = open(os.path.join(ROOT, "include", "featgraph_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(fg_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(fg.SIGNATURES), declared ^ set(fg.SIGNATURES)
+    for name in declared:
+        assert hasattr(fg.lib(), name), name
+    assert fg.lib().fg_version() >= 100
+
+
+def test_golden_vectors(fg):
+    from featgraph.util import util_convert_csr_to_dds, util_partition_adj_coo_2d
+    g = json.load(open(os.path.join(ROOT, "tests", "golden", "util_5x5.json")))
+    coo = sp.coo_matrix((np.array(g["data"], dtype="int32"), (g["row"], g["col"])), shape=(5, 5), dtype="int32")
+    s1_pos, s1_idx, vals = util_convert_csr_to_dds(coo.tocsr(), g["dds_num_col_partitions"])
+    assert vals.tolist() == g["dds_vals"]
+    assert s1_idx.tolist() == g["dds_s1_idx"]
+    assert s1_pos.tolist() == g["dds_s1_pos"]
+    before = coo.data.copy()
+    eid, row, col = util_partition_adj_coo_2d(coo, 2, 2)
+    assert eid.tolist() == g["part2d_edge_id_list"]
+    assert (coo.data == before).all()
+    assert eid.dtype == np.int32 and row.dtype == np.int32 and col.dtype == np.int32
+
+
+@pytest.mark.parametrize("shape,density", [((127, 255), 0.1), ((1000, 40), 0.3), ((3, 5000), 0.05), ((64, 64), 1.0)])
+def test_partitioners_match_oracle(fg, oracle, shape, density):
+    from featgraph_amd.util import util_convert_csr_to_dds, util_partition_adj_coo_2d
+    rng = np.random.default_rng(shape[0])
+    a = sp.random(shape[0], shape[1], density=density, format="csr", random_state=rng).astype("float32")
+    a.sort_indices()
+    for P in (1, 2, 4, 7, 32, shape[1], shape[1] + 3):
+        for x, y in zip(util_convert_csr_to_dds(a, P), oracle.csr_to_dds(a, P)):
+            assert x.dtype == y.dtype and np.array_equal(x, y)
+    coo = a.tocoo()
+    perm = rng.permutation(coo.nnz)
+    coo = sp.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+    for R, C in ((1, 1), (2, 3), (4, 4), (32, 1), (1, 32), (shape[0], shape[1]), (shape[0] + 2, 5)):
+        for x, y in zip(util_partition_adj_coo_2d(coo, R, C), oracle.partition_coo_2d(coo, R, C)):
+            assert x.dtype == y.dtype and np.array_equal(x, y)
+
+
+def test_partitioner_edge_cases(fg):
+    from featgraph_amd.util import util_convert_csr_to_dds, util_partition_adj_coo_2d
+    empty = sp.csr_matrix((4, 6), dtype="float32")
+    s1_pos, s1_idx, vals = util_convert_csr_to_dds(empty, 3)
+    assert s1_pos.tolist() == [0] * 15 and len(s1_idx) == 0 and len(vals) == 0
+    eid, r, c = util_partition_adj_coo_2d(empty.tocoo(), 2, 2)
+    assert len(eid) == 0
+    with pytest.raises(AssertionError):
+        util_convert_csr_to_dds(empty, 0)
+    with pytest.raises(AssertionError):
+        util_partition_adj_coo_2d(empty.tocoo(), 1, 0)
+    dup = sp.coo_matrix((np.ones(3, "int32"), ([0, 0, 1], [1, 1, 0])), shape=(2, 2))
+    with pytest.raises(ValueError):
+        util_partition_adj_coo_2d(dup, 2, 2)
+    f64 = sp.identity(3, dtype="float64", format="csr")
+    with pytest.raises(ValueError):
+        util_convert_csr_to_dds(f64, 2)
+    # unsorted column ids inside a row keep their stored order within each partition
+    uns = sp.csr_matrix((np.array([1, 2, 3, 4], "float32"), np.array([3, 0, 2, 1], "int32"), np.array([0, 4], "int32")),
+                        shape=(1, 4))
+    s1_pos, s1_idx, vals = util_convert_csr_to_dds(uns, 2)
+    assert s1_pos.tolist() == [0, 2, 2, 4] and s1_idx.tolist() == [0, 1, 1, 0] and vals.tolist() == [2, 4, 1, 3]
+
+
+def test_check_csr_host(fg):
+    L = fg.lib()
+    ok_ptr = np.array([0, 2, 2, 3], dtype=np.int32)
+    ok_idx = np.array([0, 4, 1], dtype=np.int32)
+    assert L.fg_check_csr_host(3, 5, fg.host_ptr(ok_ptr), fg.host_ptr(ok_idx)) == 0
+    assert L.fg_check_csr_host(3, 4, fg.host_ptr(ok_ptr), fg.host_ptr(ok_idx)) == -3
+    assert "outside" in fg.last_error()
+    bad = np.array([0, 2, 1, 3], dtype=np.int32)
+    assert L.fg_check_csr_host(3, 5, fg.host_ptr(bad), fg.host_ptr(ok_idx)) == -3
+    bad0 = np.array([1, 2, 2, 3], dtype=np.int32)
+    assert L.fg_check_csr_host(3, 5, fg.host_ptr(bad0), fg.host_ptr(ok_idx)) == -3
+    assert L.fg_check_csr_host(3, 5, None, None) == -1
+    with pytest.raises(ValueError):
+        fg.check(-3)
+
+
+def test_synthetic_graphs(fg):
+    from featgraph_amd import synthetic
+    a = synthetic.make_workload("powerlaw-23k", num_threads=1)
+    b = synthetic.make_workload("powerlaw-23k", num_threads=5)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    indptr, indices = a
+    n = indptr.shape[0] - 1
+    deg = np.diff(indptr)
+    rows = np.repeat(np.arange(n), deg)
+    keys = rows.astype(np.int64) * n + indices
+    assert (np.diff(keys) > 0).all()                      # sorted, no duplicates
+    assert indices.min() >= 0 and indices.max() < n
+    loops = np.zeros(n, bool); loops[rows[rows == indices]] = True
+    assert loops.all()
+    assert 1_000_000 < indptr[-1] < 1_200_000 and deg.max() > 1000
+    # fixed checksum: the graph is the same on every host
+    assert int(indices.astype(np.int64).sum() % 1000003) == int(b[1].astype(np.int64).sum() % 1000003)
+    c = synthetic.make_workload("powerlaw-23k", seed=7)
+    assert not np.array_equal(c[1][:1000], indices[:1000])
+    u_ptr, u_idx = synthetic.make_workload("uniform-10k")
+    assert u_ptr.shape[0] == 10001 and 160000 <= u_ptr[-1] <= 170000
+    w = synthetic.edge_weights(1000, 1)
+    assert w.dtype == np.float32 and 0 <= w.min() and w.max() < 1 and abs(w.mean() - 0.5) < 0.05
+
+
+def test_no_cpu_fallback(fg):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("this check is for hosts without a GPU")
+    from featgraph.module import VanillaSpMMx86, VanillaSDDMMx86
+    adj = sp.identity(4, dtype="float32", format="csr")
+    with pytest.raises(RuntimeError, match="GPU"):
+        VanillaSpMMx86(adj)
+    with pytest.raises(RuntimeError, match="GPU"):
+        VanillaSDDMMx86(adj)
+
+
+def test_product_does_not_import_oracle():
+    """The shipped package must not reach the CPU oracle in any way."""
+    pkg = os.path.join(ROOT, "featgraph_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cpp", ".h")):
+                text = open(os.path.join(base, f)).read()
+                assert "oracle" not in text, os.path.join(base, f)
