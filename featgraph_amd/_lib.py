@@ -21,7 +21,8 @@ _int = ctypes.c_int
 
 
 class FgPlanOpts(ctypes.Structure):
-    _fields_ = [("split_threshold", ctypes.c_int32), ("reserved", ctypes.c_int32 * 7)]
+    _fields_ = [("split_threshold", ctypes.c_int32), ("item_edges", ctypes.c_int32),
+                ("reserved", ctypes.c_int32 * 6)]
 
 
 # name -> (restype, argtypes); also the list of symbols the header declares

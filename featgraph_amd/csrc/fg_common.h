@@ -20,17 +20,21 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
             return ::fg::fail(FG_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(_e)); \
     } while (0)
 
-// One unit of wavefront work: `len` consecutive stored elements starting at `start`,
-// all belonging to output row `row`.  slot < 0: the wavefront owns the whole row
-// segment and writes the row itself.  slot >= 0: the row segment is longer than the
-// split threshold; this piece's sum goes to partial[slot] and a second kernel adds
-// the pieces.
+// One unit of wavefront work: `len` consecutive stored elements starting at `start`.
+//   info >= 0 : a piece of a row segment longer than the split threshold; all elements belong
+//               to output row `row`, the piece's sum goes to partial[info] and a second kernel
+//               adds the pieces.
+//   info <  0 : -info whole consecutive row segments, rows [row, row - info); the wavefront
+//               writes those rows itself.  Row boundaries come from the position array.
 struct Item {
     int32_t start;
     int32_t len;
     int32_t row;
-    int32_t slot;
+    int32_t info;
 };
+
+constexpr int kItemEdges = 256;   // elements staged in LDS per wavefront at a time
+constexpr int kItemRows = 64;     // most rows one multi-row item may hold
 
 // A row segment that was split: pieces partial[slot0 .. slot0 + n_pieces) add up to it.
 struct Fixup {
@@ -46,6 +50,7 @@ struct fg_spmm_plan {
     int64_t n_dst = 0, n_src = 0, nnz = 0;
     int num_col_partitions = 1;
     int split_threshold = 0;
+    int item_edges = 0;              // element budget of a multi-row item
     int device = 0;
     // per partition: [item_begin, item_end) and [fixup_begin, fixup_end)
     std::vector<int64_t> item_off, fixup_off;
@@ -56,5 +61,5 @@ struct fg_spmm_plan {
     mutable float *partial_dev = nullptr;
     mutable size_t partial_floats = 0;
     // statistics for fg_spmm_plan_describe
-    int64_t max_len = 0, n_empty = 0, n_split_rows = 0;
+    int64_t max_len = 0, n_empty = 0, n_split_rows = 0, n_multi_items = 0;
 };

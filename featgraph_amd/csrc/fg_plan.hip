@@ -25,6 +25,9 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
     if (P < 1) return fail(FG_ERR_ARG, "num_col_partitions should be larger than or equal to 1");
     if (n_dst >= INT32_MAX || n_src >= INT32_MAX) return fail(FG_ERR_SHAPE, "vertex count does not fit int32");
     int split = (opts && opts->split_threshold > 0) ? opts->split_threshold : kDefaultSplit;
+    int item_edges = (opts && opts->item_edges > 0) ? opts->item_edges : fg::kItemEdges;
+    if (item_edges > fg::kItemEdges) item_edges = fg::kItemEdges;
+    if (item_edges > split) item_edges = split;
     const int64_t d2 = n_dst + 1;
 
     // structure check: one non-decreasing run of positions across all partitions
@@ -40,7 +43,7 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
 
     auto *pl = new fg_spmm_plan();
     pl->n_dst = n_dst; pl->n_src = n_src; pl->nnz = prev;
-    pl->num_col_partitions = P; pl->split_threshold = split;
+    pl->num_col_partitions = P; pl->split_threshold = split; pl->item_edges = item_edges;
     std::vector<Item> items;
     std::vector<Fixup> fixups;
     items.reserve((size_t)(n_dst + n_dst / 8 + 16));
@@ -48,24 +51,49 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
     pl->fixup_off.push_back(0);
     for (int p = 0; p < P; ++p) {
         int32_t slot = 0;
-        for (int64_t r = 0; r < n_dst; ++r) {
-            const int32_t start = pos[p * d2 + r];
-            const int32_t len = pos[p * d2 + r + 1] - start;
+        const int32_t *pp = pos + p * d2;
+        int64_t r = 0;
+        while (r < n_dst) {
+            const int32_t start = pp[r];
+            const int32_t len = pp[r + 1] - start;
             pl->max_len = std::max<int64_t>(pl->max_len, len);
-            if (len == 0) {
-                if (p == 0) { items.push_back({start, 0, (int32_t)r, -1}); pl->n_empty++; }
-                continue;                      // later partitions only add: nothing to do
+            if (len > split) {
+                const int32_t pieces = (len + split - 1) / split;
+                // equal pieces, rounded up to whole 64-element staging rounds
+                const int32_t piece_len = (((len + pieces - 1) / pieces) + 63) / 64 * 64;
+                int32_t made = 0;
+                for (int32_t s = 0; s < len; s += piece_len, ++made)
+                    items.push_back({start + s, std::min(piece_len, len - s), (int32_t)r, slot + made});
+                fixups.push_back({(int32_t)r, slot, made, 0});
+                slot += made;
+                pl->n_split_rows++;
+                ++r;
+                continue;
             }
-            if (len <= split) { items.push_back({start, len, (int32_t)r, -1}); continue; }
-            const int32_t pieces = (len + split - 1) / split;
-            // equal pieces, rounded up to whole 64-element staging rounds
-            const int32_t piece_len = (((len + pieces - 1) / pieces) + 63) / 64 * 64;
-            int32_t made = 0;
-            for (int32_t s = 0; s < len; s += piece_len, ++made)
-                items.push_back({start + s, std::min(piece_len, len - s), (int32_t)r, slot + made});
-            fixups.push_back({(int32_t)r, slot, made, 0});
-            slot += made;
-            pl->n_split_rows++;
+            if (len > item_edges) {            // one whole row, too long to share an item
+                items.push_back({start, len, (int32_t)r, -1});
+                ++r;
+                continue;
+            }
+            // a run of short rows: at most item_edges elements and kItemRows rows
+            const int64_t r0 = r;
+            int32_t total = 0;
+            while (r < n_dst && r - r0 < fg::kItemRows) {
+                const int32_t l = pp[r + 1] - pp[r];
+                if (l > item_edges || total + l > item_edges) break;
+                if (l == 0 && p == 0) pl->n_empty++;
+                pl->max_len = std::max<int64_t>(pl->max_len, l);
+                total += l;
+                ++r;
+            }
+            if (r == r0) {                      // item_edges < 1 row: cannot happen, len <= item_edges
+                items.push_back({start, len, (int32_t)r, -1});
+                ++r;
+                continue;
+            }
+            if (total == 0 && p > 0) continue;  // later partitions only add: nothing to do
+            items.push_back({start, total, (int32_t)r0, -(int32_t)(r - r0)});
+            if (r - r0 > 1) pl->n_multi_items++;
         }
         pl->item_off.push_back((int64_t)items.size());
         pl->fixup_off.push_back((int64_t)fixups.size());
@@ -105,15 +133,15 @@ std::string spmm_launch_text(const fg_spmm_plan *plan, int F, int num_feat_parti
 
 extern "C" int fg_spmm_plan_describe(const fg_spmm_plan *pl, int F, int T, char *buf, size_t buf_len) {
     if (!pl || !buf || buf_len == 0) return fail(FG_ERR_ARG, "fg_spmm_plan_describe: bad argument");
-    char head[640];
+    char head[800];
     snprintf(head, sizeof(head),
              "featgraph-hip plan (gfx950)\n"
              "  adjacency        : %lld dst x %lld src, nnz %lld, %d source-column partition(s)\n"
-             "  work items       : %lld (one wavefront each; 4 per workgroup)\n"
+             "  work items       : %lld (one wavefront each; 4 per workgroup), %lld hold several rows (<= %d elements)\n"
              "  split threshold  : %d elements; %lld row segment(s) split into %lld piece(s)\n"
              "  longest segment  : %lld elements; %lld empty row(s)\n",
              (long long)pl->n_dst, (long long)pl->n_src, (long long)pl->nnz, pl->num_col_partitions,
-             (long long)pl->n_items, pl->split_threshold, (long long)pl->n_split_rows,
+             (long long)pl->n_items, (long long)pl->n_multi_items, pl->item_edges, pl->split_threshold, (long long)pl->n_split_rows,
              (long long)pl->n_slots, (long long)pl->max_len, (long long)pl->n_empty);
     std::string s = head;
     if (F > 0) s += fg::spmm_launch_text(pl, F, T);

@@ -4,10 +4,10 @@
 // Edge-parallel: a wavefront owns a run of consecutive stored edges.  A group of L lanes
 // covers one edge's F = H*D floats with K vector loads per operand, the 64/L groups work on
 // different edges at once, and each head's products are added across its lanes with a
-// butterfly of cross-lane shuffles.  Row/column ids are staged 64 at a time in LDS, results
-// are collected in LDS and written back as one coalesced run per 64 edges.  When the stored
-// order keeps equal row ids together (CSR order, 2-D partitioned order) the dst row already
-// held in registers is reused instead of fetched again.
+// butterfly of cross-lane shuffles.  Row/column ids are staged in LDS (up to 256 edges per
+// wavefront), results are collected in registers and written back as dense runs.  When the
+// stored order keeps equal row ids together (CSR order, 2-D partitioned order) the dst row
+// already held in registers is reused instead of fetched again.
 #include <hip/hip_runtime.h>
 
 #include "fg_common.h"
@@ -20,7 +20,7 @@ namespace {
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = 64 * kWavesPerBlock;
 constexpr int kEdgesPerWave = 256;       // COO kernel: stored edges per wavefront
-constexpr int kMaxHeadsFast = 16;        // LDS result staging holds 64 * H floats per wavefront
+constexpr int kMaxHeadsFast = 16;        // most heads the lane layouts below cover (4 loads x 4 heads)
 
 template <int V> struct Vec;
 template <> struct Vec<4> { using type = float4; };
@@ -49,8 +49,9 @@ __device__ __forceinline__ float segment_sum(float v) {
 struct SddmmArgs {
     const int32_t *row;     // COO kernel: row id per stored edge
     const int32_t *col;     // column id per stored edge
-    const Item *items;      // CSR kernel: row pieces
+    const Item *items;      // CSR kernel: plan items
     int64_t n_items;
+    const int32_t *pos;     // CSR kernel: row boundaries (indptr)
     int64_t n_edges;
     const float *src;       // gathered by col
     const float *dst;       // gathered by row
@@ -85,91 +86,106 @@ __device__ __forceinline__ void edge_heads(const typename Vec<V>::type (&s)[K], 
     }
 }
 
-// Stored-order (COO) kernel.
+// Dot products of the staged edges [0, n) of `edge` (x = column id, y = row id); results go to
+// out[j * H + head] for staged edge j.  The G lane groups take edges g, g+G, ...; U steps' src
+// loads are issued back to back.  A group keeps the dst row it fetched last and skips the
+// fetch while the row id repeats.  Per-head results are collected in registers -- the lane
+// whose position in its head segment equals the step number (mod RW) keeps that step's value
+// -- and written out every RW steps as one dense run of RW*G*H floats.
+template <int V, int L, int K, int RW, int KH, bool FULL>
+__device__ __forceinline__ void sddmm_staged(const int2 *edge, int n, int g, int li, const float *sb,
+                                             const float *db, int64_t F, const bool (&on)[K], float *out,
+                                             int32_t &held_row, typename Vec<V>::type (&dv)[K]) {
+    using S = Shape<V, L, K, RW, KH>;
+    using vec = typename S::vec;
+    constexpr int G = S::G, H = S::H, NH = S::NH;
+    constexpr int U = (K >= 2) ? 2 : 4;
+    const int seg_pos = li % RW, head0 = li / RW;
+    float res[NH];
+#pragma unroll
+    for (int kk = 0; kk < NH; ++kk) res[kk] = 0.f;
+    const int nsteps = (n + G - 1) / G;
+    for (int s0 = 0; s0 < nsteps; s0 += U) {
+        int2 rc[U];
+        bool live[U];
+        vec sv[U][K];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = (s0 + u) * G + g;
+            live[u] = j < n;
+            rc[u] = live[u] ? edge[j] : make_int2(0, -1);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (live[u] && (FULL || on[k]))
+                    sv[u][k] = *reinterpret_cast<const vec *>(sb + (int64_t)rc[u].x * F + k * L * V);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int step = s0 + u;
+            if (step < nsteps) {                       // uniform
+                if (live[u] && rc[u].y != held_row) {
+#pragma unroll
+                    for (int k = 0; k < K; ++k)
+                        if (FULL || on[k]) dv[k] = *reinterpret_cast<const vec *>(db + (int64_t)rc[u].y * F + k * L * V);
+                    held_row = rc[u].y;
+                }
+                float q[NH];
+                edge_heads<V, L, K, RW, KH, FULL>(sv[u], dv, on, q);
+                if ((step % RW) == seg_pos) {
+#pragma unroll
+                    for (int kk = 0; kk < NH; ++kk) res[kk] = q[kk];
+                }
+                if ((step % RW) == RW - 1 || step == nsteps - 1) {   // uniform: write the collected block
+                    const int my_step = (step / RW) * RW + seg_pos;
+                    const int j = my_step * G + g;
+                    if (my_step <= step && j < n) {
+#pragma unroll
+                        for (int kk = 0; kk < NH; ++kk) out[(int64_t)j * H + kk * S::HPL + head0] = res[kk];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Stored-order (COO) kernel: a wavefront takes kEdgesPerWave consecutive stored edges.
 template <int V, int L, int K, int RW, int KH, bool FULL>
 __global__ __launch_bounds__(kBlock) void sddmm_coo_kernel(const SddmmArgs a) {
     using S = Shape<V, L, K, RW, KH>;
     using vec = typename S::vec;
-    constexpr int G = S::G, H = S::H;
-    constexpr int U = (K >= 2) ? 2 : 4;
-    __shared__ int32_t s_row[kWavesPerBlock][64];
-    __shared__ int32_t s_col[kWavesPerBlock][64];
-    __shared__ float s_out[kWavesPerBlock][64 * H];
+    constexpr int H = S::H;
+    static_assert(kEdgesPerWave <= fg::kItemEdges, "staging row too small");
+    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane / L, li = lane % L;
     const int64_t e_begin = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * kEdgesPerWave;
     if (e_begin >= a.n_edges) return;
-    const int64_t e_end = min(e_begin + (int64_t)kEdgesPerWave, a.n_edges);
-    const int64_t F = a.F;
+    const int n = (int)min((int64_t)kEdgesPerWave, a.n_edges - e_begin);
     bool on[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) on[k] = FULL || (k * L * V + li * V < a.F);
-    const float *sb = a.src + li * V;
-    const float *db = a.dst + li * V;
-
-    int32_t held_row = -1;                 // row whose dst vectors are in dv[]
+    int2 *edge = s_edge[wave];
+    for (int t = lane; t < n; t += 64) edge[t] = make_int2(a.col[e_begin + t], a.row[e_begin + t]);
+    wave_lds_sync();
+    int32_t held_row = -1;
     vec dv[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) dv[k] = vec();
-
-    for (int64_t base = e_begin; base < e_end; base += 64) {
-        const int n = (int)min((int64_t)64, e_end - base);
-        int32_t r = 0, c = 0;
-        if (lane < n) { r = a.row[base + lane]; c = a.col[base + lane]; }
-        wave_lds_sync();
-        s_row[wave][lane] = r;
-        s_col[wave][lane] = c;
-        wave_lds_sync();
-
-        const int nsteps = (n + G - 1) / G;
-        for (int s0 = 0; s0 < nsteps; s0 += U) {
-            int32_t er[U], ec[U];
-            bool live[U];
-            vec sv[U][K];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int j = (s0 + u) * G + g;
-                live[u] = j < n;
-                er[u] = live[u] ? s_row[wave][j] : -1;
-                ec[u] = live[u] ? s_col[wave][j] : 0;
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int k = 0; k < K; ++k)
-                    if (live[u] && on[k]) sv[u][k] = *reinterpret_cast<const vec *>(sb + (int64_t)ec[u] * F + k * L * V);
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (live[u] && er[u] != held_row) {
-#pragma unroll
-                    for (int k = 0; k < K; ++k)
-                        if (on[k]) dv[k] = *reinterpret_cast<const vec *>(db + (int64_t)er[u] * F + k * L * V);
-                    held_row = er[u];
-                }
-                float q[K / KH];
-                edge_heads<V, L, K, RW, KH, FULL>(sv[u], dv, on, q);
-                if (live[u] && (li % RW) == 0) {
-                    const int j = (s0 + u) * G + g;
-#pragma unroll
-                    for (int kk = 0; kk < K / KH; ++kk) s_out[wave][j * H + kk * S::HPL + li / RW] = q[kk];
-                }
-            }
-        }
-        wave_lds_sync();
-        for (int t = lane; t < n * H; t += 64) a.out[base * H + t] = s_out[wave][t];
-    }
+    sddmm_staged<V, L, K, RW, KH, FULL>(edge, n, g, li, a.src + li * V, a.dst + li * V, a.F, on,
+                                        a.out + e_begin * H, held_row, dv);
 }
 
-// CSR-order kernel over plan items: edges [start, start+len) all belong to row `row`.
+// CSR-order kernel over plan items: a run of whole rows, one row, or a piece of a long row.
 template <int V, int L, int K, int RW, int KH, bool FULL>
 __global__ __launch_bounds__(kBlock) void sddmm_csr_kernel(const SddmmArgs a) {
     using S = Shape<V, L, K, RW, KH>;
     using vec = typename S::vec;
-    constexpr int G = S::G, H = S::H;
-    constexpr int U = (K >= 2) ? 2 : 4;
-    __shared__ int32_t s_col[kWavesPerBlock][64];
-    __shared__ float s_out[kWavesPerBlock][64 * H];
+    constexpr int H = S::H;
+    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges];
+    __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane / L, li = lane % L;
@@ -177,52 +193,38 @@ __global__ __launch_bounds__(kBlock) void sddmm_csr_kernel(const SddmmArgs a) {
     if (item_id >= a.n_items) return;
     const Item it = a.items[item_id];
     if (it.len == 0) return;
-    const int64_t F = a.F;
     bool on[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) on[k] = FULL || (k * L * V + li * V < a.F);
-    const float *sb = a.src + li * V;
+    int2 *edge = s_edge[wave];
+    int32_t held_row = -1;
     vec dv[K];
 #pragma unroll
-    for (int k = 0; k < K; ++k)
-        if (on[k]) dv[k] = *reinterpret_cast<const vec *>(a.dst + (int64_t)it.row * F + k * L * V + li * V);
+    for (int k = 0; k < K; ++k) dv[k] = vec();
+    const float *sb = a.src + li * V, *db = a.dst + li * V;
 
-    for (int32_t base = 0; base < it.len; base += 64) {
-        const int n = min(64, it.len - base);
-        int32_t c = 0;
-        if (lane < n) c = a.col[it.start + base + lane];
+    if (it.info < -1) {
+        // several whole rows: the row of staged edge t is the first row whose end exceeds t
+        const int nrows = -it.info;
+        if (lane < nrows) s_end[wave][lane] = a.pos[it.row + lane + 1] - it.start;
         wave_lds_sync();
-        s_col[wave][lane] = c;
-        wave_lds_sync();
-        const int nsteps = (n + G - 1) / G;
-        for (int s0 = 0; s0 < nsteps; s0 += U) {
-            int32_t ec[U];
-            bool live[U];
-            vec sv[U][K];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int j = (s0 + u) * G + g;
-                live[u] = j < n;
-                ec[u] = live[u] ? s_col[wave][j] : 0;
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int k = 0; k < K; ++k)
-                    if (live[u] && on[k]) sv[u][k] = *reinterpret_cast<const vec *>(sb + (int64_t)ec[u] * F + k * L * V);
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                float q[K / KH];
-                edge_heads<V, L, K, RW, KH, FULL>(sv[u], dv, on, q);
-                if (live[u] && (li % RW) == 0) {
-                    const int j = (s0 + u) * G + g;
-#pragma unroll
-                    for (int kk = 0; kk < K / KH; ++kk) s_out[wave][j * H + kk * S::HPL + li / RW] = q[kk];
-                }
-            }
+        for (int t = lane; t < it.len; t += 64) {
+            int lo = 0, hi = nrows - 1;
+            while (lo < hi) { const int mid = (lo + hi) >> 1; if (s_end[wave][mid] > t) hi = mid; else lo = mid + 1; }
+            edge[t] = make_int2(a.col[it.start + t], it.row + lo);
         }
         wave_lds_sync();
-        for (int t = lane; t < n * H; t += 64) a.out[((int64_t)it.start + base) * H + t] = s_out[wave][t];
+        sddmm_staged<V, L, K, RW, KH, FULL>(edge, it.len, g, li, sb, db, a.F, on, a.out + (int64_t)it.start * H,
+                                            held_row, dv);
+        return;
+    }
+    for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
+        const int n = min(fg::kItemEdges, it.len - base);
+        wave_lds_sync();
+        for (int t = lane; t < n; t += 64) edge[t] = make_int2(a.col[it.start + base + t], it.row);
+        wave_lds_sync();
+        sddmm_staged<V, L, K, RW, KH, FULL>(edge, n, g, li, sb, db, a.F, on,
+                                            a.out + ((int64_t)it.start + base) * H, held_row, dv);
     }
 }
 
@@ -353,7 +355,7 @@ int sddmm_run(const fg_spmm_plan *pl, const int32_t *row, const int32_t *col, co
     if (H < 1 || D < 1) return fail(FG_ERR_SHAPE, "heads and head length must be positive, got H=%d D=%d", H, D);
     if (n_edges < 0) return fail(FG_ERR_ARG, "negative edge count");
     if (n_edges == 0) return FG_OK;
-    if (!col || !src || !dst || !out || (!row && !pl)) return fail(FG_ERR_ARG, "null device pointer");
+    if (!col || !src || !dst || !out || (!row && !pl) || (pl && !indptr)) return fail(FG_ERR_ARG, "null device pointer");
     if ((int64_t)H * D > INT32_MAX) return fail(FG_ERR_SHAPE, "H*D too large");
     hipStream_t st = (hipStream_t)stream;
     const bool aligned16 = (((uintptr_t)src | (uintptr_t)dst) & 15) == 0;
@@ -361,6 +363,7 @@ int sddmm_run(const fg_spmm_plan *pl, const int32_t *row, const int32_t *col, co
     choose_config(H, D, aligned16, &c);
     SddmmArgs a;
     a.row = row; a.col = col; a.items = pl ? pl->items_dev : nullptr; a.n_items = pl ? pl->n_items : 0;
+    a.pos = indptr;
     a.n_edges = n_edges; a.src = src; a.dst = dst; a.out = out; a.F = H * D;
     const bool csr = pl != nullptr;
     bool launched = false;
@@ -373,7 +376,6 @@ int sddmm_run(const fg_spmm_plan *pl, const int32_t *row, const int32_t *col, co
         else launched = launch_heads(c, csr, grid, st, a);
     }
     if (!launched) {
-        if (csr && !indptr) return fail(FG_ERR_ARG, "indptr_dev is needed for this shape");
         const int64_t waves = (n_edges + 63) / 64;
         const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
         if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");

@@ -1,10 +1,10 @@
 // CSR / DDS SpMM for gfx950: out[v, :] = sum_e vals[e] * X[indices[e], :].
 //
-// One wavefront per plan item (a short row, or a piece of a long row).  The feature axis is
+// One wavefront per plan item (a run of short rows, one row, or a piece of a long row).  The feature axis is
 // spread over lanes in vectors of V floats: a group of L lanes covers V*L*K consecutive
 // floats of one source row with K coalesced vector loads, and the 64/L groups of the
 // wavefront take different elements of the row at the same time.  Column ids and weights
-// are staged 64 at a time in LDS by one coalesced load per array and read back as
+// are staged in LDS (up to 256 elements per wavefront) by coalesced loads and read back as
 // broadcasts, so no lane re-reads them from global memory.  Wide rows are cut into feature
 // tiles; the tile index is the fastest-varying part of the workgroup id, so consecutive
 // workgroups (which the dispatcher deals round-robin to the 8 XCDs) work on the same
@@ -52,6 +52,7 @@ __device__ __forceinline__ void wave_lds_sync() {
 struct SpmmArgs {
     const Item *items;
     int64_t n_items;
+    const int32_t *pos;    // this partition's position array (row boundaries), n_dst + 1 entries
     const int32_t *indices;
     const float *vals;
     const float *x;        // already offset to the partition's first source row
@@ -64,16 +65,68 @@ struct SpmmArgs {
     int accumulate;        // add to out instead of overwriting it
 };
 
+// Adds vals * X rows for the staged elements [b, e) of s_edge (x = column id, y = weight bits)
+// into acc.  The G lane groups take elements b+g, b+g+G, ...; U steps' loads are issued back to
+// back before the first use.
+template <int V, int L, int K, bool FULL, int U>
+__device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, int g, const float *xb,
+                                            int64_t F, const bool (&on)[K], typename Vec<V>::type (&acc)[K]) {
+    using vec = typename Vec<V>::type;
+    constexpr int G = 64 / L;
+    for (int s0 = b; s0 < e; s0 += G * U) {
+        int2 cw[U];
+        bool ok[U];
+        vec xv[U][K];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = s0 + u * G + g;
+            ok[u] = j < e;
+            cw[u] = ok[u] ? s_edge[j] : make_int2(0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (ok[u] && (FULL || on[k]))
+                    xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)cw[u].x * F + k * L * V);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (ok[u] && (FULL || on[k])) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
+    }
+}
+
+// Adds the lane groups' sums (group 0 gets the total) and stores / accumulates one output row.
+template <int V, int L, int K, bool FULL>
+__device__ __forceinline__ void finish_row(typename Vec<V>::type (&acc)[K], int g, const bool (&on)[K],
+                                           float *dst, bool add) {
+    using vec = typename Vec<V>::type;
+#pragma unroll
+    for (int off = L; off < 64; off <<= 1)
+#pragma unroll
+        for (int k = 0; k < K; ++k) vadd(acc[k], vshfl_xor(acc[k], off));
+    if (g == 0) {
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            if (FULL || on[k]) {
+                vec *p = reinterpret_cast<vec *>(dst + k * L * V);
+                vec r = acc[k];
+                if (add) vadd(r, *p);
+                *p = r;
+            }
+    }
+}
+
 // V: floats per lane per load; L: lanes per source row; K: loads per lane per source row;
 // FULL: every lane's columns are inside the tile (no masking needed).
 template <int V, int L, int K, bool FULL>
 __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     using vec = typename Vec<V>::type;
-    constexpr int G = 64 / L;              // elements processed per step
     constexpr int FT = V * L * K;          // floats per kernel tile
     constexpr int U = (K >= 2) ? 4 : 8;    // steps whose loads are issued back to back
-    __shared__ int32_t s_idx[kWavesPerBlock][64];
-    __shared__ float s_val[kWavesPerBlock][64];
+    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges];
+    __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -89,82 +142,45 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     bool on[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
-
-    vec acc[K];
-#pragma unroll
-    for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
     const float *xb = a.x + f_lo;
     const int64_t F = a.F;
+    int2 *edge = s_edge[wave];
+    vec acc[K];
 
-    for (int32_t base = 0; base < it.len; base += 64) {
-        const int n = min(64, it.len - base);
-        int32_t ci = 0;
-        float cw = 0.f;
-        if (lane < n) {
-            ci = a.indices[it.start + base + lane];
-            cw = a.vals[it.start + base + lane];
-        }
-        wave_lds_sync();                   // earlier reads of the staging rows are done
-        s_idx[wave][lane] = ci;
-        s_val[wave][lane] = cw;
+    if (it.info < -1) {
+        // several whole rows: stage all their elements once, then walk the rows
+        const int nrows = -it.info;
+        for (int t = lane; t < it.len; t += 64)
+            edge[t] = make_int2(a.indices[it.start + t], __float_as_int(a.vals[it.start + t]));
+        if (lane < nrows) s_end[wave][lane] = a.pos[it.row + lane + 1] - it.start;
         wave_lds_sync();
-
-        const int nfull = n / G;           // steps in which every group has an element
-        int s = 0;
-        for (; s + U <= nfull; s += U) {
-            int32_t c[U];
-            float w[U];
-            vec xv[U][K];
+        int b = 0;
+        for (int q = 0; q < nrows; ++q) {
+            const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
+            if (e > b || !a.accumulate) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                c[u] = s_idx[wave][(s + u) * G + g];
-                w[u] = s_val[wave][(s + u) * G + g];
+                for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
+                gather_rows<V, L, K, FULL, U>(edge, b, e, g, xb, F, on, acc);
+                finish_row<V, L, K, FULL>(acc, g, on, a.out + (int64_t)(it.row + q) * F + f_lo, a.accumulate != 0);
             }
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int k = 0; k < K; ++k)
-                    if (on[k]) xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)c[u] * F + k * L * V);
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int k = 0; k < K; ++k)
-                    if (on[k]) vfma(acc[k], w[u], xv[u][k]);
+            b = e;
         }
-        for (; s < nfull; ++s) {
-            const int32_t c = s_idx[wave][s * G + g];
-            const float w = s_val[wave][s * G + g];
-#pragma unroll
-            for (int k = 0; k < K; ++k)
-                if (on[k]) vfma(acc[k], w, *reinterpret_cast<const vec *>(xb + (int64_t)c * F + k * L * V));
-        }
-        if (G > 1 && nfull * G + g < n) {  // last, partly filled step
-            const int32_t c = s_idx[wave][nfull * G + g];
-            const float w = s_val[wave][nfull * G + g];
-#pragma unroll
-            for (int k = 0; k < K; ++k)
-                if (on[k]) vfma(acc[k], w, *reinterpret_cast<const vec *>(xb + (int64_t)c * F + k * L * V));
-        }
+        return;
     }
 
-    // add the groups' sums; group 0 ends up with the row's sum
+    // one row, or one piece of a long row: stage kItemEdges elements at a time
 #pragma unroll
-    for (int off = L; off < 64; off <<= 1)
-#pragma unroll
-        for (int k = 0; k < K; ++k) vadd(acc[k], vshfl_xor(acc[k], off));
-
-    if (g == 0) {
-        float *dst = (it.slot < 0 ? a.out + (int64_t)it.row * F : a.partial + (int64_t)it.slot * F) + f_lo;
-        const bool add = a.accumulate && it.slot < 0;
-#pragma unroll
-        for (int k = 0; k < K; ++k)
-            if (on[k]) {
-                vec *p = reinterpret_cast<vec *>(dst + k * L * V);
-                vec r = acc[k];
-                if (add) vadd(r, *p);
-                *p = r;
-            }
+    for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
+    for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
+        const int n = min(fg::kItemEdges, it.len - base);
+        wave_lds_sync();                   // earlier reads of the staging row are done
+        for (int t = lane; t < n; t += 64)
+            edge[t] = make_int2(a.indices[it.start + base + t], __float_as_int(a.vals[it.start + base + t]));
+        wave_lds_sync();
+        gather_rows<V, L, K, FULL, U>(edge, 0, n, g, xb, F, on, acc);
     }
+    float *dst = (it.info < 0 ? a.out + (int64_t)it.row * F : a.partial + (int64_t)it.info * F) + f_lo;
+    finish_row<V, L, K, FULL>(acc, g, on, dst, a.accumulate && it.info < 0);
 }
 
 // out[row, :] (+)= sum of the row's pieces, in piece order.  One lane per V columns.
@@ -245,11 +261,11 @@ int ensure_partial(const fg_spmm_plan *pl, int F) {
     return FG_OK;
 }
 
-int spmm_run(const fg_spmm_plan *pl, const int32_t *idx, const float *vals, const float *x,
-             float *out, int F, int T, void *stream) {
+int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
+             const float *x, float *out, int F, int T, void *stream) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (pl->n_dst == 0) return FG_OK;
-    if (!out || (pl->nnz > 0 && (!idx || !vals || !x))) return fail(FG_ERR_ARG, "null device pointer");
+    if (!out || !pos || (pl->nnz > 0 && (!idx || !vals || !x))) return fail(FG_ERR_ARG, "null device pointer");
     const bool aligned16 = (((uintptr_t)x | (uintptr_t)out) & 15) == 0;
     SpmmConfig c;
     int rc = choose_config(F, T, aligned16, &c);
@@ -263,6 +279,7 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *idx, const float *vals, cons
         if (i1 > i0) {
             SpmmArgs a;
             a.items = pl->items_dev + i0; a.n_items = i1 - i0;
+            a.pos = pos + (int64_t)p * (pl->n_dst + 1);
             a.indices = idx; a.vals = vals;
             a.x = x + (int64_t)p * width * F;
             a.out = out; a.partial = pl->partial_dev;
@@ -313,15 +330,13 @@ std::string spmm_launch_text(const fg_spmm_plan *pl, int F, int T) {
 extern "C" int fg_spmm_csr_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev,
                                const int32_t *indices_dev, const float *vals_dev, const float *x_dev,
                                float *out_dev, int F, int num_feat_partitions, void *stream) {
-    (void)indptr_dev;   // row boundaries live in the plan's items
     if (plan && plan->num_col_partitions != 1)
         return fail(FG_ERR_ARG, "fg_spmm_csr_f32 needs a plan with one column partition; use fg_spmm_dds_f32");
-    return spmm_run(plan, indices_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
+    return spmm_run(plan, indptr_dev, indices_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
 }
 
 extern "C" int fg_spmm_dds_f32(const fg_spmm_plan *plan, const int32_t *s1_pos_dev,
                                const int32_t *s1_idx_dev, const float *vals_dev, const float *x_dev,
                                float *out_dev, int F, int num_feat_partitions, void *stream) {
-    (void)s1_pos_dev;
-    return spmm_run(plan, s1_idx_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
+    return spmm_run(plan, s1_pos_dev, s1_idx_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
 }
