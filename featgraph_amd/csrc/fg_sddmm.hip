@@ -228,6 +228,192 @@ __global__ __launch_bounds__(kBlock) void sddmm_csr_kernel(const SddmmArgs a) {
     }
 }
 
+// ---- feature-tiled, source-column-partitioned traversal ---------------------------------------
+//
+// For graphs whose feature matrices do not fit the L2 caches.  The edge list is a DDS copy of
+// the adjacency (column partition by column partition, CSR inside a partition) and the feature
+// axis is cut into tiles of L*4 floats; workgroup id = item block * n_tiles + tile, so the 8
+// XCDs (dealt workgroups round-robin) work on the same edges but different tiles and each L2
+// holds one tile's slice of one partition's src rows.  A head (RW lanes) must lie inside a tile.
+// One head per edge in total means the tiles hold partial dot products: they go to
+// partial[tile][e'] and sddmm_tile_sum_kernel adds them; with whole heads per tile the results
+// go straight to out.  Results are scattered to the caller's edge order through edge_pos.
+
+struct SddmmTiledArgs {
+    const Item *items;
+    int64_t n_items;
+    const int32_t *pos;       // this partition's row boundaries
+    const int32_t *col;       // partition-local column ids, DDS order
+    const int32_t *edge_pos;  // DDS position -> position in the caller's edge order
+    const float *src;         // offset to the partition's first src row
+    const float *dst;
+    float *out;               // out (direct mode) or partial (tile-sum mode)
+    int64_t out_edge_stride;  // floats between consecutive edges in out
+    int64_t out_tile_stride;  // floats between consecutive tiles in out
+    int F;
+    int n_tiles;
+};
+
+// One batch: U edges of one row for this lane group (edge j0 + u*jstride, u < U, those below
+// `e`), all U src loads issued back to back; lanes without an edge re-read edge e-1.  Every
+// head's U results end up one per lane (lane position u of the head segment keeps result u) and
+// are stored by those lanes.
+template <int L, int RW, int U, bool SCATTER>
+__device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int jstride, int e, const float *sb,
+                                                 int64_t F, const float4 &dv, float *out, int64_t estride,
+                                                 int64_t e_base, int seg_pos) {
+    static_assert(U <= RW, "one result per lane of a head segment");
+    int2 ce[U];
+    float4 sv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int j = j0 + u * jstride;
+        ce[u] = edge[j < e ? j : e - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) sv[u] = *reinterpret_cast<const float4 *>(sb + (int64_t)ce[u].x * F);
+    float mine = 0.f;
+    int my_pos = 0;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const float p = segment_sum<RW>(vdot(sv[u], dv));
+        if (seg_pos == u) { mine = p; my_pos = ce[u].y; }
+    }
+    const int ju = j0 + seg_pos * jstride;
+    if (seg_pos < U && ju < e) {
+        const int64_t at = SCATTER ? (int64_t)my_pos : e_base + ju;
+        out[at * estride] = mine;
+    }
+}
+
+template <int L, int RW, bool SCATTER>
+__global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArgs a) {
+    constexpr int G = 64 / L;
+    constexpr int U = RW < 8 ? RW : 8;
+    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges];     // x = column id, y = edge_pos
+    __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
+    __shared__ int32_t s_next[kWavesPerBlock];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane / L, li = lane % L;
+    const int tile = (int)(blockIdx.x % (unsigned)a.n_tiles);
+    const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_tiles) * kWavesPerBlock + wave;
+    if (item_id >= a.n_items) return;
+    const Item it = a.items[item_id];
+    if (it.len == 0) return;
+    const int64_t F = a.F;
+    const int f_lo = tile * (L * 4) + li * 4;
+    const float *sb = a.src + f_lo;
+    const float *db = a.dst + f_lo;
+    const int seg_pos = li % RW;
+    float *out = a.out + (int64_t)tile * a.out_tile_stride + li / RW;
+    int2 *edge = s_edge[wave];
+
+    auto stage = [&](int64_t base, int n) {
+        int2 r[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = min(lane + 64 * i, n - 1);
+            r[i] = make_int2(a.col[base + t], SCATTER ? a.edge_pos[base + t] : 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) edge[lane + 64 * i] = r[i];
+    };
+
+    if (it.info < -1) {
+        const int nrows = -it.info;
+        stage(it.start, it.len);
+        s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        if (lane == 0) s_next[wave] = 0;
+        wave_lds_sync();
+        if (nrows < 2 * G) {
+            // few, longer rows: all lane groups share each row in turn
+            int b = 0;
+            for (int q = 0; q < nrows; ++q) {
+                const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
+                if (e > b) {
+                    const float4 dv = *reinterpret_cast<const float4 *>(db + (int64_t)(it.row + q) * F);
+                    for (int s0 = b; s0 < e; s0 += G * U)
+                        sddmm_tile_batch<L, RW, U, SCATTER>(edge, s0 + g, G, e, sb, F, dv, out, a.out_edge_stride,
+                                                            it.start, seg_pos);
+                }
+                b = e;
+            }
+            return;
+        }
+        // many short rows: every lane group walks rows of its own
+        int q = -1, j = 0, e = 0;
+        bool done = false;
+        float4 dv = vzero4();
+        for (;;) {
+            if (!done && j >= e) {
+                int qn = 0;
+                if (li == 0) qn = atomicAdd(&s_next[wave], 1);
+                q = __shfl(qn, g * L);
+                if (q >= nrows) {
+                    done = true;
+                } else {
+                    j = q ? s_end[wave][q - 1] : 0;
+                    e = s_end[wave][q];
+                    if (e > j) dv = *reinterpret_cast<const float4 *>(db + (int64_t)(it.row + q) * F);
+                }
+            }
+            if (__all(done)) break;
+            if (!done && j < e) {
+                sddmm_tile_batch<L, RW, U, SCATTER>(edge, j, 1, e, sb, F, dv, out, a.out_edge_stride, it.start, seg_pos);
+                j += U;
+            }
+        }
+        return;
+    }
+    // one row, or one piece of a long row
+    const float4 dv = *reinterpret_cast<const float4 *>(db + (int64_t)it.row * F);
+    for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
+        const int n = min(fg::kItemEdges, it.len - base);
+        wave_lds_sync();
+        stage((int64_t)it.start + base, n);
+        wave_lds_sync();
+        for (int s0 = 0; s0 < n; s0 += G * U)
+            sddmm_tile_batch<L, RW, U, SCATTER>(edge, s0 + g, G, n, sb, F, dv, out, a.out_edge_stride,
+                                                (int64_t)it.start + base, seg_pos);
+    }
+}
+
+// out[edge_pos[e']] = sum over tiles of partial[tile][e'], tiles added in ascending order.
+__global__ __launch_bounds__(256) void sddmm_tile_sum_kernel(const float *partial, const int32_t *edge_pos,
+                                                             float *out, int64_t n_edges, int n_tiles) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n_edges) return;
+    float s = partial[e];
+    for (int t = 1; t < n_tiles; ++t) s += partial[(int64_t)t * n_edges + e];
+    out[edge_pos[e]] = s;
+}
+
+template <int L, bool SCATTER>
+bool launch_tiled(int RW, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
+    switch (RW) {
+        case 2: if constexpr (L >= 2) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 2, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
+        case 4: if constexpr (L >= 4) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 4, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
+        case 8: if constexpr (L >= 8) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 8, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
+        case 16: if constexpr (L >= 16) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 16, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
+        case 32: if constexpr (L >= 32) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 32, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
+        case 64: if constexpr (L >= 64) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 64, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
+    }
+    return false;
+}
+
+template <bool SCATTER>
+bool launch_tiled_l(int L, int RW, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
+    switch (L) {
+        case 4: return launch_tiled<4, SCATTER>(RW, grid, st, a);
+        case 8: return launch_tiled<8, SCATTER>(RW, grid, st, a);
+        case 16: return launch_tiled<16, SCATTER>(RW, grid, st, a);
+        case 32: return launch_tiled<32, SCATTER>(RW, grid, st, a);
+        case 64: return launch_tiled<64, SCATTER>(RW, grid, st, a);
+    }
+    return false;
+}
+
 // Any H, D (odd lengths, unaligned pointers): one edge at a time per wavefront, lanes stride
 // over the head's D floats, full-wavefront reduction per head.
 __global__ __launch_bounds__(kBlock) void sddmm_generic_kernel(const int32_t *row, const int32_t *col,
@@ -402,4 +588,77 @@ extern "C" int fg_sddmm_csr_f32(const fg_spmm_plan *plan, const int32_t *indptr_
     if (plan->num_col_partitions != 1) return fail(FG_ERR_ARG, "fg_sddmm_csr_f32 needs a plan with one column partition");
     return sddmm_run(plan, nullptr, indices_dev, indptr_dev, plan->n_dst, plan->nnz, src_dev, dst_dev,
                      out_dev, H, D, stream);
+}
+
+namespace {
+int ensure_floats(const fg_spmm_plan *pl, size_t need) {
+    if (need <= pl->partial_floats) return FG_OK;
+    if (pl->partial_dev) FG_HIP_TRY(hipFree(pl->partial_dev));
+    pl->partial_dev = nullptr; pl->partial_floats = 0;
+    FG_HIP_TRY(hipMalloc((void **)&pl->partial_dev, need * sizeof(float)));
+    pl->partial_floats = need;
+    return FG_OK;
+}
+}  // namespace
+
+extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_dev, const int32_t *s1_idx_dev,
+                                const int32_t *edge_pos_dev, const float *src_dev, const float *dst_dev,
+                                float *out_dev, int H, int D, int num_feat_partitions, void *stream) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (H < 1 || D < 1) return fail(FG_ERR_SHAPE, "heads and head length must be positive, got H=%d D=%d", H, D);
+    if (pl->nnz == 0) return FG_OK;
+    if (!s1_pos_dev || !s1_idx_dev || !edge_pos_dev || !src_dev || !dst_dev || !out_dev)
+        return fail(FG_ERR_ARG, "null device pointer");
+    if ((((uintptr_t)src_dev | (uintptr_t)dst_dev) & 15) != 0) return fail(FG_ERR_ARG, "src/dst must be 16-byte aligned");
+    const int64_t F64 = (int64_t)H * D;
+    if (F64 > INT32_MAX) return fail(FG_ERR_SHAPE, "H*D too large");
+    const int F = (int)F64;
+    const int T = num_feat_partitions;
+    if (T < 1 || F % T != 0) return fail(FG_ERR_SHAPE, "feature length %d is not divisible by num_feat_partitions %d", F, T);
+    const int tile_w = F / T;
+    if (tile_w % 4 != 0 || tile_w > 256 || !is_pow2(tile_w / 4) || tile_w < 16)
+        return fail(FG_ERR_SHAPE, "feature tile of %d floats: need a power of two between 16 and 256", tile_w);
+    const int L = tile_w / 4;
+    int RW;                       // lanes per head inside a tile
+    bool tile_sum;                // tiles hold partial sums of one head
+    if (D >= tile_w) {
+        if (D % tile_w != 0) return fail(FG_ERR_SHAPE, "head length %d is not a multiple of the %d-float tile", D, tile_w);
+        if (D > tile_w && H != 1) return fail(FG_ERR_SHAPE, "a head spanning several tiles needs H == 1");
+        RW = L; tile_sum = D > tile_w;
+    } else {
+        if (tile_w % D != 0 || D % 4 != 0 || !is_pow2(D / 4) || D < 8)
+            return fail(FG_ERR_SHAPE, "head length %d does not pack into a %d-float tile", D, tile_w);
+        RW = D / 4; tile_sum = false;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    SddmmTiledArgs a;
+    a.col = s1_idx_dev; a.edge_pos = edge_pos_dev; a.dst = dst_dev; a.F = F; a.n_tiles = T;
+    if (tile_sum) {
+        int rc = ensure_floats(pl, (size_t)T * (size_t)pl->nnz);
+        if (rc != FG_OK) return rc;
+        a.out = pl->partial_dev; a.out_edge_stride = 1; a.out_tile_stride = pl->nnz;
+    } else {
+        a.out = out_dev; a.out_edge_stride = H; a.out_tile_stride = tile_w / D;
+    }
+    const int P = pl->num_col_partitions;
+    const int64_t width = (pl->n_src + P - 1) / P;
+    for (int p = 0; p < P; ++p) {
+        const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
+        if (i1 == i0) continue;
+        a.items = pl->items_dev + i0; a.n_items = i1 - i0;
+        a.pos = s1_pos_dev + (int64_t)p * (pl->n_dst + 1);
+        a.src = src_dev + (int64_t)p * width * F;
+        const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * T;
+        if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
+        const bool ok = tile_sum ? launch_tiled_l<false>(L, RW, dim3((unsigned)blocks), st, a)
+                                 : launch_tiled_l<true>(L, RW, dim3((unsigned)blocks), st, a);
+        if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d RW=%d", L, RW);
+    }
+    if (tile_sum) {
+        const unsigned blocks = (unsigned)((pl->nnz + 255) / 256);
+        hipLaunchKernelGGL(sddmm_tile_sum_kernel, dim3(blocks), dim3(256), 0, st, pl->partial_dev, edge_pos_dev,
+                           out_dev, pl->nnz, T);
+    }
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
 }

@@ -65,15 +65,38 @@ struct SpmmArgs {
     int accumulate;        // add to out instead of overwriting it
 };
 
+__device__ __forceinline__ float4 vselect(bool c, const float4 &a) {
+    return make_float4(c ? a.x : 0.f, c ? a.y : 0.f, c ? a.z : 0.f, c ? a.w : 0.f);
+}
+__device__ __forceinline__ float vselect(bool c, const float &a) { return c ? a : 0.f; }
+
 // Adds vals * X rows for the staged elements [b, e) of s_edge (x = column id, y = weight bits)
 // into acc.  The G lane groups take elements b+g, b+g+G, ...; U steps' loads are issued back to
-// back before the first use.
+// back before the first use.  No load sits under a branch: in the last, partly filled batch a
+// lane without an element re-reads the row's last element and its value is replaced by zero.
 template <int V, int L, int K, bool FULL, int U>
 __device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, int g, const float *xb,
                                             int64_t F, const bool (&on)[K], typename Vec<V>::type (&acc)[K]) {
     using vec = typename Vec<V>::type;
     constexpr int G = 64 / L;
-    for (int s0 = b; s0 < e; s0 += G * U) {
+    int s0 = b;
+    for (; s0 + G * U <= e; s0 += G * U) {
+        int2 cw[U];
+        vec xv[U][K];
+#pragma unroll
+        for (int u = 0; u < U; ++u) cw[u] = s_edge[s0 + u * G + g];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (FULL || on[k]) xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)cw[u].x * F + k * L * V);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (FULL || on[k]) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
+    }
+    if (s0 < e) {                          // uniform: fewer than G*U elements left
         int2 cw[U];
         bool ok[U];
         vec xv[U][K];
@@ -81,26 +104,26 @@ __device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, in
         for (int u = 0; u < U; ++u) {
             const int j = s0 + u * G + g;
             ok[u] = j < e;
-            cw[u] = ok[u] ? s_edge[j] : make_int2(0, 0);
+            cw[u] = s_edge[ok[u] ? j : e - 1];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int k = 0; k < K; ++k)
-                if (ok[u] && (FULL || on[k]))
-                    xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)cw[u].x * F + k * L * V);
+                if (FULL || on[k]) xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)cw[u].x * F + k * L * V);
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int k = 0; k < K; ++k)
-                if (ok[u] && (FULL || on[k])) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
+                if (FULL || on[k]) vfma(acc[k], ok[u] ? __int_as_float(cw[u].y) : 0.f, vselect(ok[u], xv[u][k]));
     }
 }
 
-// Adds the lane groups' sums (group 0 gets the total) and stores / accumulates one output row.
-template <int V, int L, int K, bool FULL>
-__device__ __forceinline__ void finish_row(typename Vec<V>::type (&acc)[K], int g, const bool (&on)[K],
-                                           float *dst, bool add) {
+// Adds the lane groups' sums (group 0 gets the total) and stores one output row; `old` is what
+// the row held before (only read when ADD).
+template <int V, int L, int K, bool FULL, bool ADD>
+__device__ __forceinline__ void finish_row(typename Vec<V>::type (&acc)[K], const typename Vec<V>::type (&old)[K],
+                                           int g, const bool (&on)[K], float *dst) {
     using vec = typename Vec<V>::type;
 #pragma unroll
     for (int off = L; off < 64; off <<= 1)
@@ -110,23 +133,40 @@ __device__ __forceinline__ void finish_row(typename Vec<V>::type (&acc)[K], int 
 #pragma unroll
         for (int k = 0; k < K; ++k)
             if (FULL || on[k]) {
-                vec *p = reinterpret_cast<vec *>(dst + k * L * V);
                 vec r = acc[k];
-                if (add) vadd(r, *p);
-                *p = r;
+                if (ADD) vadd(r, old[k]);
+                *reinterpret_cast<vec *>(dst + k * L * V) = r;
             }
     }
 }
 
+// Loads elements [base, base + min(n, 256)) of (indices, vals) into registers, 4 per lane; lanes
+// past the end re-read the last element so that no load is conditional.  n >= 1.
+__device__ __forceinline__ void stage_load(const int32_t *indices, const float *vals, int64_t base, int n,
+                                           int lane, int2 (&r)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int t = min(lane + 64 * i, n - 1);
+        r[i] = make_int2(indices[base + t], __float_as_int(vals[base + t]));
+    }
+}
+__device__ __forceinline__ void stage_store(int2 *edge, int lane, const int2 (&r)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) edge[lane + 64 * i] = r[i];
+}
+
 // V: floats per lane per load; L: lanes per source row; K: loads per lane per source row;
-// FULL: every lane's columns are inside the tile (no masking needed).
-template <int V, int L, int K, bool FULL>
+// FULL: every lane's columns are inside the tile (no masking needed); ACC: add to out.
+template <int V, int L, int K, bool FULL, bool ACC>
 __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     using vec = typename Vec<V>::type;
+    static_assert(fg::kItemEdges == 256, "stage_load/stage_store move 4 x 64 elements");
     constexpr int FT = V * L * K;          // floats per kernel tile
+    constexpr int G = 64 / L;              // lane groups per wavefront
     constexpr int U = (K >= 2) ? 4 : 8;    // steps whose loads are issued back to back
     __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges];
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
+    __shared__ int32_t s_next[kWavesPerBlock];
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -145,42 +185,125 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     const float *xb = a.x + f_lo;
     const int64_t F = a.F;
     int2 *edge = s_edge[wave];
-    vec acc[K];
+    vec acc[K], old[K];
+    int2 regs[4];
 
     if (it.info < -1) {
-        // several whole rows: stage all their elements once, then walk the rows
+        // Several whole rows: stage all their elements once.
         const int nrows = -it.info;
-        for (int t = lane; t < it.len; t += 64)
-            edge[t] = make_int2(a.indices[it.start + t], __float_as_int(a.vals[it.start + t]));
-        if (lane < nrows) s_end[wave][lane] = a.pos[it.row + lane + 1] - it.start;
+        if (it.len > 0) {
+            stage_load(a.indices, a.vals, it.start, it.len, lane, regs);
+            stage_store(edge, lane, regs);
+        }
+        s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        if (lane == 0) s_next[wave] = 0;
         wave_lds_sync();
-        int b = 0;
-        for (int q = 0; q < nrows; ++q) {
-            const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
-            if (e > b || !a.accumulate) {
+        if (nrows < 2 * G) {
+            // Few, longer rows: all lane groups share each row in turn.
+            int b = 0;
+            for (int q = 0; q < nrows; ++q) {
+                const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
+                if (e > b || !ACC) {
+                    float *dst = a.out + (int64_t)(it.row + q) * F + f_lo;
+                    if (ACC) {
 #pragma unroll
-                for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
-                gather_rows<V, L, K, FULL, U>(edge, b, e, g, xb, F, on, acc);
-                finish_row<V, L, K, FULL>(acc, g, on, a.out + (int64_t)(it.row + q) * F + f_lo, a.accumulate != 0);
+                        for (int k = 0; k < K; ++k)
+                            if (FULL || on[k]) old[k] = *reinterpret_cast<const vec *>(dst + k * L * V);
+                    }
+#pragma unroll
+                    for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
+                    gather_rows<V, L, K, FULL, U>(edge, b, e, g, xb, F, on, acc);
+                    finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
+                }
+                b = e;
             }
-            b = e;
+            return;
+        }
+        // Many short rows: every lane group takes rows of its own (next free row from a counter
+        // in LDS), walks each row's elements U at a time and writes the row itself, so G rows
+        // are in flight per wavefront and no sums cross lane groups.
+        int q = -1, j = 0, e = 0;
+        bool done = false, nonempty = false;
+        for (;;) {
+            if (!done && j >= e) {
+                if (q >= 0 && (!ACC || nonempty)) {       // the row this group just finished
+                    float *dst = a.out + (int64_t)(it.row + q) * F + f_lo;
+#pragma unroll
+                    for (int k = 0; k < K; ++k)
+                        if (FULL || on[k]) {
+                            vec r = acc[k];
+                            if (ACC) vadd(r, old[k]);
+                            *reinterpret_cast<vec *>(dst + k * L * V) = r;
+                        }
+                }
+                int qn = 0;
+                if (li == 0) qn = atomicAdd(&s_next[wave], 1);
+                q = __shfl(qn, g * L);
+                if (q >= nrows) {
+                    done = true;
+                } else {
+                    j = q ? s_end[wave][q - 1] : 0;
+                    e = s_end[wave][q];
+                    nonempty = e > j;
+#pragma unroll
+                    for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
+                    if (ACC && nonempty) {
+                        const float *src = a.out + (int64_t)(it.row + q) * F + f_lo;
+#pragma unroll
+                        for (int k = 0; k < K; ++k)
+                            if (FULL || on[k]) old[k] = *reinterpret_cast<const vec *>(src + k * L * V);
+                    }
+                }
+            }
+            if (__all(done)) break;
+            if (!done && j < e) {
+                int2 cw[U];
+                bool ok[U];
+                vec xv[U][K];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    ok[u] = j + u < e;
+                    cw[u] = edge[ok[u] ? j + u : e - 1];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int k = 0; k < K; ++k)
+                        if (FULL || on[k]) xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)cw[u].x * F + k * L * V);
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int k = 0; k < K; ++k)
+                        if (FULL || on[k]) vfma(acc[k], ok[u] ? __int_as_float(cw[u].y) : 0.f, vselect(ok[u], xv[u][k]));
+                j += U;
+            }
         }
         return;
     }
 
-    // one row, or one piece of a long row: stage kItemEdges elements at a time
+    // one row, or one piece of a long row: 256 elements at a time, the next 256 on their way
+    // while the current ones are used
+    float *dst = (it.info < 0 ? a.out + (int64_t)it.row * F : a.partial + (int64_t)it.info * F) + f_lo;
+    const bool add = ACC && it.info < 0;
 #pragma unroll
     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
+    if (it.len > 0) stage_load(a.indices, a.vals, it.start, it.len, lane, regs);
+    if (ACC) {
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            if (FULL || on[k]) old[k] = add ? *reinterpret_cast<const vec *>(dst + k * L * V) : vzero(vec());
+    }
     for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
         const int n = min(fg::kItemEdges, it.len - base);
         wave_lds_sync();                   // earlier reads of the staging row are done
-        for (int t = lane; t < n; t += 64)
-            edge[t] = make_int2(a.indices[it.start + base + t], __float_as_int(a.vals[it.start + base + t]));
+        stage_store(edge, lane, regs);
         wave_lds_sync();
+        if (base + fg::kItemEdges < it.len)
+            stage_load(a.indices, a.vals, (int64_t)it.start + base + fg::kItemEdges,
+                       it.len - base - fg::kItemEdges, lane, regs);
         gather_rows<V, L, K, FULL, U>(edge, 0, n, g, xb, F, on, acc);
     }
-    float *dst = (it.info < 0 ? a.out + (int64_t)it.row * F : a.partial + (int64_t)it.info * F) + f_lo;
-    finish_row<V, L, K, FULL>(acc, g, on, dst, a.accumulate && it.info < 0);
+    finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
 }
 
 // out[row, :] (+)= sum of the row's pieces, in piece order.  One lane per V columns.
@@ -232,8 +355,13 @@ int choose_config(int F, int T, bool aligned16, SpmmConfig *c) {
 
 template <int V, int L, int K>
 void launch_vlk(bool full, dim3 grid, hipStream_t st, const SpmmArgs &a) {
-    if (full) hipLaunchKernelGGL((spmm_items_kernel<V, L, K, true>), grid, dim3(kBlock), 0, st, a);
-    else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, false>), grid, dim3(kBlock), 0, st, a);
+    if (a.accumulate) {
+        if (full) hipLaunchKernelGGL((spmm_items_kernel<V, L, K, true, true>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, false, true>), grid, dim3(kBlock), 0, st, a);
+    } else {
+        if (full) hipLaunchKernelGGL((spmm_items_kernel<V, L, K, true, false>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, false, false>), grid, dim3(kBlock), 0, st, a);
+    }
 }
 
 template <int V>
@@ -317,7 +445,7 @@ std::string spmm_launch_text(const fg_spmm_plan *pl, int F, int T) {
     const int64_t per_part = pl->item_off.size() > 1 ? pl->item_off[1] - pl->item_off[0] : 0;
     snprintf(b, sizeof(b),
              "  feature length   : %d, %d requested tile(s) of %d, %d kernel tile(s) of %d floats\n"
-             "  kernel           : spmm_items_kernel<V=%d, L=%d, K=%d, FULL=%d>; %d element(s) per step\n"
+             "  kernel           : spmm_items_kernel<V=%d, L=%d, K=%d, FULL=%d, ACC=pass>0>; %d element(s) per step\n"
              "  launch           : %d pass(es); first pass grid %lld x block %d; fixup rows %lld\n",
              F, c.n_ftiles / c.sub_per_tile, c.tile_w, c.n_ftiles, c.V * c.L * c.K, c.V, c.L, c.K,
              (int)c.full, 64 / c.L, pl->num_col_partitions,

@@ -6,7 +6,8 @@ import numpy as np
 import torch
 
 from .. import _lib
-from ..util import util_partition_adj_coo_2d
+from .. import tuning
+from ..util import util_convert_csr_to_dds, util_partition_adj_coo_2d
 from . import common
 
 
@@ -72,9 +73,12 @@ class SDDMMbase(object):
             with torch.cuda.device(self._ctx):
                 _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(indptr), self._num_rows, self._num_cols,
                                                           1, None, ctypes.byref(self._plan)))
+        # source-column-partitioned copies of the edge list for the tiled traversal, by P
+        self._dds = {}
         # To be updated in self.build
         self._func = None
         self._placeholders = None
+        self._tiled = None
         self._heads = 1
         self._head_len = None
         self._use_csr = False
@@ -82,13 +86,43 @@ class SDDMMbase(object):
         self.out_tvm = None
 
     def __del__(self):
-        plan = getattr(self, "_plan", None)
-        if plan is not None and plan.value:
-            try:
-                _lib.lib().fg_spmm_plan_destroy(plan)
-            except Exception:
-                pass
-            self._plan = None
+        plans = [getattr(self, "_plan", None)] + [d['plan'] for d in getattr(self, "_dds", {}).values()]
+        for plan in plans:
+            if plan is not None and plan.value:
+                try:
+                    _lib.lib().fg_spmm_plan_destroy(plan)
+                except Exception:
+                    pass
+                plan.value = None
+
+    def _dds_layout(self, P):
+        """DDS copy of the stored edges (P source-column partitions, CSR inside each) with, per
+        traversed edge, its position in the stored order; device arrays + plan, built once per P."""
+        if P in self._dds:
+            return self._dds[P]
+        import scipy.sparse
+        nnz = self._adj_row_indices.shape[0]
+        if self._row_sorted:
+            order = None                        # stored order is already CSR order
+            indptr = np.zeros(self._num_rows + 1, dtype=np.int32)
+            np.cumsum(np.bincount(self._adj_row_indices, minlength=self._num_rows), out=indptr[1:])
+            indices = self._adj_col_indices
+            positions = np.arange(nnz, dtype=np.int32)
+        else:
+            order = np.lexsort((self._adj_col_indices, self._adj_row_indices)).astype(np.int32)
+            indptr = np.zeros(self._num_rows + 1, dtype=np.int32)
+            np.cumsum(np.bincount(self._adj_row_indices, minlength=self._num_rows), out=indptr[1:])
+            indices = self._adj_col_indices[order]
+            positions = order
+        csr = scipy.sparse.csr_matrix((positions, indices, indptr), shape=(self._num_rows, self._num_cols))
+        s1_pos, s1_idx, edge_pos = util_convert_csr_to_dds(csr, P)
+        d = {'P': P, 'pos': common.to_device_i32(s1_pos, self._ctx), 'idx': common.to_device_i32(s1_idx, self._ctx),
+             'edge_pos': common.to_device_i32(edge_pos, self._ctx), 'plan': ctypes.c_void_p()}
+        with torch.cuda.device(self._ctx):
+            _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(s1_pos), self._num_rows, self._num_cols, P, None,
+                                                      ctypes.byref(d['plan'])))
+        self._dds[P] = d
+        return d
 
     def _preprocess_adj(self, adj_scipy_coo, num_row_partitions=1, num_col_partitions=1):
         return util_partition_adj_coo_2d(adj_scipy_coo, num_row_partitions, num_col_partitions)
@@ -129,12 +163,24 @@ class SDDMMbase(object):
                 "num_cuda_blocks must be smaller than num_edges, which is {}.".format(self._adj_row_indices.shape[0])
             notes.append("num_cuda_blocks has no counterpart: the grid follows the edge count")
         order = schedule_args.get('order', 'auto')
-        if order not in ('auto', 'csr', 'coo'):
-            raise ValueError("order must be 'auto', 'csr' or 'coo'")
+        if order not in ('auto', 'csr', 'coo', 'tiled'):
+            raise ValueError("order must be 'auto', 'csr', 'coo' or 'tiled'")
         if order == 'csr' and not self._row_sorted:
             raise ValueError("order='csr' needs stored edges with non-decreasing row ids")
         use_csr = self._row_sorted and order != 'coo'
-        return [src_ph, dst_ph], H, D, use_csr, notes
+        # Tiled traversal for feature matrices beyond the L2: (source partitions, feature tiles)
+        tiled = None
+        nnz = self._adj_row_indices.shape[0]
+        if order in ('auto', 'tiled') and nnz > 0:
+            tiled = tuning.choose_sddmm(self._num_rows, self._num_cols, nnz, H, D)
+            p_arg, t_arg = schedule_args.get('num_src_partitions'), schedule_args.get('num_feat_tiles')
+            if order == 'tiled' or p_arg is not None or t_arg is not None:
+                base = tiled or (1, 1)
+                tiled = (int(p_arg) if p_arg is not None else base[0], int(t_arg) if t_arg is not None else base[1])
+            if tiled is not None:
+                notes.append("tiled traversal: %d source-column partitions x %d feature tiles; results are "
+                             "written back in the stored edge order" % tiled)
+        return [src_ph, dst_ph], H, D, use_csr, tiled, notes
 
     def build(self, input_placeholders, compute_args, schedule_args):
         """Fix the feature shape and kernel variant, allocate the output once.
@@ -148,12 +194,17 @@ class SDDMMbase(object):
             {'num_feat_partitions': T} is accepted (see lower_to_ir for what it maps to)
 
         schedule_args : dict
-            'num_feat_partitions', 'num_cuda_blocks' (reference keys) and 'order' in
-            {'auto', 'csr', 'coo'}: which kernel walks the stored edges
+            'num_feat_partitions', 'num_cuda_blocks' (reference keys); 'order' in
+            {'auto', 'csr', 'coo', 'tiled'}: which kernel walks the edges ('auto' picks the tiled
+            traversal when the feature matrices exceed the L2); 'num_src_partitions' /
+            'num_feat_tiles': override the tiled traversal's shape
         """
-        phs, H, D, use_csr, notes = self._resolve(input_placeholders, compute_args, schedule_args)
+        phs, H, D, use_csr, tiled, notes = self._resolve(input_placeholders, compute_args, schedule_args)
         self._placeholders = phs
         self._heads, self._head_len, self._use_csr, self._notes = H, D, use_csr, notes
+        self._tiled = None
+        if tiled is not None:
+            self._tiled = (self._dds_layout(tiled[0]), tiled[1])
         self._func = _lib.lib().fg_sddmm_csr_f32 if use_csr else _lib.lib().fg_sddmm_coo_f32
         nnz = self._adj_row_indices.shape[0]
         oshape = (nnz,) if self._out_1d else (nnz, H)
@@ -161,13 +212,14 @@ class SDDMMbase(object):
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         """Return a text description of the launch. This can be useful for debug."""
-        _, H, D, use_csr, notes = self._resolve(input_placeholders, compute_args, schedule_args)
+        _, H, D, use_csr, tiled, notes = self._resolve(input_placeholders, compute_args, schedule_args)
         nnz = self._adj_row_indices.shape[0]
         text = "featgraph-hip SDDMM (gfx950)\n"
         text += "  adjacency        : %d x %d, %d stored edges, %d x %d partition blocks\n" % (
             self._num_rows, self._num_cols, nnz, self._num_row_partitions, self._num_col_partitions)
         text += "  features         : %d head(s) x %d floats\n" % (H, D)
-        text += "  kernel           : %s\n" % ("sddmm_csr_kernel over row pieces (dst row held in registers)"
+        text += "  kernel           : %s\n" % ("sddmm_tiled_kernel over a source-column-partitioned edge list" if tiled
+                                               else "sddmm_csr_kernel over row pieces (dst row held in registers)"
                                                if use_csr else "sddmm_coo_kernel, 256 stored edges per wavefront")
         for n in notes:
             text += "  note             : %s\n" % n
@@ -175,7 +227,13 @@ class SDDMMbase(object):
 
     def _launch(self, src_feat, dst_feat):
         s = common.stream_ptr()
-        if self._use_csr:
+        if self._tiled is not None:
+            d, T = self._tiled
+            _lib.check(_lib.lib().fg_sddmm_dds_f32(d['plan'], _lib.dev_ptr(d['pos']), _lib.dev_ptr(d['idx']),
+                                                   _lib.dev_ptr(d['edge_pos']), _lib.dev_ptr(src_feat),
+                                                   _lib.dev_ptr(dst_feat), _lib.dev_ptr(self.out_tvm),
+                                                   self._heads, self._head_len, T, s))
+        elif self._use_csr:
             _lib.check(self._func(self._plan, _lib.dev_ptr(self._adj_indptr_dev), _lib.dev_ptr(self._adj_col_indices_dev),
                                   _lib.dev_ptr(src_feat), _lib.dev_ptr(dst_feat), _lib.dev_ptr(self.out_tvm),
                                   self._heads, self._head_len, s))
@@ -221,7 +279,7 @@ class SDDMMbase(object):
 class VanillaSDDMMhip(SDDMMbase):
     """Edge-wise dot product on gfx950, optionally over a 2-D partitioned edge order."""
     _compute_keys = ('num_feat_partitions',)
-    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order')
+    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles')
     _out_1d = True
 
     def __init__(self, adj_scipy, num_row_partitions=1, num_col_partitions=1):
@@ -235,13 +293,13 @@ class VanillaSDDMMhip(SDDMMbase):
 class VanillaSDDMMx86(VanillaSDDMMhip):
     """Constructor and knobs of the reference's VanillaSDDMMx86
     (python/featgraph/module/sddmm.py:168-176); the partitioned traversal runs on the GPU."""
-    _schedule_keys = ('num_feat_partitions', 'order')
+    _schedule_keys = ('num_feat_partitions', 'order', 'num_src_partitions', 'num_feat_tiles')
 
 
 class VanillaSDDMMcuda(VanillaSDDMMhip):
     """Constructor and knobs of the reference's VanillaSDDMMcuda
     (python/featgraph/module/sddmm.py:179-187): no partitioning, hence no edge_mapping."""
-    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order')
+    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles')
 
     def __init__(self, adj_scipy):
         super(VanillaSDDMMcuda, self).__init__(adj_scipy, num_row_partitions=1, num_col_partitions=1)

@@ -6,6 +6,7 @@ import numpy as np
 import torch
 
 from .. import _lib
+from .. import tuning
 from ..util import util_convert_csr_to_dds
 from . import common
 
@@ -35,37 +36,29 @@ class SpMMbase(object):
         self._target = None
         self._ctx = None
         self._register()
-        L = _lib.lib()
         indptr = np.ascontiguousarray(adj_scipy_csr.indptr, dtype=np.int32)
         indices = np.ascontiguousarray(adj_scipy_csr.indices, dtype=np.int32)
-        _lib.check(L.fg_check_csr_host(self._num_rows, self._num_cols, _lib.host_ptr(indptr),
-                                       _lib.host_ptr(indices)))
-        self._plan = ctypes.c_void_p()
+        _lib.check(_lib.lib().fg_check_csr_host(self._num_rows, self._num_cols, _lib.host_ptr(indptr),
+                                                _lib.host_ptr(indices)))
+        self._adj_scipy_csr = adj_scipy_csr
+        self._adj_indptr = indptr
+        self._adj_indices = indices
+        self._adj_vals = np.ascontiguousarray(adj_scipy_csr.data, dtype=np.float32)
+        # device layouts by number of source-column partitions: 1 = CSR, P > 1 = DDS
+        self._layouts = {}
         # 1D graph partitioning
         if self._num_col_partitions > 1:
-            adj_s1_pos, adj_s1_idx, adj_vals = self._preprocess_adj(adj_scipy_csr, self._num_col_partitions)
-            self._adj_s1_pos = adj_s1_pos
-            self._adj_s1_idx = adj_s1_idx
-            self._adj_vals = np.ascontiguousarray(adj_vals, dtype=np.float32)
-            self._adj_s1_pos_dev = common.to_device_i32(self._adj_s1_pos, self._ctx)
-            self._adj_s1_idx_dev = common.to_device_i32(self._adj_s1_idx, self._ctx)
-            self._adj_vals_dev = common.to_device_f32(self._adj_vals, self._ctx)
+            lay = self._layout(self._num_col_partitions)
+            self._adj_s1_pos, self._adj_s1_idx, self._adj_vals = lay['host']
+            self._adj_s1_pos_dev, self._adj_s1_idx_dev, self._adj_vals_dev = lay['pos'], lay['idx'], lay['vals']
             self._adj_d1_size = self._num_col_partitions
             self._adj_d2_size = self._num_rows + 1
-            pos_host = self._adj_s1_pos
         else:
-            self._adj_indptr = indptr
-            self._adj_indices = indices
-            self._adj_vals = np.ascontiguousarray(adj_scipy_csr.data, dtype=np.float32)
-            self._adj_indptr_dev = common.to_device_i32(self._adj_indptr, self._ctx)
-            self._adj_indices_dev = common.to_device_i32(self._adj_indices, self._ctx)
-            self._adj_vals_dev = common.to_device_f32(self._adj_vals, self._ctx)
-            pos_host = self._adj_indptr
-        with torch.cuda.device(self._ctx):
-            _lib.check(L.fg_spmm_plan_create(_lib.host_ptr(pos_host), self._num_rows, self._num_cols,
-                                             self._num_col_partitions, None, ctypes.byref(self._plan)))
+            lay = self._layout(1)
+            self._adj_indptr_dev, self._adj_indices_dev, self._adj_vals_dev = lay['pos'], lay['idx'], lay['vals']
         # To be updated in self.build
         self._func = None
+        self._active = None
         self._placeholders = None
         self._feat_len = None
         self._num_feat_partitions = 0
@@ -73,14 +66,33 @@ class SpMMbase(object):
         # To be updated in self.build; the same tensor is returned by every run()
         self.out_tvm = None
 
+    def _layout(self, P):
+        """Device arrays + load-balance plan for P source-column partitions (built once per P)."""
+        if P in self._layouts:
+            return self._layouts[P]
+        if P > 1:
+            pos, idx, vals = self._preprocess_adj(self._adj_scipy_csr, P)
+            vals = np.ascontiguousarray(vals, dtype=np.float32)
+        else:
+            pos, idx, vals = self._adj_indptr, self._adj_indices, self._adj_vals
+        lay = {'P': P, 'host': (pos, idx, vals),
+               'pos': common.to_device_i32(pos, self._ctx), 'idx': common.to_device_i32(idx, self._ctx),
+               'vals': common.to_device_f32(vals, self._ctx), 'plan': ctypes.c_void_p()}
+        with torch.cuda.device(self._ctx):
+            _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(pos), self._num_rows, self._num_cols, P, None,
+                                                      ctypes.byref(lay['plan'])))
+        self._layouts[P] = lay
+        return lay
+
     def __del__(self):
-        plan = getattr(self, "_plan", None)
-        if plan is not None and plan.value:
-            try:
-                _lib.lib().fg_spmm_plan_destroy(plan)
-            except Exception:
-                pass
-            self._plan = None
+        for lay in getattr(self, "_layouts", {}).values():
+            plan = lay.get('plan')
+            if plan is not None and plan.value:
+                try:
+                    _lib.lib().fg_spmm_plan_destroy(plan)
+                except Exception:
+                    pass
+                lay['plan'] = None
 
     def _preprocess_adj(self, adj_scipy_csr, num_col_partitions=1):
         return util_convert_csr_to_dds(adj_scipy_csr, num_col_partitions)
@@ -112,7 +124,20 @@ class SpMMbase(object):
             notes.append("num_cuda_blocks has no counterpart: work items, not row blocks, are balanced")
         if T < 0 or (T > 0 and feat_len % T != 0):
             raise ValueError("feat_len %d is not divisible by num_feat_partitions %d" % (feat_len, T))
-        return ph, feat_len, int(T), notes
+        # Source-column partitions: the constructor's count when it was given, else chosen for
+        # the L2 size (the product is the same; later partitions add to the output in place).
+        P = self._num_col_partitions
+        src_parts = schedule_args.get('num_src_partitions', 'auto')
+        if P == 1 and src_parts is not None:
+            auto_p, auto_t = tuning.choose_spmm(self._num_rows, self._num_cols, self._adj_indices.shape[0], feat_len)
+            P = auto_p if src_parts == 'auto' else int(src_parts)
+            if P < 1:
+                raise ValueError("num_src_partitions must be >= 1")
+            if T == 0:
+                T = auto_t
+            if P > 1:
+                notes.append("%d source-column partitions chosen for the L2 size" % P)
+        return ph, feat_len, int(T), P, notes
 
     def build(self, input_placeholders, compute_args, schedule_args):
         """Fix the feature length and kernel variant, allocate the output once.
@@ -126,33 +151,32 @@ class SpMMbase(object):
             e.g. {'num_feat_partitions': T}: feature tiles handled by different workgroups
 
         schedule_args : dict
-            The reference's CUDA keys 'num_cuda_blocks' / 'num_threads_per_cuda_block' are accepted
+            The reference's CUDA keys 'num_cuda_blocks' / 'num_threads_per_cuda_block' are accepted.
+            'num_src_partitions': 'auto' (default) | int | None -- source-column partitions used
+            when the constructor was left at one partition (None: plain CSR).
         """
-        ph, feat_len, T, notes = self._resolve(input_placeholders, compute_args, schedule_args)
+        ph, feat_len, T, P, notes = self._resolve(input_placeholders, compute_args, schedule_args)
         self._placeholders = [ph]
         self._feat_len = feat_len
         self._num_feat_partitions = T
         self._notes = notes
-        self._func = (_lib.lib().fg_spmm_dds_f32 if self._num_col_partitions > 1
-                      else _lib.lib().fg_spmm_csr_f32)
+        self._active = self._layout(P)
+        self._func = _lib.lib().fg_spmm_dds_f32 if P > 1 else _lib.lib().fg_spmm_csr_f32
         self.out_tvm = torch.zeros((self._num_rows, feat_len), dtype=torch.float32, device=self._ctx)
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         """Return a text description of the plan and launch. This can be useful for debug."""
-        _, feat_len, T, notes = self._resolve(input_placeholders, compute_args, schedule_args)
+        _, feat_len, T, P, notes = self._resolve(input_placeholders, compute_args, schedule_args)
         buf = ctypes.create_string_buffer(4096)
-        _lib.check(_lib.lib().fg_spmm_plan_describe(self._plan, feat_len, T, buf, len(buf)))
+        _lib.check(_lib.lib().fg_spmm_plan_describe(self._layout(P)['plan'], feat_len, T, buf, len(buf)))
         text = buf.value.decode()
         for n in notes:
             text += "  note             : %s\n" % n
         return text
 
     def _launch(self, src_feat):
-        if self._num_col_partitions > 1:
-            pos, idx = self._adj_s1_pos_dev, self._adj_s1_idx_dev
-        else:
-            pos, idx = self._adj_indptr_dev, self._adj_indices_dev
-        _lib.check(self._func(self._plan, _lib.dev_ptr(pos), _lib.dev_ptr(idx), _lib.dev_ptr(self._adj_vals_dev),
+        lay = self._active
+        _lib.check(self._func(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(lay['vals']),
                               _lib.dev_ptr(src_feat), _lib.dev_ptr(self.out_tvm), self._feat_len,
                               self._num_feat_partitions, common.stream_ptr()))
 
@@ -196,7 +220,7 @@ class SpMMbase(object):
 class VanillaSpMMhip(SpMMbase):
     """CSR (or, with num_col_partitions > 1, DDS) SpMM on gfx950."""
     _compute_keys = ('num_feat_partitions',)
-    _schedule_keys = ('num_cuda_blocks', 'num_threads_per_cuda_block')
+    _schedule_keys = ('num_cuda_blocks', 'num_threads_per_cuda_block', 'num_src_partitions')
 
     def __init__(self, adj_scipy, num_col_partitions=1):
         super(VanillaSpMMhip, self).__init__(adj_scipy, num_col_partitions)
@@ -210,7 +234,7 @@ class VanillaSpMMx86(VanillaSpMMhip):
     """Constructor and knobs of the reference's VanillaSpMMx86
     (python/featgraph/module/spmm.py:197-209): source-column partitions at init,
     'num_feat_partitions' at build.  Both partitionings are carried out on the GPU."""
-    _schedule_keys = ()
+    _schedule_keys = ('num_src_partitions',)
 
 
 class VanillaSpMMcuda(VanillaSpMMhip):

@@ -1,0 +1,72 @@
+"""Default tiling / partitioning choices for gfx950 (MI355X: 8 XCDs, 4 MB of L2 each).
+
+A gathered feature row is useful to an XCD only through that XCD's L2, and workgroups are
+dealt to XCDs round-robin, so a kernel tile index that varies fastest with the workgroup id
+gives every XCD its own slice of the feature axis.  Source-column partitions then bound how
+many source rows an XCD touches per pass.  The numbers below come from sweeps on the
+232,965-node / 114.8M-edge power-law graph (feature lengths 32..512).
+"""
+
+TILE_FLOATS = 64                 # feature tile per workgroup: 256 B of every gathered row
+SPMM_SLICE_BYTES = 7.5e6         # per-XCD slice of X per pass (out is re-read every pass, so few passes)
+SDDMM_SLICE_BYTES = 2.0e6        # no read-modify-write per pass: the slice can really fit the L2
+MAX_PARTITIONS = 64
+
+
+def _pow2_floor(v):
+    p = 1
+    while p * 2 <= v:
+        p *= 2
+    return p
+
+
+def feature_tiles(feat_len):
+    """Number of feature tiles: tiles of TILE_FLOATS floats when that divides feat_len."""
+    if feat_len % TILE_FLOATS == 0:
+        return feat_len // TILE_FLOATS
+    return 1
+
+
+def _partitions(n_src, row_bytes, nnz, n_rows, slice_bytes, min_segment):
+    want = (n_src * row_bytes) / slice_bytes
+    if want <= 1.0:
+        return 1
+    p = _pow2_floor(int(want + 0.5)) if want >= 2 else 2
+    # keep row segments long enough to amortise the per-row work
+    avg_deg = nnz / max(1, n_rows)
+    while p > 1 and avg_deg / p < min_segment:
+        p //= 2
+    return max(1, min(MAX_PARTITIONS, p))
+
+
+def choose_spmm(n_dst, n_src, nnz, feat_len):
+    """(num_col_partitions, num_feat_partitions) for an SpMM of this size."""
+    t = feature_tiles(feat_len)
+    row_bytes = 4 * feat_len / min(t, 8) if t > 1 else 4 * feat_len
+    p = _partitions(n_src, row_bytes, nnz, n_dst, SPMM_SLICE_BYTES, min_segment=24)
+    return p, (t if t > 1 else 0)
+
+
+def choose_sddmm(n_rows, n_cols, nnz, heads, head_len):
+    """(num_src_partitions, num_feat_tiles) for the tiled traversal, or None when the plain
+    kernels should be used (small feature matrices, or a shape the tiled kernel does not take)."""
+    feat_len = heads * head_len
+    tile = None
+    for cand in (64, 128, 256, 32, 16):
+        if feat_len % cand != 0:
+            continue
+        if heads == 1 or cand % head_len == 0 or (head_len == cand):
+            if heads > 1 and (head_len % 4 != 0 or head_len < 8 or (head_len & (head_len - 1)) != 0):
+                continue
+            tile = cand
+            break
+    if tile is None:
+        return None
+    t = feat_len // tile
+    row_bytes = 4 * feat_len / min(t, 8)
+    if n_cols * row_bytes <= 2 * SDDMM_SLICE_BYTES:
+        return None
+    p = _partitions(n_cols, row_bytes, nnz, n_rows, SDDMM_SLICE_BYTES, min_segment=8)
+    if p == 1 and t == 1:
+        return None
+    return p, t

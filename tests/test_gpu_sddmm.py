@@ -132,6 +132,61 @@ def test_multihead(torch_cuda, oracle, H, D, order):
         np.testing.assert_allclose(out[:, 0], flat.cpu().numpy(), rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("order", ["csr", "shuffled"])
+@pytest.mark.parametrize("feat_len,P,T", [(512, 4, 8), (512, 1, 8), (128, 3, 2), (64, 1, 1), (256, 2, 1), (32, 5, 2),
+                                           (1024, 2, 8), (2048, 3, 8), (128, 64, 8)])
+def test_tiled_traversal(torch_cuda, oracle, feat_len, P, T, order):
+    """Source-column-partitioned, feature-tiled traversal (per-tile partial sums added by a second
+    kernel): same values, in the stored edge order, for CSR-ordered and arbitrarily ordered edges."""
+    from featgraph_amd.module import VanillaSDDMMhip
+    rng = np.random.default_rng(31 * feat_len + P)
+    coo = _rand_coo(rng, 140, 1500, 0.03).tolil()
+    coo[[0, 70, 139], :] = 0
+    coo[9, rng.choice(1500, 1400, replace=False)] = 1          # longer than the split threshold
+    coo = coo.tocsr(); coo.eliminate_zeros(); coo.sort_indices(); coo = coo.tocoo()
+    if order == "shuffled":
+        p = rng.permutation(coo.nnz)
+        coo = sp.coo_matrix((coo.data[p], (coo.row[p], coo.col[p])), shape=coo.shape)
+    src = rng.standard_normal((1500, feat_len)).astype("float32")
+    dst = rng.standard_normal((140, feat_len)).astype("float32")
+    m, out = _run(torch_cuda, VanillaSDDMMhip, coo, src, dst, {},
+                  {'order': 'tiled', 'num_src_partitions': P, 'num_feat_tiles': T})
+    assert m._tiled is not None and "tiled" in m.lower_to_ir(m._placeholders, {}, {'order': 'tiled'})
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([torch_cuda.from_numpy(src).cuda(), torch_cuda.from_numpy(dst).cuda()]).cpu().numpy()
+    assert_sum_close(out, oracle.sddmm_f64(coo.row, coo.col, src, dst), sddmm_mass(coo.row, coo.col, src, dst),
+                     "F=%d P=%d T=%d %s" % (feat_len, P, T, order))
+
+
+@pytest.mark.parametrize("H,D,P,T", [(8, 64, 4, 8), (4, 32, 2, 2), (8, 32, 3, 1), (2, 8, 2, 1), (4, 64, 1, 4),
+                                     (16, 16, 2, 4), (4, 256, 2, 4)])
+def test_tiled_multihead(torch_cuda, oracle, H, D, P, T):
+    """Whole heads per feature tile: results go straight to out[edge, head]."""
+    from featgraph_amd.module import MultiHeadSDDMMhip
+    rng = np.random.default_rng(H * 1000 + D)
+    coo = _rand_coo(rng, 150, 900, 0.05, shuffle=True)
+    src = rng.standard_normal((900, H, D)).astype("float32")
+    dst = rng.standard_normal((150, H, D)).astype("float32")
+    m, out = _run(torch_cuda, MultiHeadSDDMMhip, coo, src, dst, {},
+                  {'order': 'tiled', 'num_src_partitions': P, 'num_feat_tiles': T})
+    assert m._tiled is not None
+    expect = np.einsum("ehd,ehd->eh", src[coo.col].astype("f8"), dst[coo.row].astype("f8"))
+    assert_sum_close(out.cpu().numpy(), expect, sddmm_mass(coo.row, coo.col, src, dst), "H=%d D=%d" % (H, D))
+
+
+def test_tiled_rejects_bad_shapes(torch_cuda):
+    from featgraph_amd.module import VanillaSDDMMhip, MultiHeadSDDMMhip, placeholder
+    rng = np.random.default_rng(1)
+    coo = _rand_coo(rng, 20, 30, 0.3)
+    torch = torch_cuda
+    for cls, shp, T in ((VanillaSDDMMhip, (100,), 1), (VanillaSDDMMhip, (96,), 2), (MultiHeadSDDMMhip, (2, 128), 4),
+                        (MultiHeadSDDMMhip, (3, 20), 1)):
+        m = cls(coo)
+        m.build([placeholder((30,) + shp), placeholder((20,) + shp)], {}, {'order': 'tiled', 'num_feat_tiles': T})
+        with pytest.raises(ValueError):
+            m.run([torch.zeros((30,) + shp, device="cuda"), torch.zeros((20,) + shp, device="cuda")])
+
+
 @pytest.mark.parametrize("R,C", [(1, 5), (3, 1), (4, 4), (7, 2), (127, 255)])
 def test_partitioned_orders(torch_cuda, oracle, R, C):
     """COO order, CSR order and every 2-D partitioned order give the same values after
@@ -200,7 +255,10 @@ def test_powerlaw_23k(torch_cuda, oracle, feat_len):
     ref = oracle.sddmm_f64(coo.row, coo.col, src, dst)
     mass = sddmm_mass(coo.row, coo.col, src, dst)
     ref32 = oracle.sddmm_x86(coo.row, coo.col, src, dst)
-    for sched, ctor in (({'order': 'csr'}, ()), ({'order': 'coo'}, ()), ({}, (8, 8))):
+    tiles = max(1, feat_len // 64)
+    for sched, ctor in (({'order': 'csr'}, ()), ({'order': 'coo'}, ()), ({}, (8, 8)),
+                        ({'order': 'tiled', 'num_src_partitions': 4, 'num_feat_tiles': tiles}, ()),
+                        ({'order': 'tiled', 'num_src_partitions': 16, 'num_feat_tiles': tiles}, (3, 3))):
         m, out = _run(torch_cuda, VanillaSDDMMhip, coo, src, dst, {}, sched, *ctor)
         got = out.cpu().numpy()
         if ctor:
@@ -236,6 +294,12 @@ def test_full_size_properties(torch_cuda):
     assert ((out.double() - expect).abs() <= ATOL + RTOL * expect.abs() + 1e-6 * src.double().abs().sum(1)[col_d]).all()
 
     out_csr = m.run([src, dst]).clone()
+    m3 = VanillaSDDMMhip(adj)
+    m3.build([placeholder((n, F)), placeholder((n, F))], {}, {})        # default: tiled traversal at this size
+    assert m3._tiled is not None
+    out_tiled = m3.run([src, dst])
+    assert ((out_csr - out_tiled).abs() <= ATOL + RTOL * out_tiled.abs() + 1e-4).all()
+    del m3, out_tiled
     m2 = VanillaSDDMMhip(adj)
     m2.build([placeholder((n, F)), placeholder((n, F))], {}, {'order': 'coo'})
     out_coo = m2.run([src, dst])

@@ -128,6 +128,20 @@ def test_tilings_and_partitions(torch_cuda, oracle, feat_len, T, P):
     assert "spmm_items_kernel" in text and "work items" in text
 
 
+@pytest.mark.parametrize("src_parts", [None, 1, 3, 'auto'])
+def test_internal_source_partitions(torch_cuda, oracle, src_parts):
+    """The constructor's single partition can be replaced by internal source-column partitions
+    at build time; the CSR copy on the device stays bit-exact."""
+    from featgraph_amd.module import VanillaSpMMhip
+    rng = np.random.default_rng(77)
+    adj = _adj_with_long_and_empty_rows(rng, 200, 2500, 1800)
+    x = rng.standard_normal((2500, 128)).astype("float32")
+    m, out = _run(torch_cuda, VanillaSpMMhip, adj, x, {}, {'num_src_partitions': src_parts})
+    assert_sum_close(out.cpu().numpy(), oracle.spmm_f64(adj, x), spmm_mass(adj, x))
+    assert np.array_equal(m._adj_indices_dev.cpu().numpy(), adj.indices)
+    assert m._active['P'] == (3 if src_parts == 3 else 1)
+
+
 def test_output_fully_overwritten_and_reused(torch_cuda, oracle):
     """run() returns the same tensor every time and writes every element (no stale data),
     also rows without edges (module/spmm.py:161; te.sum over an empty range is 0)."""
