@@ -3,14 +3,17 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One step = one weighted CSR SpMM followed by one edge-wise SDDMM (CSR edge order), both at
+One step = one weighted CSR SpMM followed by one edge-wise SDDMM (edges stored in CSR order), both at
 feature length 512 on the seeded 232,965-node / ~114.8M-edge power-law graph, graph and
 features resident in HBM, outputs preallocated (the protocol of measure_average_time,
 python/featgraph/module/spmm.py:179-186).  Prints ONE JSON line; `value` is
 2 * (2 * nnz * F) flops per step over the measured step time.
 
-`roofline` prices the slower of the two launches against the 8 TB/s HBM peak with the
-compulsory-traffic byte model:
+`roofline` prices the slower of the two operators against the 8 TB/s HBM peak with the
+compulsory-traffic byte model (an operator is one C-ABI call; on this graph it is several
+launches of one kernel, one per source-column partition, so `achieved` = the operator's
+algorithmic bytes / the HIP-event time of all its launches, and `avg_launch_ms` is that time
+divided by the number of launches):
     SpMM  : 4(N+1) + 8 nnz + 4 N F (X once) + 4 N F (out once)
     SDDMM : 4(N+1) + 4 nnz (CSR order; 8 nnz in COO order) + 8 N F + 4 nnz H
 `cpu_baseline` times the CPU oracle (a C restatement of the reference's x86 schedules: SpMM
@@ -133,7 +136,7 @@ def main():
     spmm = VanillaSpMMhip(adj, args.num_col_partitions)
     spmm.build([placeholder((n, F))], {'num_feat_partitions': args.num_feat_partitions}, {})
     sddmm = VanillaSDDMMhip(adj)
-    sddmm.build([placeholder((n, F)), placeholder((n, F))], {}, {'order': 'csr'})
+    sddmm.build([placeholder((n, F)), placeholder((n, F))], {}, {})
     del adj
 
     def step(ev=None):
@@ -165,10 +168,14 @@ def main():
     ops = {
         "spmm": {"ms": t_spmm, "gflops": flops_op / t_spmm / 1e6, "compulsory_gb": b_spmm / 1e9,
                  "hbm_gbs": b_spmm / t_spmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_spmm / 1e6,
-                 "kernel": "spmm_items_kernel"},
+                 "kernel": "spmm_items_kernel", "launches": spmm._active['P'],
+                 "num_col_partitions": spmm._active['P'], "num_feat_partitions": spmm._num_feat_partitions},
         "sddmm": {"ms": t_sddmm, "gflops": flops_op / t_sddmm / 1e6, "compulsory_gb": b_sddmm / 1e9,
                   "hbm_gbs": b_sddmm / t_sddmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_sddmm / 1e6,
-                  "kernel": "sddmm_csr_kernel"},
+                  "kernel": "sddmm_tiled_kernel" if sddmm._tiled else "sddmm_csr_kernel",
+                  "launches": sddmm._tiled[0]['P'] if sddmm._tiled else 1,
+                  "num_src_partitions": sddmm._tiled[0]['P'] if sddmm._tiled else 1,
+                  "num_feat_tiles": sddmm._tiled[1] if sddmm._tiled else 1},
     }
     for o in ops.values():
         o["pct_hbm_roofline"] = 100.0 * o["hbm_gbs"] / HBM_PEAK_GBS
@@ -181,13 +188,14 @@ def main():
     roofline = {"bound": "hbm", "kernel": ops[dom]["kernel"], "achieved": round(ops[dom]["hbm_gbs"], 2),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ops[dom]["hbm_gbs"] / HBM_PEAK_GBS, 5),
                 "traffic": traffic, "algorithmic_bytes": int(b_spmm if dom == "spmm" else b_sddmm),
-                "avg_launch_ms": round(ops[dom]["ms"], 4)}
+                "launches": ops[dom]["launches"], "op_ms": round(ops[dom]["ms"], 4),
+                "avg_launch_ms": round(ops[dom]["ms"] / ops[dom]["launches"], 4)}
 
     line = {
         "metric": METRIC, "value": round(2 * flops_op / (ms_per_step * 1e6), 2), "unit": "GFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "%s: CSR SpMM + CSR-order SDDMM, F=%d, fp32, int32 indices" % (args.workload, F),
+        "config": {"workload": "%s: weighted CSR SpMM + SDDMM over the same edges, F=%d, fp32, int32 indices" % (args.workload, F),
                    "nodes": n, "edges": nnz, "max_in_degree": int(deg.max()), "median_in_degree": float(np.median(deg)),
                    "feat_len": F, "num_feat_partitions": args.num_feat_partitions,
                    "num_col_partitions": args.num_col_partitions, "seeds": {"graph": 0xFEA7, "weights": 1, "features": 2}},

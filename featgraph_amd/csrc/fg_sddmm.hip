@@ -38,11 +38,24 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// v from another lane of the same 16-lane row, chosen by a DPP control word (no LDS traffic).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
 // Sum over the RW consecutive lanes of a head segment; every lane of the segment gets it.
+// Inside a 16-lane row the butterfly runs on DPP moves: swap neighbours, swap pairs, mirror
+// the half row (the other quad's sum), mirror the row (the other half's sum); only the 32- and
+// 64-lane steps go through the LDS crossbar.
 template <int RW>
 __device__ __forceinline__ float segment_sum(float v) {
-#pragma unroll
-    for (int off = 1; off < RW; off <<= 1) v += __shfl_xor(v, off);
+    if (RW >= 2) v += dpp_move<0xB1>(v);     // quad_perm [1,0,3,2]
+    if (RW >= 4) v += dpp_move<0x4E>(v);     // quad_perm [2,3,0,1]
+    if (RW >= 8) v += dpp_move<0x141>(v);    // row_half_mirror
+    if (RW >= 16) v += dpp_move<0x140>(v);   // row_mirror
+    if (RW >= 32) v += __shfl_xor(v, 16);
+    if (RW >= 64) v += __shfl_xor(v, 32);
     return v;
 }
 
@@ -258,10 +271,10 @@ struct SddmmTiledArgs {
 // `e`), all U src loads issued back to back; lanes without an edge re-read edge e-1.  Every
 // head's U results end up one per lane (lane position u of the head segment keeps result u) and
 // are stored by those lanes.
-template <int L, int RW, int U, bool SCATTER>
-__device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int jstride, int e, const float *sb,
-                                                 int64_t F, const float4 &dv, float *out, int64_t estride,
-                                                 int64_t e_base, int seg_pos) {
+template <int L, int RW, int U, bool SCATTER, bool OFF32>
+__device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int jstride, int e, const float *src,
+                                                 uint32_t lane_bytes, int64_t F, const float4 &dv, float *out,
+                                                 int64_t estride, int64_t e_base, int seg_pos) {
     static_assert(U <= RW, "one result per lane of a head segment");
     int2 ce[U];
     float4 sv[U];
@@ -271,7 +284,11 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
         ce[u] = edge[j < e ? j : e - 1];
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u) sv[u] = *reinterpret_cast<const float4 *>(sb + (int64_t)ce[u].x * F);
+    for (int u = 0; u < U; ++u) {
+        const char *base = reinterpret_cast<const char *>(src);
+        sv[u] = OFF32 ? *reinterpret_cast<const float4 *>(base + ((uint32_t)ce[u].x + lane_bytes))
+                      : *reinterpret_cast<const float4 *>(base + (int64_t)ce[u].x * F * 4 + lane_bytes);
+    }
     float mine = 0.f;
     int my_pos = 0;
 #pragma unroll
@@ -286,7 +303,7 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
     }
 }
 
-template <int L, int RW, bool SCATTER>
+template <int L, int RW, bool SCATTER, bool OFF32>
 __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArgs a) {
     constexpr int G = 64 / L;
     constexpr int U = RW < 8 ? RW : 8;
@@ -303,7 +320,8 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     if (it.len == 0) return;
     const int64_t F = a.F;
     const int f_lo = tile * (L * 4) + li * 4;
-    const float *sb = a.src + f_lo;
+    const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
+    const uint32_t scale = OFF32 ? (uint32_t)a.F * 4u : 1u;
     const float *db = a.dst + f_lo;
     const int seg_pos = li % RW;
     float *out = a.out + (int64_t)tile * a.out_tile_stride + li / RW;
@@ -314,7 +332,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int t = min(lane + 64 * i, n - 1);
-            r[i] = make_int2(a.col[base + t], SCATTER ? a.edge_pos[base + t] : 0);
+            r[i] = make_int2((int)((uint32_t)a.col[base + t] * scale), SCATTER ? a.edge_pos[base + t] : 0);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) edge[lane + 64 * i] = r[i];
@@ -334,8 +352,8 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
                 if (e > b) {
                     const float4 dv = *reinterpret_cast<const float4 *>(db + (int64_t)(it.row + q) * F);
                     for (int s0 = b; s0 < e; s0 += G * U)
-                        sddmm_tile_batch<L, RW, U, SCATTER>(edge, s0 + g, G, e, sb, F, dv, out, a.out_edge_stride,
-                                                            it.start, seg_pos);
+                        sddmm_tile_batch<L, RW, U, SCATTER, OFF32>(edge, s0 + g, G, e, a.src, lane_bytes, F, dv, out,
+                                                                   a.out_edge_stride, it.start, seg_pos);
                 }
                 b = e;
             }
@@ -360,7 +378,8 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
             }
             if (__all(done)) break;
             if (!done && j < e) {
-                sddmm_tile_batch<L, RW, U, SCATTER>(edge, j, 1, e, sb, F, dv, out, a.out_edge_stride, it.start, seg_pos);
+                sddmm_tile_batch<L, RW, U, SCATTER, OFF32>(edge, j, 1, e, a.src, lane_bytes, F, dv, out,
+                                                           a.out_edge_stride, it.start, seg_pos);
                 j += U;
             }
         }
@@ -374,8 +393,8 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         stage((int64_t)it.start + base, n);
         wave_lds_sync();
         for (int s0 = 0; s0 < n; s0 += G * U)
-            sddmm_tile_batch<L, RW, U, SCATTER>(edge, s0 + g, G, n, sb, F, dv, out, a.out_edge_stride,
-                                                (int64_t)it.start + base, seg_pos);
+            sddmm_tile_batch<L, RW, U, SCATTER, OFF32>(edge, s0 + g, G, n, a.src, lane_bytes, F, dv, out,
+                                                       a.out_edge_stride, (int64_t)it.start + base, seg_pos);
     }
 }
 
@@ -389,27 +408,33 @@ __global__ __launch_bounds__(256) void sddmm_tile_sum_kernel(const float *partia
     out[edge_pos[e]] = s;
 }
 
+template <int L, int RW, bool SCATTER>
+void launch_tiled_off(bool off32, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
+    if (off32) hipLaunchKernelGGL((sddmm_tiled_kernel<L, RW, SCATTER, true>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((sddmm_tiled_kernel<L, RW, SCATTER, false>), grid, dim3(kBlock), 0, st, a);
+}
+
 template <int L, bool SCATTER>
-bool launch_tiled(int RW, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
+bool launch_tiled(int RW, bool off32, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
     switch (RW) {
-        case 2: if constexpr (L >= 2) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 2, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
-        case 4: if constexpr (L >= 4) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 4, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
-        case 8: if constexpr (L >= 8) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 8, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
-        case 16: if constexpr (L >= 16) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 16, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
-        case 32: if constexpr (L >= 32) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 32, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
-        case 64: if constexpr (L >= 64) { hipLaunchKernelGGL((sddmm_tiled_kernel<L, 64, SCATTER>), grid, dim3(kBlock), 0, st, a); return true; } break;
+        case 2: if constexpr (L >= 2) { launch_tiled_off<L, 2, SCATTER>(off32, grid, st, a); return true; } break;
+        case 4: if constexpr (L >= 4) { launch_tiled_off<L, 4, SCATTER>(off32, grid, st, a); return true; } break;
+        case 8: if constexpr (L >= 8) { launch_tiled_off<L, 8, SCATTER>(off32, grid, st, a); return true; } break;
+        case 16: if constexpr (L >= 16) { launch_tiled_off<L, 16, SCATTER>(off32, grid, st, a); return true; } break;
+        case 32: if constexpr (L >= 32) { launch_tiled_off<L, 32, SCATTER>(off32, grid, st, a); return true; } break;
+        case 64: if constexpr (L >= 64) { launch_tiled_off<L, 64, SCATTER>(off32, grid, st, a); return true; } break;
     }
     return false;
 }
 
 template <bool SCATTER>
-bool launch_tiled_l(int L, int RW, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
+bool launch_tiled_l(int L, int RW, bool off32, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
     switch (L) {
-        case 4: return launch_tiled<4, SCATTER>(RW, grid, st, a);
-        case 8: return launch_tiled<8, SCATTER>(RW, grid, st, a);
-        case 16: return launch_tiled<16, SCATTER>(RW, grid, st, a);
-        case 32: return launch_tiled<32, SCATTER>(RW, grid, st, a);
-        case 64: return launch_tiled<64, SCATTER>(RW, grid, st, a);
+        case 4: return launch_tiled<4, SCATTER>(RW, off32, grid, st, a);
+        case 8: return launch_tiled<8, SCATTER>(RW, off32, grid, st, a);
+        case 16: return launch_tiled<16, SCATTER>(RW, off32, grid, st, a);
+        case 32: return launch_tiled<32, SCATTER>(RW, off32, grid, st, a);
+        case 64: return launch_tiled<64, SCATTER>(RW, off32, grid, st, a);
     }
     return false;
 }
@@ -650,8 +675,9 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
         a.src = src_dev + (int64_t)p * width * F;
         const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * T;
         if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
-        const bool ok = tile_sum ? launch_tiled_l<false>(L, RW, dim3((unsigned)blocks), st, a)
-                                 : launch_tiled_l<true>(L, RW, dim3((unsigned)blocks), st, a);
+        const bool off32 = (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
+        const bool ok = tile_sum ? launch_tiled_l<false>(L, RW, off32, dim3((unsigned)blocks), st, a)
+                                 : launch_tiled_l<true>(L, RW, off32, dim3((unsigned)blocks), st, a);
         if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d RW=%d", L, RW);
     }
     if (tile_sum) {

@@ -70,13 +70,24 @@ __device__ __forceinline__ float4 vselect(bool c, const float4 &a) {
 }
 __device__ __forceinline__ float vselect(bool c, const float &a) { return c ? a : 0.f; }
 
-// Adds vals * X rows for the staged elements [b, e) of s_edge (x = column id, y = weight bits)
-// into acc.  The G lane groups take elements b+g, b+g+G, ...; U steps' loads are issued back to
-// back before the first use.  No load sits under a branch: in the last, partly filled batch a
-// lane without an element re-reads the row's last element and its value is replaced by zero.
-template <int V, int L, int K, bool FULL, int U>
-__device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, int g, const float *xb,
-                                            int64_t F, const bool (&on)[K], typename Vec<V>::type (&acc)[K]) {
+// Address of this lane's part of a staged source row.  OFF32: the staged word is the row's byte
+// offset from the (wave-uniform) start of X and fits 32 bits, so the load takes a scalar base
+// plus a 32-bit lane offset and no 64-bit multiply is left in the loop; otherwise it is the
+// column id.
+template <bool OFF32>
+__device__ __forceinline__ const float *row_ptr(const float *x, uint32_t lane_bytes, int64_t F, int staged) {
+    if (OFF32) return reinterpret_cast<const float *>(reinterpret_cast<const char *>(x) + ((uint32_t)staged + lane_bytes));
+    return reinterpret_cast<const float *>(reinterpret_cast<const char *>(x + (int64_t)staged * F) + lane_bytes);
+}
+
+// Adds vals * X rows for the staged elements [b, e) of s_edge (x = staged column word, y =
+// weight bits) into acc.  The G lane groups take elements b+g, b+g+G, ...; U steps' loads are
+// issued back to back before the first use.  No load sits under a branch: in the last, partly
+// filled batch a lane without an element re-reads the row's last element with weight zero.
+template <int V, int L, int K, bool FULL, int U, bool OFF32>
+__device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, int g, const float *x,
+                                            uint32_t lane_bytes, int64_t F, const bool (&on)[K],
+                                            typename Vec<V>::type (&acc)[K]) {
     using vec = typename Vec<V>::type;
     constexpr int G = 64 / L;
     int s0 = b;
@@ -89,7 +100,8 @@ __device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, in
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int k = 0; k < K; ++k)
-                if (FULL || on[k]) xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)cw[u].x * F + k * L * V);
+                if (FULL || on[k])
+                    xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<OFF32>(x, lane_bytes, F, cw[u].x) + k * L * V);
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -98,24 +110,24 @@ __device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, in
     }
     if (s0 < e) {                          // uniform: fewer than G*U elements left
         int2 cw[U];
-        bool ok[U];
         vec xv[U][K];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int j = s0 + u * G + g;
-            ok[u] = j < e;
-            cw[u] = s_edge[ok[u] ? j : e - 1];
+            cw[u] = s_edge[j < e ? j : e - 1];
+            if (j >= e) cw[u].y = 0;
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int k = 0; k < K; ++k)
-                if (FULL || on[k]) xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)cw[u].x * F + k * L * V);
+                if (FULL || on[k])
+                    xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<OFF32>(x, lane_bytes, F, cw[u].x) + k * L * V);
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int k = 0; k < K; ++k)
-                if (FULL || on[k]) vfma(acc[k], ok[u] ? __int_as_float(cw[u].y) : 0.f, vselect(ok[u], xv[u][k]));
+                if (FULL || on[k]) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
     }
 }
 
@@ -142,12 +154,13 @@ __device__ __forceinline__ void finish_row(typename Vec<V>::type (&acc)[K], cons
 
 // Loads elements [base, base + min(n, 256)) of (indices, vals) into registers, 4 per lane; lanes
 // past the end re-read the last element so that no load is conditional.  n >= 1.
+// `scale` turns a column id into the staged word: the row's byte size (OFF32) or 1.
 __device__ __forceinline__ void stage_load(const int32_t *indices, const float *vals, int64_t base, int n,
-                                           int lane, int2 (&r)[4]) {
+                                           int lane, uint32_t scale, int2 (&r)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int t = min(lane + 64 * i, n - 1);
-        r[i] = make_int2(indices[base + t], __float_as_int(vals[base + t]));
+        r[i] = make_int2((int)((uint32_t)indices[base + t] * scale), __float_as_int(vals[base + t]));
     }
 }
 __device__ __forceinline__ void stage_store(int2 *edge, int lane, const int2 (&r)[4]) {
@@ -156,8 +169,9 @@ __device__ __forceinline__ void stage_store(int2 *edge, int lane, const int2 (&r
 }
 
 // V: floats per lane per load; L: lanes per source row; K: loads per lane per source row;
-// FULL: every lane's columns are inside the tile (no masking needed); ACC: add to out.
-template <int V, int L, int K, bool FULL, bool ACC>
+// FULL: every lane's columns are inside the tile (no masking needed); ACC: add to out;
+// OFF32: X spans less than 4 GiB, rows are addressed by 32-bit byte offsets.
+template <int V, int L, int K, bool FULL, bool ACC, bool OFF32>
 __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     using vec = typename Vec<V>::type;
     static_assert(fg::kItemEdges == 256, "stage_load/stage_store move 4 x 64 elements");
@@ -182,7 +196,8 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     bool on[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
-    const float *xb = a.x + f_lo;
+    const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
+    const uint32_t scale = OFF32 ? (uint32_t)a.F * 4u : 1u;
     const int64_t F = a.F;
     int2 *edge = s_edge[wave];
     vec acc[K], old[K];
@@ -192,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
         // Several whole rows: stage all their elements once.
         const int nrows = -it.info;
         if (it.len > 0) {
-            stage_load(a.indices, a.vals, it.start, it.len, lane, regs);
+            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, regs);
             stage_store(edge, lane, regs);
         }
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
@@ -212,7 +227,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
                     }
 #pragma unroll
                     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
-                    gather_rows<V, L, K, FULL, U>(edge, b, e, g, xb, F, on, acc);
+                    gather_rows<V, L, K, FULL, U, OFF32>(edge, b, e, g, a.x, lane_bytes, F, on, acc);
                     finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
                 }
                 b = e;
@@ -258,23 +273,23 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
             if (__all(done)) break;
             if (!done && j < e) {
                 int2 cw[U];
-                bool ok[U];
                 vec xv[U][K];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    ok[u] = j + u < e;
-                    cw[u] = edge[ok[u] ? j + u : e - 1];
+                    cw[u] = edge[j + u < e ? j + u : e - 1];
+                    if (j + u >= e) cw[u].y = 0;
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u)
 #pragma unroll
                     for (int k = 0; k < K; ++k)
-                        if (FULL || on[k]) xv[u][k] = *reinterpret_cast<const vec *>(xb + (int64_t)cw[u].x * F + k * L * V);
+                        if (FULL || on[k])
+                            xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<OFF32>(a.x, lane_bytes, F, cw[u].x) + k * L * V);
 #pragma unroll
                 for (int u = 0; u < U; ++u)
 #pragma unroll
                     for (int k = 0; k < K; ++k)
-                        if (FULL || on[k]) vfma(acc[k], ok[u] ? __int_as_float(cw[u].y) : 0.f, vselect(ok[u], xv[u][k]));
+                        if (FULL || on[k]) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
                 j += U;
             }
         }
@@ -287,7 +302,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     const bool add = ACC && it.info < 0;
 #pragma unroll
     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
-    if (it.len > 0) stage_load(a.indices, a.vals, it.start, it.len, lane, regs);
+    if (it.len > 0) stage_load(a.indices, a.vals, it.start, it.len, lane, scale, regs);
     if (ACC) {
 #pragma unroll
         for (int k = 0; k < K; ++k)
@@ -300,8 +315,8 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
         wave_lds_sync();
         if (base + fg::kItemEdges < it.len)
             stage_load(a.indices, a.vals, (int64_t)it.start + base + fg::kItemEdges,
-                       it.len - base - fg::kItemEdges, lane, regs);
-        gather_rows<V, L, K, FULL, U>(edge, 0, n, g, xb, F, on, acc);
+                       it.len - base - fg::kItemEdges, lane, scale, regs);
+        gather_rows<V, L, K, FULL, U, OFF32>(edge, 0, n, g, a.x, lane_bytes, F, on, acc);
     }
     finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
 }
@@ -329,6 +344,7 @@ struct SpmmConfig {
     int V, L, K;
     int tile_w, sub_per_tile, n_ftiles;
     bool full;
+    bool off32;     // every source row starts less than 4 GiB into X
 };
 
 int pow2_ceil(int v) { int p = 1; while (p < v) p <<= 1; return p; }
@@ -353,14 +369,20 @@ int choose_config(int F, int T, bool aligned16, SpmmConfig *c) {
     return FG_OK;
 }
 
+template <int V, int L, int K, bool FULL, bool ACC>
+void launch_off(bool off32, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+    if (off32) hipLaunchKernelGGL((spmm_items_kernel<V, L, K, FULL, ACC, true>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, FULL, ACC, false>), grid, dim3(kBlock), 0, st, a);
+}
+
 template <int V, int L, int K>
-void launch_vlk(bool full, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+void launch_vlk(bool full, bool off32, dim3 grid, hipStream_t st, const SpmmArgs &a) {
     if (a.accumulate) {
-        if (full) hipLaunchKernelGGL((spmm_items_kernel<V, L, K, true, true>), grid, dim3(kBlock), 0, st, a);
-        else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, false, true>), grid, dim3(kBlock), 0, st, a);
+        if (full) launch_off<V, L, K, true, true>(off32, grid, st, a);
+        else launch_off<V, L, K, false, true>(off32, grid, st, a);
     } else {
-        if (full) hipLaunchKernelGGL((spmm_items_kernel<V, L, K, true, false>), grid, dim3(kBlock), 0, st, a);
-        else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, false, false>), grid, dim3(kBlock), 0, st, a);
+        if (full) launch_off<V, L, K, true, false>(off32, grid, st, a);
+        else launch_off<V, L, K, false, false>(off32, grid, st, a);
     }
 }
 
@@ -368,14 +390,14 @@ template <int V>
 int launch_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs &a) {
     if (c.K == 1) {
         switch (c.L) {
-            case 4: launch_vlk<V, 4, 1>(c.full, grid, st, a); return FG_OK;
-            case 8: launch_vlk<V, 8, 1>(c.full, grid, st, a); return FG_OK;
-            case 16: launch_vlk<V, 16, 1>(c.full, grid, st, a); return FG_OK;
-            case 32: launch_vlk<V, 32, 1>(c.full, grid, st, a); return FG_OK;
-            case 64: launch_vlk<V, 64, 1>(c.full, grid, st, a); return FG_OK;
+            case 4: launch_vlk<V, 4, 1>(c.full, c.off32, grid, st, a); return FG_OK;
+            case 8: launch_vlk<V, 8, 1>(c.full, c.off32, grid, st, a); return FG_OK;
+            case 16: launch_vlk<V, 16, 1>(c.full, c.off32, grid, st, a); return FG_OK;
+            case 32: launch_vlk<V, 32, 1>(c.full, c.off32, grid, st, a); return FG_OK;
+            case 64: launch_vlk<V, 64, 1>(c.full, c.off32, grid, st, a); return FG_OK;
         }
-    } else if (c.L == 64 && c.K == 2) { launch_vlk<V, 64, 2>(c.full, grid, st, a); return FG_OK; }
-    else if (c.L == 64 && c.K == 4) { launch_vlk<V, 64, 4>(c.full, grid, st, a); return FG_OK; }
+    } else if (c.L == 64 && c.K == 2) { launch_vlk<V, 64, 2>(c.full, c.off32, grid, st, a); return FG_OK; }
+    else if (c.L == 64 && c.K == 4) { launch_vlk<V, 64, 4>(c.full, c.off32, grid, st, a); return FG_OK; }
     return fail(FG_ERR_SHAPE, "no SpMM kernel for V=%d L=%d K=%d", V, c.L, c.K);
 }
 
@@ -399,6 +421,7 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
     int rc = choose_config(F, T, aligned16, &c);
     if (rc != FG_OK) return rc;
     if ((rc = ensure_partial(pl, F)) != FG_OK) return rc;
+    c.off32 = (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;

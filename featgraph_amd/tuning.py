@@ -9,7 +9,7 @@ many source rows an XCD touches per pass.  The numbers below come from sweeps on
 
 TILE_FLOATS = 64                 # feature tile per workgroup: 256 B of every gathered row
 SPMM_SLICE_BYTES = 7.5e6         # per-XCD slice of X per pass (out is re-read every pass, so few passes)
-SDDMM_SLICE_BYTES = 2.0e6        # no read-modify-write per pass: the slice can really fit the L2
+SDDMM_SLICE_BYTES = 7.5e6        # same optimum measured for SDDMM: shorter row segments cost more than misses
 MAX_PARTITIONS = 64
 
 
@@ -64,9 +64,9 @@ def choose_sddmm(n_rows, n_cols, nnz, heads, head_len):
         return None
     t = feat_len // tile
     row_bytes = 4 * feat_len / min(t, 8)
-    if n_cols * row_bytes <= 2 * SDDMM_SLICE_BYTES:
+    if n_cols * row_bytes <= SDDMM_SLICE_BYTES:
         return None
-    p = _partitions(n_cols, row_bytes, nnz, n_rows, SDDMM_SLICE_BYTES, min_segment=8)
+    p = _partitions(n_cols, row_bytes, nnz, n_rows, SDDMM_SLICE_BYTES, min_segment=24)
     if p == 1 and t == 1:
         return None
     return p, t
