@@ -30,6 +30,13 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# Fabric-side bytes (rocprofv3 FETCH_SIZE x2 + WRITE_SIZE, scaled by the X copy of the same run) moved
+# by all launches of the named kernel in one operator call, at the default tiling; from
+# profiles/bench_powerlaw233k_f512_rocprofv3.txt.  Other configurations have no measurement: null.
+MEASURED_TRAFFIC = {
+    ("spmm", "powerlaw-233k", 512, 8, 8): 67.6e9,      # 8 x spmm_items_kernel (+ fix-ups)
+    ("sddmm", "powerlaw-233k", 512, 8, 8): 66.2e9,     # 8 x sddmm_tiled_kernel (tile sum: +5.1e9)
+}
 METRIC = "SpMM/SDDMM GFLOP/s + achieved HBM GB/s (% roofline), 233k-node graph, feat 512"
 
 
@@ -149,6 +156,12 @@ def main():
         if ev is not None:
             ev[2].record()
 
+    # One plain device copy of X (reads and writes n*F*4 bytes each): the reference point that
+    # rocprofv3's FETCH_SIZE / WRITE_SIZE counters of the kernels are scaled by.
+    x_copy = torch.empty_like(x_d)
+    x_copy.copy_(x_d)
+    del x_copy
+
     for _ in range(args.warmup):
         step()
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
@@ -180,11 +193,9 @@ def main():
     for o in ops.values():
         o["pct_hbm_roofline"] = 100.0 * o["hbm_gbs"] / HBM_PEAK_GBS
     dom = "spmm" if t_spmm >= t_sddmm else "sddmm"
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic_%s_f%d_%s.json" % (dom, F, args.workload))
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch")
+    key = (dom, args.workload, F, ops[dom]["launches"],
+           ops[dom].get("num_feat_partitions", ops[dom].get("num_feat_tiles")))
+    traffic = MEASURED_TRAFFIC.get(key)
     roofline = {"bound": "hbm", "kernel": ops[dom]["kernel"], "achieved": round(ops[dom]["hbm_gbs"], 2),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ops[dom]["hbm_gbs"] / HBM_PEAK_GBS, 5),
                 "traffic": traffic, "algorithmic_bytes": int(b_spmm if dom == "spmm" else b_sddmm),
