@@ -245,7 +245,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_csr_kernel(const SddmmArgs a) {
 //
 // For graphs whose feature matrices do not fit the L2 caches.  The edge list is a DDS copy of
 // the adjacency (column partition by column partition, CSR inside a partition) and the feature
-// axis is cut into tiles of L*4 floats; workgroup id = item block * n_tiles + tile, so the 8
+// axis is cut into tiles of L*K*4 floats; workgroup id = item block * n_tiles + tile, so the 8
 // XCDs (dealt workgroups round-robin) work on the same edges but different tiles and each L2
 // holds one tile's slice of one partition's src rows.  A head (RW lanes) must lie inside a tile.
 // One head per edge in total means the tiles hold partial dot products: they go to
@@ -268,16 +268,17 @@ struct SddmmTiledArgs {
 };
 
 // One batch: U edges of one row for this lane group (edge j0 + u*jstride, u < U, those below
-// `e`), all U src loads issued back to back; lanes without an edge re-read edge e-1.  Every
+// `e`), all U*K src loads issued back to back; lanes without an edge re-read edge e-1.  Every
 // head's U results end up one per lane (lane position u of the head segment keeps result u) and
 // are stored by those lanes.
-template <int L, int RW, int U, bool SCATTER, bool OFF32>
+template <int L, int K, int RW, int KH, int U, bool SCATTER, bool OFF32>
 __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int jstride, int e, const float *src,
-                                                 uint32_t lane_bytes, int64_t F, const float4 &dv, float *out,
+                                                 uint32_t lane_bytes, int64_t F, const float4 (&dv)[K], float *out,
                                                  int64_t estride, int64_t e_base, int seg_pos) {
     static_assert(U <= RW, "one result per lane of a head segment");
+    constexpr int NH = K / KH, HPL = L / RW;
     int2 ce[U];
-    float4 sv[U];
+    float4 sv[U][K];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int j = j0 + u * jstride;
@@ -286,28 +287,42 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const char *base = reinterpret_cast<const char *>(src);
-        sv[u] = OFF32 ? *reinterpret_cast<const float4 *>(base + ((uint32_t)ce[u].x + lane_bytes))
-                      : *reinterpret_cast<const float4 *>(base + (int64_t)ce[u].x * F * 4 + lane_bytes);
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            sv[u][k] = OFF32 ? *reinterpret_cast<const float4 *>(base + ((uint32_t)ce[u].x + lane_bytes) + k * L * 16)
+                             : *reinterpret_cast<const float4 *>(base + (int64_t)ce[u].x * F * 4 + lane_bytes + k * L * 16);
     }
-    float mine = 0.f;
+    float mine[NH];
     int my_pos = 0;
 #pragma unroll
+    for (int kk = 0; kk < NH; ++kk) mine[kk] = 0.f;
+#pragma unroll
     for (int u = 0; u < U; ++u) {
-        const float p = segment_sum<RW>(vdot(sv[u], dv));
-        if (seg_pos == u) { mine = p; my_pos = ce[u].y; }
+#pragma unroll
+        for (int kk = 0; kk < NH; ++kk) {
+            float p = 0.f;
+#pragma unroll
+            for (int k = kk * KH; k < (kk + 1) * KH; ++k) p += vdot(sv[u][k], dv[k]);
+            p = segment_sum<RW>(p);
+            if (seg_pos == u) mine[kk] = p;
+        }
+        if (seg_pos == u) my_pos = ce[u].y;
     }
     const int ju = j0 + seg_pos * jstride;
     if (seg_pos < U && ju < e) {
         const int64_t at = SCATTER ? (int64_t)my_pos : e_base + ju;
-        out[at * estride] = mine;
+#pragma unroll
+        for (int kk = 0; kk < NH; ++kk) out[at * estride + kk * HPL] = mine[kk];
     }
 }
 
-template <int L, int RW, bool SCATTER, bool OFF32>
+// L lanes x K loads cover one tile of L*K*4 floats of an edge's operands; RW lanes per head inside
+// one load (KH == 1) or a head spanning KH loads (RW == L).
+template <int L, int K, int RW, int KH, bool SCATTER, bool OFF32>
 __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArgs a) {
     constexpr int G = 64 / L;
-    constexpr int U = RW < 8 ? RW : 8;
-    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges];     // x = column id, y = edge_pos
+    constexpr int U = (RW < 8 ? RW : 8) / (K >= 2 ? 2 : 1) > 0 ? (RW < 8 ? RW : 8) / (K >= 2 ? 2 : 1) : 1;
+    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges];     // x = column word, y = edge_pos
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
     __shared__ int32_t s_next[kWavesPerBlock];
 
@@ -319,13 +334,14 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     const Item it = a.items[item_id];
     if (it.len == 0) return;
     const int64_t F = a.F;
-    const int f_lo = tile * (L * 4) + li * 4;
+    const int f_lo = tile * (L * K * 4) + li * 4;
     const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
     const uint32_t scale = OFF32 ? (uint32_t)a.F * 4u : 1u;
     const float *db = a.dst + f_lo;
     const int seg_pos = li % RW;
     float *out = a.out + (int64_t)tile * a.out_tile_stride + li / RW;
     int2 *edge = s_edge[wave];
+    float4 dv[K];
 
     auto stage = [&](int64_t base, int n) {
         int2 r[4];
@@ -336,6 +352,10 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) edge[lane + 64 * i] = r[i];
+    };
+    auto load_dst = [&](int64_t row) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) dv[k] = *reinterpret_cast<const float4 *>(db + row * F + k * L * 4);
     };
 
     if (it.info < -1) {
@@ -350,10 +370,10 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
             for (int q = 0; q < nrows; ++q) {
                 const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
                 if (e > b) {
-                    const float4 dv = *reinterpret_cast<const float4 *>(db + (int64_t)(it.row + q) * F);
+                    load_dst(it.row + q);
                     for (int s0 = b; s0 < e; s0 += G * U)
-                        sddmm_tile_batch<L, RW, U, SCATTER, OFF32>(edge, s0 + g, G, e, a.src, lane_bytes, F, dv, out,
-                                                                   a.out_edge_stride, it.start, seg_pos);
+                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32>(edge, s0 + g, G, e, a.src, lane_bytes, F, dv,
+                                                                          out, a.out_edge_stride, it.start, seg_pos);
                 }
                 b = e;
             }
@@ -362,7 +382,8 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         // many short rows: every lane group walks rows of its own
         int q = -1, j = 0, e = 0;
         bool done = false;
-        float4 dv = vzero4();
+#pragma unroll
+        for (int k = 0; k < K; ++k) dv[k] = vzero4();
         for (;;) {
             if (!done && j >= e) {
                 int qn = 0;
@@ -373,28 +394,28 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
                 } else {
                     j = q ? s_end[wave][q - 1] : 0;
                     e = s_end[wave][q];
-                    if (e > j) dv = *reinterpret_cast<const float4 *>(db + (int64_t)(it.row + q) * F);
+                    if (e > j) load_dst(it.row + q);
                 }
             }
             if (__all(done)) break;
             if (!done && j < e) {
-                sddmm_tile_batch<L, RW, U, SCATTER, OFF32>(edge, j, 1, e, a.src, lane_bytes, F, dv, out,
-                                                           a.out_edge_stride, it.start, seg_pos);
+                sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32>(edge, j, 1, e, a.src, lane_bytes, F, dv, out,
+                                                                  a.out_edge_stride, it.start, seg_pos);
                 j += U;
             }
         }
         return;
     }
     // one row, or one piece of a long row
-    const float4 dv = *reinterpret_cast<const float4 *>(db + (int64_t)it.row * F);
+    load_dst(it.row);
     for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
         const int n = min(fg::kItemEdges, it.len - base);
         wave_lds_sync();
         stage((int64_t)it.start + base, n);
         wave_lds_sync();
         for (int s0 = 0; s0 < n; s0 += G * U)
-            sddmm_tile_batch<L, RW, U, SCATTER, OFF32>(edge, s0 + g, G, n, a.src, lane_bytes, F, dv, out,
-                                                       a.out_edge_stride, (int64_t)it.start + base, seg_pos);
+            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32>(edge, s0 + g, G, n, a.src, lane_bytes, F, dv, out,
+                                                              a.out_edge_stride, (int64_t)it.start + base, seg_pos);
     }
 }
 
@@ -408,33 +429,47 @@ __global__ __launch_bounds__(256) void sddmm_tile_sum_kernel(const float *partia
     out[edge_pos[e]] = s;
 }
 
-template <int L, int RW, bool SCATTER>
+template <int L, int K, int RW, int KH, bool SCATTER>
 void launch_tiled_off(bool off32, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
-    if (off32) hipLaunchKernelGGL((sddmm_tiled_kernel<L, RW, SCATTER, true>), grid, dim3(kBlock), 0, st, a);
-    else hipLaunchKernelGGL((sddmm_tiled_kernel<L, RW, SCATTER, false>), grid, dim3(kBlock), 0, st, a);
+    if (off32) hipLaunchKernelGGL((sddmm_tiled_kernel<L, K, RW, KH, SCATTER, true>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((sddmm_tiled_kernel<L, K, RW, KH, SCATTER, false>), grid, dim3(kBlock), 0, st, a);
 }
 
-template <int L, bool SCATTER>
-bool launch_tiled(int RW, bool off32, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
+// heads narrower than one load: RW lanes per head, KH == 1
+template <int L, int K, bool SCATTER>
+bool launch_tiled_rw(int RW, bool off32, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
     switch (RW) {
-        case 2: if constexpr (L >= 2) { launch_tiled_off<L, 2, SCATTER>(off32, grid, st, a); return true; } break;
-        case 4: if constexpr (L >= 4) { launch_tiled_off<L, 4, SCATTER>(off32, grid, st, a); return true; } break;
-        case 8: if constexpr (L >= 8) { launch_tiled_off<L, 8, SCATTER>(off32, grid, st, a); return true; } break;
-        case 16: if constexpr (L >= 16) { launch_tiled_off<L, 16, SCATTER>(off32, grid, st, a); return true; } break;
-        case 32: if constexpr (L >= 32) { launch_tiled_off<L, 32, SCATTER>(off32, grid, st, a); return true; } break;
-        case 64: if constexpr (L >= 64) { launch_tiled_off<L, 64, SCATTER>(off32, grid, st, a); return true; } break;
+        case 2: if constexpr (L >= 2) { launch_tiled_off<L, K, 2, 1, SCATTER>(off32, grid, st, a); return true; } break;
+        case 4: if constexpr (L >= 4) { launch_tiled_off<L, K, 4, 1, SCATTER>(off32, grid, st, a); return true; } break;
+        case 8: if constexpr (L >= 8) { launch_tiled_off<L, K, 8, 1, SCATTER>(off32, grid, st, a); return true; } break;
+        case 16: if constexpr (L >= 16) { launch_tiled_off<L, K, 16, 1, SCATTER>(off32, grid, st, a); return true; } break;
+        case 32: if constexpr (L >= 32) { launch_tiled_off<L, K, 32, 1, SCATTER>(off32, grid, st, a); return true; } break;
     }
     return false;
 }
 
+// KH: loads per head (0 = heads narrower than a load, RW lanes each)
+template <int L, int K, bool SCATTER>
+bool launch_tiled_lk(int RW, int KH, bool off32, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
+    if (KH == 0) return launch_tiled_rw<L, K, SCATTER>(RW, off32, grid, st, a);
+    if (KH == 1) { launch_tiled_off<L, K, L, 1, SCATTER>(off32, grid, st, a); return true; }
+    if constexpr (K >= 2) { if (KH == 2) { launch_tiled_off<L, K, L, 2, SCATTER>(off32, grid, st, a); return true; } }
+    return false;
+}
+
 template <bool SCATTER>
-bool launch_tiled_l(int L, int RW, bool off32, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
-    switch (L) {
-        case 4: return launch_tiled<4, SCATTER>(RW, off32, grid, st, a);
-        case 8: return launch_tiled<8, SCATTER>(RW, off32, grid, st, a);
-        case 16: return launch_tiled<16, SCATTER>(RW, off32, grid, st, a);
-        case 32: return launch_tiled<32, SCATTER>(RW, off32, grid, st, a);
-        case 64: return launch_tiled<64, SCATTER>(RW, off32, grid, st, a);
+bool launch_tiled_l(int L, int K, int RW, int KH, bool off32, dim3 grid, hipStream_t st, const SddmmTiledArgs &a) {
+    if (K == 1) {
+        switch (L) {
+            case 4: return launch_tiled_lk<4, 1, SCATTER>(RW, KH, off32, grid, st, a);
+            case 8: return launch_tiled_lk<8, 1, SCATTER>(RW, KH, off32, grid, st, a);
+            case 16: return launch_tiled_lk<16, 1, SCATTER>(RW, KH, off32, grid, st, a);
+        }
+    } else if (K == 2) {
+        switch (L) {
+            case 16: return launch_tiled_lk<16, 2, SCATTER>(RW, KH, off32, grid, st, a);
+            case 32: return launch_tiled_lk<32, 2, SCATTER>(RW, KH, off32, grid, st, a);
+        }
     }
     return false;
 }
@@ -643,17 +678,23 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
     const int tile_w = F / T;
     if (tile_w % 4 != 0 || tile_w > 256 || !is_pow2(tile_w / 4) || tile_w < 16)
         return fail(FG_ERR_SHAPE, "feature tile of %d floats: need a power of two between 16 and 256", tile_w);
-    const int L = tile_w / 4;
-    int RW;                       // lanes per head inside a tile
+    // tile = L lanes x K loads x 4 floats: two loads per lane from 128 floats up, so that a lane's own
+    // share of the dot product is longer and the cross-lane sum is paid once per 8 floats
+    const int K = tile_w >= 128 ? 2 : 1;
+    const int L = tile_w / 4 / K;
+    const int load_w = L * 4;     // floats covered by one load of the lane group
+    int RW, KH;                   // lanes per head inside a load / loads per head (0: head narrower than a load)
     bool tile_sum;                // tiles hold partial sums of one head
     if (D >= tile_w) {
         if (D % tile_w != 0) return fail(FG_ERR_SHAPE, "head length %d is not a multiple of the %d-float tile", D, tile_w);
         if (D > tile_w && H != 1) return fail(FG_ERR_SHAPE, "a head spanning several tiles needs H == 1");
-        RW = L; tile_sum = D > tile_w;
+        RW = L; KH = K; tile_sum = D > tile_w;
     } else {
         if (tile_w % D != 0 || D % 4 != 0 || !is_pow2(D / 4) || D < 8)
             return fail(FG_ERR_SHAPE, "head length %d does not pack into a %d-float tile", D, tile_w);
-        RW = D / 4; tile_sum = false;
+        if (D >= load_w) { RW = L; KH = D / load_w; }
+        else { RW = D / 4; KH = 0; }
+        tile_sum = false;
     }
     hipStream_t st = (hipStream_t)stream;
     SddmmTiledArgs a;
@@ -676,9 +717,9 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
         const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * T;
         if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
         const bool off32 = (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
-        const bool ok = tile_sum ? launch_tiled_l<false>(L, RW, off32, dim3((unsigned)blocks), st, a)
-                                 : launch_tiled_l<true>(L, RW, off32, dim3((unsigned)blocks), st, a);
-        if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d RW=%d", L, RW);
+        const bool ok = tile_sum ? launch_tiled_l<false>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a)
+                                 : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
+        if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);
     }
     if (tile_sum) {
         const unsigned blocks = (unsigned)((pl->nnz + 255) / 256);

@@ -61,7 +61,8 @@ struct SpmmArgs {
     int F;                 // row stride of x / out in floats
     int tile_w;            // floats per requested feature tile (F / num_feat_partitions)
     int sub_per_tile;      // kernel tiles (V*L*K floats each) per requested tile
-    int n_ftiles;          // num_feat_partitions * sub_per_tile
+    int n_ftiles;          // kernel tiles handled by this launch (consecutive, starting at tile_base)
+    int tile_base;
     int accumulate;        // add to out instead of overwriting it
 };
 
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int tile = (int)(blockIdx.x % (unsigned)a.n_ftiles);
+    const int tile = a.tile_base + (int)(blockIdx.x % (unsigned)a.n_ftiles);
     const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_ftiles) * kWavesPerBlock + wave;
     if (item_id >= a.n_items) return;      // uniform per wavefront; no workgroup barriers below
     const Item it = a.items[item_id];
@@ -434,12 +435,19 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
             a.indices = idx; a.vals = vals;
             a.x = x + (int64_t)p * width * F;
             a.out = out; a.partial = pl->partial_dev;
-            a.F = F; a.tile_w = c.tile_w; a.sub_per_tile = c.sub_per_tile; a.n_ftiles = c.n_ftiles;
+            a.F = F; a.tile_w = c.tile_w; a.sub_per_tile = c.sub_per_tile;
             a.accumulate = p > 0;
-            const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * c.n_ftiles;
-            if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
-            rc = (c.V == 4) ? launch_v<4>(c, dim3((unsigned)blocks), st, a) : launch_v<1>(c, dim3((unsigned)blocks), st, a);
-            if (rc != FG_OK) return rc;
+            // More than 8 tiles: 8 at a time (one per XCD), so that an XCD's L2 serves one tile's
+            // slice of this partition per launch; the partition's index arrays stay in the
+            // memory-side cache between the launches.
+            const int per_launch = (c.n_ftiles > 8 && c.n_ftiles % 8 == 0) ? 8 : c.n_ftiles;
+            for (int tb = 0; tb < c.n_ftiles; tb += per_launch) {
+                a.n_ftiles = per_launch; a.tile_base = tb;
+                const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
+                if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
+                rc = (c.V == 4) ? launch_v<4>(c, dim3((unsigned)blocks), st, a) : launch_v<1>(c, dim3((unsigned)blocks), st, a);
+                if (rc != FG_OK) return rc;
+            }
         }
         const int64_t x0 = pl->fixup_off[p], x1 = pl->fixup_off[p + 1];
         if (x1 > x0) {
