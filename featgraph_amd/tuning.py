@@ -44,6 +44,10 @@ def choose_spmm(n_dst, n_src, nnz, feat_len):
     t = feature_tiles(feat_len)
     row_bytes = 4 * feat_len / min(t, 8) if t > 1 else 4 * feat_len
     p = _partitions(n_src, row_bytes, nnz, n_dst, SPMM_SLICE_BYTES, min_segment=24)
+    if p == 1 and feat_len <= 256:
+        # rows too short to partition: nothing is reused through the L2 anyway, and whole rows per
+        # wavefront cost the fewest index reads (measured on the 2.45M-node / 61.9M-edge graph)
+        return 1, 1
     return p, (t if t > 1 else 0)
 
 
@@ -67,6 +71,11 @@ def choose_sddmm(n_rows, n_cols, nnz, heads, head_len):
     if n_cols * row_bytes <= SDDMM_SLICE_BYTES:
         return None
     p = _partitions(n_cols, row_bytes, nnz, n_rows, SDDMM_SLICE_BYTES, min_segment=24)
-    if p == 1 and t == 1:
-        return None
+    if p == 1:
+        # rows too short to partition: one tile per edge when the kernel takes the whole row
+        if feat_len <= 256 and (feat_len & (feat_len - 1)) == 0 and feat_len >= 16 and \
+                (heads == 1 or feat_len % head_len == 0):
+            return 1, 1
+        if t == 1:
+            return None
     return p, t

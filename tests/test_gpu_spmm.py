@@ -305,3 +305,50 @@ def test_full_size_properties(torch_cuda):
         e = slice(indptr[v], indptr[v + 1])
         terms = vals[e].astype(np.float64)[:, None] * xh[indices[e]].astype(np.float64)
         assert_sum_close(outh[v], terms.sum(0), np.abs(terms).sum(0), "row %d" % v)
+
+
+def test_low_degree_large_graph_properties(torch_cuda):
+    """2.45M nodes / ~61.9M edges (average degree 25), F = 128: SpMM followed by SDDMM on the same
+    edges, checked through a column-sum checksum, all-ones row sums and sampled edges."""
+    from featgraph_amd import synthetic
+    from featgraph_amd.module import VanillaSpMMhip, VanillaSDDMMhip, placeholder
+    torch = torch_cuda
+    indptr, indices = synthetic.make_workload("powerlaw-2.45M")
+    n = indptr.shape[0] - 1
+    nnz = indices.shape[0]
+    F = 128
+    g = torch.Generator(device="cuda"); g.manual_seed(5)
+    vals_d = torch.rand(nnz, generator=g, device="cuda", dtype=torch.float32)
+    vals = vals_d.cpu().numpy()
+    adj = sp.csr_matrix((vals, indices, indptr), shape=(n, n))
+    x = torch.randn((n, F), generator=g, device="cuda")
+    y = torch.randn((n, F), generator=g, device="cuda")
+    idx_d = torch.from_numpy(indices).cuda().long()
+
+    m = VanillaSpMMhip(adj)
+    m.build([placeholder((n, F))], {}, {})
+    assert np.array_equal(m._adj_indptr_dev.cpu().numpy(), indptr)
+    out = m.run([x])
+    col_w = torch.zeros(n, device="cuda", dtype=torch.float64)
+    col_w.index_add_(0, idx_d, vals_d.double())
+    expect = (col_w[:, None] * x.double()).sum(0)
+    scale = (col_w[:, None] * x.double().abs()).sum(0)
+    assert ((out.double().sum(0) - expect).abs() <= 1e-5 * scale).all()
+    ones = torch.ones((n, F), device="cuda")
+    row_sum = np.add.reduceat(vals.astype(np.float64), indptr[:-1])
+    got = m.run([ones]).cpu().numpy()
+    np.testing.assert_allclose(got[:, 0], row_sum, rtol=RTOL, atol=ATOL)
+    assert (got[:, -1] == got[:, 0]).all()
+
+    s = VanillaSDDMMhip(adj)
+    s.build([placeholder((n, F)), placeholder((n, F))], {}, {})
+    e_out = s.run([x, y])
+    pick = torch.randint(0, nnz, (300000,), generator=g, device="cuda")
+    r = s._adj_row_indices_dev.long()[pick]
+    c = s._adj_col_indices_dev.long()[pick]
+    prod = x[c].double() * y[r].double()
+    ref = prod.sum(1)
+    assert ((e_out[pick].double() - ref).abs() <= ATOL + RTOL * ref.abs() + 1e-6 * prod.abs().sum(1)).all()
+    for e in (0, nnz - 1):
+        rr, cc = int(s._adj_row_indices[e]), int(s._adj_col_indices[e])
+        assert abs(e_out[e].item() - float((x[cc].double() * y[rr].double()).sum())) <= 1e-3
