@@ -271,7 +271,8 @@ struct SddmmTiledArgs {
 // `e`), all U*K src loads issued back to back; lanes without an edge re-read edge e-1.  Every
 // head's U results end up one per lane (lane position u of the head segment keeps result u) and
 // are stored by those lanes.
-template <int L, int K, int RW, int KH, int U, bool SCATTER, bool OFF32>
+constexpr int kTilePad = 8;   // staging slots past the last edge that the unclamped walk may read
+template <int L, int K, int RW, int KH, int U, bool SCATTER, bool OFF32, bool CLAMP>
 __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int jstride, int e, const float *src,
                                                  uint32_t lane_bytes, int64_t F, const float4 (&dv)[K], float *out,
                                                  int64_t estride, int64_t e_base, int seg_pos) {
@@ -282,7 +283,9 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int j = j0 + u * jstride;
-        ce[u] = edge[j < e ? j : e - 1];
+        // !CLAMP (consecutive edges): slots past the row's end hold later rows' edges or the
+        // padding -- loadable, and their results are not stored
+        ce[u] = edge[(!CLAMP || j < e) ? j : e - 1];
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -322,7 +325,8 @@ template <int L, int K, int RW, int KH, bool SCATTER, bool OFF32>
 __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArgs a) {
     constexpr int G = 64 / L;
     constexpr int U = (RW < 8 ? RW : 8) / (K >= 2 ? 2 : 1) > 0 ? (RW < 8 ? RW : 8) / (K >= 2 ? 2 : 1) : 1;
-    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges];     // x = column word, y = edge_pos
+    static_assert(U <= kTilePad, "unclamped reads must stay inside the padded staging row");
+    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges + kTilePad];     // x = column word, y = edge_pos
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
     __shared__ int32_t s_next[kWavesPerBlock];
 
@@ -352,6 +356,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) edge[lane + 64 * i] = r[i];
+        if (lane < kTilePad) edge[fg::kItemEdges + lane] = r[3];
     };
     auto load_dst = [&](int64_t row) {
 #pragma unroll
@@ -372,7 +377,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
                 if (e > b) {
                     load_dst(it.row + q);
                     for (int s0 = b; s0 < e; s0 += G * U)
-                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32>(edge, s0 + g, G, e, a.src, lane_bytes, F, dv,
+                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, true>(edge, s0 + g, G, e, a.src, lane_bytes, F, dv,
                                                                           out, a.out_edge_stride, it.start, seg_pos);
                 }
                 b = e;
@@ -399,7 +404,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
             }
             if (__all(done)) break;
             if (!done && j < e) {
-                sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32>(edge, j, 1, e, a.src, lane_bytes, F, dv, out,
+                sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false>(edge, j, 1, e, a.src, lane_bytes, F, dv, out,
                                                                   a.out_edge_stride, it.start, seg_pos);
                 j += U;
             }
@@ -414,7 +419,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         stage((int64_t)it.start + base, n);
         wave_lds_sync();
         for (int s0 = 0; s0 < n; s0 += G * U)
-            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32>(edge, s0 + g, G, n, a.src, lane_bytes, F, dv, out,
+            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, true>(edge, s0 + g, G, n, a.src, lane_bytes, F, dv, out,
                                                               a.out_edge_stride, (int64_t)it.start + base, seg_pos);
     }
 }

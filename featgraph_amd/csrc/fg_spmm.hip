@@ -23,6 +23,7 @@ namespace {
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = 64 * kWavesPerBlock;
+constexpr int kPad = 8;
 
 template <int V> struct Vec;
 template <> struct Vec<4> { using type = float4; };
@@ -167,6 +168,7 @@ __device__ __forceinline__ void stage_load(const int32_t *indices, const float *
 __device__ __forceinline__ void stage_store(int2 *edge, int lane, const int2 (&r)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) edge[lane + 64 * i] = r[i];
+    if (lane < kPad) edge[fg::kItemEdges + lane] = r[3];      // a valid element: slots past the end stay loadable
 }
 
 // V: floats per lane per load; L: lanes per source row; K: loads per lane per source row;
@@ -178,8 +180,10 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     static_assert(fg::kItemEdges == 256, "stage_load/stage_store move 4 x 64 elements");
     constexpr int FT = V * L * K;          // floats per kernel tile
     constexpr int G = 64 / L;              // lane groups per wavefront
-    constexpr int U = (K >= 2) ? 4 : 8;    // steps whose loads are issued back to back
-    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges];
+    constexpr int U = (K >= 2) ? 2 : (L <= 8 ? 8 : 4);   // steps whose loads are issued back to back
+    static_assert(U <= kPad, "reads past a row's end must stay inside the padded staging row");
+    // kPad extra slots: the lane-group-per-row walk may read up to U - 1 slots past a row's end
+    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
     __shared__ int32_t s_next[kWavesPerBlock];
 
@@ -277,7 +281,9 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
                 vec xv[U][K];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    cw[u] = edge[j + u < e ? j + u : e - 1];
+                    // past the row's end this is a later row's element (or the padding): a valid
+                    // source row, given weight zero
+                    cw[u] = edge[j + u];
                     if (j + u >= e) cw[u].y = 0;
                 }
 #pragma unroll
