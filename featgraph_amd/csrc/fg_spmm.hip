@@ -65,6 +65,8 @@ struct SpmmArgs {
     int n_ftiles;          // kernel tiles handled by this launch (consecutive, starting at tile_base)
     int tile_base;
     int accumulate;        // add to out instead of overwriting it
+    int heads;             // weights are [nnz, heads]; a kernel tile lies inside one head
+    int head_len;          // floats per head (F / heads)
 };
 
 __device__ __forceinline__ float4 vselect(bool c, const float4 &a) {
@@ -156,13 +158,15 @@ __device__ __forceinline__ void finish_row(typename Vec<V>::type (&acc)[K], cons
 
 // Loads elements [base, base + min(n, 256)) of (indices, vals) into registers, 4 per lane; lanes
 // past the end re-read the last element so that no load is conditional.  n >= 1.
-// `scale` turns a column id into the staged word: the row's byte size (OFF32) or 1.
+// `scale` turns a column id into the staged word: the row's byte size (OFF32) or 1.  The weight of
+// element t is vals[t * vstride + voff] (one weight per head), or 1 when there are no weights.
 __device__ __forceinline__ void stage_load(const int32_t *indices, const float *vals, int64_t base, int n,
-                                           int lane, uint32_t scale, int2 (&r)[4]) {
+                                           int lane, uint32_t scale, int vstride, int voff, int2 (&r)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int t = min(lane + 64 * i, n - 1);
-        r[i] = make_int2((int)((uint32_t)indices[base + t] * scale), __float_as_int(vals[base + t]));
+        const float w = vals ? vals[(base + t) * vstride + voff] : 1.0f;
+        r[i] = make_int2((int)((uint32_t)indices[base + t] * scale), __float_as_int(w));
     }
 }
 __device__ __forceinline__ void stage_store(int2 *edge, int lane, const int2 (&r)[4]) {
@@ -203,6 +207,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
     const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
     const uint32_t scale = OFF32 ? (uint32_t)a.F * 4u : 1u;
+    const int voff = (rt * a.tile_w + st * FT) / a.head_len;     // head of this kernel tile
     const int64_t F = a.F;
     int2 *edge = s_edge[wave];
     vec acc[K], old[K];
@@ -212,7 +217,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
         // Several whole rows: stage all their elements once.
         const int nrows = -it.info;
         if (it.len > 0) {
-            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, regs);
+            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.heads, voff, regs);
             stage_store(edge, lane, regs);
         }
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
@@ -309,7 +314,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     const bool add = ACC && it.info < 0;
 #pragma unroll
     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
-    if (it.len > 0) stage_load(a.indices, a.vals, it.start, it.len, lane, scale, regs);
+    if (it.len > 0) stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.heads, voff, regs);
     if (ACC) {
 #pragma unroll
         for (int k = 0; k < K; ++k)
@@ -322,10 +327,155 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
         wave_lds_sync();
         if (base + fg::kItemEdges < it.len)
             stage_load(a.indices, a.vals, (int64_t)it.start + base + fg::kItemEdges,
-                       it.len - base - fg::kItemEdges, lane, scale, regs);
+                       it.len - base - fg::kItemEdges, lane, scale, a.heads, voff, regs);
         gather_rows<V, L, K, FULL, U, OFF32>(edge, 0, n, g, a.x, lane_bytes, F, on, acc);
     }
     finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
+}
+
+// ---- max / min aggregation ------------------------------------------------------------------------
+//
+// out[v, f] = max (or min) over the row's elements of vals[e] * X[indices[e], f]; a row without
+// elements gives 0.  Same items, staging and lane layout as the sum kernel; all lane groups share
+// each row in turn and a lane without an element in the last batch keeps its running extreme.
+
+template <bool IS_MAX> __device__ __forceinline__ float ext_identity() { return IS_MAX ? -INFINITY : INFINITY; }
+template <bool IS_MAX> __device__ __forceinline__ float ext_op(float a, float b) { return IS_MAX ? fmaxf(a, b) : fminf(a, b); }
+template <bool IS_MAX> __device__ __forceinline__ void vext(float4 &a, const float4 &b) {
+    a.x = ext_op<IS_MAX>(a.x, b.x); a.y = ext_op<IS_MAX>(a.y, b.y);
+    a.z = ext_op<IS_MAX>(a.z, b.z); a.w = ext_op<IS_MAX>(a.w, b.w);
+}
+template <bool IS_MAX> __device__ __forceinline__ void vext(float &a, const float &b) { a = ext_op<IS_MAX>(a, b); }
+__device__ __forceinline__ float4 vscale(float w, const float4 &x) { return make_float4(w * x.x, w * x.y, w * x.z, w * x.w); }
+__device__ __forceinline__ float vscale(float w, const float &x) { return w * x; }
+__device__ __forceinline__ float4 vsplat(float4, float v) { return make_float4(v, v, v, v); }
+__device__ __forceinline__ float vsplat(float, float v) { return v; }
+__device__ __forceinline__ float4 vpick(bool c, const float4 &a, const float4 &b) {
+    return make_float4(c ? a.x : b.x, c ? a.y : b.y, c ? a.z : b.z, c ? a.w : b.w);
+}
+__device__ __forceinline__ float vpick(bool c, const float &a, const float &b) { return c ? a : b; }
+
+template <int V, int L, int K, bool FULL, bool OFF32, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void gspmm_extreme_kernel(const SpmmArgs a) {
+    using vec = typename Vec<V>::type;
+    constexpr int FT = V * L * K;
+    constexpr int G = 64 / L;
+    constexpr int U = (K >= 2) ? 2 : 4;
+    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
+    __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int tile = a.tile_base + (int)(blockIdx.x % (unsigned)a.n_ftiles);
+    const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_ftiles) * kWavesPerBlock + wave;
+    if (item_id >= a.n_items) return;
+    const Item it = a.items[item_id];
+    const int g = lane / L, li = lane % L;
+    const int rt = tile / a.sub_per_tile, st = tile % a.sub_per_tile;
+    const int f_end = (rt + 1) * a.tile_w;
+    const int f_lo = rt * a.tile_w + st * FT + li * V;
+    bool on[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
+    const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
+    const uint32_t scale = OFF32 ? (uint32_t)a.F * 4u : 1u;
+    const int voff = (rt * a.tile_w + st * FT) / a.head_len;
+    const int64_t F = a.F;
+    int2 *edge = s_edge[wave];
+    int2 regs[4];
+    vec acc[K];
+
+    // running extreme over staged elements [b, e)
+    auto walk = [&](int b, int e) {
+        for (int s0 = b; s0 < e; s0 += G * U) {
+            int2 cw[U];
+            bool ok[U];
+            vec xv[U][K];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int j = s0 + u * G + g;
+                ok[u] = j < e;
+                cw[u] = edge[ok[u] ? j : e - 1];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    if (FULL || on[k])
+                        xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<OFF32>(a.x, lane_bytes, F, cw[u].x) + k * L * V);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    if (FULL || on[k]) {
+                        vec m = acc[k];
+                        vext<IS_MAX>(m, vscale(__int_as_float(cw[u].y), xv[u][k]));
+                        acc[k] = vpick(ok[u], m, acc[k]);
+                    }
+        }
+    };
+    auto reset = [&]() {
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc[k] = vsplat(vec(), ext_identity<IS_MAX>());
+    };
+    // combine the lane groups, store (an empty row stores 0)
+    auto finish = [&](float *dst, bool empty) {
+#pragma unroll
+        for (int off = L; off < 64; off <<= 1)
+#pragma unroll
+            for (int k = 0; k < K; ++k) vext<IS_MAX>(acc[k], vshfl_xor(acc[k], off));
+        if (g == 0) {
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (FULL || on[k]) *reinterpret_cast<vec *>(dst + k * L * V) = empty ? vzero(vec()) : acc[k];
+        }
+    };
+
+    if (it.info < -1) {
+        const int nrows = -it.info;
+        if (it.len > 0) {
+            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.heads, voff, regs);
+            stage_store(edge, lane, regs);
+        }
+        s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        wave_lds_sync();
+        int b = 0;
+        for (int q = 0; q < nrows; ++q) {
+            const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
+            reset();
+            walk(b, e);
+            finish(a.out + (int64_t)(it.row + q) * F + f_lo, e == b);
+            b = e;
+        }
+        return;
+    }
+    reset();
+    for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
+        const int n = min(fg::kItemEdges, it.len - base);
+        wave_lds_sync();
+        stage_load(a.indices, a.vals, (int64_t)it.start + base, n, lane, scale, a.heads, voff, regs);
+        stage_store(edge, lane, regs);
+        wave_lds_sync();
+        walk(0, n);
+    }
+    float *dst = (it.info < 0 ? a.out + (int64_t)it.row * F : a.partial + (int64_t)it.info * F) + f_lo;
+    finish(dst, it.len == 0);
+}
+
+// out[row, :] = max / min over the row's pieces.
+template <int V, bool IS_MAX>
+__global__ __launch_bounds__(256) void gspmm_extreme_fixup_kernel(const Fixup *fixups, int64_t n_fixups,
+                                                                  const float *partial, float *out, int F) {
+    using vec = typename Vec<V>::type;
+    const int per_row = F / V;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_fixups * per_row) return;
+    const Fixup fx = fixups[t / per_row];
+    const int f = (int)(t % per_row) * V;
+    vec m = *reinterpret_cast<const vec *>(partial + (int64_t)fx.slot0 * F + f);
+    for (int p = 1; p < fx.n_pieces; ++p)
+        vext<IS_MAX>(m, *reinterpret_cast<const vec *>(partial + (int64_t)(fx.slot0 + p) * F + f));
+    *reinterpret_cast<vec *>(out + (int64_t)fx.row * F + f) = m;
 }
 
 // out[row, :] (+)= sum of the row's pieces, in piece order.  One lane per V columns.
@@ -408,6 +558,32 @@ int launch_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs &a) 
     return fail(FG_ERR_SHAPE, "no SpMM kernel for V=%d L=%d K=%d", V, c.L, c.K);
 }
 
+template <int V, int L, int K, bool IS_MAX>
+void launch_ext_vlk(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+    if (c.full) {
+        if (c.off32) hipLaunchKernelGGL((gspmm_extreme_kernel<V, L, K, true, true, IS_MAX>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((gspmm_extreme_kernel<V, L, K, true, false, IS_MAX>), grid, dim3(kBlock), 0, st, a);
+    } else {
+        if (c.off32) hipLaunchKernelGGL((gspmm_extreme_kernel<V, L, K, false, true, IS_MAX>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((gspmm_extreme_kernel<V, L, K, false, false, IS_MAX>), grid, dim3(kBlock), 0, st, a);
+    }
+}
+
+template <int V, bool IS_MAX>
+int launch_ext_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+    if (c.K == 1) {
+        switch (c.L) {
+            case 4: launch_ext_vlk<V, 4, 1, IS_MAX>(c, grid, st, a); return FG_OK;
+            case 8: launch_ext_vlk<V, 8, 1, IS_MAX>(c, grid, st, a); return FG_OK;
+            case 16: launch_ext_vlk<V, 16, 1, IS_MAX>(c, grid, st, a); return FG_OK;
+            case 32: launch_ext_vlk<V, 32, 1, IS_MAX>(c, grid, st, a); return FG_OK;
+            case 64: launch_ext_vlk<V, 64, 1, IS_MAX>(c, grid, st, a); return FG_OK;
+        }
+    } else if (c.L == 64 && c.K == 2) { launch_ext_vlk<V, 64, 2, IS_MAX>(c, grid, st, a); return FG_OK; }
+    else if (c.L == 64 && c.K == 4) { launch_ext_vlk<V, 64, 4, IS_MAX>(c, grid, st, a); return FG_OK; }
+    return fail(FG_ERR_SHAPE, "no max/min kernel for V=%d L=%d K=%d", V, c.L, c.K);
+}
+
 int ensure_partial(const fg_spmm_plan *pl, int F) {
     const size_t need = (size_t)pl->max_slots_in_partition * (size_t)F;
     if (need <= pl->partial_floats) return FG_OK;
@@ -418,12 +594,31 @@ int ensure_partial(const fg_spmm_plan *pl, int F) {
     return FG_OK;
 }
 
+// reduce: FG_REDUCE_SUM / MAX / MIN.  heads > 1: vals is [nnz, heads] and every kernel tile must
+// lie inside one head.  vals == nullptr with allow_no_vals: every weight is 1.
 int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
-             const float *x, float *out, int F, int T, void *stream) {
+             const float *x, float *out, int F, int T, void *stream, int heads = 1,
+             int reduce = FG_REDUCE_SUM, bool allow_no_vals = false) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (pl->n_dst == 0) return FG_OK;
-    if (!out || !pos || (pl->nnz > 0 && (!idx || !vals || !x))) return fail(FG_ERR_ARG, "null device pointer");
+    if (!out || !pos || (pl->nnz > 0 && (!idx || (!vals && !allow_no_vals) || !x)))
+        return fail(FG_ERR_ARG, "null device pointer");
+    if (reduce != FG_REDUCE_SUM && reduce != FG_REDUCE_MAX && reduce != FG_REDUCE_MIN)
+        return fail(FG_ERR_ARG, "unknown reduce op %d", reduce);
+    if (reduce != FG_REDUCE_SUM && pl->num_col_partitions != 1)
+        return fail(FG_ERR_ARG, "max / min aggregation needs a plan with one column partition");
+    if (heads < 1 || F % heads != 0) return fail(FG_ERR_SHAPE, "feature length %d is not divisible by %d heads", F, heads);
     const bool aligned16 = (((uintptr_t)x | (uintptr_t)out) & 15) == 0;
+    if (heads > 1) {
+        // tiles must not straddle heads: tile = the head, or 64 floats when that divides the head
+        const int D = F / heads;
+        const int want = (D % 64 == 0) ? 64 : D;
+        if (want % 4 != 0 || want < 16 || (want & (want - 1)) != 0 || !aligned16)
+            return fail(FG_ERR_SHAPE, "per-head weights need a head length that is a power of two >= 16 or a multiple of 64, got %d", D);
+        if (T == 0) T = F / want;
+        if (T < 1 || F % T != 0 || D % (F / T) != 0 || (((F / T) & (F / T - 1)) != 0) || F / T > 256)
+            return fail(FG_ERR_SHAPE, "num_feat_partitions %d does not cut %d-float heads into power-of-two tiles", T, D);
+    }
     SpmmConfig c;
     int rc = choose_config(F, T, aligned16, &c);
     if (rc != FG_OK) return rc;
@@ -442,6 +637,7 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
             a.x = x + (int64_t)p * width * F;
             a.out = out; a.partial = pl->partial_dev;
             a.F = F; a.tile_w = c.tile_w; a.sub_per_tile = c.sub_per_tile;
+            a.heads = heads; a.head_len = F / heads;
             a.accumulate = p > 0;
             // More than 8 tiles: 8 at a time (one per XCD), so that an XCD's L2 serves one tile's
             // slice of this partition per launch; the partition's index arrays stay in the
@@ -451,7 +647,10 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
                 a.n_ftiles = per_launch; a.tile_base = tb;
                 const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
                 if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
-                rc = (c.V == 4) ? launch_v<4>(c, dim3((unsigned)blocks), st, a) : launch_v<1>(c, dim3((unsigned)blocks), st, a);
+                const dim3 grid((unsigned)blocks);
+                if (reduce == FG_REDUCE_SUM) rc = (c.V == 4) ? launch_v<4>(c, grid, st, a) : launch_v<1>(c, grid, st, a);
+                else if (reduce == FG_REDUCE_MAX) rc = (c.V == 4) ? launch_ext_v<4, true>(c, grid, st, a) : launch_ext_v<1, true>(c, grid, st, a);
+                else rc = (c.V == 4) ? launch_ext_v<4, false>(c, grid, st, a) : launch_ext_v<1, false>(c, grid, st, a);
                 if (rc != FG_OK) return rc;
             }
         }
@@ -460,12 +659,17 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
             const int fv = (aligned16 && F % 4 == 0) ? 4 : 1;
             const int64_t threads = (x1 - x0) * (F / fv);
             const unsigned blocks = (unsigned)((threads + 255) / 256);
-            if (fv == 4)
-                hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, pl->fixups_dev + x0,
-                                   x1 - x0, pl->partial_dev, out, F, (int)(p > 0));
-            else
-                hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, pl->fixups_dev + x0,
-                                   x1 - x0, pl->partial_dev, out, F, (int)(p > 0));
+            const Fixup *fx = pl->fixups_dev + x0;
+            if (reduce == FG_REDUCE_SUM) {
+                if (fv == 4) hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F, (int)(p > 0));
+                else hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F, (int)(p > 0));
+            } else if (reduce == FG_REDUCE_MAX) {
+                if (fv == 4) hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<4, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F);
+                else hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<1, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F);
+            } else {
+                if (fv == 4) hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<4, false>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F);
+                else hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<1, false>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F);
+            }
         }
     }
     FG_HIP_TRY(hipGetLastError());
@@ -504,4 +708,11 @@ extern "C" int fg_spmm_dds_f32(const fg_spmm_plan *plan, const int32_t *s1_pos_d
                                const int32_t *s1_idx_dev, const float *vals_dev, const float *x_dev,
                                float *out_dev, int F, int num_feat_partitions, void *stream) {
     return spmm_run(plan, s1_pos_dev, s1_idx_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
+}
+
+extern "C" int fg_gspmm_f32(const fg_spmm_plan *plan, const int32_t *pos_dev, const int32_t *idx_dev,
+                            const float *vals_dev, const float *x_dev, float *out_dev, int F, int heads,
+                            int reduce, int num_feat_partitions, void *stream) {
+    return spmm_run(plan, pos_dev, idx_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream, heads,
+                    reduce, /*allow_no_vals=*/true);
 }

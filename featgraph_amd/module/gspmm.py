@@ -1,0 +1,127 @@
+"""Generalised SpMM: aggregation by sum / mean / max / min, with one weight per edge, one weight
+per edge and head, or none.  The reference snapshot has no such operator (its README.md:9-11
+points to a branch with "generalized SpMM"); the class follows the build()/run() conventions of
+the reference's SpMM modules (python/featgraph/module/spmm.py:81-161)."""
+import ctypes
+
+import numpy as np
+import scipy.sparse
+import torch
+
+from .. import _lib
+from .. import tuning
+from ..util import util_convert_csr_to_dds
+from . import common
+from .spmm import VanillaSpMMhip
+
+_REDUCE = {'sum': 0, 'mean': 0, 'max': 1, 'min': 2}
+
+
+class GSpMMhip(VanillaSpMMhip):
+    """out[v, h, :] = reduce_{e in row v} w[e, h] * SrcFeat[indices[e], h, :].
+
+    compute_args: 'reduce' in {'sum', 'mean', 'max', 'min'} (default 'sum'); 'msg' in
+    {'u_mul_e', 'copy_u'} (default 'u_mul_e': the adjacency values, or the edge weights given
+    to run(); 'copy_u': weight 1); 'num_feat_partitions' as for VanillaSpMMhip.
+    SrcFeat is (num_cols, F) or (num_cols, H, D); with H > 1 the weights are (nnz, H) and must
+    be passed to run() as a second input, in the adjacency's CSR edge order.
+    Rows without edges give 0 for every reduce.
+    """
+    _compute_keys = ('num_feat_partitions', 'reduce', 'msg')
+
+    def build(self, input_placeholders, compute_args, schedule_args):
+        compute_args = dict(compute_args)
+        reduce = compute_args.pop('reduce', 'sum')
+        msg = compute_args.pop('msg', 'u_mul_e')
+        if reduce not in _REDUCE:
+            raise ValueError("reduce must be one of %s" % sorted(_REDUCE))
+        if msg not in ('u_mul_e', 'copy_u'):
+            raise ValueError("msg must be 'u_mul_e' or 'copy_u'")
+        if len(input_placeholders) not in (1, 2):
+            raise ValueError("GSpMM takes SrcFeat and optionally the edge weights")
+        src_ph = input_placeholders[0]
+        if len(src_ph.shape) not in (2, 3) or src_ph.shape[0] != self._num_cols:
+            raise ValueError("SrcFeat must be (num_cols=%d, F) or (num_cols, H, D), got %s" % (self._num_cols, src_ph.shape))
+        heads = src_ph.shape[1] if len(src_ph.shape) == 3 else 1
+        feat_len = int(np.prod(src_ph.shape[1:]))
+        nnz = self._adj_indices.shape[0]
+        weights_at_run = len(input_placeholders) == 2
+        if weights_at_run:
+            want = (nnz,) if heads == 1 else (nnz, heads)
+            if tuple(input_placeholders[1].shape) not in (want, (nnz, heads)):
+                raise ValueError("edge weights must have shape %s, got %s" % (want, input_placeholders[1].shape))
+            if msg == 'copy_u':
+                raise ValueError("msg='copy_u' takes no edge weights")
+        elif heads > 1 and msg == 'u_mul_e':
+            raise ValueError("per-head weights (nnz, H) must be passed to run() as a second input")
+        if reduce in ('max', 'min'):
+            schedule_args = dict(schedule_args, num_src_partitions=None)
+            if self._num_col_partitions != 1:
+                raise ValueError("max / min aggregation needs num_col_partitions == 1")
+        flat = common.placeholder((self._num_cols, feat_len))
+        _, _, T, P, notes = self._resolve([flat], compute_args, schedule_args)
+        self._placeholders = list(input_placeholders)
+        self._feat_len, self._heads, self._num_feat_partitions = feat_len, heads, (0 if heads > 1 and 'num_feat_partitions' not in compute_args else T)
+        self._reduce, self._msg, self._weights_at_run, self._notes = reduce, msg, weights_at_run, notes
+        self._active = self._glayout(P)
+        self._func = _lib.lib().fg_gspmm_f32
+        self._inv_deg_edge = None
+        if reduce == 'mean':
+            deg = np.diff(self._adj_indptr).astype(np.float32)
+            inv = np.where(deg > 0, 1.0 / np.maximum(deg, 1), 0).astype(np.float32)
+            self._inv_deg_edge = common.to_device_f32(np.repeat(inv, np.diff(self._adj_indptr)), self._ctx)
+        self.out_tvm = torch.zeros((self._num_rows,) + tuple(src_ph.shape[1:]), dtype=torch.float32, device=self._ctx)
+
+    def _glayout(self, P):
+        """Layout for P source partitions plus, for P > 1, each DDS element's CSR position (so that
+        weights given in CSR order can be brought into DDS order on the device)."""
+        lay = self._layout(P)
+        if P > 1 and 'edge_pos' not in lay:
+            nnz = self._adj_indices.shape[0]
+            csr = scipy.sparse.csr_matrix((np.arange(nnz, dtype=np.int32), self._adj_indices, self._adj_indptr),
+                                          shape=(self._num_rows, self._num_cols))
+            _, _, edge_pos = util_convert_csr_to_dds(csr, P)
+            lay['edge_pos'] = torch.from_numpy(edge_pos.astype(np.int64)).to(self._ctx)
+        return lay
+
+    def _weights(self, given):
+        """Device weights in the active layout's element order, or None for weight 1."""
+        lay = self._active
+        if self._msg == 'copy_u':
+            w = None
+        elif given is not None:
+            w = given.reshape(given.shape[0], -1)
+        else:
+            w = self._layouts[1]['vals'].reshape(-1, 1) if 1 in self._layouts else None
+            if w is None:
+                w = common.to_device_f32(self._adj_scipy_csr.data, self._ctx).reshape(-1, 1)
+        if self._inv_deg_edge is not None:
+            w = self._inv_deg_edge.reshape(-1, 1) if w is None else w * self._inv_deg_edge.reshape(-1, 1)
+        if w is not None and lay['P'] > 1:
+            w = w.index_select(0, lay['edge_pos'])
+        return None if w is None else w.contiguous()
+
+    def _launch(self, src_feat, weights=None):
+        lay = self._active
+        w = self._weights(weights)
+        heads = self._heads if (w is not None and w.shape[1] > 1) else 1
+        self._w_keepalive = w
+        _lib.check(self._func(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(w),
+                              _lib.dev_ptr(src_feat), _lib.dev_ptr(self.out_tvm), self._feat_len, heads,
+                              _REDUCE[self._reduce], self._num_feat_partitions, common.stream_ptr()))
+
+    def run(self, input_tvm_ndarrays):
+        """[SrcFeat] or [SrcFeat, edge_weights]; returns self.out_tvm (overwritten in place)."""
+        if self._func is None:
+            raise RuntimeError("call build() before run()")
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        self._launch(input_tvm_ndarrays[0], input_tvm_ndarrays[1] if self._weights_at_run else None)
+        return self.out_tvm
+
+    def measure_average_time(self, input_tvm_ndarrays, num_runs):
+        if self._func is None:
+            raise RuntimeError("call build() before measure_average_time()")
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        x = input_tvm_ndarrays[0]
+        w = input_tvm_ndarrays[1] if self._weights_at_run else None
+        return common.timed_mean_seconds(lambda: self._launch(x, w), num_runs)

@@ -22,6 +22,11 @@
  *   orc_csr_to_dds, orc_partition_coo_2d
  *       the reference's stored vectors (tests/test_util.py:22-24, :43), scipy
  *       sub-matrix slicing on random matrices, brute-force invariants.
+ *   orc_gspmm
+ *       PARITY UNPINNED by the reference: max / min / per-head-weighted aggregation is what
+ *       README.md:9-11 points to ("generalized SpMM") but the snapshot holds no code, test or
+ *       vector for it.  Pinned by numpy maximum/minimum.reduceat closed forms, by reduce == sum
+ *       with H == 1 equalling orc_spmm_csr_rowwise bit-exactly, and by brute force on tiny inputs.
  *   orc_sddmm_multihead
  *       PARITY UNPINNED by the reference: the reference snapshot holds no
  *       multi-head op, test or vector (python/featgraph/op/__init__.py:1-5).
@@ -124,6 +129,36 @@ int orc_spmm_csr_rowwise(int64_t n_dst, int F, const int32_t *indptr,
             const float w = vals[e];
             const float *xr = x + (int64_t)indices[e] * F;
             for (int f = 0; f < F; ++f) o[f] += w * xr[f];
+        }
+    }
+    return ORC_OK;
+}
+
+/*
+ * Generalised aggregation.  NOT IN THE REFERENCE (parity unpinned, see the header):
+ *   out[v, h, d] = reduce over the row's elements e of w(e, h) * X[indices[e], h, d]
+ * reduce: 0 sum, 1 max, 2 min; w(e, h) = vals[e * H + h], or 1 when vals is NULL; a row without
+ * elements gives 0 for every reduce.  Elements are visited in stored order.
+ */
+int orc_gspmm(int64_t n_dst, int F, int H, const int32_t *indptr, const int32_t *indices,
+              const float *vals, const float *x, float *out, int reduce, int nthreads) {
+    if (F < 1 || H < 1 || F % H != 0 || reduce < 0 || reduce > 2 || nthreads < 1) return ORC_EARG;
+    const int D = F / H;
+#pragma omp parallel for num_threads(nthreads) schedule(dynamic, 64)
+    for (int64_t row = 0; row < n_dst; ++row) {
+        float *o = out + row * F;
+        const int32_t b = indptr[row], e = indptr[row + 1];
+        for (int f = 0; f < F; ++f) o[f] = 0.0f;
+        for (int32_t k = b; k < e; ++k) {
+            const float *xr = x + (int64_t)indices[k] * F;
+            for (int f = 0; f < F; ++f) {
+                const float w = vals ? vals[(int64_t)k * H + f / D] : 1.0f;
+                const float m = w * xr[f];
+                if (reduce == 0) o[f] += m;
+                else if (k == b) o[f] = m;
+                else if (reduce == 1) o[f] = m > o[f] ? m : o[f];
+                else o[f] = m < o[f] ? m : o[f];
+            }
         }
     }
     return ORC_OK;

@@ -51,6 +51,7 @@ def lib():
         L.orc_spmm_csr_x86.argtypes = [_i64, _i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int]
         L.orc_spmm_csr_rowwise.argtypes = [_i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int]
         L.orc_spmm_dds_x86.argtypes = [_i64, _i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int]
+        L.orc_gspmm.argtypes = [_i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int]
         L.orc_sddmm_x86.argtypes = [_i64, _i64, _i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int, _int]
         L.orc_sddmm_multihead.argtypes = [_i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int]
         L.orc_csr_to_dds.argtypes = [_i64, _i64, _i32p, _i32p, _u32p, _int, _i32p, _i32p, _u32p]
@@ -115,6 +116,30 @@ def spmm_dds_x86(s1_pos, s1_idx, vals, x, n_dst, num_col_partitions,
                                   _p(s1_idx, _i32p), _p(vals, _f32p), _p(x, _f32p),
                                   _p(out, _f32p), num_feat_partitions, nthreads), "spmm_dds_x86")
     return out
+
+
+REDUCE = {"sum": 0, "max": 1, "min": 2}
+
+
+def gspmm(indptr, indices, vals, x, reduce="sum", nthreads=1):
+    """out[v,h,:] = reduce_e vals[e,h] * x[indices[e],h,:]; x is [n, F] or [n, H, D], vals is None
+    (weight 1), [nnz] or [nnz, H].  Not in the reference (README.md:9-11 only names it)."""
+    indptr = _c(indptr, np.int32); indices = _c(indices, np.int32)
+    x = _c(x, np.float32)
+    shape = x.shape
+    H = shape[1] if x.ndim == 3 else 1
+    x2 = x.reshape(shape[0], -1)
+    F = x2.shape[1]
+    vp = None
+    if vals is not None:
+        vals = _c(vals, np.float32).reshape(indices.shape[0], -1)
+        assert vals.shape[1] == H
+        vp = _p(vals, _f32p)
+    n_dst = indptr.shape[0] - 1
+    out = np.empty((n_dst, F), dtype=np.float32)
+    _check(lib().orc_gspmm(n_dst, F, H, _p(indptr, _i32p), _p(indices, _i32p), vp, _p(x2, _f32p),
+                           _p(out, _f32p), REDUCE[reduce], nthreads), "gspmm")
+    return out.reshape((n_dst,) + shape[1:])
 
 
 def sddmm_x86(row, col, src, dst, num_feat_partitions=1, parallel_edges=False, nthreads=1):

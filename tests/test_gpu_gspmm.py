@@ -1,0 +1,125 @@
+"""GPU tests of the generalised SpMM (sum / mean / max / min aggregation, per-head weights,
+copy_u).  The reference has no such operator, so parity is unpinned by it; the checks are the
+CPU oracle's closed forms (numpy reduceat, see tests/test_oracle.py) and reductions to the plain
+SpMM."""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+from helpers import RTOL, ATOL, assert_sum_close, spmm_mass
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+def _graph(rng, n_rows=260, n_cols=3000, long_len=2700):
+    a = sp.random(n_rows, n_cols, density=0.02, format="csr", random_state=rng,
+                  data_rvs=lambda k: rng.standard_normal(k)).astype("float32").tolil()
+    a[[0, n_rows // 2, n_rows - 1], :] = 0
+    cols = rng.choice(n_cols, size=long_len, replace=False)
+    a[5, cols] = rng.standard_normal(long_len).astype("float32") + 3.0
+    a = a.tocsr().astype("float32"); a.eliminate_zeros(); a.sort_indices()
+    return a
+
+
+@pytest.mark.parametrize("reduce", ["max", "min"])
+@pytest.mark.parametrize("feat_len", [1, 4, 7, 32, 64, 100, 128, 256, 512, 1024])
+def test_extreme_aggregation(torch_cuda, oracle, reduce, feat_len):
+    """max / min are exact: every kernel shape, split hub row, empty rows -> 0, negative weights."""
+    from featgraph_amd.module import GSpMMhip, placeholder
+    torch = torch_cuda
+    rng = np.random.default_rng(feat_len)
+    adj = _graph(rng)
+    x = rng.standard_normal((3000, feat_len)).astype("float32")
+    for msg in ("u_mul_e", "copy_u"):
+        m = GSpMMhip(adj)
+        m.build([placeholder(x.shape)], {'reduce': reduce, 'msg': msg}, {})
+        m.out_tvm.fill_(float("nan"))
+        out = m.run([torch.from_numpy(x).cuda()]).cpu().numpy()
+        ref = oracle.gspmm(adj.indptr, adj.indices, adj.data if msg == "u_mul_e" else None, x, reduce, 2)
+        assert np.array_equal(out, ref), (reduce, msg, feat_len)
+        assert (out[np.diff(adj.indptr) == 0] == 0).all()
+
+
+@pytest.mark.parametrize("reduce,P", [("sum", None), ("sum", 3), ("mean", None), ("mean", 4), ("sum", 'auto')])
+def test_sum_and_mean(torch_cuda, oracle, reduce, P):
+    from featgraph_amd.module import GSpMMhip, VanillaSpMMhip, placeholder
+    torch = torch_cuda
+    rng = np.random.default_rng(3)
+    adj = _graph(rng)
+    x = rng.standard_normal((3000, 96)).astype("float32")
+    m = GSpMMhip(adj)
+    m.build([placeholder(x.shape)], {'reduce': reduce}, {'num_src_partitions': P})
+    out = m.run([torch.from_numpy(x).cuda()]).cpu().numpy()
+    ref64 = oracle.spmm_f64(adj, x)
+    mass = spmm_mass(adj, x)
+    if reduce == "mean":
+        deg = np.maximum(np.diff(adj.indptr), 1)[:, None]
+        ref64, mass = ref64 / deg, mass / deg
+    assert_sum_close(out, ref64, mass, "%s P=%s" % (reduce, P))
+    if reduce == "sum" and P is None:
+        v = VanillaSpMMhip(adj)
+        v.build([placeholder(x.shape)], {}, {'num_src_partitions': None})
+        assert np.array_equal(out, v.run([torch.from_numpy(x).cuda()]).cpu().numpy())
+    # copy_u mean = plain average of the gathered rows
+    m.build([placeholder(x.shape)], {'reduce': 'mean', 'msg': 'copy_u'}, {'num_src_partitions': P})
+    out = m.run([torch.from_numpy(x).cuda()]).cpu().numpy()
+    ones = sp.csr_matrix((np.ones(adj.nnz, "float32"), adj.indices, adj.indptr), shape=adj.shape)
+    deg = np.maximum(np.diff(adj.indptr), 1)[:, None]
+    assert_sum_close(out, oracle.spmm_f64(ones, x) / deg, spmm_mass(ones, x) / deg)
+
+
+@pytest.mark.parametrize("H,D,reduce,P", [(4, 64, "sum", None), (8, 64, "sum", 3), (4, 32, "sum", None), (2, 16, "max", None),
+                                          (8, 128, "sum", None), (4, 64, "min", None), (4, 32, "mean", 2), (1, 48, "sum", None)])
+def test_per_head_weights(torch_cuda, oracle, H, D, reduce, P):
+    """out[v,h,:] = reduce_e w[e,h] * x[u,h,:] with weights handed to run() in CSR edge order."""
+    from featgraph_amd.module import GSpMMhip, placeholder
+    torch = torch_cuda
+    rng = np.random.default_rng(H * 100 + D)
+    adj = _graph(rng, 200, 1500, 1300)
+    x = rng.standard_normal((1500, H, D)).astype("float32")
+    w = rng.standard_normal((adj.nnz, H)).astype("float32")
+    m = GSpMMhip(adj)
+    wshape = (adj.nnz, H) if H > 1 else (adj.nnz,)
+    m.build([placeholder(x.shape), placeholder(wshape)], {'reduce': reduce}, {'num_src_partitions': P})
+    out = m.run([torch.from_numpy(x).cuda(), torch.from_numpy(w.reshape(wshape)).cuda()]).cpu().numpy()
+    assert out.shape == (200, H, D)
+    if reduce in ("max", "min"):
+        assert np.array_equal(out, oracle.gspmm(adj.indptr, adj.indices, w, x, reduce))
+        return
+    ref = np.zeros((200, H, D)); mass = np.zeros((200, H, D))
+    for h in range(H):
+        ah = sp.csr_matrix((w[:, h], adj.indices, adj.indptr), shape=adj.shape)
+        ref[:, h] = oracle.spmm_f64(ah, x[:, h]); mass[:, h] = spmm_mass(ah, x[:, h])
+    if reduce == "mean":
+        deg = np.maximum(np.diff(adj.indptr), 1)[:, None, None]
+        ref, mass = ref / deg, mass / deg
+    assert_sum_close(out, ref, mass, "H=%d D=%d" % (H, D))
+    np.testing.assert_allclose(out, oracle.gspmm(adj.indptr, adj.indices, w, x, "sum") /
+                               (np.maximum(np.diff(adj.indptr), 1)[:, None, None] if reduce == "mean" else 1),
+                               rtol=1e-3, atol=1e-3)
+
+
+def test_gspmm_errors(torch_cuda):
+    from featgraph_amd.module import GSpMMhip, placeholder
+    rng = np.random.default_rng(0)
+    adj = _graph(rng, 50, 200, 150)
+    m = GSpMMhip(adj)
+    with pytest.raises(ValueError):
+        m.build([placeholder((200, 8))], {'reduce': 'prod'}, {})
+    with pytest.raises(ValueError):
+        m.build([placeholder((200, 4, 16))], {}, {})                         # per-head weights missing
+    with pytest.raises(ValueError):
+        m.build([placeholder((200, 8)), placeholder((7,))], {}, {})          # wrong weight shape
+    with pytest.raises(ValueError):
+        GSpMMhip(adj, 2).build([placeholder((200, 8))], {'reduce': 'max'}, {})
+    m.build([placeholder((200, 4, 6)), placeholder((adj.nnz, 4))], {}, {})   # head length 6: no kernel tile
+    import torch
+    with pytest.raises(ValueError):
+        m.run([torch.zeros((200, 4, 6), device="cuda"), torch.zeros((adj.nnz, 4), device="cuda")])

@@ -254,3 +254,33 @@ def test_multihead_closed_form(oracle):
         np.testing.assert_allclose(out.sum(1), flat, rtol=1e-4, atol=1e-4)
         if H == 1:
             assert np.array_equal(out[:, 0], flat)
+
+
+def test_gspmm_closed_forms(oracle):
+    """Max / min / per-head aggregation (no counterpart in the reference): numpy reduceat over
+    the gathered messages, sum with one head == the plain SpMM restatement, empty rows give 0."""
+    rng = np.random.default_rng(9)
+    a = _rand_csr(rng, 60, 80, 0.15).tolil()
+    a[[3, 59], :] = 0
+    a = a.tocsr().astype("float32"); a.eliminate_zeros(); a.sort_indices()
+    nonempty = np.diff(a.indptr) > 0
+    starts = a.indptr[:-1][nonempty]
+    for H, D in ((1, 24), (4, 16), (3, 5)):
+        x = rng.standard_normal((80, H, D)).astype("float32")
+        w = rng.standard_normal((a.nnz, H)).astype("float32")
+        msg = w[:, :, None] * x[a.indices]
+        for red, fn in (("max", np.maximum), ("min", np.minimum), ("sum", np.add)):
+            expect = np.zeros((60, H, D), "float32")
+            expect[nonempty] = fn.reduceat(msg, starts, axis=0)
+            got = oracle.gspmm(a.indptr, a.indices, w, x, red, nthreads=2)
+            if red == "sum":
+                np.testing.assert_allclose(got, expect, rtol=1e-4, atol=1e-5)
+            else:
+                assert np.array_equal(got, expect)
+            assert (got[~nonempty] == 0).all()
+        plain = oracle.gspmm(a.indptr, a.indices, None, x, "max")
+        e2 = np.zeros((60, H, D), "float32"); e2[nonempty] = np.maximum.reduceat(x[a.indices], starts, axis=0)
+        assert np.array_equal(plain, e2)
+    x = rng.standard_normal((80, 24)).astype("float32")
+    assert np.array_equal(oracle.gspmm(a.indptr, a.indices, a.data, x, "sum"),
+                          oracle.spmm_csr_rowwise(a.indptr, a.indices, a.data, x))
