@@ -319,3 +319,32 @@ class MultiHeadSDDMMhip(VanillaSDDMMhip):
             raise ValueError("multi-head SrcFeat / DstFeat must be 3-D [n, H, D], got %s and %s"
                              % (src_ph.shape, dst_ph.shape))
         return src_ph.shape[1], src_ph.shape[2]
+
+
+class GSDDMMhip(VanillaSDDMMhip):
+    """Generalised SDDMM: compute_args {'op': 'dot' | 'add' | 'sub' | 'mul'}.  'dot' is
+    VanillaSDDMMhip; the others give out[e, :] = SrcFeat[col[e], :] op DstFeat[row[e], :] with
+    shape (num_edges, feat_len), in the stored edge order.  Not present in the reference."""
+    _compute_keys = ('num_feat_partitions', 'op')
+    _EDGE_OPS = {'add': 0, 'sub': 1, 'mul': 2}
+
+    def build(self, input_placeholders, compute_args, schedule_args):
+        compute_args = dict(compute_args)
+        self._op = compute_args.pop('op', 'dot')
+        if self._op == 'dot':
+            return super(GSDDMMhip, self).build(input_placeholders, compute_args, schedule_args)
+        if self._op not in self._EDGE_OPS:
+            raise ValueError("op must be 'dot', 'add', 'sub' or 'mul'")
+        phs, H, D, _, _, notes = self._resolve(input_placeholders, compute_args, dict(schedule_args, order='coo'))
+        self._placeholders, self._heads, self._head_len, self._notes = phs, H, D, notes
+        self._tiled, self._use_csr = None, False
+        self._func = _lib.lib().fg_gsddmm_elementwise_f32
+        self.out_tvm = torch.zeros((self._adj_row_indices.shape[0], H * D), dtype=torch.float32, device=self._ctx)
+
+    def _launch(self, src_feat, dst_feat):
+        if getattr(self, '_op', 'dot') == 'dot':
+            return super(GSDDMMhip, self)._launch(src_feat, dst_feat)
+        _lib.check(self._func(_lib.dev_ptr(self._adj_row_indices_dev), _lib.dev_ptr(self._adj_col_indices_dev),
+                              self._adj_row_indices.shape[0], _lib.dev_ptr(src_feat), _lib.dev_ptr(dst_feat),
+                              _lib.dev_ptr(self.out_tvm), self._heads * self._head_len,
+                              self._EDGE_OPS[self._op], common.stream_ptr()))
