@@ -1,0 +1,93 @@
+"""Default-configuration timings of every benchmark configuration on one GPU.
+
+    python -m featgraph_amd.benchmark.bench_configs [--quick]
+
+Configurations: weighted CSR SpMM and SDDMM (CSR-ordered and shuffled COO edges) at feature
+lengths 32..512 and multi-head SDDMM (H in {4, 8}, D in {32, 64}) on the 232,965-node power-law
+graph; SpMM followed by SDDMM at feature length 128 on the 2.45M-node low-degree graph; SpMM on the
+10,000-node uniform graph.  One JSON line per measurement (mean of 5 launches after a warm-up).
+"""
+import argparse
+import json
+
+import numpy as np
+import scipy.sparse as sp
+import torch
+
+from .. import synthetic
+from ..module import VanillaSpMMhip, VanillaSDDMMhip, MultiHeadSDDMMhip, placeholder
+
+HBM_PEAK_GBS = 8000.0
+
+
+def _line(workload, op, knobs, seconds, nnz, feat_len, bytes_model):
+    out = dict(workload=workload, op=op, **knobs)
+    out.update(ms=round(seconds * 1e3, 4), gflops=round(2.0 * nnz * feat_len / seconds / 1e9, 1),
+               compulsory_gb=round(bytes_model / 1e9, 3), compulsory_gbs=round(bytes_model / seconds / 1e9, 1),
+               pct_hbm_roofline=round(100.0 * bytes_model / seconds / 1e9 / HBM_PEAK_GBS, 3),
+               gathered_tbs=round(4.0 * nnz * feat_len / seconds / 1e12, 2))
+    print(json.dumps(out), flush=True)
+
+
+def run_workload(name, feat_lens, head_shapes, shuffled_coo):
+    indptr, indices = synthetic.make_workload(name)
+    n = indptr.shape[0] - 1
+    nnz = int(indptr[-1])
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    vals = torch.rand(nnz, generator=gen, device="cuda").cpu().numpy()
+    adj = sp.csr_matrix((vals, indices, indptr), shape=(n, n))
+    spmm = VanillaSpMMhip(adj)
+    sddmm = VanillaSDDMMhip(adj)
+    for F in feat_lens:
+        gen.manual_seed(2)
+        x = torch.randn((n, F), generator=gen, device="cuda")
+        y = torch.randn((n, F), generator=gen, device="cuda")
+        spmm.build([placeholder((n, F))], {}, {})
+        t = spmm.measure_average_time([x], 5)
+        _line(name, "spmm", {"feat_len": F, "partitions": spmm._active['P'], "tiles": spmm._num_feat_partitions},
+              t, nnz, F, 4 * (n + 1) + 8 * nnz + 8 * n * F)
+        sddmm.build([placeholder((n, F)), placeholder((n, F))], {}, {})
+        t = sddmm.measure_average_time([x, y], 5)
+        tiled = (sddmm._tiled[0]['P'], sddmm._tiled[1]) if sddmm._tiled else None
+        _line(name, "sddmm_csr_order", {"feat_len": F, "tiled": tiled}, t, nnz, F,
+              4 * (n + 1) + 4 * nnz + 8 * n * F + 4 * nnz)
+        del x, y
+    for H, D in head_shapes:
+        gen.manual_seed(2)
+        x = torch.randn((n, H, D), generator=gen, device="cuda")
+        y = torch.randn((n, H, D), generator=gen, device="cuda")
+        mh = MultiHeadSDDMMhip(adj)
+        mh.build([placeholder((n, H, D)), placeholder((n, H, D))], {}, {})
+        t = mh.measure_average_time([x, y], 5)
+        tiled = (mh._tiled[0]['P'], mh._tiled[1]) if mh._tiled else None
+        _line(name, "sddmm_multihead", {"heads": H, "head_len": D, "tiled": tiled}, t, nnz, H * D,
+              4 * (n + 1) + 4 * nnz + 8 * n * H * D + 4 * nnz * H)
+        del mh, x, y
+    if shuffled_coo:
+        coo = adj.tocoo()
+        perm = torch.randperm(nnz, generator=torch.Generator().manual_seed(3)).numpy()
+        coo = sp.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+        m = VanillaSDDMMhip(coo)
+        for F in shuffled_coo:
+            gen.manual_seed(2)
+            x = torch.randn((n, F), generator=gen, device="cuda")
+            y = torch.randn((n, F), generator=gen, device="cuda")
+            for order in ("coo", "auto"):
+                m.build([placeholder((n, F)), placeholder((n, F))], {}, {'order': order})
+                t = m.measure_average_time([x, y], 5)
+                _line(name, "sddmm_shuffled_coo", {"feat_len": F, "order": order}, t, nnz, F,
+                      8 * nnz + 8 * n * F + 4 * nnz)
+            del x, y
+
+
+if __name__ == '__main__':
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--quick", action="store_true", help="small graphs only")
+    args = ap.parse_args()
+    run_workload("uniform-10k", [32], [], [])
+    if args.quick:
+        run_workload("powerlaw-23k", [32, 128, 512], [(4, 32), (8, 64)], [128])
+    else:
+        run_workload("powerlaw-233k", [32, 64, 128, 256, 512], [(4, 32), (4, 64), (8, 32), (8, 64)], [128])
+        run_workload("powerlaw-2.45M", [128], [], [])
