@@ -1,0 +1,109 @@
+"""Differentiable SpMM / SDDMM built from the forward kernels.
+
+The backward passes are the same two operators on the transposed graph:
+  y = A(w) x            dx = A(w)^T dy          dw[e] = <dy[row e], x[col e]>       (an SDDMM)
+  s[e] = <src[col e], dst[row e]>    ddst = A(ds) src    dsrc = A(ds)^T dst         (two SpMMs)
+so `Graph` keeps plans for the adjacency in CSR order and for its transpose, and the permutation
+between the two edge orders.  The reference has no autograd layer; this is the consumer-side API
+its README (README.md:13-14, DGL integration) points at.
+"""
+import numpy as np
+import scipy.sparse
+import torch
+
+from .module import GSpMMhip, VanillaSDDMMhip, placeholder
+
+
+class Graph(object):
+    """Structure of one adjacency (rows = destinations, columns = sources) for differentiable ops.
+
+    Edge weights and edge outputs are 1-D tensors in the adjacency's CSR edge order.
+    """
+
+    def __init__(self, adj_scipy):
+        csr = adj_scipy.tocsr().astype(np.float32)
+        csr.sort_indices()
+        self.shape = csr.shape
+        self.nnz = csr.nnz
+        pos = scipy.sparse.csr_matrix((np.arange(1, csr.nnz + 1, dtype=np.int64), csr.indices, csr.indptr),
+                                      shape=csr.shape)
+        tr = pos.T.tocsr()
+        tr.sort_indices()
+        self._csr = csr
+        self._tr = scipy.sparse.csr_matrix((np.ones(csr.nnz, np.float32), tr.indices.astype(np.int32),
+                                            tr.indptr.astype(np.int32)), shape=tr.shape)
+        self._tr_pos_host = (tr.data - 1).astype(np.int64)      # transposed edge order -> CSR position
+        self._tr_pos = None
+        self._mods = {}
+
+    def _tr_perm(self, device):
+        if self._tr_pos is None or self._tr_pos.device != device:
+            self._tr_pos = torch.from_numpy(self._tr_pos_host).to(device)
+        return self._tr_pos
+
+    def _spmm_mod(self, transposed, feat_len):
+        key = ('spmm', transposed, feat_len)
+        if key not in self._mods:
+            adj = self._tr if transposed else self._csr
+            m = GSpMMhip(adj)
+            m.build([placeholder((adj.shape[1], feat_len)), placeholder((self.nnz,))], {}, {})
+            self._mods[key] = m
+        return self._mods[key]
+
+    def _sddmm_mod(self, feat_len):
+        key = ('sddmm', feat_len)
+        if key not in self._mods:
+            m = VanillaSDDMMhip(self._csr)
+            m.build([placeholder((self.shape[1], feat_len)), placeholder((self.shape[0], feat_len))], {}, {})
+            self._mods[key] = m
+        return self._mods[key]
+
+    # raw (non-differentiable) building blocks; each returns a fresh tensor
+    def _spmm_raw(self, x, w, transposed=False):
+        x = x.contiguous()
+        if transposed:
+            w = w.index_select(0, self._tr_perm(w.device))
+        return self._spmm_mod(transposed, x.shape[1]).run([x, w.contiguous()]).clone()
+
+    def _sddmm_raw(self, src, dst):
+        return self._sddmm_mod(src.shape[1]).run([src.contiguous(), dst.contiguous()]).clone()
+
+    def spmm(self, x, w):
+        """y[v,:] = sum_e w[e] x[col e,:]; x (num_cols, F), w (nnz,); differentiable in both."""
+        return _SpMM.apply(self, x, w)
+
+    def sddmm(self, src, dst):
+        """s[e] = <src[col e,:], dst[row e,:]>; src (num_cols, F), dst (num_rows, F)."""
+        return _SDDMM.apply(self, src, dst)
+
+
+class _SpMM(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, g, x, w):
+        ctx.g = g
+        ctx.save_for_backward(x, w)
+        return g._spmm_raw(x, w)
+
+    @staticmethod
+    def backward(ctx, dy):
+        g = ctx.g
+        x, w = ctx.saved_tensors
+        dx = g._spmm_raw(dy, w, transposed=True) if ctx.needs_input_grad[1] else None
+        dw = g._sddmm_raw(x, dy) if ctx.needs_input_grad[2] else None
+        return None, dx, dw
+
+
+class _SDDMM(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, g, src, dst):
+        ctx.g = g
+        ctx.save_for_backward(src, dst)
+        return g._sddmm_raw(src, dst)
+
+    @staticmethod
+    def backward(ctx, ds):
+        g = ctx.g
+        src, dst = ctx.saved_tensors
+        dsrc = g._spmm_raw(dst, ds, transposed=True) if ctx.needs_input_grad[1] else None
+        ddst = g._spmm_raw(src, ds) if ctx.needs_input_grad[2] else None
+        return None, dsrc, ddst
