@@ -365,10 +365,26 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
 
     if (it.info < -1) {
         const int nrows = -it.info;
+        // The destination rows of this item are read once here, one word per 128 bytes, while the
+        // edges are on their way.  Loads return in order, so a row fetched from memory at the moment
+        // it is needed would hold up every gather issued after it; fetched here, all rows' misses
+        // overlap each other and the staging loads, and the later reads hit the cache.
+        constexpr int kLines = (L * K * 16 + 127) / 128;
+        constexpr int kTouch = (fg::kItemRows * kLines + 63) / 64;
+        float touched[kTouch];
+#pragma unroll
+        for (int i = 0; i < kTouch; ++i) {
+            const int t = lane + 64 * i;
+            const int r = min(t / kLines, nrows - 1);
+            const int f = min((t % kLines) * 32, L * K * 4 - 1);
+            touched[i] = a.dst[(int64_t)(it.row + r) * F + tile * (L * K * 4) + f];
+        }
         stage(it.start, it.len);
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
         if (lane == 0) s_next[wave] = 0;
         wave_lds_sync();
+#pragma unroll
+        for (int i = 0; i < kTouch; ++i) asm volatile("" ::"v"(touched[i]));    // keeps the loads
         if (nrows < 2 * G) {
             // few, longer rows: all lane groups share each row in turn
             int b = 0;

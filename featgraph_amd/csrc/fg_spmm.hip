@@ -216,6 +216,24 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     if (it.info < -1) {
         // Several whole rows: stage all their elements once.
         const int nrows = -it.info;
+        // ACC: the rows this item adds to are read once here, one word per 128 bytes, while the
+        // elements are on their way.  Loads return in order, so a row of `out` fetched from memory
+        // at the moment it is needed would hold up every gather issued after it; fetched here, all
+        // rows' misses overlap each other and the staging loads, and the later reads hit the cache.
+        constexpr int kLines = (FT * 4 + 127) / 128;
+        constexpr int kTouch = ACC ? (fg::kItemRows * kLines + 63) / 64 : 1;
+        float touched[kTouch];
+        if (ACC) {
+            const int f_tile = rt * a.tile_w + st * FT;
+            const int f_last = min(f_tile + FT, f_end) - 1;
+#pragma unroll
+            for (int i = 0; i < kTouch; ++i) {
+                const int t = lane + 64 * i;
+                const int r = min(t / kLines, nrows - 1);
+                const int f = min(f_tile + (t % kLines) * 32, f_last);
+                touched[i] = a.out[(int64_t)(it.row + r) * F + f];
+            }
+        }
         if (it.len > 0) {
             stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.heads, voff, regs);
             stage_store(edge, lane, regs);
@@ -223,6 +241,10 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
         if (lane == 0) s_next[wave] = 0;
         wave_lds_sync();
+        if (ACC) {
+#pragma unroll
+            for (int i = 0; i < kTouch; ++i) asm volatile("" ::"v"(touched[i]));    // keeps the loads
+        }
         if (nrows < 2 * G) {
             // Few, longer rows: all lane groups share each row in turn.
             int b = 0;
