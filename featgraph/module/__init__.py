@@ -1,3 +1,3 @@
 from featgraph_amd.module import (VanillaSpMMhip, VanillaSpMMx86, VanillaSpMMcuda,
                                   VanillaSDDMMhip, VanillaSDDMMx86, VanillaSDDMMcuda,
-                                  MultiHeadSDDMMhip, GSpMMhip, GSDDMMhip, placeholder)
+                                  MultiHeadSDDMMhip, GSpMMhip, GSDDMMhip, EdgeSoftmaxhip, placeholder)

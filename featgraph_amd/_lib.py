@@ -42,6 +42,8 @@ SIGNATURES = {
     "fg_sddmm_csr_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
     "fg_sddmm_dds_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
     "fg_gsddmm_elementwise_f32": (_int, [_vp, _vp, _i64, _vp, _vp, _vp, _int, _int, _vp]),
+    "fg_edge_softmax_f32": (_int, [_vp, _vp, _vp, _vp, _int, _vp]),
+    "fg_edge_softmax_backward_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp]),
     "fg_synth_powerlaw_csr": (_int, [_i64, _vp, _vp, _vp, ctypes.c_uint64, _int, _vp, _vp]),
 }
 

@@ -1,8 +1,10 @@
-"""Differentiable SpMM / SDDMM built from the forward kernels.
+"""Differentiable SpMM / SDDMM / edge softmax built from the forward kernels.
 
 The backward passes are the same two operators on the transposed graph:
   y = A(w) x            dx = A(w)^T dy          dw[e] = <dy[row e], x[col e]>       (an SDDMM)
   s[e] = <src[col e], dst[row e]>    ddst = A(ds) src    dsrc = A(ds)^T dst         (two SpMMs)
+(with heads: x, src, dst are (n, H, D), w and s are (nnz, H), and every identity holds per head);
+  a = edge_softmax(s)   ds = a * (da - sum over the row of a * da)
 so `Graph` keeps plans for the adjacency in CSR order and for its transpose, and the permutation
 between the two edge orders.  The reference has no autograd layer; this is the consumer-side API
 its README (README.md:13-14, DGL integration) points at.
@@ -11,13 +13,14 @@ import numpy as np
 import scipy.sparse
 import torch
 
-from .module import GSpMMhip, VanillaSDDMMhip, placeholder
+from .module import EdgeSoftmaxhip, GSpMMhip, MultiHeadSDDMMhip, VanillaSDDMMhip, placeholder
 
 
 class Graph(object):
     """Structure of one adjacency (rows = destinations, columns = sources) for differentiable ops.
 
-    Edge weights and edge outputs are 1-D tensors in the adjacency's CSR edge order.
+    Edge weights and edge outputs are (nnz,) tensors, or (nnz, H) with heads, in the adjacency's CSR
+    edge order.
     """
 
     def __init__(self, adj_scipy):
@@ -41,40 +44,60 @@ class Graph(object):
             self._tr_pos = torch.from_numpy(self._tr_pos_host).to(device)
         return self._tr_pos
 
-    def _spmm_mod(self, transposed, feat_len):
-        key = ('spmm', transposed, feat_len)
+    def _spmm_mod(self, transposed, tail, w_heads):
+        key = ('spmm', transposed, tail, w_heads)
         if key not in self._mods:
             adj = self._tr if transposed else self._csr
             m = GSpMMhip(adj)
-            m.build([placeholder((adj.shape[1], feat_len)), placeholder((self.nnz,))], {}, {})
+            w_shape = (self.nnz,) if w_heads == 0 else (self.nnz, w_heads)
+            m.build([placeholder((adj.shape[1],) + tail), placeholder(w_shape)], {}, {})
             self._mods[key] = m
         return self._mods[key]
 
-    def _sddmm_mod(self, feat_len):
-        key = ('sddmm', feat_len)
+    def _sddmm_mod(self, tail):
+        key = ('sddmm', tail)
         if key not in self._mods:
-            m = VanillaSDDMMhip(self._csr)
-            m.build([placeholder((self.shape[1], feat_len)), placeholder((self.shape[0], feat_len))], {}, {})
+            m = (MultiHeadSDDMMhip if len(tail) == 2 else VanillaSDDMMhip)(self._csr)
+            m.build([placeholder((self.shape[1],) + tail), placeholder((self.shape[0],) + tail)], {}, {})
+            self._mods[key] = m
+        return self._mods[key]
+
+    def _softmax_mod(self, shape):
+        key = ('softmax', shape)
+        if key not in self._mods:
+            m = EdgeSoftmaxhip(self._csr)
+            m.build([placeholder(shape)])
             self._mods[key] = m
         return self._mods[key]
 
     # raw (non-differentiable) building blocks; each returns a fresh tensor
     def _spmm_raw(self, x, w, transposed=False):
         x = x.contiguous()
+        if x.dim() == 3 and (w.dim() != 2 or w.shape[1] != x.shape[1]):
+            raise ValueError("with x of shape (n, H, D) the weights must be (nnz, H)")
+        if x.dim() == 2 and w.dim() != 1:
+            raise ValueError("with x of shape (n, F) the weights must be (nnz,)")
         if transposed:
             w = w.index_select(0, self._tr_perm(w.device))
-        return self._spmm_mod(transposed, x.shape[1]).run([x, w.contiguous()]).clone()
+        mod = self._spmm_mod(transposed, tuple(x.shape[1:]), 0 if w.dim() == 1 else w.shape[1])
+        return mod.run([x, w.contiguous()]).clone()
 
     def _sddmm_raw(self, src, dst):
-        return self._sddmm_mod(src.shape[1]).run([src.contiguous(), dst.contiguous()]).clone()
+        return self._sddmm_mod(tuple(src.shape[1:])).run([src.contiguous(), dst.contiguous()]).clone()
 
     def spmm(self, x, w):
-        """y[v,:] = sum_e w[e] x[col e,:]; x (num_cols, F), w (nnz,); differentiable in both."""
+        """y[v,:] = sum_e w[e] x[col e,:]; x (num_cols, F) with w (nnz,), or x (num_cols, H, D) with
+        w (nnz, H); differentiable in both."""
         return _SpMM.apply(self, x, w)
 
     def sddmm(self, src, dst):
-        """s[e] = <src[col e,:], dst[row e,:]>; src (num_cols, F), dst (num_rows, F)."""
+        """s[e] = <src[col e,:], dst[row e,:]>; src (num_cols, F), dst (num_rows, F) -> (nnz,), or
+        (n, H, D) operands -> (nnz, H)."""
         return _SDDMM.apply(self, src, dst)
+
+    def edge_softmax(self, scores):
+        """Softmax of scores, (nnz,) or (nnz, H), over the edges of each destination row, per head."""
+        return _EdgeSoftmax.apply(self, scores)
 
 
 class _SpMM(torch.autograd.Function):
@@ -107,3 +130,17 @@ class _SDDMM(torch.autograd.Function):
         dsrc = g._spmm_raw(dst, ds, transposed=True) if ctx.needs_input_grad[1] else None
         ddst = g._spmm_raw(src, ds) if ctx.needs_input_grad[2] else None
         return None, dsrc, ddst
+
+
+class _EdgeSoftmax(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, g, scores):
+        ctx.g = g
+        a = g._softmax_mod(tuple(scores.shape)).run([scores.contiguous()]).clone()
+        ctx.save_for_backward(a)
+        return a
+
+    @staticmethod
+    def backward(ctx, da):
+        (a,) = ctx.saved_tensors
+        return None, ctx.g._softmax_mod(tuple(a.shape)).backward(a, da.contiguous()).clone()

@@ -63,3 +63,9 @@ struct fg_spmm_plan {
     // statistics for fg_spmm_plan_describe
     int64_t max_len = 0, n_empty = 0, n_split_rows = 0, n_multi_items = 0;
 };
+
+namespace fg {
+// Makes plan->partial_dev hold at least floats_per_piece floats for every piece of split rows of
+// one partition (grown on demand, never shrunk).
+int ensure_partial(const fg_spmm_plan *plan, size_t floats_per_piece);
+}  // namespace fg

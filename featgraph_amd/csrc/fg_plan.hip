@@ -127,6 +127,15 @@ extern "C" void fg_spmm_plan_destroy(fg_spmm_plan *pl) {
 }
 
 namespace fg {
+int ensure_partial(const fg_spmm_plan *pl, size_t floats_per_piece) {
+    const size_t need = (size_t)pl->max_slots_in_partition * floats_per_piece;
+    if (need <= pl->partial_floats) return FG_OK;
+    if (pl->partial_dev) FG_HIP_TRY(hipFree(pl->partial_dev));
+    pl->partial_dev = nullptr; pl->partial_floats = 0;
+    FG_HIP_TRY(hipMalloc((void **)&pl->partial_dev, need * sizeof(float)));
+    pl->partial_floats = need;
+    return FG_OK;
+}
 // Declared in fg_spmm.hip: text of the launch the SpMM entry points would use.
 std::string spmm_launch_text(const fg_spmm_plan *plan, int F, int num_feat_partitions);
 }

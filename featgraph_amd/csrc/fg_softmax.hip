@@ -1,0 +1,404 @@
+// Softmax over the stored elements of every CSR row, per head, and its gradient (gfx950).
+//
+//   forward : y[e, h] = exp(x[e, h] - m[v, h]) / sum_{e' in row v} exp(x[e', h] - m[v, h]),  m = row maximum
+//   backward: dx[e, h] = a[e, h] * (g[e, h] - sum_{e' in row v} a[e', h] * g[e', h])
+//
+// x, y are [nnz, H] row-major, so a row's values are one contiguous run of len * H floats.  The
+// work is cut by the same plan items as SpMM: one wavefront per run of short rows, per row, or
+// per piece of a long row.  A row of up to 1024 floats is read once and finished in registers, a
+// run of short rows is finished in LDS, a longer row is swept twice (statistics, then result).  Pieces of a split row write
+// (max, sum) per head, a small kernel merges them per row, and a second launch of the main
+// kernel normalises the pieces.  Both operators move 2 * nnz * H * 4 bytes at best (read + write;
+// the gradient reads two arrays): they are bound by HBM bandwidth.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "fg_common.h"
+
+using fg::fail;
+using fg::Fixup;
+using fg::Item;
+
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = 64 * kWavesPerBlock;
+constexpr int kStage = 1024;          // floats of a multi-row item staged in LDS per wavefront
+
+// Orders this wavefront's LDS writes before its later LDS reads (and the reverse); the staging
+// buffers are private to one wavefront, so no workgroup barrier is involved.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+struct SoftmaxArgs {
+    const Item *items;
+    int64_t n_items;
+    const int32_t *indptr;
+    const float *x;       // forward: scores; backward: the softmax output a
+    const float *g;       // backward: dL/da
+    float *y;
+    float2 *stats;        // per (piece, head): forward (max, sum of exp); backward (sum of a * g, 0)
+    int H;
+};
+
+// Combines `v` over the lanes that hold the same head (lane % H, H a power of two <= 64), or over
+// the whole wavefront when H == 1.
+template <bool IS_MAX>
+__device__ __forceinline__ float head_reduce(float v, int H) {
+    for (int off = 32; off >= H; off >>= 1) {
+        const float o = __shfl_xor(v, off);
+        v = IS_MAX ? fmaxf(v, o) : v + o;
+    }
+    return v;
+}
+
+
+// A whole row of n <= 64 * R floats (H a power of two <= 64, so lane i always meets head i % H):
+// every lane's R loads are issued back to back, the row is read from memory once and the result
+// is formed in registers.  No load sits under a branch: lanes past the end re-read the last float.
+template <bool BWD, int R>
+__device__ __forceinline__ void row_in_registers(const float *x, const float *g, float *y, int n, int lane, int H) {
+    float v[R], w[BWD ? R : 1];
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        const int i = min(lane + 64 * k, n - 1);
+        v[k] = x[i];
+        if (BWD) w[k] = g[i];
+    }
+    if (!BWD) {
+        float m = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < R; ++k) m = (lane + 64 * k < n) ? fmaxf(m, v[k]) : m;
+        m = head_reduce<true>(m, H);
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < R; ++k) {
+            v[k] = (lane + 64 * k < n) ? __expf(v[k] - m) : 0.f;
+            s += v[k];
+        }
+        s = head_reduce<false>(s, H);
+        const float inv = 1.0f / s;
+#pragma unroll
+        for (int k = 0; k < R; ++k)
+            if (lane + 64 * k < n) y[lane + 64 * k] = v[k] * inv;
+    } else {
+        float d = 0.f;
+#pragma unroll
+        for (int k = 0; k < R; ++k) d += (lane + 64 * k < n) ? v[k] * w[k] : 0.f;
+        d = head_reduce<false>(d, H);
+#pragma unroll
+        for (int k = 0; k < R; ++k)
+            if (lane + 64 * k < n) y[lane + 64 * k] = v[k] * (w[k] - d);
+    }
+}
+
+// One run of `len` elements starting at element e0, all lanes together.
+//   LANEHEAD: H divides 64, lane i always meets head i % H, values are read as one coalesced run.
+//   otherwise: one head at a time, lanes stride over the elements.
+// STATS_ONLY: write (max, sum) / (dot, 0) to stats[slot * H + h] instead of the result.
+// NORMALISE : the row statistics come from stats[slot * H + h] (merged over the row's pieces).
+template <bool BWD, bool LANEHEAD, bool STATS_ONLY, bool NORMALISE>
+__device__ __forceinline__ void run_together(const SoftmaxArgs &a, int64_t e0, int len, int lane, int slot) {
+    const int H = a.H;
+    const int64_t base = e0 * H;
+    const float *x = a.x + base;
+    const float *g = BWD ? a.g + base : nullptr;
+    float *y = a.y + base;
+    if (LANEHEAD) {
+        const int n = len * H;
+        if (!STATS_ONLY && !NORMALISE) {
+            if (n <= 64 * 2) { row_in_registers<BWD, 2>(x, g, y, n, lane, H); return; }
+            if (n <= 64 * 4) { row_in_registers<BWD, 4>(x, g, y, n, lane, H); return; }
+            if (n <= 64 * 8) { row_in_registers<BWD, 8>(x, g, y, n, lane, H); return; }
+        }
+        // longer runs: sweeps of 8 loads per lane issued back to back (lanes past the end re-read
+        // the last float, so no load sits under a branch)
+        constexpr int U = 8;
+        const int h = lane & (H - 1);
+        float m = 0.f, s = 0.f;
+        if (NORMALISE) {
+            const float2 st = a.stats[(int64_t)slot * H + h];
+            m = st.x; s = st.y;
+        } else if (!BWD) {
+            // one sweep: running maximum, the sum rescaled whenever the maximum grows
+            m = -INFINITY;
+            for (int i0 = lane; i0 < n + lane; i0 += 64 * U) {
+                float v[U];
+#pragma unroll
+                for (int k = 0; k < U; ++k) v[k] = x[min(i0 + 64 * k, n - 1)];
+#pragma unroll
+                for (int k = 0; k < U; ++k) {
+                    const float vk = (i0 + 64 * k < n) ? v[k] : -INFINITY;
+                    const float mn = fmaxf(m, vk);
+                    s = (m == mn ? s : s * __expf(m - mn)) + (vk == -INFINITY ? 0.f : __expf(vk - mn));
+                    m = mn;
+                }
+            }
+            const float mw = head_reduce<true>(m, H);
+            s = (m == -INFINITY) ? 0.f : s * __expf(m - mw);
+            m = mw;
+            s = head_reduce<false>(s, H);
+        } else {
+            for (int i0 = lane; i0 < n + lane; i0 += 64 * U) {
+                float v[U], w[U];
+#pragma unroll
+                for (int k = 0; k < U; ++k) { const int i = min(i0 + 64 * k, n - 1); v[k] = x[i]; w[k] = g[i]; }
+#pragma unroll
+                for (int k = 0; k < U; ++k) m += (i0 + 64 * k < n) ? v[k] * w[k] : 0.f;
+            }
+            m = head_reduce<false>(m, H);
+        }
+        if (STATS_ONLY) {
+            if (lane < H) a.stats[(int64_t)slot * H + lane] = make_float2(m, s);
+            return;
+        }
+        if (!BWD) {
+            const float inv = 1.0f / s;
+            for (int i0 = lane; i0 < n + lane; i0 += 64 * U) {
+                float v[U];
+#pragma unroll
+                for (int k = 0; k < U; ++k) v[k] = x[min(i0 + 64 * k, n - 1)];
+#pragma unroll
+                for (int k = 0; k < U; ++k)
+                    if (i0 + 64 * k < n) y[i0 + 64 * k] = __expf(v[k] - m) * inv;
+            }
+        } else {
+            for (int i0 = lane; i0 < n + lane; i0 += 64 * U) {
+                float v[U], w[U];
+#pragma unroll
+                for (int k = 0; k < U; ++k) { const int i = min(i0 + 64 * k, n - 1); v[k] = x[i]; w[k] = g[i]; }
+#pragma unroll
+                for (int k = 0; k < U; ++k)
+                    if (i0 + 64 * k < n) y[i0 + 64 * k] = v[k] * (w[k] - m);
+            }
+        }
+        return;
+    }
+    for (int h = 0; h < H; ++h) {
+        float m = 0.f, s = 0.f;
+        if (NORMALISE) {
+            const float2 st = a.stats[(int64_t)slot * H + h];
+            m = st.x; s = st.y;
+        } else if (!BWD) {
+            m = -INFINITY;
+            for (int j = lane; j < len; j += 64) m = fmaxf(m, x[(int64_t)j * H + h]);
+            m = head_reduce<true>(m, 1);
+            for (int j = lane; j < len; j += 64) s += __expf(x[(int64_t)j * H + h] - m);
+            s = head_reduce<false>(s, 1);
+        } else {
+            for (int j = lane; j < len; j += 64) m += x[(int64_t)j * H + h] * g[(int64_t)j * H + h];
+            m = head_reduce<false>(m, 1);
+        }
+        if (STATS_ONLY) {
+            if (lane == 0) a.stats[(int64_t)slot * H + h] = make_float2(m, s);
+            continue;
+        }
+        if (!BWD) {
+            const float inv = 1.0f / s;
+            for (int j = lane; j < len; j += 64) y[(int64_t)j * H + h] = __expf(x[(int64_t)j * H + h] - m) * inv;
+        } else {
+            for (int j = lane; j < len; j += 64) y[(int64_t)j * H + h] = x[(int64_t)j * H + h] * (g[(int64_t)j * H + h] - m);
+        }
+    }
+}
+
+// PIECES == false: rows held whole by an item are finished, pieces write their statistics.
+// PIECES == true : pieces only, normalised with the merged statistics of their row.
+template <bool BWD, bool LANEHEAD, bool PIECES>
+__device__ __forceinline__ void edge_softmax_body(const SoftmaxArgs &a) {
+    __shared__ float s_x[kWavesPerBlock][kStage];
+    __shared__ float s_g[BWD ? kWavesPerBlock : 1][BWD ? kStage : 1];
+    const int lane = threadIdx.x & 63;
+    const int64_t item_id = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (item_id >= a.n_items) return;         // uniform per wavefront; no workgroup barriers below
+    const Item it = a.items[item_id];
+    if (it.len == 0) return;
+    if (it.info >= 0) {
+        if (PIECES) run_together<BWD, LANEHEAD, false, true>(a, it.start, it.len, lane, it.info);
+        else run_together<BWD, LANEHEAD, true, false>(a, it.start, it.len, lane, it.info);
+        return;
+    }
+    if (PIECES) return;
+    if (it.info == -1) {
+        run_together<BWD, LANEHEAD, false, false>(a, it.start, it.len, lane, 0);
+        return;
+    }
+    // several whole rows: lane q keeps the end of row q
+    const int nrows = -it.info;
+    const int H = a.H;
+    const int ends = a.indptr[it.row + min(lane, nrows - 1) + 1];
+    const int nf = it.len * H;
+    if (nf <= kStage) {
+        // The item's values are one contiguous run: copy it to LDS with coalesced loads, let one
+        // lane per (row, head) work on its row there, and copy the result out the same way.
+        float *sx = s_x[threadIdx.x >> 6];
+        float *sg = s_g[BWD ? (threadIdx.x >> 6) : 0];
+        const int64_t base = (int64_t)it.start * H;
+        for (int i0 = 0; i0 < nf; i0 += 256) {
+            float v[4], w[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int i = min(i0 + lane + 64 * k, nf - 1);
+                v[k] = a.x[base + i];
+                if (BWD) w[k] = a.g[base + i];
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int i = i0 + lane + 64 * k;
+                if (i < nf) { sx[i] = v[k]; if (BWD) sg[i] = w[k]; }
+            }
+        }
+        wave_lds_sync();
+        const int tasks = nrows * H;
+        for (int t0 = 0; t0 < tasks; t0 += 64) {
+            const int t = min(t0 + lane, tasks - 1);
+            const int q = t / H, h = t - q * H;
+            const int prev = __shfl(ends, max(q - 1, 0));
+            const int e = __shfl(ends, q) - it.start;
+            const int b = q ? prev - it.start : 0;
+            if (t0 + lane < tasks && e > b) {
+                float *r = sx + b * H + h;
+                const int len = e - b;
+                if (!BWD) {
+                    float m = r[0];
+                    for (int j = 1; j < len; ++j) m = fmaxf(m, r[j * H]);
+                    float sum = 0.f;
+                    for (int j = 0; j < len; ++j) { const float ex = __expf(r[j * H] - m); r[j * H] = ex; sum += ex; }
+                    const float inv = 1.0f / sum;
+                    for (int j = 0; j < len; ++j) r[j * H] *= inv;
+                } else {
+                    const float *gr = sg + b * H + h;
+                    float d = 0.f;
+                    for (int j = 0; j < len; ++j) d += r[j * H] * gr[j * H];
+                    for (int j = 0; j < len; ++j) r[j * H] *= gr[j * H] - d;
+                }
+            }
+        }
+        wave_lds_sync();
+        for (int i = lane; i < nf; i += 64) a.y[base + i] = sx[i];
+        return;
+    }
+    if ((int64_t)it.len * H >= 32 * (int64_t)nrows) {
+        // long enough rows: the wavefront takes them one after the other
+        int b = it.start;
+        for (int q = 0; q < nrows; ++q) {
+            const int e = __shfl(ends, q);
+            if (e > b) run_together<BWD, LANEHEAD, false, false>(a, b, e - b, lane, 0);
+            b = e;
+        }
+        return;
+    }
+    // short rows: one lane per (row, head), walking that row's values for its head
+    const int tasks = nrows * H;
+    for (int t0 = 0; t0 < tasks; t0 += 64) {
+        const int t = min(t0 + lane, tasks - 1);
+        const int q = t / H, h = t - q * H;
+        const int prev = __shfl(ends, max(q - 1, 0));
+        const int e = __shfl(ends, q);
+        const int b = q ? prev : it.start;
+        if (t0 + lane < tasks && e > b) {
+            const float *x = a.x + (int64_t)b * H + h;
+            float *y = a.y + (int64_t)b * H + h;
+            const int len = e - b;
+            if (!BWD) {
+                float m = x[0];
+                for (int j = 1; j < len; ++j) m = fmaxf(m, x[(int64_t)j * H]);
+                float s = 0.f;
+                for (int j = 0; j < len; ++j) s += __expf(x[(int64_t)j * H] - m);
+                const float inv = 1.0f / s;
+                for (int j = 0; j < len; ++j) y[(int64_t)j * H] = __expf(x[(int64_t)j * H] - m) * inv;
+            } else {
+                const float *g = a.g + (int64_t)b * H + h;
+                float d = 0.f;
+                for (int j = 0; j < len; ++j) d += x[(int64_t)j * H] * g[(int64_t)j * H];
+                for (int j = 0; j < len; ++j) y[(int64_t)j * H] = x[(int64_t)j * H] * (g[(int64_t)j * H] - d);
+            }
+        }
+    }
+}
+
+// The forward kernel is held to 64 registers (8 wavefronts per SIMD); the gradient kernel is bound
+// by its two LDS staging rows per wavefront instead.
+template <bool LANEHEAD, bool PIECES>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void edge_softmax_kernel(const SoftmaxArgs a) {
+    edge_softmax_body<false, LANEHEAD, PIECES>(a);
+}
+template <bool LANEHEAD, bool PIECES>
+__global__ __launch_bounds__(kBlock) void edge_softmax_backward_kernel(const SoftmaxArgs a) {
+    edge_softmax_body<true, LANEHEAD, PIECES>(a);
+}
+
+// Merges the pieces' statistics of every split row, in piece order, and writes the row's
+// statistics back to each of its pieces.  One lane per (split row, head).
+template <bool BWD>
+__global__ __launch_bounds__(256) void edge_softmax_merge_kernel(const Fixup *fixups, int64_t n_fixups,
+                                                                 float2 *stats, int H) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_fixups * H) return;
+    const Fixup fx = fixups[t / H];
+    const int h = (int)(t % H);
+    float2 *s = stats + (int64_t)fx.slot0 * H + h;
+    float m, sum = 0.f;
+    if (!BWD) {
+        m = s[0].x;
+        for (int p = 1; p < fx.n_pieces; ++p) m = fmaxf(m, s[(int64_t)p * H].x);
+        for (int p = 0; p < fx.n_pieces; ++p) sum += s[(int64_t)p * H].y * __expf(s[(int64_t)p * H].x - m);
+    } else {
+        m = 0.f;
+        for (int p = 0; p < fx.n_pieces; ++p) m += s[(int64_t)p * H].x;
+    }
+    for (int p = 0; p < fx.n_pieces; ++p) s[(int64_t)p * H] = make_float2(m, sum);
+}
+
+template <bool BWD, bool LANEHEAD>
+void launch_both(const fg_spmm_plan *pl, const SoftmaxArgs &a, hipStream_t st) {
+    const dim3 grid((unsigned)((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock));
+    if (BWD) hipLaunchKernelGGL((edge_softmax_backward_kernel<LANEHEAD, false>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((edge_softmax_kernel<LANEHEAD, false>), grid, dim3(kBlock), 0, st, a);
+    if (pl->n_fixups > 0) {
+        const int64_t threads = pl->n_fixups * a.H;
+        hipLaunchKernelGGL(edge_softmax_merge_kernel<BWD>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
+                           pl->fixups_dev, pl->n_fixups, a.stats, a.H);
+        if (BWD) hipLaunchKernelGGL((edge_softmax_backward_kernel<LANEHEAD, true>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((edge_softmax_kernel<LANEHEAD, true>), grid, dim3(kBlock), 0, st, a);
+    }
+}
+
+int softmax_run(const fg_spmm_plan *pl, const int32_t *indptr, const float *x, const float *g, float *y,
+                int H, void *stream, bool bwd) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (pl->num_col_partitions != 1) return fail(FG_ERR_ARG, "edge softmax needs a plan with one column partition");
+    if (H < 1) return fail(FG_ERR_SHAPE, "number of heads must be positive, got %d", H);
+    if (pl->nnz == 0 || pl->n_items == 0) return FG_OK;
+    if (!indptr || !x || !y || (bwd && !g)) return fail(FG_ERR_ARG, "null device pointer");
+    if ((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock > 0x7fffffffLL)
+        return fail(FG_ERR_SHAPE, "too many work items for one grid");
+    int rc = fg::ensure_partial(pl, (size_t)2 * (size_t)H);
+    if (rc != FG_OK) return rc;
+    SoftmaxArgs a;
+    a.items = pl->items_dev; a.n_items = pl->n_items; a.indptr = indptr;
+    a.x = x; a.g = g; a.y = y; a.stats = reinterpret_cast<float2 *>(pl->partial_dev); a.H = H;
+    hipStream_t st = (hipStream_t)stream;
+    const bool lanehead = H <= 64 && (H & (H - 1)) == 0;
+    if (bwd) { if (lanehead) launch_both<true, true>(pl, a, st); else launch_both<true, false>(pl, a, st); }
+    else { if (lanehead) launch_both<false, true>(pl, a, st); else launch_both<false, false>(pl, a, st); }
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
+}
+
+}  // namespace
+
+extern "C" int fg_edge_softmax_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev, const float *scores_dev,
+                                   float *out_dev, int heads, void *stream) {
+    return softmax_run(plan, indptr_dev, scores_dev, nullptr, out_dev, heads, stream, false);
+}
+
+extern "C" int fg_edge_softmax_backward_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev,
+                                            const float *softmax_dev, const float *grad_softmax_dev,
+                                            float *grad_scores_dev, int heads, void *stream) {
+    return softmax_run(plan, indptr_dev, softmax_dev, grad_softmax_dev, grad_scores_dev, heads, stream, true);
+}

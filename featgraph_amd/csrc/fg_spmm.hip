@@ -606,16 +606,6 @@ int launch_ext_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs 
     return fail(FG_ERR_SHAPE, "no max/min kernel for V=%d L=%d K=%d", V, c.L, c.K);
 }
 
-int ensure_partial(const fg_spmm_plan *pl, int F) {
-    const size_t need = (size_t)pl->max_slots_in_partition * (size_t)F;
-    if (need <= pl->partial_floats) return FG_OK;
-    if (pl->partial_dev) FG_HIP_TRY(hipFree(pl->partial_dev));
-    pl->partial_dev = nullptr; pl->partial_floats = 0;
-    FG_HIP_TRY(hipMalloc((void **)&pl->partial_dev, need * sizeof(float)));
-    pl->partial_floats = need;
-    return FG_OK;
-}
-
 // reduce: FG_REDUCE_SUM / MAX / MIN.  heads > 1: vals is [nnz, heads] and every kernel tile must
 // lie inside one head.  vals == nullptr with allow_no_vals: every weight is 1.
 int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
@@ -644,7 +634,7 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
     SpmmConfig c;
     int rc = choose_config(F, T, aligned16, &c);
     if (rc != FG_OK) return rc;
-    if ((rc = ensure_partial(pl, F)) != FG_OK) return rc;
+    if ((rc = fg::ensure_partial(pl, (size_t)F)) != FG_OK) return rc;
     c.off32 = (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;

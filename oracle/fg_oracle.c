@@ -27,12 +27,18 @@
  *       README.md:9-11 points to ("generalized SpMM") but the snapshot holds no code, test or
  *       vector for it.  Pinned by numpy maximum/minimum.reduceat closed forms, by reduce == sum
  *       with H == 1 equalling orc_spmm_csr_rowwise bit-exactly, and by brute force on tiny inputs.
+ *   orc_edge_softmax, orc_edge_softmax_backward
+ *       PARITY UNPINNED by the reference: the snapshot has no attention / softmax operator at all.
+ *       Pinned by scipy.special.softmax per row in float64, rows summing to 1, invariance under a
+ *       per-row shift, one-element rows giving 1, and for the backward pass by torch's float64
+ *       autograd of a dense masked softmax and by central finite differences.
  *   orc_sddmm_multihead
  *       PARITY UNPINNED by the reference: the reference snapshot holds no
  *       multi-head op, test or vector (python/featgraph/op/__init__.py:1-5).
  *       It is pinned only by its closed form (einsum 'ehd,ehd->eh'), by H=1
  *       reducing to orc_sddmm_x86, and by head sums equalling the flat SDDMM.
  */
+#include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -159,6 +165,50 @@ int orc_gspmm(int64_t n_dst, int F, int H, const int32_t *indptr, const int32_t 
                 else if (reduce == 1) o[f] = m > o[f] ? m : o[f];
                 else o[f] = m < o[f] ? m : o[f];
             }
+        }
+    }
+    return ORC_OK;
+}
+
+/*
+ * Softmax over each row's stored elements, separately per head.  NOT IN THE REFERENCE (parity
+ * unpinned, see the header):
+ *   out[e, h] = exp(x[e, h] - m[v, h]) / sum over the row's e' of exp(x[e', h] - m[v, h]),
+ *   m[v, h] = max over the row's elements, v = the row of e.
+ * Elements are visited in stored order; a row without elements writes nothing.
+ */
+int orc_edge_softmax(int64_t n_rows, int H, const int32_t *indptr, const float *x, float *out,
+                     int nthreads) {
+    if (H < 1 || nthreads < 1) return ORC_EARG;
+#pragma omp parallel for num_threads(nthreads) schedule(dynamic, 64)
+    for (int64_t row = 0; row < n_rows; ++row) {
+        const int64_t b = indptr[row], e = indptr[row + 1];
+        for (int h = 0; h < H; ++h) {
+            if (e <= b) continue;
+            float m = x[b * H + h];
+            for (int64_t k = b + 1; k < e; ++k) m = x[k * H + h] > m ? x[k * H + h] : m;
+            float s = 0.0f;
+            for (int64_t k = b; k < e; ++k) s += expf(x[k * H + h] - m);
+            for (int64_t k = b; k < e; ++k) out[k * H + h] = expf(x[k * H + h] - m) / s;
+        }
+    }
+    return ORC_OK;
+}
+
+/*
+ * Gradient of orc_edge_softmax with respect to x, given a = its output and g = dL/da:
+ *   dx[e, h] = a[e, h] * (g[e, h] - sum over the row's e' of a[e', h] * g[e', h]).
+ */
+int orc_edge_softmax_backward(int64_t n_rows, int H, const int32_t *indptr, const float *a,
+                              const float *g, float *dx, int nthreads) {
+    if (H < 1 || nthreads < 1) return ORC_EARG;
+#pragma omp parallel for num_threads(nthreads) schedule(dynamic, 64)
+    for (int64_t row = 0; row < n_rows; ++row) {
+        const int64_t b = indptr[row], e = indptr[row + 1];
+        for (int h = 0; h < H; ++h) {
+            float d = 0.0f;
+            for (int64_t k = b; k < e; ++k) d += a[k * H + h] * g[k * H + h];
+            for (int64_t k = b; k < e; ++k) dx[k * H + h] = a[k * H + h] * (g[k * H + h] - d);
         }
     }
     return ORC_OK;

@@ -52,6 +52,8 @@ def lib():
         L.orc_spmm_csr_rowwise.argtypes = [_i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int]
         L.orc_spmm_dds_x86.argtypes = [_i64, _i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int]
         L.orc_gspmm.argtypes = [_i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int]
+        L.orc_edge_softmax.argtypes = [_i64, _int, _i32p, _f32p, _f32p, _int]
+        L.orc_edge_softmax_backward.argtypes = [_i64, _int, _i32p, _f32p, _f32p, _f32p, _int]
         L.orc_sddmm_x86.argtypes = [_i64, _i64, _i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int, _int]
         L.orc_sddmm_multihead.argtypes = [_i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int]
         L.orc_csr_to_dds.argtypes = [_i64, _i64, _i32p, _i32p, _u32p, _int, _i32p, _i32p, _u32p]
@@ -140,6 +142,29 @@ def gspmm(indptr, indices, vals, x, reduce="sum", nthreads=1):
     _check(lib().orc_gspmm(n_dst, F, H, _p(indptr, _i32p), _p(indices, _i32p), vp, _p(x2, _f32p),
                            _p(out, _f32p), REDUCE[reduce], nthreads), "gspmm")
     return out.reshape((n_dst,) + shape[1:])
+
+
+def edge_softmax(indptr, x, nthreads=1):
+    """Softmax of x ([nnz] or [nnz, H]) over each row's elements, per head.  Not in the reference."""
+    indptr = _c(indptr, np.int32)
+    x = _c(x, np.float32)
+    H = x.shape[1] if x.ndim == 2 else 1
+    out = np.zeros_like(x)
+    _check(lib().orc_edge_softmax(indptr.shape[0] - 1, H, _p(indptr, _i32p), _p(x, _f32p), _p(out, _f32p),
+                                  nthreads), "edge_softmax")
+    return out
+
+
+def edge_softmax_backward(indptr, a, g, nthreads=1):
+    """Gradient of edge_softmax with respect to its input, given its output a and dL/da = g."""
+    indptr = _c(indptr, np.int32)
+    a = _c(a, np.float32); g = _c(g, np.float32)
+    assert a.shape == g.shape
+    H = a.shape[1] if a.ndim == 2 else 1
+    out = np.zeros_like(a)
+    _check(lib().orc_edge_softmax_backward(indptr.shape[0] - 1, H, _p(indptr, _i32p), _p(a, _f32p),
+                                           _p(g, _f32p), _p(out, _f32p), nthreads), "edge_softmax_backward")
+    return out
 
 
 def sddmm_x86(row, col, src, dst, num_feat_partitions=1, parallel_edges=False, nthreads=1):
@@ -235,4 +260,16 @@ def sddmm_multihead_f64(row, col, src, dst, chunk=1 << 18):
         e = slice(s, s + chunk)
         out[e] = np.einsum("ehd,ehd->eh", src[col[e]].astype(np.float64),
                            dst[row[e]].astype(np.float64))
+    return out
+
+
+def edge_softmax_f64(indptr, x):
+    """scipy.special.softmax over each row's slice, float64."""
+    import scipy.special
+    x64 = np.asarray(x, dtype=np.float64)
+    out = np.zeros_like(x64)
+    for r in range(len(indptr) - 1):
+        b, e = int(indptr[r]), int(indptr[r + 1])
+        if e > b:
+            out[b:e] = scipy.special.softmax(x64[b:e], axis=0)
     return out

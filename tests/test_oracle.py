@@ -284,3 +284,72 @@ def test_gspmm_closed_forms(oracle):
     x = rng.standard_normal((80, 24)).astype("float32")
     assert np.array_equal(oracle.gspmm(a.indptr, a.indices, a.data, x, "sum"),
                           oracle.spmm_csr_rowwise(a.indptr, a.indices, a.data, x))
+
+
+# ---- edge softmax (not in the reference: pinned by library routines and invariants) ---------
+
+def _ragged_indptr(rng, n_rows, max_len):
+    lens = rng.integers(0, max_len, size=n_rows)
+    lens[::7] = 0                       # empty rows
+    lens[3] = 1                         # a one-element row
+    lens[5] = 4 * max_len               # a long row
+    return np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+
+
+@pytest.mark.parametrize("H", [1, 3, 4])
+def test_edge_softmax_closed_forms(oracle, H):
+    import scipy.special
+    rng = np.random.default_rng(11 + H)
+    indptr = _ragged_indptr(rng, 60, 40)
+    nnz = int(indptr[-1])
+    x = (rng.standard_normal((nnz, H)) * 3).astype(np.float32)
+    got = oracle.edge_softmax(indptr, x)
+    np.testing.assert_allclose(got, oracle.edge_softmax_f64(indptr, x), rtol=2e-6, atol=1e-7)
+    # dense masked softmax through scipy on the whole matrix at once (a second, differently shaped route)
+    for h in range(H):
+        dense = np.full((60, int(np.diff(indptr).max())), -np.inf)
+        for r in range(60):
+            dense[r, :indptr[r + 1] - indptr[r]] = x[indptr[r]:indptr[r + 1], h]
+        with np.errstate(invalid="ignore"):
+            sm = scipy.special.softmax(dense, axis=1)
+        for r in range(60):
+            np.testing.assert_allclose(got[indptr[r]:indptr[r + 1], h], sm[r, :indptr[r + 1] - indptr[r]],
+                                       rtol=2e-6, atol=1e-7)
+    # every non-empty row sums to one per head; a one-element row is exactly one
+    sums = np.add.reduceat(got.astype(np.float64), indptr[:-1][np.diff(indptr) > 0], axis=0)
+    np.testing.assert_allclose(sums, 1.0, rtol=0, atol=1e-5)
+    assert np.all(got[indptr[3]:indptr[4]] == 1.0)
+    # adding a per-row, per-head constant changes nothing beyond rounding; large inputs do not overflow
+    shift = np.repeat(rng.standard_normal((60, H)).astype(np.float32) * 50, np.diff(indptr), axis=0)
+    np.testing.assert_allclose(oracle.edge_softmax(indptr, x + shift), got, rtol=2e-4, atol=1e-6)
+    assert np.isfinite(oracle.edge_softmax(indptr, x * 1e4)).all()
+    # 1-D input is the one-head case
+    if H == 1:
+        assert np.array_equal(oracle.edge_softmax(indptr, x[:, 0]), got[:, 0])
+
+
+def test_edge_softmax_backward_closed_forms(oracle):
+    import torch
+    rng = np.random.default_rng(5)
+    H = 2
+    indptr = _ragged_indptr(rng, 30, 12)
+    nnz = int(indptr[-1])
+    x = rng.standard_normal((nnz, H)).astype(np.float32)
+    g = rng.standard_normal((nnz, H)).astype(np.float32)
+    a = oracle.edge_softmax(indptr, x)
+    got = oracle.edge_softmax_backward(indptr, a, g)
+    # float64 autograd of torch.softmax applied row by row
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    pieces = [torch.softmax(xt[indptr[r]:indptr[r + 1]], dim=0) for r in range(30) if indptr[r + 1] > indptr[r]]
+    (torch.cat(pieces) * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    np.testing.assert_allclose(got, xt.grad.numpy(), rtol=1e-4, atol=1e-6)
+    # central finite differences of the float64 closed form, a few coordinates
+    def loss(xx):
+        return float((oracle.edge_softmax_f64(indptr, xx) * g).sum())
+    for (e, h) in [(0, 0), (int(indptr[5]) + 3, 1), (nnz - 1, 0)]:
+        xp = x.astype(np.float64).copy(); xm = xp.copy()
+        xp[e, h] += 1e-5; xm[e, h] -= 1e-5
+        np.testing.assert_allclose(got[e, h], (loss(xp) - loss(xm)) / 2e-5, rtol=1e-3, atol=1e-6)
+    # the gradient of each row sums to zero per head (softmax is shift-invariant)
+    rows = indptr[:-1][np.diff(indptr) > 0]
+    np.testing.assert_allclose(np.add.reduceat(got.astype(np.float64), rows, axis=0), 0.0, atol=1e-6)
