@@ -37,7 +37,8 @@ SIGNATURES = {
     "fg_spmm_plan_describe": (_int, [_vp, _int, _int, ctypes.c_char_p, ctypes.c_size_t]),
     "fg_spmm_csr_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
     "fg_spmm_dds_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
-    "fg_gspmm_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp]),
+    "fg_gspmm_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp]),
+    "fg_edge_values_head_major_f32": (_int, [_vp, _vp, _i64, _int, _vp, _vp]),
     "fg_sddmm_coo_f32": (_int, [_vp, _vp, _i64, _vp, _vp, _vp, _int, _int, _vp]),
     "fg_sddmm_csr_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
     "fg_sddmm_dds_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]),

@@ -4,8 +4,9 @@
 
 Configurations: weighted CSR SpMM and SDDMM (CSR-ordered and shuffled COO edges) at feature
 lengths 32..512 and multi-head SDDMM (H in {4, 8}, D in {32, 64}) on the 232,965-node power-law
-graph; SpMM followed by SDDMM at feature length 128 on the 2.45M-node low-degree graph; SpMM on the
-10,000-node uniform graph.  One JSON line per measurement (mean of 5 launches after a warm-up).
+graph, plus the other two steps of an attention layer there (edge softmax and its gradient for
+H in {1, 4, 8}, per-head weighted SpMM for the same head shapes); SpMM followed by SDDMM at feature
+length 128 on the 2.45M-node low-degree graph; SpMM on the 10,000-node uniform graph.  One JSON line per measurement (mean of 5 launches after a warm-up).
 """
 import argparse
 import json
@@ -15,7 +16,9 @@ import scipy.sparse as sp
 import torch
 
 from .. import synthetic
-from ..module import VanillaSpMMhip, VanillaSDDMMhip, MultiHeadSDDMMhip, placeholder
+from ..module import common
+from ..module import (VanillaSpMMhip, VanillaSDDMMhip, MultiHeadSDDMMhip, GSpMMhip, EdgeSoftmaxhip,
+                      placeholder)
 
 HBM_PEAK_GBS = 8000.0
 
@@ -29,7 +32,45 @@ def _line(workload, op, knobs, seconds, nnz, feat_len, bytes_model):
     print(json.dumps(out), flush=True)
 
 
-def run_workload(name, feat_lens, head_shapes, shuffled_coo):
+def _stream_line(workload, op, knobs, seconds, bytes_model):
+    """An operator without gathers: bytes that must move / time against the HBM peak."""
+    out = dict(workload=workload, op=op, **knobs)
+    out.update(ms=round(seconds * 1e3, 4), compulsory_gb=round(bytes_model / 1e9, 3),
+               compulsory_gbs=round(bytes_model / seconds / 1e9, 1),
+               pct_hbm_roofline=round(100.0 * bytes_model / seconds / 1e9 / HBM_PEAK_GBS, 3))
+    print(json.dumps(out), flush=True)
+
+
+def run_attention_steps(name, adj, softmax_heads, head_shapes):
+    n = adj.shape[0]
+    nnz = adj.nnz
+    gen = torch.Generator(device="cuda")
+    sm = EdgeSoftmaxhip(adj)
+    for H in softmax_heads:
+        gen.manual_seed(4)
+        shape = (nnz,) if H == 1 else (nnz, H)
+        s = torch.randn(shape, generator=gen, device="cuda")
+        sm.build([placeholder(shape)])
+        t = sm.measure_average_time([s], 5)
+        _stream_line(name, "edge_softmax", {"heads": H}, t, 4 * (n + 1) + 8 * nnz * H)
+        a = sm.run([s]).clone()
+        t = common.timed_mean_seconds(lambda: sm.backward(a, s), 5)
+        _stream_line(name, "edge_softmax_backward", {"heads": H}, t, 4 * (n + 1) + 12 * nnz * H)
+        del s, a
+    for H, D in head_shapes:
+        gen.manual_seed(2)
+        x = torch.randn((n, H, D), generator=gen, device="cuda")
+        w = torch.rand((nnz, H), generator=gen, device="cuda")
+        m = GSpMMhip(adj)
+        m.build([placeholder((n, H, D)), placeholder((nnz, H))], {}, {})
+        t = m.measure_average_time([x, w], 5)
+        _line(name, "spmm_per_head_weights", {"heads": H, "head_len": D, "partitions": m._active['P'],
+                                              "tiles": m._num_feat_partitions}, t, nnz, H * D,
+              4 * (n + 1) + 4 * nnz + 4 * nnz * H + 8 * n * H * D)
+        del m, x, w
+
+
+def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):
     indptr, indices = synthetic.make_workload(name)
     n = indptr.shape[0] - 1
     nnz = int(indptr[-1])
@@ -64,6 +105,8 @@ def run_workload(name, feat_lens, head_shapes, shuffled_coo):
         _line(name, "sddmm_multihead", {"heads": H, "head_len": D, "tiled": tiled}, t, nnz, H * D,
               4 * (n + 1) + 4 * nnz + 8 * n * H * D + 4 * nnz * H)
         del mh, x, y
+    if softmax_heads:
+        run_attention_steps(name, adj, softmax_heads, head_shapes)
     if shuffled_coo:
         coo = adj.tocoo()
         perm = torch.randperm(nnz, generator=torch.Generator().manual_seed(3)).numpy()
@@ -87,7 +130,7 @@ if __name__ == '__main__':
     args = ap.parse_args()
     run_workload("uniform-10k", [32], [], [])
     if args.quick:
-        run_workload("powerlaw-23k", [32, 128, 512], [(4, 32), (8, 64)], [128])
+        run_workload("powerlaw-23k", [32, 128, 512], [(4, 32), (8, 64)], [128], (1, 4))
     else:
-        run_workload("powerlaw-233k", [32, 64, 128, 256, 512], [(4, 32), (4, 64), (8, 32), (8, 64)], [128])
+        run_workload("powerlaw-233k", [32, 64, 128, 256, 512], [(4, 32), (4, 64), (8, 32), (8, 64)], [128], (1, 4, 8))
         run_workload("powerlaw-2.45M", [128], [], [])

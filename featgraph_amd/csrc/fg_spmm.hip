@@ -67,6 +67,8 @@ struct SpmmArgs {
     int accumulate;        // add to out instead of overwriting it
     int heads;             // weights are [nnz, heads]; a kernel tile lies inside one head
     int head_len;          // floats per head (F / heads)
+    int vstride;           // weight of element t, head h: vals[t * vstride + h * head_stride]
+    int64_t head_stride;
 };
 
 __device__ __forceinline__ float4 vselect(bool c, const float4 &a) {
@@ -161,7 +163,7 @@ __device__ __forceinline__ void finish_row(typename Vec<V>::type (&acc)[K], cons
 // `scale` turns a column id into the staged word: the row's byte size (OFF32) or 1.  The weight of
 // element t is vals[t * vstride + voff] (one weight per head), or 1 when there are no weights.
 __device__ __forceinline__ void stage_load(const int32_t *indices, const float *vals, int64_t base, int n,
-                                           int lane, uint32_t scale, int vstride, int voff, int2 (&r)[4]) {
+                                           int lane, uint32_t scale, int vstride, int64_t voff, int2 (&r)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int t = min(lane + 64 * i, n - 1);
@@ -207,7 +209,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
     const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
     const uint32_t scale = OFF32 ? (uint32_t)a.F * 4u : 1u;
-    const int voff = (rt * a.tile_w + st * FT) / a.head_len;     // head of this kernel tile
+    const int64_t voff = (int64_t)((rt * a.tile_w + st * FT) / a.head_len) * a.head_stride;     // head of this kernel tile
     const int64_t F = a.F;
     int2 *edge = s_edge[wave];
     vec acc[K], old[K];
@@ -235,7 +237,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
             }
         }
         if (it.len > 0) {
-            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.heads, voff, regs);
+            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
             stage_store(edge, lane, regs);
         }
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     const bool add = ACC && it.info < 0;
 #pragma unroll
     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
-    if (it.len > 0) stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.heads, voff, regs);
+    if (it.len > 0) stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
     if (ACC) {
 #pragma unroll
         for (int k = 0; k < K; ++k)
@@ -349,7 +351,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
         wave_lds_sync();
         if (base + fg::kItemEdges < it.len)
             stage_load(a.indices, a.vals, (int64_t)it.start + base + fg::kItemEdges,
-                       it.len - base - fg::kItemEdges, lane, scale, a.heads, voff, regs);
+                       it.len - base - fg::kItemEdges, lane, scale, a.vstride, voff, regs);
         gather_rows<V, L, K, FULL, U, OFF32>(edge, 0, n, g, a.x, lane_bytes, F, on, acc);
     }
     finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
@@ -401,7 +403,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_extreme_kernel(const SpmmArgs a)
     for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
     const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
     const uint32_t scale = OFF32 ? (uint32_t)a.F * 4u : 1u;
-    const int voff = (rt * a.tile_w + st * FT) / a.head_len;
+    const int64_t voff = (int64_t)((rt * a.tile_w + st * FT) / a.head_len) * a.head_stride;
     const int64_t F = a.F;
     int2 *edge = s_edge[wave];
     int2 regs[4];
@@ -456,7 +458,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_extreme_kernel(const SpmmArgs a)
     if (it.info < -1) {
         const int nrows = -it.info;
         if (it.len > 0) {
-            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.heads, voff, regs);
+            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
             stage_store(edge, lane, regs);
         }
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
@@ -475,7 +477,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_extreme_kernel(const SpmmArgs a)
     for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
         const int n = min(fg::kItemEdges, it.len - base);
         wave_lds_sync();
-        stage_load(a.indices, a.vals, (int64_t)it.start + base, n, lane, scale, a.heads, voff, regs);
+        stage_load(a.indices, a.vals, (int64_t)it.start + base, n, lane, scale, a.vstride, voff, regs);
         stage_store(edge, lane, regs);
         wave_lds_sync();
         walk(0, n);
@@ -606,11 +608,11 @@ int launch_ext_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs 
     return fail(FG_ERR_SHAPE, "no max/min kernel for V=%d L=%d K=%d", V, c.L, c.K);
 }
 
-// reduce: FG_REDUCE_SUM / MAX / MIN.  heads > 1: vals is [nnz, heads] and every kernel tile must
-// lie inside one head.  vals == nullptr with allow_no_vals: every weight is 1.
+// reduce: FG_REDUCE_SUM / MAX / MIN.  heads > 1: vals is [nnz, heads] (or [heads, nnz] when
+// head_major) and every kernel tile must lie inside one head.  vals == nullptr with allow_no_vals: every weight is 1.
 int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
              const float *x, float *out, int F, int T, void *stream, int heads = 1,
-             int reduce = FG_REDUCE_SUM, bool allow_no_vals = false) {
+             int reduce = FG_REDUCE_SUM, bool allow_no_vals = false, bool head_major = false) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (pl->n_dst == 0) return FG_OK;
     if (!out || !pos || (pl->nnz > 0 && (!idx || (!vals && !allow_no_vals) || !x)))
@@ -650,6 +652,7 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
             a.out = out; a.partial = pl->partial_dev;
             a.F = F; a.tile_w = c.tile_w; a.sub_per_tile = c.sub_per_tile;
             a.heads = heads; a.head_len = F / heads;
+            a.vstride = head_major ? 1 : heads; a.head_stride = head_major ? pl->nnz : 1;
             a.accumulate = p > 0;
             // More than 8 tiles: 8 at a time (one per XCD), so that an XCD's L2 serves one tile's
             // slice of this partition per launch; the partition's index arrays stay in the
@@ -724,7 +727,32 @@ extern "C" int fg_spmm_dds_f32(const fg_spmm_plan *plan, const int32_t *s1_pos_d
 
 extern "C" int fg_gspmm_f32(const fg_spmm_plan *plan, const int32_t *pos_dev, const int32_t *idx_dev,
                             const float *vals_dev, const float *x_dev, float *out_dev, int F, int heads,
-                            int reduce, int num_feat_partitions, void *stream) {
+                            int vals_head_major, int reduce, int num_feat_partitions, void *stream) {
     return spmm_run(plan, pos_dev, idx_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream, heads,
-                    reduce, /*allow_no_vals=*/true);
+                    reduce, /*allow_no_vals=*/true, vals_head_major != 0);
+}
+
+namespace {
+// dst[h, e] = src[pos[e], h] (pos == nullptr: src[e, h]): one lane per element, the element's
+// heads are read together and written to the heads' own contiguous arrays.
+__global__ __launch_bounds__(256) void edge_values_head_major_kernel(const float *src, const int32_t *pos,
+                                                                     int64_t n, int H, float *dst) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    const float *s = src + (pos ? (int64_t)pos[e] : e) * H;
+    for (int h = 0; h < H; ++h) dst[(int64_t)h * n + e] = s[h];
+}
+}  // namespace
+
+extern "C" int fg_edge_values_head_major_f32(const float *src_dev, const int32_t *edge_pos_dev, int64_t n_edges,
+                                             int heads, float *dst_dev, void *stream) {
+    if (n_edges < 0 || heads < 1) return fail(FG_ERR_ARG, "fg_edge_values_head_major_f32: bad size");
+    if (n_edges == 0) return FG_OK;
+    if (!src_dev || !dst_dev) return fail(FG_ERR_ARG, "null device pointer");
+    const int64_t blocks = (n_edges + 255) / 256;
+    if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "too many edges for one grid");
+    hipLaunchKernelGGL(edge_values_head_major_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       src_dev, edge_pos_dev, n_edges, heads, dst_dev);
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
 }

@@ -66,6 +66,7 @@ class GSpMMhip(VanillaSpMMhip):
         self._active = self._glayout(P)
         self._func = _lib.lib().fg_gspmm_f32
         self._inv_deg_edge = None
+        self._w_head_major = None
         if reduce == 'mean':
             deg = np.diff(self._adj_indptr).astype(np.float32)
             inv = np.where(deg > 0, 1.0 / np.maximum(deg, 1), 0).astype(np.float32)
@@ -82,10 +83,13 @@ class GSpMMhip(VanillaSpMMhip):
                                           shape=(self._num_rows, self._num_cols))
             _, _, edge_pos = util_convert_csr_to_dds(csr, P)
             lay['edge_pos'] = torch.from_numpy(edge_pos.astype(np.int64)).to(self._ctx)
+            lay['edge_pos32'] = torch.from_numpy(edge_pos.astype(np.int32)).to(self._ctx)
         return lay
 
     def _weights(self, given):
-        """Device weights in the active layout's element order, or None for weight 1."""
+        """(device weights in the active layout's element order or None for weight 1, head-major flag).
+        One weight per edge: a 1-D array in element order.  One weight per edge and head: the
+        library's relayout kernel writes them head-major (each head contiguous) in element order."""
         lay = self._active
         if self._msg == 'copy_u':
             w = None
@@ -97,17 +101,28 @@ class GSpMMhip(VanillaSpMMhip):
                 w = common.to_device_f32(self._adj_scipy_csr.data, self._ctx).reshape(-1, 1)
         if self._inv_deg_edge is not None:
             w = self._inv_deg_edge.reshape(-1, 1) if w is None else w * self._inv_deg_edge.reshape(-1, 1)
-        if w is not None and lay['P'] > 1:
+        if w is None:
+            return None, 0
+        if w.shape[1] > 1:
+            w = w.contiguous()
+            if self._w_head_major is None or self._w_head_major.shape != (w.shape[1], w.shape[0]):
+                self._w_head_major = torch.empty((w.shape[1], w.shape[0]), dtype=torch.float32, device=self._ctx)
+            pos = lay['edge_pos32'] if lay['P'] > 1 else None
+            _lib.check(_lib.lib().fg_edge_values_head_major_f32(_lib.dev_ptr(w), _lib.dev_ptr(pos), w.shape[0],
+                                                                w.shape[1], _lib.dev_ptr(self._w_head_major),
+                                                                common.stream_ptr()))
+            return self._w_head_major, 1
+        if lay['P'] > 1:
             w = w.index_select(0, lay['edge_pos'])
-        return None if w is None else w.contiguous()
+        return w.contiguous(), 0
 
     def _launch(self, src_feat, weights=None):
         lay = self._active
-        w = self._weights(weights)
-        heads = self._heads if (w is not None and w.shape[1] > 1) else 1
+        w, head_major = self._weights(weights)
+        heads = self._heads if head_major else 1
         self._w_keepalive = w
         _lib.check(self._func(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(w),
-                              _lib.dev_ptr(src_feat), _lib.dev_ptr(self.out_tvm), self._feat_len, heads,
+                              _lib.dev_ptr(src_feat), _lib.dev_ptr(self.out_tvm), self._feat_len, heads, head_major,
                               _REDUCE[self._reduce], self._num_feat_partitions, common.stream_ptr()))
 
     def run(self, input_tvm_ndarrays):
