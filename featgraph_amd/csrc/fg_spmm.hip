@@ -90,8 +90,10 @@ __device__ __forceinline__ const float *row_ptr(const float *x, uint32_t lane_by
 // weight bits) into acc.  The G lane groups take elements b+g, b+g+G, ...; U steps' loads are
 // issued back to back before the first use.  No load sits under a branch: in the last, partly
 // filled batch a lane without an element re-reads the row's last element with weight zero.
-template <int V, int L, int K, bool FULL, int U, bool OFF32>
-__device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, int g, const float *x,
+// HPT > 1: the kernel tile holds HPT heads and the lane's weight is wrow[slot] (its head's staged
+// weights) instead of the word staged next to the column.
+template <int V, int L, int K, bool FULL, int U, bool OFF32, int HPT>
+__device__ __forceinline__ void gather_rows(const int2 *s_edge, const float *wrow, int b, int e, int g, const float *x,
                                             uint32_t lane_bytes, int64_t F, const bool (&on)[K],
                                             typename Vec<V>::type (&acc)[K]) {
     using vec = typename Vec<V>::type;
@@ -101,7 +103,10 @@ __device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, in
         int2 cw[U];
         vec xv[U][K];
 #pragma unroll
-        for (int u = 0; u < U; ++u) cw[u] = s_edge[s0 + u * G + g];
+        for (int u = 0; u < U; ++u) {
+            cw[u] = s_edge[s0 + u * G + g];
+            if (HPT > 1) cw[u].y = __float_as_int(wrow[s0 + u * G + g]);
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -121,6 +126,7 @@ __device__ __forceinline__ void gather_rows(const int2 *s_edge, int b, int e, in
         for (int u = 0; u < U; ++u) {
             const int j = s0 + u * G + g;
             cw[u] = s_edge[j < e ? j : e - 1];
+            if (HPT > 1) cw[u].y = __float_as_int(wrow[j < e ? j : e - 1]);
             if (j >= e) cw[u].y = 0;
         }
 #pragma unroll
@@ -177,10 +183,33 @@ __device__ __forceinline__ void stage_store(int2 *edge, int lane, const int2 (&r
     if (lane < kPad) edge[fg::kItemEdges + lane] = r[3];      // a valid element: slots past the end stay loadable
 }
 
+// The same for the weights of the HPT heads of a kernel tile (head h of the tile: vals[t * vstride + voff + h * hstride]).
+template <int HPT>
+__device__ __forceinline__ void stage_load_w(const float *vals, int64_t base, int n, int lane, int vstride,
+                                             int64_t voff, int64_t hstride, float (&w)[HPT][4]) {
+#pragma unroll
+    for (int h = 0; h < HPT; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = min(lane + 64 * i, n - 1);
+            w[h][i] = vals ? vals[(base + t) * vstride + voff + h * hstride] : 1.0f;
+        }
+}
+template <int HPT, int ROW>
+__device__ __forceinline__ void stage_store_w(float (*rows)[ROW], int lane, const float (&w)[HPT][4]) {
+#pragma unroll
+    for (int h = 0; h < HPT; ++h) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rows[h][lane + 64 * i] = w[h][i];
+        if (lane < kPad) rows[h][fg::kItemEdges + lane] = w[h][3];
+    }
+}
+
 // V: floats per lane per load; L: lanes per source row; K: loads per lane per source row;
 // FULL: every lane's columns are inside the tile (no masking needed); ACC: add to out;
-// OFF32: X spans less than 4 GiB, rows are addressed by 32-bit byte offsets.
-template <int V, int L, int K, bool FULL, bool ACC, bool OFF32>
+// OFF32: X spans less than 4 GiB, rows are addressed by 32-bit byte offsets; HPT: heads (with
+// their own weights) per kernel tile, each covered by L / HPT lanes.
+template <int V, int L, int K, bool FULL, bool ACC, bool OFF32, int HPT = 1>
 __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     using vec = typename Vec<V>::type;
     static_assert(fg::kItemEdges == 256, "stage_load/stage_store move 4 x 64 elements");
@@ -192,6 +221,9 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
     __shared__ int32_t s_next[kWavesPerBlock];
+    constexpr int kWRow = HPT > 1 ? fg::kItemEdges + kPad : 1;
+    __shared__ float s_w[kWavesPerBlock][HPT][kWRow];
+    static_assert(HPT == 1 || (L % HPT == 0 && K == 1 && FULL), "heads of a tile split its lanes evenly");
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -212,8 +244,11 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     const int64_t voff = (int64_t)((rt * a.tile_w + st * FT) / a.head_len) * a.head_stride;     // head of this kernel tile
     const int64_t F = a.F;
     int2 *edge = s_edge[wave];
+    const float *wrow = s_w[wave][HPT > 1 ? (lane % L) / (L / HPT) : 0];
+    const float *col_vals = HPT > 1 ? nullptr : a.vals;     // HPT > 1: weights are staged per head instead
     vec acc[K], old[K];
     int2 regs[4];
+    float wregs[HPT][4];
 
     if (it.info < -1) {
         // Several whole rows: stage all their elements once.
@@ -237,8 +272,10 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
             }
         }
         if (it.len > 0) {
-            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
+            stage_load(a.indices, col_vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
+            if (HPT > 1) stage_load_w<HPT>(a.vals, it.start, it.len, lane, a.vstride, voff, a.head_stride, wregs);
             stage_store(edge, lane, regs);
+            if (HPT > 1) stage_store_w<HPT>(s_w[wave], lane, wregs);
         }
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
         if (lane == 0) s_next[wave] = 0;
@@ -261,7 +298,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
                     }
 #pragma unroll
                     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
-                    gather_rows<V, L, K, FULL, U, OFF32>(edge, b, e, g, a.x, lane_bytes, F, on, acc);
+                    gather_rows<V, L, K, FULL, U, OFF32, HPT>(edge, wrow, b, e, g, a.x, lane_bytes, F, on, acc);
                     finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
                 }
                 b = e;
@@ -313,6 +350,7 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
                     // past the row's end this is a later row's element (or the padding): a valid
                     // source row, given weight zero
                     cw[u] = edge[j + u];
+                    if (HPT > 1) cw[u].y = __float_as_int(wrow[j + u]);
                     if (j + u >= e) cw[u].y = 0;
                 }
 #pragma unroll
@@ -338,7 +376,10 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
     const bool add = ACC && it.info < 0;
 #pragma unroll
     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
-    if (it.len > 0) stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
+    if (it.len > 0) {
+        stage_load(a.indices, col_vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
+        if (HPT > 1) stage_load_w<HPT>(a.vals, it.start, it.len, lane, a.vstride, voff, a.head_stride, wregs);
+    }
     if (ACC) {
 #pragma unroll
         for (int k = 0; k < K; ++k)
@@ -348,11 +389,16 @@ __global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
         const int n = min(fg::kItemEdges, it.len - base);
         wave_lds_sync();                   // earlier reads of the staging row are done
         stage_store(edge, lane, regs);
+        if (HPT > 1) stage_store_w<HPT>(s_w[wave], lane, wregs);
         wave_lds_sync();
-        if (base + fg::kItemEdges < it.len)
-            stage_load(a.indices, a.vals, (int64_t)it.start + base + fg::kItemEdges,
+        if (base + fg::kItemEdges < it.len) {
+            stage_load(a.indices, col_vals, (int64_t)it.start + base + fg::kItemEdges,
                        it.len - base - fg::kItemEdges, lane, scale, a.vstride, voff, regs);
-        gather_rows<V, L, K, FULL, U, OFF32>(edge, 0, n, g, a.x, lane_bytes, F, on, acc);
+            if (HPT > 1)
+                stage_load_w<HPT>(a.vals, (int64_t)it.start + base + fg::kItemEdges, it.len - base - fg::kItemEdges,
+                                  lane, a.vstride, voff, a.head_stride, wregs);
+        }
+        gather_rows<V, L, K, FULL, U, OFF32, HPT>(edge, wrow, 0, n, g, a.x, lane_bytes, F, on, acc);
     }
     finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
 }
@@ -526,6 +572,7 @@ struct SpmmConfig {
     int tile_w, sub_per_tile, n_ftiles;
     bool full;
     bool off32;     // every source row starts less than 4 GiB into X
+    int hpt = 1;    // heads (with their own weights) per kernel tile
 };
 
 int pow2_ceil(int v) { int p = 1; while (p < v) p <<= 1; return p; }
@@ -556,6 +603,18 @@ void launch_off(bool off32, dim3 grid, hipStream_t st, const SpmmArgs &a) {
     else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, FULL, ACC, false>), grid, dim3(kBlock), 0, st, a);
 }
 
+// tiles of HPT heads: 128-bit lanes, one load per lane, no masking
+template <int L, int HPT>
+void launch_hpt(bool off32, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+    if (a.accumulate) {
+        if (off32) hipLaunchKernelGGL((spmm_items_kernel<4, L, 1, true, true, true, HPT>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((spmm_items_kernel<4, L, 1, true, true, false, HPT>), grid, dim3(kBlock), 0, st, a);
+    } else {
+        if (off32) hipLaunchKernelGGL((spmm_items_kernel<4, L, 1, true, false, true, HPT>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((spmm_items_kernel<4, L, 1, true, false, false, HPT>), grid, dim3(kBlock), 0, st, a);
+    }
+}
+
 template <int V, int L, int K>
 void launch_vlk(bool full, bool off32, dim3 grid, hipStream_t st, const SpmmArgs &a) {
     if (a.accumulate) {
@@ -569,6 +628,15 @@ void launch_vlk(bool full, bool off32, dim3 grid, hipStream_t st, const SpmmArgs
 
 template <int V>
 int launch_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+    if (c.hpt > 1) {
+        if (V == 4 && c.K == 1 && c.full) {
+            if (c.L == 16 && c.hpt == 2) { launch_hpt<16, 2>(c.off32, grid, st, a); return FG_OK; }
+            if (c.L == 16 && c.hpt == 4) { launch_hpt<16, 4>(c.off32, grid, st, a); return FG_OK; }
+            if (c.L == 8 && c.hpt == 4) { launch_hpt<8, 4>(c.off32, grid, st, a); return FG_OK; }
+            if (c.L == 4 && c.hpt == 4) { launch_hpt<4, 4>(c.off32, grid, st, a); return FG_OK; }
+        }
+        return fail(FG_ERR_SHAPE, "no SpMM kernel for %d heads per tile with V=%d L=%d K=%d", c.hpt, V, c.L, c.K);
+    }
     if (c.K == 1) {
         switch (c.L) {
             case 4: launch_vlk<V, 4, 1>(c.full, c.off32, grid, st, a); return FG_OK;
@@ -623,19 +691,37 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
         return fail(FG_ERR_ARG, "max / min aggregation needs a plan with one column partition");
     if (heads < 1 || F % heads != 0) return fail(FG_ERR_SHAPE, "feature length %d is not divisible by %d heads", F, heads);
     const bool aligned16 = (((uintptr_t)x | (uintptr_t)out) & 15) == 0;
+    int hpt = 1;
     if (heads > 1) {
-        // tiles must not straddle heads: tile = the head, or 64 floats when that divides the head
+        // A kernel tile holds whole heads or lies inside one: 64 floats when the head length divides
+        // or is a multiple of 64, else (short heads) 4 heads; the sum kernel stages one weight per
+        // head of the tile.
         const int D = F / heads;
-        const int want = (D % 64 == 0) ? 64 : D;
-        if (want % 4 != 0 || want < 16 || (want & (want - 1)) != 0 || !aligned16)
-            return fail(FG_ERR_SHAPE, "per-head weights need a head length that is a power of two >= 16 or a multiple of 64, got %d", D);
-        if (T == 0) T = F / want;
-        if (T < 1 || F % T != 0 || D % (F / T) != 0 || (((F / T) & (F / T - 1)) != 0) || F / T > 256)
-            return fail(FG_ERR_SHAPE, "num_feat_partitions %d does not cut %d-float heads into power-of-two tiles", T, D);
+        if (D % 4 != 0 || !aligned16) return fail(FG_ERR_SHAPE, "per-head weights need a head length that is a multiple of 4 and 16-byte aligned arrays, got %d", D);
+        int tile;
+        if (T == 0) {
+            if (D % 64 == 0) tile = 64;
+            else if ((D & (D - 1)) != 0) return fail(FG_ERR_SHAPE, "per-head weights need a head length that is a power of two or a multiple of 64, got %d", D);
+            else if (D >= 16) tile = (reduce == FG_REDUCE_SUM && 64 % D == 0 && F % 64 == 0) ? 64 : D;
+            else tile = (reduce == FG_REDUCE_SUM && heads % 4 == 0) ? 4 * D : 0;
+            if (tile == 0) return fail(FG_ERR_SHAPE, "no kernel for %d heads of %d floats with this aggregation", heads, D);
+            T = F / tile;
+        } else {
+            if (T < 1 || F % T != 0) return fail(FG_ERR_SHAPE, "feature length %d is not divisible by num_feat_partitions %d", F, T);
+            tile = F / T;
+        }
+        if ((tile & (tile - 1)) != 0 || tile > 256 || tile < 16 || !(tile % D == 0 || D % tile == 0))
+            return fail(FG_ERR_SHAPE, "num_feat_partitions %d does not cut %d-float heads into power-of-two tiles of 16..256 floats", T, D);
+        if (tile > D) {
+            hpt = tile / D;
+            if (reduce != FG_REDUCE_SUM || !(hpt == 2 || hpt == 4) || tile > 64 || (tile == 64 ? false : hpt != 4))
+                return fail(FG_ERR_SHAPE, "no kernel for tiles of %d floats holding %d heads", tile, hpt);
+        }
     }
     SpmmConfig c;
     int rc = choose_config(F, T, aligned16, &c);
     if (rc != FG_OK) return rc;
+    c.hpt = hpt;
     if ((rc = fg::ensure_partial(pl, (size_t)F)) != FG_OK) return rc;
     c.off32 = (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
     hipStream_t st = (hipStream_t)stream;

@@ -76,7 +76,9 @@ def test_sum_and_mean(torch_cuda, oracle, reduce, P):
 
 
 @pytest.mark.parametrize("H,D,reduce,P", [(4, 64, "sum", None), (8, 64, "sum", 3), (4, 32, "sum", None), (2, 16, "max", None),
-                                          (8, 128, "sum", None), (4, 64, "min", None), (4, 32, "mean", 2), (1, 48, "sum", None)])
+                                          (8, 128, "sum", None), (4, 64, "min", None), (4, 32, "mean", 2), (1, 48, "sum", None),
+                                          (8, 8, "sum", None), (8, 8, "sum", 3), (4, 16, "sum", 2), (16, 4, "sum", None),
+                                          (2, 32, "sum", 4), (3, 32, "sum", None), (8, 16, "mean", None)])
 def test_per_head_weights(torch_cuda, oracle, H, D, reduce, P):
     """out[v,h,:] = reduce_e w[e,h] * x[u,h,:] with weights handed to run() in CSR edge order."""
     from featgraph_amd.module import GSpMMhip, placeholder
