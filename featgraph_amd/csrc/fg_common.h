@@ -68,4 +68,6 @@ namespace fg {
 // Makes plan->partial_dev hold at least floats_per_piece floats for every piece of split rows of
 // one partition (grown on demand, never shrunk).
 int ensure_partial(const fg_spmm_plan *plan, size_t floats_per_piece);
+// FG_OK when the calling thread's current device is the one the plan was created on.
+int check_device(const fg_spmm_plan *plan);
 }  // namespace fg

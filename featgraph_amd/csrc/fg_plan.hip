@@ -127,6 +127,13 @@ extern "C" void fg_spmm_plan_destroy(fg_spmm_plan *pl) {
 }
 
 namespace fg {
+int check_device(const fg_spmm_plan *pl) {
+    int dev = -1;
+    FG_HIP_TRY(hipGetDevice(&dev));
+    if (dev != pl->device)
+        return fail(FG_ERR_ARG, "the plan lives on device %d but the current device is %d", pl->device, dev);
+    return FG_OK;
+}
 int ensure_partial(const fg_spmm_plan *pl, size_t floats_per_piece) {
     const size_t need = (size_t)pl->max_slots_in_partition * floats_per_piece;
     if (need <= pl->partial_floats) return FG_OK;

@@ -698,6 +698,7 @@ extern "C" int fg_sddmm_csr_f32(const fg_spmm_plan *plan, const int32_t *indptr_
                                 const int32_t *indices_dev, const float *src_dev, const float *dst_dev,
                                 float *out_dev, int H, int D, void *stream) {
     if (!plan) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(plan)) return drc;
     if (plan->num_col_partitions != 1) return fail(FG_ERR_ARG, "fg_sddmm_csr_f32 needs a plan with one column partition");
     return sddmm_run(plan, nullptr, indices_dev, indptr_dev, plan->n_dst, plan->nnz, src_dev, dst_dev,
                      out_dev, H, D, stream);
@@ -718,6 +719,7 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
                                 const int32_t *edge_pos_dev, const float *src_dev, const float *dst_dev,
                                 float *out_dev, int H, int D, int num_feat_partitions, void *stream) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
     if (H < 1 || D < 1) return fail(FG_ERR_SHAPE, "heads and head length must be positive, got H=%d D=%d", H, D);
     if (pl->nnz == 0) return FG_OK;
     if (!s1_pos_dev || !s1_idx_dev || !edge_pos_dev || !src_dev || !dst_dev || !out_dev)

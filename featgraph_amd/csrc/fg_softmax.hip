@@ -371,6 +371,7 @@ void launch_both(const fg_spmm_plan *pl, const SoftmaxArgs &a, hipStream_t st) {
 int softmax_run(const fg_spmm_plan *pl, const int32_t *indptr, const float *x, const float *g, float *y,
                 int H, void *stream, bool bwd) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
     if (pl->num_col_partitions != 1) return fail(FG_ERR_ARG, "edge softmax needs a plan with one column partition");
     if (H < 1) return fail(FG_ERR_SHAPE, "number of heads must be positive, got %d", H);
     if (pl->nnz == 0 || pl->n_items == 0) return FG_OK;

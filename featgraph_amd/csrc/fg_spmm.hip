@@ -682,6 +682,7 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
              const float *x, float *out, int F, int T, void *stream, int heads = 1,
              int reduce = FG_REDUCE_SUM, bool allow_no_vals = false, bool head_major = false) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
     if (pl->n_dst == 0) return FG_OK;
     if (!out || !pos || (pl->nnz > 0 && (!idx || (!vals && !allow_no_vals) || !x)))
         return fail(FG_ERR_ARG, "null device pointer");

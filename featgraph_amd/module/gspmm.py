@@ -77,12 +77,11 @@ class GSpMMhip(VanillaSpMMhip):
         """Layout for P source partitions plus, for P > 1, each DDS element's CSR position (so that
         weights given in CSR order can be brought into DDS order on the device)."""
         lay = self._layout(P)
-        if P > 1 and 'edge_pos' not in lay:
+        if P > 1 and 'edge_pos32' not in lay:
             nnz = self._adj_indices.shape[0]
             csr = scipy.sparse.csr_matrix((np.arange(nnz, dtype=np.int32), self._adj_indices, self._adj_indptr),
                                           shape=(self._num_rows, self._num_cols))
             _, _, edge_pos = util_convert_csr_to_dds(csr, P)
-            lay['edge_pos'] = torch.from_numpy(edge_pos.astype(np.int64)).to(self._ctx)
             lay['edge_pos32'] = torch.from_numpy(edge_pos.astype(np.int32)).to(self._ctx)
         return lay
 
@@ -103,7 +102,7 @@ class GSpMMhip(VanillaSpMMhip):
             w = self._inv_deg_edge.reshape(-1, 1) if w is None else w * self._inv_deg_edge.reshape(-1, 1)
         if w is None:
             return None, 0
-        if w.shape[1] > 1:
+        if w.shape[1] > 1 or lay['P'] > 1:
             w = w.contiguous()
             if self._w_head_major is None or self._w_head_major.shape != (w.shape[1], w.shape[0]):
                 self._w_head_major = torch.empty((w.shape[1], w.shape[0]), dtype=torch.float32, device=self._ctx)
@@ -112,14 +111,12 @@ class GSpMMhip(VanillaSpMMhip):
                                                                 w.shape[1], _lib.dev_ptr(self._w_head_major),
                                                                 common.stream_ptr()))
             return self._w_head_major, 1
-        if lay['P'] > 1:
-            w = w.index_select(0, lay['edge_pos'])
         return w.contiguous(), 0
 
     def _launch(self, src_feat, weights=None):
         lay = self._active
         w, head_major = self._weights(weights)
-        heads = self._heads if head_major else 1
+        heads = w.shape[0] if head_major else 1
         self._w_keepalive = w
         _lib.check(self._func(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(w),
                               _lib.dev_ptr(src_feat), _lib.dev_ptr(self.out_tvm), self._feat_len, heads, head_major,
