@@ -161,7 +161,8 @@ def test_tiled_traversal(torch_cuda, oracle, feat_len, P, T, order):
 @pytest.mark.parametrize("H,D,P,T", [(8, 64, 4, 8), (4, 32, 2, 2), (8, 32, 3, 1), (2, 8, 2, 1), (4, 64, 1, 4),
                                      (16, 16, 2, 4), (4, 256, 2, 4)])
 def test_tiled_multihead(torch_cuda, oracle, H, D, P, T):
-    """Whole heads per feature tile: results go straight to out[edge, head]."""
+    """Whole heads per feature tile: results go straight to out[edge, head], or (one head per tile,
+    four heads or more) through a per-tile staging array and a last kernel that writes each edge's heads."""
     from featgraph_amd.module import MultiHeadSDDMMhip
     rng = np.random.default_rng(H * 1000 + D)
     coo = _rand_coo(rng, 150, 900, 0.05, shuffle=True)
