@@ -71,10 +71,6 @@ struct SpmmArgs {
     int64_t head_stride;
 };
 
-__device__ __forceinline__ float4 vselect(bool c, const float4 &a) {
-    return make_float4(c ? a.x : 0.f, c ? a.y : 0.f, c ? a.z : 0.f, c ? a.w : 0.f);
-}
-__device__ __forceinline__ float vselect(bool c, const float &a) { return c ? a : 0.f; }
 
 // Address of this lane's part of a staged source row.  OFF32: the staged word is the row's byte
 // offset from the (wave-uniform) start of X and fits 32 bits, so the load takes a scalar base
