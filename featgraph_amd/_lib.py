@@ -22,7 +22,15 @@ _int = ctypes.c_int
 
 class FgPlanOpts(ctypes.Structure):
     _fields_ = [("split_threshold", ctypes.c_int32), ("item_edges", ctypes.c_int32),
-                ("reserved", ctypes.c_int32 * 6)]
+                ("wide_offsets", ctypes.c_int32), ("reserved", ctypes.c_int32 * 5)]
+
+
+# Options every module passes to fg_spmm_plan_create (None: the library's defaults).
+plan_opts = None
+
+
+def plan_opts_ptr():
+    return ctypes.byref(plan_opts) if plan_opts is not None else None
 
 
 # name -> (restype, argtypes); also the list of symbols the header declares

@@ -51,6 +51,7 @@ struct fg_spmm_plan {
     int num_col_partitions = 1;
     int split_threshold = 0;
     int item_edges = 0;              // element budget of a multi-row item
+    bool wide_offsets = false;       // never use 32-bit byte offsets into the feature matrices
     int device = 0;
     // per partition: [item_begin, item_end) and [fixup_begin, fixup_end)
     std::vector<int64_t> item_off, fixup_off;

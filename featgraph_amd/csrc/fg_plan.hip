@@ -44,6 +44,7 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
     auto *pl = new fg_spmm_plan();
     pl->n_dst = n_dst; pl->n_src = n_src; pl->nnz = prev;
     pl->num_col_partitions = P; pl->split_threshold = split; pl->item_edges = item_edges;
+    pl->wide_offsets = opts && opts->wide_offsets != 0;
     std::vector<Item> items;
     std::vector<Fixup> fixups;
     items.reserve((size_t)(n_dst + n_dst / 8 + 16));

@@ -795,7 +795,7 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
         a.src = src_dev + (int64_t)p * width * F;
         const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * T;
         if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
-        const bool off32 = (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
+        const bool off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
         const bool ok = (tile_sum || staged) ? launch_tiled_l<false>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a)
                                  : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
         if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);

@@ -720,7 +720,7 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
     if (rc != FG_OK) return rc;
     c.hpt = hpt;
     if ((rc = fg::ensure_partial(pl, (size_t)F)) != FG_OK) return rc;
-    c.off32 = (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
+    c.off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;

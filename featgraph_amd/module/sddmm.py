@@ -72,7 +72,7 @@ class SDDMMbase(object):
             self._adj_indptr_dev = common.to_device_i32(indptr, self._ctx)
             with torch.cuda.device(self._ctx):
                 _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(indptr), self._num_rows, self._num_cols,
-                                                          1, None, ctypes.byref(self._plan)))
+                                                          1, _lib.plan_opts_ptr(), ctypes.byref(self._plan)))
         # source-column-partitioned copies of the edge list for the tiled traversal, by P
         self._dds = {}
         # To be updated in self.build
@@ -119,7 +119,7 @@ class SDDMMbase(object):
         d = {'P': P, 'pos': common.to_device_i32(s1_pos, self._ctx), 'idx': common.to_device_i32(s1_idx, self._ctx),
              'edge_pos': common.to_device_i32(edge_pos, self._ctx), 'plan': ctypes.c_void_p()}
         with torch.cuda.device(self._ctx):
-            _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(s1_pos), self._num_rows, self._num_cols, P, None,
+            _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(s1_pos), self._num_rows, self._num_cols, P, _lib.plan_opts_ptr(),
                                                       ctypes.byref(d['plan'])))
         self._dds[P] = d
         return d

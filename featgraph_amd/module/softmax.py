@@ -34,7 +34,7 @@ class EdgeSoftmaxhip(object):
         self._plan = ctypes.c_void_p()
         with torch.cuda.device(self._ctx):
             _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(self._indptr), self._num_rows, self._num_cols,
-                                                      1, None, ctypes.byref(self._plan)))
+                                                      1, _lib.plan_opts_ptr(), ctypes.byref(self._plan)))
         self._placeholders = None
         self._heads = None
         self.out_tvm = None

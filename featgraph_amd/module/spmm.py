@@ -79,7 +79,7 @@ class SpMMbase(object):
                'pos': common.to_device_i32(pos, self._ctx), 'idx': common.to_device_i32(idx, self._ctx),
                'vals': common.to_device_f32(vals, self._ctx), 'plan': ctypes.c_void_p()}
         with torch.cuda.device(self._ctx):
-            _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(pos), self._num_rows, self._num_cols, P, None,
+            _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(pos), self._num_rows, self._num_cols, P, _lib.plan_opts_ptr(),
                                                       ctypes.byref(lay['plan'])))
         self._layouts[P] = lay
         return lay
