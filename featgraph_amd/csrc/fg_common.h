@@ -57,6 +57,7 @@ struct fg_spmm_plan {
     std::vector<int64_t> item_off, fixup_off;
     int64_t n_items = 0, n_fixups = 0, n_slots = 0, max_slots_in_partition = 0;
     fg::Item *items_dev = nullptr;
+    int64_t *item_off_dev = nullptr;     // item_off on the device (num_col_partitions + 1 entries)
     fg::Fixup *fixups_dev = nullptr;
     // partial sums of split rows; grown on demand to max_slots_in_partition * F floats
     mutable float *partial_dev = nullptr;

@@ -108,6 +108,9 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
     if (e == hipSuccess && pl->n_items) e = hipMalloc((void **)&pl->items_dev, sizeof(Item) * items.size());
     if (e == hipSuccess && pl->n_items)
         e = hipMemcpy(pl->items_dev, items.data(), sizeof(Item) * items.size(), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMalloc((void **)&pl->item_off_dev, sizeof(int64_t) * pl->item_off.size());
+    if (e == hipSuccess)
+        e = hipMemcpy(pl->item_off_dev, pl->item_off.data(), sizeof(int64_t) * pl->item_off.size(), hipMemcpyHostToDevice);
     if (e == hipSuccess && pl->n_fixups) e = hipMalloc((void **)&pl->fixups_dev, sizeof(Fixup) * fixups.size());
     if (e == hipSuccess && pl->n_fixups)
         e = hipMemcpy(pl->fixups_dev, fixups.data(), sizeof(Fixup) * fixups.size(), hipMemcpyHostToDevice);
@@ -122,6 +125,7 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
 extern "C" void fg_spmm_plan_destroy(fg_spmm_plan *pl) {
     if (!pl) return;
     if (pl->items_dev) (void)hipFree(pl->items_dev);
+    if (pl->item_off_dev) (void)hipFree(pl->item_off_dev);
     if (pl->fixups_dev) (void)hipFree(pl->fixups_dev);
     if (pl->partial_dev) (void)hipFree(pl->partial_dev);
     delete pl;

@@ -10,6 +10,8 @@
 // already held in registers is reused instead of fetched again.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "fg_common.h"
 
 using fg::fail;
@@ -253,12 +255,15 @@ __global__ __launch_bounds__(kBlock) void sddmm_csr_kernel(const SddmmArgs a) {
 // go straight to out.  Results are scattered to the caller's edge order through edge_pos.
 
 struct SddmmTiledArgs {
-    const Item *items;
-    int64_t n_items;
-    const int32_t *pos;       // this partition's row boundaries
+    const Item *items;        // all partitions' items
+    const int64_t *item_off;  // [n_parts + 1]: partition p owns items [item_off[p], item_off[p + 1])
+    const int32_t *pos;       // row boundaries, one array of pos_stride entries per partition
+    int64_t pos_stride;
     const int32_t *col;       // partition-local column ids, DDS order
     const int32_t *edge_pos;  // DDS position -> position in the caller's edge order
-    const float *src;         // offset to the partition's first src row
+    const float *src;         // partition p's first src row is src + p * src_stride
+    int64_t src_stride;
+    int first_part, conc, n_parts;   // this launch works on partitions [first_part, first_part + conc)
     const float *dst;
     float *out;               // out (direct mode) or partial (tile-sum mode)
     int64_t out_edge_stride;  // floats between consecutive edges in out
@@ -356,10 +361,19 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane / L, li = lane % L;
-    const int tile = (int)(blockIdx.x % (unsigned)a.n_tiles);
-    const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_tiles) * kWavesPerBlock + wave;
-    if (item_id >= a.n_items) return;
-    const Item it = a.items[item_id];
+    // workgroup id = (item block, partition in flight, tile), tile fastest: with n_tiles * conc == 8
+    // every XCD works on one tile of one partition
+    const unsigned per = (unsigned)(a.n_tiles * a.conc);
+    const int slot = (int)(blockIdx.x % per);
+    const int tile = slot % a.n_tiles;
+    const int part = a.first_part + slot / a.n_tiles;
+    if (part >= a.n_parts) return;
+    const int64_t i0 = a.item_off[part];
+    const int64_t item_id = (int64_t)(blockIdx.x / per) * kWavesPerBlock + wave;
+    if (item_id >= a.item_off[part + 1] - i0) return;
+    const Item it = a.items[i0 + item_id];
+    const int32_t *pos = a.pos + part * a.pos_stride;
+    const float *src = a.src + part * a.src_stride;
     if (it.len == 0) return;
     const int64_t F = a.F;
     const int f_lo = tile * (L * K * 4) + li * 4;
@@ -404,7 +418,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
             touched[i] = a.dst[(int64_t)(it.row + r) * F + tile * (L * K * 4) + f];
         }
         stage(it.start, it.len);
-        s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        s_end[wave][lane] = pos[it.row + min(lane, nrows - 1) + 1] - it.start;
         if (lane == 0) s_next[wave] = 0;
         wave_lds_sync();
 #pragma unroll
@@ -418,10 +432,10 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
                     load_dst(it.row + q);
                     int s0 = b;
                     for (; s0 + G * U <= e; s0 += G * U)
-                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, e, a.src, lane_bytes, F, dv,
+                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, e, src, lane_bytes, F, dv,
                                                                                  out, a.out_edge_stride, it.start, seg_pos);
                     if (s0 < e)
-                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, true>(edge, s0 + g, G, e, a.src, lane_bytes, F, dv,
+                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, true>(edge, s0 + g, G, e, src, lane_bytes, F, dv,
                                                                           out, a.out_edge_stride, it.start, seg_pos);
                 }
                 b = e;
@@ -448,7 +462,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
             }
             if (__all(done)) break;
             if (!done && j < e) {
-                sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false>(edge, j, 1, e, a.src, lane_bytes, F, dv, out,
+                sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false>(edge, j, 1, e, src, lane_bytes, F, dv, out,
                                                                   a.out_edge_stride, it.start, seg_pos);
                 j += U;
             }
@@ -464,10 +478,10 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         wave_lds_sync();
         int s0 = 0;
         for (; s0 + G * U <= n; s0 += G * U)
-            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, n, a.src, lane_bytes, F, dv, out,
+            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
                                                                      a.out_edge_stride, (int64_t)it.start + base, seg_pos);
         if (s0 < n)
-            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, true>(edge, s0 + g, G, n, a.src, lane_bytes, F, dv, out,
+            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, true>(edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
                                                               a.out_edge_stride, (int64_t)it.start + base, seg_pos);
     }
 }
@@ -787,17 +801,25 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
     }
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
-    for (int p = 0; p < P; ++p) {
-        const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
-        if (i1 == i0) continue;
-        a.items = pl->items_dev + i0; a.n_items = i1 - i0;
-        a.pos = s1_pos_dev + (int64_t)p * (pl->n_dst + 1);
-        a.src = src_dev + (int64_t)p * width * F;
-        const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * T;
+    a.items = pl->items_dev; a.item_off = pl->item_off_dev;
+    a.pos = s1_pos_dev; a.pos_stride = pl->n_dst + 1;
+    a.src = src_dev; a.src_stride = width * F; a.n_parts = P;
+    // Fewer than 8 tiles: 8 / T partitions per launch, so that every XCD still has one tile of one
+    // partition to itself (no two L2s hold the same slice) and a partition's slice can be smaller
+    // at the same number of launches.  Edges of different partitions write different results.
+    // (232,965-node graph: 3.93 -> 3.71 ms at F=128, 7.89 -> 7.56 ms at F=256, 1.96 -> 1.82 ms at F=64.)
+    const int conc = (T < 8 && 8 % T == 0) ? std::max(1, std::min(8 / T, P)) : 1;
+    a.conc = conc;
+    const bool off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
+    for (int p0 = 0; p0 < P; p0 += conc) {
+        int64_t most = 0;
+        for (int p = p0; p < std::min(P, p0 + conc); ++p) most = std::max(most, pl->item_off[p + 1] - pl->item_off[p]);
+        if (most == 0) continue;
+        a.first_part = p0;
+        const int64_t blocks = ((most + kWavesPerBlock - 1) / kWavesPerBlock) * T * conc;
         if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
-        const bool off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
         const bool ok = (tile_sum || staged) ? launch_tiled_l<false>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a)
-                                 : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
+                                             : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
         if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);
     }
     if (tile_sum) {
