@@ -348,6 +348,23 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
     }
 }
 
+// The last, partly filled batch of a row: exactly `nu` steps (1 <= nu <= U, uniform over the
+// wavefront) are loaded and reduced, instead of U steps padded with re-reads of the last edge --
+// a re-read costs the same cache bandwidth as a gather.
+template <int L, int K, int RW, int KH, int NU, bool SCATTER, bool OFF32>
+__device__ __forceinline__ void sddmm_tile_tail(int nu, const int2 *edge, int j0, int jstride, int e, const float *src,
+                                                uint32_t lane_bytes, int64_t F, const float4 (&dv)[K], float *out,
+                                                int64_t estride, int64_t e_base, int seg_pos) {
+    if (nu >= NU) {
+        sddmm_tile_batch<L, K, RW, KH, NU, SCATTER, OFF32, true>(edge, j0, jstride, e, src, lane_bytes, F, dv, out, estride,
+                                                                  e_base, seg_pos);
+        return;
+    }
+    if constexpr (NU > 1)
+        sddmm_tile_tail<L, K, RW, KH, NU - 1, SCATTER, OFF32>(nu, edge, j0, jstride, e, src, lane_bytes, F, dv, out, estride,
+                                                              e_base, seg_pos);
+}
+
 // L lanes x K loads cover one tile of L*K*4 floats of an edge's operands; RW lanes per head inside
 // one load (KH == 1) or a head spanning KH loads (RW == L).
 template <int L, int K, int RW, int KH, bool SCATTER, bool OFF32>
@@ -435,8 +452,8 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
                         sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, e, src, lane_bytes, F, dv,
                                                                                  out, a.out_edge_stride, it.start, seg_pos);
                     if (s0 < e)
-                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, true>(edge, s0 + g, G, e, src, lane_bytes, F, dv,
-                                                                          out, a.out_edge_stride, it.start, seg_pos);
+                        sddmm_tile_tail<L, K, RW, KH, U, SCATTER, OFF32>((e - s0 + G - 1) / G, edge, s0 + g, G, e, src, lane_bytes,
+                                                                         F, dv, out, a.out_edge_stride, it.start, seg_pos);
                 }
                 b = e;
             }
@@ -481,8 +498,8 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
             sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
                                                                      a.out_edge_stride, (int64_t)it.start + base, seg_pos);
         if (s0 < n)
-            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, true>(edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
-                                                              a.out_edge_stride, (int64_t)it.start + base, seg_pos);
+            sddmm_tile_tail<L, K, RW, KH, U, SCATTER, OFF32>((n - s0 + G - 1) / G, edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
+                                                             a.out_edge_stride, (int64_t)it.start + base, seg_pos);
     }
 }
 

@@ -82,6 +82,41 @@ __device__ __forceinline__ const float *row_ptr(const float *x, uint32_t lane_by
     return reinterpret_cast<const float *>(reinterpret_cast<const char *>(x + (int64_t)staged * F) + lane_bytes);
 }
 
+// The last, partly filled batch of gather_rows: exactly `nu` steps (1 <= nu <= NU, uniform over
+// the wavefront), so that no step is spent re-reading the row's last element; inside the last
+// step a lane without an element still re-reads it with weight zero (no load under a branch).
+template <int V, int L, int K, bool FULL, int NU, bool OFF32, int HPT>
+__device__ __forceinline__ void gather_tail(int nu, const int2 *s_edge, const float *wrow, int s0, int e, int g,
+                                            const float *x, uint32_t lane_bytes, int64_t F, const bool (&on)[K],
+                                            typename Vec<V>::type (&acc)[K]) {
+    using vec = typename Vec<V>::type;
+    constexpr int G = 64 / L;
+    if (nu < NU) {
+        if constexpr (NU > 1) gather_tail<V, L, K, FULL, NU - 1, OFF32, HPT>(nu, s_edge, wrow, s0, e, g, x, lane_bytes, F, on, acc);
+        return;
+    }
+    int2 cw[NU];
+    vec xv[NU][K];
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        const int j = s0 + u * G + g;
+        cw[u] = s_edge[j < e ? j : e - 1];
+        if (HPT > 1) cw[u].y = __float_as_int(wrow[j < e ? j : e - 1]);
+        if (j >= e) cw[u].y = 0;
+    }
+#pragma unroll
+    for (int u = 0; u < NU; ++u)
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            if (FULL || on[k])
+                xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<OFF32>(x, lane_bytes, F, cw[u].x) + k * L * V);
+#pragma unroll
+    for (int u = 0; u < NU; ++u)
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            if (FULL || on[k]) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
+}
+
 // Adds vals * X rows for the staged elements [b, e) of s_edge (x = staged column word, y =
 // weight bits) into acc.  The G lane groups take elements b+g, b+g+G, ...; U steps' loads are
 // issued back to back before the first use.  No load sits under a branch: in the last, partly
@@ -115,28 +150,8 @@ __device__ __forceinline__ void gather_rows(const int2 *s_edge, const float *wro
             for (int k = 0; k < K; ++k)
                 if (FULL || on[k]) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
     }
-    if (s0 < e) {                          // uniform: fewer than G*U elements left
-        int2 cw[U];
-        vec xv[U][K];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int j = s0 + u * G + g;
-            cw[u] = s_edge[j < e ? j : e - 1];
-            if (HPT > 1) cw[u].y = __float_as_int(wrow[j < e ? j : e - 1]);
-            if (j >= e) cw[u].y = 0;
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int k = 0; k < K; ++k)
-                if (FULL || on[k])
-                    xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<OFF32>(x, lane_bytes, F, cw[u].x) + k * L * V);
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int k = 0; k < K; ++k)
-                if (FULL || on[k]) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
-    }
+    if (s0 < e)                            // uniform: fewer than G*U elements left
+        gather_tail<V, L, K, FULL, U, OFF32, HPT>((e - s0 + G - 1) / G, s_edge, wrow, s0, e, g, x, lane_bytes, F, on, acc);
 }
 
 // Adds the lane groups' sums (group 0 gets the total) and stores one output row; `old` is what
