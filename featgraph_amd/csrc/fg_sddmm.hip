@@ -503,14 +503,28 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     }
 }
 
-// out[edge_pos[e']] = sum over tiles of partial[tile][e'], tiles added in ascending order.
+// out[edge_pos[e']] = sum over tiles of partial[tile][e'], tiles added in ascending order.  Four
+// edges per lane: the tiles' arrays start `stride` floats apart (a multiple of 4, 16-byte aligned)
+// and are read as 128-bit loads.
 __global__ __launch_bounds__(256) void sddmm_tile_sum_kernel(const float *partial, const int32_t *edge_pos,
-                                                             float *out, int64_t n_edges, int n_tiles) {
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+                                                             float *out, int64_t n_edges, int64_t stride, int n_tiles) {
+    const int64_t e = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (e >= n_edges) return;
-    float s = partial[e];
-    for (int t = 1; t < n_tiles; ++t) s += partial[(int64_t)t * n_edges + e];
-    out[edge_pos[e]] = s;
+    if (e + 4 <= n_edges) {
+        float4 s = *reinterpret_cast<const float4 *>(partial + e);
+        for (int t = 1; t < n_tiles; ++t) {
+            const float4 v = *reinterpret_cast<const float4 *>(partial + (int64_t)t * stride + e);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        const int4 at = *reinterpret_cast<const int4 *>(edge_pos + e);
+        out[at.x] = s.x; out[at.y] = s.y; out[at.z] = s.z; out[at.w] = s.w;
+        return;
+    }
+    for (int64_t i = e; i < n_edges; ++i) {
+        float s = partial[i];
+        for (int t = 1; t < n_tiles; ++t) s += partial[(int64_t)t * stride + i];
+        out[edge_pos[i]] = s;
+    }
 }
 
 // out[edge_pos[e'], t * hpt + h] = staged[t][e'][h]: the heads of every edge, computed tile by tile
@@ -806,9 +820,10 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
     const int hpt = D >= tile_w ? 1 : tile_w / D;
     const bool staged = !tile_sum && hpt == 1 && H >= 4 && T > 1;
     if (tile_sum) {
-        int rc = ensure_floats(pl, (size_t)T * (size_t)pl->nnz);
+        const int64_t stride = (pl->nnz + 3) & ~(int64_t)3;
+        int rc = ensure_floats(pl, (size_t)T * (size_t)stride);
         if (rc != FG_OK) return rc;
-        a.out = pl->partial_dev; a.out_edge_stride = 1; a.out_tile_stride = pl->nnz;
+        a.out = pl->partial_dev; a.out_edge_stride = 1; a.out_tile_stride = stride;
     } else if (staged) {
         int rc = ensure_floats(pl, (size_t)H * (size_t)pl->nnz);
         if (rc != FG_OK) return rc;
@@ -840,9 +855,10 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
         if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);
     }
     if (tile_sum) {
-        const unsigned blocks = (unsigned)((pl->nnz + 255) / 256);
+        if ((uintptr_t)edge_pos_dev & 15) return fail(FG_ERR_ARG, "edge_pos must be 16-byte aligned");
+        const unsigned blocks = (unsigned)((pl->nnz + 1023) / 1024);
         hipLaunchKernelGGL(sddmm_tile_sum_kernel, dim3(blocks), dim3(256), 0, st, pl->partial_dev, edge_pos_dev,
-                           out_dev, pl->nnz, T);
+                           out_dev, pl->nnz, (pl->nnz + 3) & ~(int64_t)3, T);
     } else if (staged) {
         const unsigned blocks = (unsigned)((pl->nnz + 255) / 256);
         hipLaunchKernelGGL(sddmm_tile_heads_kernel, dim3(blocks), dim3(256), 0, st, pl->partial_dev, edge_pos_dev,
