@@ -11,9 +11,11 @@ python/featgraph/module/spmm.py:179-186).  Prints ONE JSON line; `value` is
 
 `roofline` prices the slower of the two operators against the 8 TB/s HBM peak with the
 compulsory-traffic byte model (an operator is one C-ABI call; on this graph it is several
-launches of one kernel, one per source-column partition, so `achieved` = the operator's
-algorithmic bytes / the HIP-event time of all its launches, and `avg_launch_ms` is that time
-divided by the number of launches):
+launches of one kernel, one per source-column partition, plus a short closing kernel -- the
+fix-ups of split rows for SpMM, the sum over feature tiles for SDDMM -- so `achieved` = the
+operator's algorithmic bytes / the HIP-event time of all its launches; `kernels` lists them and
+`avg_launch_ms` is that time divided by the number of launches of the gather kernel, i.e. it
+carries the closing kernel's share as well):
     SpMM  : 4(N+1) + 8 nnz + 4 N F (X once) + 4 N F (out once)
     SDDMM : 4(N+1) + 4 nnz (CSR order; 8 nnz in COO order) + 8 N F + 4 nnz H
 `cpu_baseline` times the CPU oracle (a C restatement of the reference's x86 schedules: SpMM
@@ -203,11 +205,14 @@ def main():
         "spmm": {"ms": t_spmm, "gflops": flops_op / t_spmm / 1e6, "compulsory_gb": b_spmm / 1e9,
                  "hbm_gbs": b_spmm / t_spmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_spmm / 1e6,
                  "kernel": "spmm_items_kernel", "launches": spmm._active['P'],
+                 "kernels": {"spmm_items_kernel": spmm._active['P'], "spmm_fixup_kernel": spmm._active['P']},
                  "num_col_partitions": spmm._active['P'], "num_feat_partitions": spmm._num_feat_partitions},
         "sddmm": {"ms": t_sddmm, "gflops": flops_op / t_sddmm / 1e6, "compulsory_gb": b_sddmm / 1e9,
                   "hbm_gbs": b_sddmm / t_sddmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_sddmm / 1e6,
                   "kernel": "sddmm_tiled_kernel" if sddmm._tiled else "sddmm_csr_kernel",
                   "launches": sddmm._tiled[0]['P'] if sddmm._tiled else 1,
+                  "kernels": ({"sddmm_tiled_kernel": sddmm._tiled[0]['P'], "sddmm_tile_sum_kernel": 1}
+                              if sddmm._tiled else {"sddmm_csr_kernel": 1}),
                   "num_src_partitions": sddmm._tiled[0]['P'] if sddmm._tiled else 1,
                   "num_feat_tiles": sddmm._tiled[1] if sddmm._tiled else 1},
     }
@@ -220,7 +225,7 @@ def main():
     roofline = {"bound": "hbm", "kernel": ops[dom]["kernel"], "achieved": round(ops[dom]["hbm_gbs"], 2),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ops[dom]["hbm_gbs"] / HBM_PEAK_GBS, 5),
                 "traffic": traffic, "algorithmic_bytes": int(b_spmm if dom == "spmm" else b_sddmm),
-                "launches": ops[dom]["launches"], "op_ms": round(ops[dom]["ms"], 4),
+                "launches": ops[dom]["launches"], "kernels": ops[dom]["kernels"], "op_ms": round(ops[dom]["ms"], 4),
                 "avg_launch_ms": round(ops[dom]["ms"] / ops[dom]["launches"], 4)}
 
     line = {
