@@ -127,7 +127,15 @@ def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):
 if __name__ == '__main__':
     ap = argparse.ArgumentParser()
     ap.add_argument("--quick", action="store_true", help="small graphs only")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="only the edge softmax / per-head SpMM steps on the 232,965-node graph")
     args = ap.parse_args()
+    if args.attention_only:
+        indptr, indices = synthetic.make_workload("powerlaw-233k")
+        n = indptr.shape[0] - 1
+        adj = sp.csr_matrix((np.ones(int(indptr[-1]), np.float32), indices, indptr), shape=(n, n))
+        run_attention_steps("powerlaw-233k", adj, (1, 4, 8), [(4, 64), (8, 64)])
+        raise SystemExit(0)
     run_workload("uniform-10k", [32], [], [])
     if args.quick:
         run_workload("powerlaw-23k", [32, 128, 512], [(4, 32), (8, 64)], [128], (1, 4))
