@@ -72,16 +72,25 @@ extern "C" int fg_csr_to_dds(int64_t n_rows, int64_t n_cols, const int32_t *indp
     uint32_t *vals = static_cast<uint32_t *>(vals32);
     const int64_t d2 = n_rows + 1;
     const int64_t width = (n_cols + P - 1) / P;          // columns per partition
-    auto part_of = [&](int32_t c) { return width > 0 ? (int64_t)c / width : 0; };
+    if (n_cols >= INT32_MAX) return fail(FG_ERR_SHAPE, "fg_csr_to_dds: column count does not fit int32");
+    const uint32_t w32 = (uint32_t)std::max<int64_t>(width, 1);
+    auto part_of = [&](int32_t c) { return (int64_t)((uint32_t)c / w32); };
+    const int nt = fg::default_threads();
 
-    // cursor[p*d2 + r] = number of elements of row r in partition p, then their offsets
+    // cursor[p*d2 + r] = number of elements of row r in partition p, then their offsets.  Rows are
+    // independent in both passes (a cell belongs to one row), so they run over row ranges in parallel.
     std::vector<int64_t> cursor((size_t)P * d2, 0);
-    for (int64_t r = 0; r < n_rows; ++r)
-        for (int32_t e = indptr[r]; e < indptr[r + 1]; ++e) {
-            const int32_t c = indices[e];
-            if (c < 0 || c >= n_cols) return fail(FG_ERR_GRAPH, "indices[%d] = %d outside [0, %lld)", e, c, (long long)n_cols);
-            cursor[part_of(c) * d2 + r]++;
-        }
+    std::vector<int64_t> bad_at((size_t)nt, -1);
+    fg::parallel_ranges(n_rows, nt, [&](int t, int64_t r0, int64_t r1) {
+        for (int64_t r = r0; r < r1; ++r)
+            for (int32_t e = indptr[r]; e < indptr[r + 1]; ++e) {
+                const int32_t c = indices[e];
+                if (c < 0 || c >= n_cols) { if (bad_at[t] < 0) bad_at[t] = e; continue; }
+                cursor[part_of(c) * d2 + r]++;
+            }
+    });
+    for (int64_t e : bad_at)
+        if (e >= 0) return fail(FG_ERR_GRAPH, "indices[%lld] = %d outside [0, %lld)", (long long)e, indices[e], (long long)n_cols);
     int64_t run = 0;
     for (int p = 0; p < P; ++p) {
         for (int64_t r = 0; r < n_rows; ++r) {
@@ -92,14 +101,16 @@ extern "C" int fg_csr_to_dds(int64_t n_rows, int64_t n_cols, const int32_t *indp
         }
         s1_pos[p * d2 + n_rows] = (int32_t)run;
     }
-    for (int64_t r = 0; r < n_rows; ++r)
-        for (int32_t e = indptr[r]; e < indptr[r + 1]; ++e) {
-            const int32_t c = indices[e];
-            const int64_t p = part_of(c);
-            const int64_t at = cursor[p * d2 + r]++;
-            s1_idx[at] = (int32_t)(c - p * width);
-            vals[at] = data[e];
-        }
+    fg::parallel_ranges(n_rows, nt, [&](int, int64_t r0, int64_t r1) {
+        for (int64_t r = r0; r < r1; ++r)
+            for (int32_t e = indptr[r]; e < indptr[r + 1]; ++e) {
+                const int32_t c = indices[e];
+                const int64_t p = part_of(c);
+                const int64_t at = cursor[p * d2 + r]++;
+                s1_idx[at] = (int32_t)(c - p * width);
+                vals[at] = data[e];
+            }
+    });
     return FG_OK;
 }
 
