@@ -198,6 +198,14 @@ def main():
     t_spmm = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps      # ms, HIP events on the launch stream
     t_sddmm = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
 
+    def sddmm_launches():
+        """Launches of the tiled kernel: with T < 8 tiles, 8 / T partitions share a launch."""
+        if not sddmm._tiled:
+            return 1
+        P, T = sddmm._tiled[0]['P'], sddmm._tiled[1]
+        conc = min(8 // T, P) if (T < 8 and 8 % T == 0) else 1
+        return (P + conc - 1) // conc
+
     flops_op = 2.0 * nnz * F
     b_spmm = spmm_bytes(n, n, nnz, F)
     b_sddmm = sddmm_bytes(n, nnz, F, 1, csr=True)
@@ -210,8 +218,8 @@ def main():
         "sddmm": {"ms": t_sddmm, "gflops": flops_op / t_sddmm / 1e6, "compulsory_gb": b_sddmm / 1e9,
                   "hbm_gbs": b_sddmm / t_sddmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_sddmm / 1e6,
                   "kernel": "sddmm_tiled_kernel" if sddmm._tiled else "sddmm_csr_kernel",
-                  "launches": sddmm._tiled[0]['P'] if sddmm._tiled else 1,
-                  "kernels": ({"sddmm_tiled_kernel": sddmm._tiled[0]['P'], "sddmm_tile_sum_kernel": 1}
+                  "launches": sddmm_launches(),
+                  "kernels": ({"sddmm_tiled_kernel": sddmm_launches(), "sddmm_tile_sum_kernel": 1}
                               if sddmm._tiled else {"sddmm_csr_kernel": 1}),
                   "num_src_partitions": sddmm._tiled[0]['P'] if sddmm._tiled else 1,
                   "num_feat_tiles": sddmm._tiled[1] if sddmm._tiled else 1},
@@ -219,7 +227,7 @@ def main():
     for o in ops.values():
         o["pct_hbm_roofline"] = 100.0 * o["hbm_gbs"] / HBM_PEAK_GBS
     dom = "spmm" if t_spmm >= t_sddmm else "sddmm"
-    key = (dom, args.workload, F, ops[dom]["launches"],
+    key = (dom, args.workload, F, ops[dom].get("num_col_partitions", ops[dom].get("num_src_partitions")),
            ops[dom].get("num_feat_partitions", ops[dom].get("num_feat_tiles")))
     traffic = MEASURED_TRAFFIC.get(key)
     roofline = {"bound": "hbm", "kernel": ops[dom]["kernel"], "achieved": round(ops[dom]["hbm_gbs"], 2),

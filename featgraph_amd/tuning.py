@@ -56,7 +56,10 @@ def choose_sddmm(n_rows, n_cols, nnz, heads, head_len):
     kernels should be used (small feature matrices, or a shape the tiled kernel does not take)."""
     feat_len = heads * head_len
     tile = None
-    for cand in (64, 128, 256, 32, 16):
+    # one head of 256 floats or more: 128-float tiles halve the per-tile partial sums, and with fewer
+    # than 8 tiles the kernel runs 8 / tiles partitions per launch, so the slice an XCD holds stays the same
+    order = (128, 64, 256, 32, 16) if (heads == 1 and feat_len >= 256) else (64, 128, 256, 32, 16)
+    for cand in order:
         if feat_len % cand != 0:
             continue
         if heads == 1 or cand % head_len == 0 or (head_len == cand):
@@ -71,6 +74,8 @@ def choose_sddmm(n_rows, n_cols, nnz, heads, head_len):
     if n_cols * row_bytes <= SDDMM_SLICE_BYTES:
         return None
     p = _partitions(n_cols, row_bytes, nnz, n_rows, SDDMM_SLICE_BYTES, min_segment=24)
+    if p > 1 and t < 8 and 8 % t == 0:
+        p = max(p, 8 // t)          # at least one partition per XCD: a single launch covers them all
     if p == 1:
         # rows too short to partition: one tile per edge when the kernel takes the whole row
         if feat_len <= 256 and (feat_len & (feat_len - 1)) == 0 and feat_len >= 16 and \
