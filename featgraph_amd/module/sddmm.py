@@ -221,6 +221,11 @@ class SDDMMbase(object):
         text += "  kernel           : %s\n" % ("sddmm_tiled_kernel over a source-column-partitioned edge list" if tiled
                                                else "sddmm_csr_kernel over row pieces (dst row held in registers)"
                                                if use_csr else "sddmm_coo_kernel, 256 stored edges per wavefront")
+        if tiled:
+            P, T = tiled
+            conc = min(8 // T, P) if (T < 8 and 8 % T == 0) else 1
+            text += "  traversal        : %d source-column partition(s) x %d feature tile(s) of %d floats; %d partition(s) per launch, %d launch(es)\n" % (
+                P, T, H * D // T, conc, (P + conc - 1) // conc)
         for n in notes:
             text += "  note             : %s\n" % n
         return text
