@@ -150,3 +150,30 @@ def test_product_does_not_import_oracle():
             if f.endswith((".py", ".hip", ".cpp", ".h")):
                 text = open(os.path.join(base, f)).read()
                 assert "oracle" not in text, os.path.join(base, f)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more ends with a message instead of a run."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr
+
+
+def test_default_tilings():
+    """The defaults the modules pick for the benchmark shapes (pure arithmetic, no GPU)."""
+    from featgraph_amd import tuning
+    n, nnz = 232965, 114766039
+    assert tuning.choose_spmm(n, n, nnz, 512) == (8, 8)
+    assert tuning.choose_spmm(n, n, nnz, 128) == (8, 2)
+    assert tuning.choose_spmm(2450000, 2450000, 61903880, 128) == (1, 1)     # rows too short to partition
+    assert tuning.choose_sddmm(n, n, nnz, 1, 512) == (16, 4)
+    assert tuning.choose_sddmm(n, n, nnz, 8, 64) == (16, 4)
+    assert tuning.choose_sddmm(n, n, nnz, 4, 32) == (8, 2)
+    assert tuning.choose_sddmm(10000, 10000, 170000, 1, 32) is None           # fits the caches: plain kernels
+    for F in (32, 64, 128, 256, 512):
+        p, t = tuning.choose_sddmm(n, n, nnz, 1, F)
+        assert F % t == 0 and p >= 1
