@@ -1,0 +1,81 @@
+"""Status codes and messages of the device entry points of the C ABI, called directly through ctypes
+with raw device pointers (no module layer): bad arguments must come back as negative codes with a
+message, never as a launch."""
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+FG_OK, FG_ERR_ARG, FG_ERR_SHAPE, FG_ERR_GRAPH = 0, -1, -2, -3
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    from featgraph_amd import _lib
+    L = _lib.lib()
+    indptr = np.array([0, 2, 2, 5, 6], dtype=np.int32)
+    indices = np.array([0, 3, 1, 2, 4, 0], dtype=np.int32)
+    plan = ctypes.c_void_p()
+    assert L.fg_spmm_plan_create(_lib.host_ptr(indptr), 4, 5, 1, None, ctypes.byref(plan)) == FG_OK
+    s1_pos = np.array([0, 1, 1, 2, 3, 3, 4, 4, 6, 6], dtype=np.int32)        # P = 2 over the same matrix
+    plan2 = ctypes.c_void_p()
+    assert L.fg_spmm_plan_create(_lib.host_ptr(s1_pos), 4, 5, 2, None, ctypes.byref(plan2)) == FG_OK
+    dev = lambda a: torch.from_numpy(a).cuda()
+    t = dict(indptr=dev(indptr), indices=dev(indices), vals=torch.ones(6, device="cuda"),
+             x=torch.ones((5, 8), device="cuda"), y=torch.ones((4, 8), device="cuda"),
+             out=torch.zeros((4, 8), device="cuda"), e=torch.zeros(6, device="cuda"))
+    yield L, _lib, plan, plan2, t
+    L.fg_spmm_plan_destroy(plan)
+    L.fg_spmm_plan_destroy(plan2)
+
+
+def test_spmm_arguments(env):
+    L, lib, plan, plan2, t = env
+    p = lib.dev_ptr
+    ok = L.fg_spmm_csr_f32(plan, p(t['indptr']), p(t['indices']), p(t['vals']), p(t['x']), p(t['out']), 8, 0, None)
+    assert ok == FG_OK
+    assert L.fg_spmm_csr_f32(None, p(t['indptr']), p(t['indices']), p(t['vals']), p(t['x']), p(t['out']), 8, 0, None) == FG_ERR_ARG
+    assert b"plan" in L.fg_last_error()
+    assert L.fg_spmm_csr_f32(plan, p(t['indptr']), None, p(t['vals']), p(t['x']), p(t['out']), 8, 0, None) == FG_ERR_ARG
+    assert L.fg_spmm_csr_f32(plan, p(t['indptr']), p(t['indices']), p(t['vals']), p(t['x']), p(t['out']), 0, 0, None) == FG_ERR_SHAPE
+    assert L.fg_spmm_csr_f32(plan, p(t['indptr']), p(t['indices']), p(t['vals']), p(t['x']), p(t['out']), 8, 3, None) == FG_ERR_SHAPE
+    assert b"divisible" in L.fg_last_error()
+    # a plan with column partitions does not fit the CSR entry point
+    assert L.fg_spmm_csr_f32(plan2, p(t['indptr']), p(t['indices']), p(t['vals']), p(t['x']), p(t['out']), 8, 0, None) == FG_ERR_ARG
+    # max / min aggregation needs one partition; unknown reduce
+    assert L.fg_gspmm_f32(plan2, p(t['indptr']), p(t['indices']), p(t['vals']), p(t['x']), p(t['out']), 8, 1, 0, 1, 0, None) == FG_ERR_ARG
+    assert L.fg_gspmm_f32(plan, p(t['indptr']), p(t['indices']), p(t['vals']), p(t['x']), p(t['out']), 8, 1, 0, 7, 0, None) == FG_ERR_ARG
+    assert L.fg_gspmm_f32(plan, p(t['indptr']), p(t['indices']), p(t['vals']), p(t['x']), p(t['out']), 8, 3, 0, 0, 0, None) == FG_ERR_SHAPE
+
+
+def test_sddmm_and_softmax_arguments(env):
+    L, lib, plan, plan2, t = env
+    p = lib.dev_ptr
+    assert L.fg_sddmm_csr_f32(plan, p(t['indptr']), p(t['indices']), p(t['x']), p(t['y']), p(t['e']), 1, 8, None) == FG_OK
+    assert L.fg_sddmm_csr_f32(plan, p(t['indptr']), p(t['indices']), None, p(t['y']), p(t['e']), 1, 8, None) == FG_ERR_ARG
+    assert L.fg_sddmm_csr_f32(plan, p(t['indptr']), p(t['indices']), p(t['x']), p(t['y']), p(t['e']), 0, 8, None) == FG_ERR_SHAPE
+    assert L.fg_sddmm_coo_f32(None, p(t['indices']), 6, p(t['x']), p(t['y']), p(t['e']), 1, 8, None) == FG_ERR_ARG
+    assert L.fg_sddmm_coo_f32(p(t['indices']), p(t['indices']), -1, p(t['x']), p(t['y']), p(t['e']), 1, 8, None) == FG_ERR_ARG
+    # tiled traversal: a tile must be a power of two between 16 and 256 floats
+    assert L.fg_sddmm_dds_f32(plan, p(t['indptr']), p(t['indices']), p(t['indices']), p(t['x']), p(t['y']), p(t['e']),
+                              1, 8, 1, None) == FG_ERR_SHAPE
+    assert L.fg_edge_softmax_f32(plan, p(t['indptr']), p(t['e']), p(t['e']), 1, None) == FG_OK
+    assert L.fg_edge_softmax_f32(plan, p(t['indptr']), p(t['e']), p(t['e']), 0, None) == FG_ERR_SHAPE
+    assert L.fg_edge_softmax_f32(plan2, p(t['indptr']), p(t['e']), p(t['e']), 1, None) == FG_ERR_ARG
+    assert L.fg_edge_softmax_f32(plan, p(t['indptr']), None, p(t['e']), 1, None) == FG_ERR_ARG
+    assert L.fg_edge_softmax_backward_f32(plan, p(t['indptr']), p(t['e']), None, p(t['e']), 1, None) == FG_ERR_ARG
+    assert L.fg_edge_values_head_major_f32(p(t['e']), None, 6, 0, p(t['e']), None) == FG_ERR_ARG
+    assert L.fg_gsddmm_elementwise_f32(p(t['indices']), p(t['indices']), 6, p(t['x']), p(t['y']), p(t['out']), 8, 9, None) == FG_ERR_ARG
+
+
+def test_plan_rejects_bad_positions(env):
+    L, lib, plan, plan2, t = env
+    bad = ctypes.c_void_p()
+    dec = np.array([0, 3, 2, 5], dtype=np.int32)
+    assert L.fg_spmm_plan_create(lib.host_ptr(dec), 3, 4, 1, None, ctypes.byref(bad)) == FG_ERR_GRAPH
+    assert not bad.value
+    assert L.fg_spmm_plan_create(lib.host_ptr(dec), 3, 4, 0, None, ctypes.byref(bad)) == FG_ERR_ARG
+    assert L.fg_spmm_plan_create(None, 3, 4, 1, None, ctypes.byref(bad)) == FG_ERR_ARG
