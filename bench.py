@@ -36,8 +36,8 @@ HBM_PEAK_GBS = 8000.0
 # by all launches of the named kernel in one operator call, at the default tiling; from
 # profiles/bench_powerlaw233k_f512_rocprofv3.txt.  Other configurations have no measurement: null.
 MEASURED_TRAFFIC = {
-    ("spmm", "powerlaw-233k", 512, 8, 8): 72.4e9,      # 8 x spmm_items_kernel (+ fix-ups)
-    ("sddmm", "powerlaw-233k", 512, 8, 8): 70.4e9,     # 8 x sddmm_tiled_kernel (tile sum: +4.7e9)
+    ("spmm", "powerlaw-233k", 512, 8, 8): 72.5e9,      # 8 x spmm_items_kernel (+ fix-ups)
+    ("sddmm", "powerlaw-233k", 512, 16, 4): 78.3e9,    # 8 x sddmm_tiled_kernel (tile sum: +2.9e9)
 }
 METRIC = "SpMM/SDDMM GFLOP/s + achieved HBM GB/s (% roofline), 233k-node graph, feat 512"
 
