@@ -177,3 +177,44 @@ def test_default_tilings():
     for F in (32, 64, 128, 256, 512):
         p, t = tuning.choose_sddmm(n, n, nnz, 1, F)
         assert F % t == 0 and p >= 1
+
+
+def test_partitioners_property_based(fg, oracle):
+    """Random small matrices, partition counts and storage orders: the library's partitioners agree with
+    the oracle bit for bit, the DDS arrays expand back to the matrix, and the 2-D edge ids are a
+    permutation that argsort inverts."""
+    from hypothesis import given, settings, strategies as st
+    from featgraph_amd.util import util_convert_csr_to_dds, util_partition_adj_coo_2d
+
+    @settings(max_examples=150, deadline=None)
+    @given(st.integers(1, 12), st.integers(1, 12), st.integers(0, 2 ** 31 - 1), st.floats(0.0, 1.0),
+           st.integers(1, 15), st.integers(1, 15))
+    def check(n_rows, n_cols, seed, density, a_parts, b_parts):
+        rng = np.random.default_rng(seed)
+        mask = rng.random((n_rows, n_cols)) < density
+        dense = np.where(mask, rng.integers(1, 1000, size=(n_rows, n_cols)), 0).astype(np.int32)
+        csr = sp.csr_matrix(dense)
+        csr.sort_indices()
+        got = util_convert_csr_to_dds(csr, a_parts)
+        for x, y in zip(got, oracle.csr_to_dds(csr, a_parts)):
+            assert np.array_equal(x, y)
+        s1_pos, s1_idx, vals = got
+        width = -(-n_cols // a_parts)
+        rebuilt = np.zeros_like(dense)
+        for p in range(a_parts):
+            for r in range(n_rows):
+                for k in range(s1_pos[p * (n_rows + 1) + r], s1_pos[p * (n_rows + 1) + r + 1]):
+                    rebuilt[r, s1_idx[k] + p * width] = vals[k]
+        assert np.array_equal(rebuilt, dense)
+        coo = csr.tocoo()
+        perm = rng.permutation(coo.nnz)
+        coo = sp.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+        eid, row, col = util_partition_adj_coo_2d(coo, a_parts, b_parts)
+        for x, y in zip((eid, row, col), oracle.partition_coo_2d(coo, a_parts, b_parts)):
+            assert np.array_equal(x, y)
+        assert sorted(eid.tolist()) == list(range(1, coo.nnz + 1))
+        assert np.array_equal(row, coo.row[eid - 1]) and np.array_equal(col, coo.col[eid - 1])
+        mapping = np.argsort(eid)
+        assert np.array_equal(eid[mapping], np.arange(1, coo.nnz + 1))
+
+    check()
