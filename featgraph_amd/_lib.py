@@ -46,6 +46,7 @@ SIGNATURES = {
     "fg_spmm_csr_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
     "fg_spmm_dds_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
     "fg_gspmm_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp]),
+    "fg_gspmm_arg_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _vp]),
     "fg_edge_values_head_major_f32": (_int, [_vp, _vp, _i64, _int, _vp, _vp]),
     "fg_sddmm_coo_f32": (_int, [_vp, _vp, _i64, _vp, _vp, _vp, _int, _int, _vp]),
     "fg_sddmm_csr_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),

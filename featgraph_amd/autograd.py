@@ -95,6 +95,33 @@ class Graph(object):
         (n, H, D) operands -> (nnz, H)."""
         return _SDDMM.apply(self, src, dst)
 
+    def aggregate(self, x, reduce="sum"):
+        """y[v,:] = reduce over the edges e into v of x[col e,:], reduce in {'sum', 'mean', 'max', 'min'}
+        (rows without edges give 0); x (num_cols, F); differentiable in x."""
+        if reduce not in ("sum", "mean", "max", "min"):
+            raise ValueError("reduce must be 'sum', 'mean', 'max' or 'min'")
+        return _Aggregate.apply(self, x, reduce)
+
+    def _aggregate_mod(self, feat_len, reduce):
+        key = ('aggregate', feat_len, reduce)
+        if key not in self._mods:
+            m = GSpMMhip(self._csr)
+            args = {'reduce': reduce, 'msg': 'copy_u'}
+            if reduce in ('max', 'min'):
+                args['return_arg'] = True
+            m.build([placeholder((self.shape[1], feat_len))], args, {})
+            self._mods[key] = m
+        return self._mods[key]
+
+    def _mean_weights(self, device):
+        if getattr(self, "_inv_deg", None) is None or self._inv_deg.device != device:
+            deg = np.diff(self._csr.indptr).astype(np.float32)
+            inv = np.where(deg > 0, 1.0 / np.maximum(deg, 1), 0).astype(np.float32)
+            self._inv_deg = torch.from_numpy(np.repeat(inv, np.diff(self._csr.indptr))).to(device)
+            self._ones = torch.ones(self.nnz, device=device)
+            self._cols = torch.from_numpy(self._csr.indices.astype(np.int64)).to(device)
+        return self._inv_deg
+
     def edge_softmax(self, scores):
         """Softmax of scores, (nnz,) or (nnz, H), over the edges of each destination row, per head."""
         return _EdgeSoftmax.apply(self, scores)
@@ -144,3 +171,33 @@ class _EdgeSoftmax(torch.autograd.Function):
     def backward(ctx, da):
         (a,) = ctx.saved_tensors
         return None, ctx.g._softmax_mod(tuple(a.shape)).backward(a, da.contiguous()).clone()
+
+
+class _Aggregate(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, g, x, reduce):
+        ctx.g, ctx.reduce = g, reduce
+        x = x.contiguous()
+        mod = g._aggregate_mod(x.shape[1], reduce)
+        y = mod.run([x]).clone()
+        if reduce in ("max", "min"):
+            ctx.save_for_backward(mod.arg_tvm.clone())
+        ctx.x_shape = tuple(x.shape)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        g, reduce = ctx.g, ctx.reduce
+        dy = dy.contiguous()
+        if reduce in ("sum", "mean"):
+            w = g._mean_weights(dy.device)
+            return None, g._spmm_raw(dy, w if reduce == "mean" else g._ones, transposed=True), None
+        (arg,) = ctx.saved_tensors
+        g._mean_weights(dy.device)
+        n_src, F = ctx.x_shape
+        valid = arg >= 0
+        src = g._cols[arg.clamp(min=0).long()]                               # source vertex of the selected edge
+        flat = (src * F + torch.arange(F, device=dy.device)[None, :])[valid]
+        dx = torch.zeros(n_src * F, dtype=dy.dtype, device=dy.device)
+        dx.index_add_(0, flat, dy[valid])
+        return None, dx.view(n_src, F), None

@@ -11,6 +11,7 @@
 // elements but different feature tiles, and every XCD's L2 holds only its tiles' slice of X.
 #include <hip/hip_runtime.h>
 
+#include <climits>
 #include <string>
 
 #include "fg_common.h"
@@ -67,6 +68,7 @@ struct SpmmArgs {
     int accumulate;        // add to out instead of overwriting it
     int heads;             // weights are [nnz, heads]; a kernel tile lies inside one head
     int head_len;          // floats per head (F / heads)
+    int32_t *arg;          // arg kernel: stored position of the element that gave out[v, f]
     int vstride;           // weight of element t, head h: vals[t * vstride + h * head_stride]
     int64_t head_stride;
 };
@@ -559,6 +561,184 @@ __global__ __launch_bounds__(256) void gspmm_extreme_fixup_kernel(const Fixup *f
     *reinterpret_cast<vec *>(out + (int64_t)fx.row * F + f) = m;
 }
 
+// ---- which element gave the extreme -------------------------------------------------------------
+//
+// arg[v, f] = stored position of the first element e of row v with vals[e] * X[indices[e], f] ==
+// out[v, f] (out as written by the max / min kernel; -1 for a row without elements).  Same items
+// and lane layout; the products are formed by the same multiplication, so the comparison is exact.
+// Pieces of split rows combine through atomicMin on arg (set to INT_MAX beforehand).
+
+__device__ __forceinline__ int4 imin4(const int4 &a, const int4 &b) {
+    return make_int4(min(a.x, b.x), min(a.y, b.y), min(a.z, b.z), min(a.w, b.w));
+}
+__device__ __forceinline__ int imin4(const int &a, const int &b) { return min(a, b); }
+__device__ __forceinline__ int4 imatch(const float4 &m, const float4 &t, int e, const int4 &cur) {
+    return make_int4(m.x == t.x ? min(cur.x, e) : cur.x, m.y == t.y ? min(cur.y, e) : cur.y,
+                     m.z == t.z ? min(cur.z, e) : cur.z, m.w == t.w ? min(cur.w, e) : cur.w);
+}
+__device__ __forceinline__ int imatch(const float &m, const float &t, int e, const int &cur) { return m == t ? min(cur, e) : cur; }
+__device__ __forceinline__ int4 ishfl_xor(const int4 &a, int off) {
+    return make_int4(__shfl_xor(a.x, off), __shfl_xor(a.y, off), __shfl_xor(a.z, off), __shfl_xor(a.w, off));
+}
+__device__ __forceinline__ int ishfl_xor(const int &a, int off) { return __shfl_xor(a, off); }
+__device__ __forceinline__ int4 isplat(int4, int v) { return make_int4(v, v, v, v); }
+__device__ __forceinline__ int isplat(int, int v) { return v; }
+__device__ __forceinline__ int4 inone(const int4 &a) {      // INT_MAX (no match) -> -1
+    return make_int4(a.x == INT_MAX ? -1 : a.x, a.y == INT_MAX ? -1 : a.y, a.z == INT_MAX ? -1 : a.z, a.w == INT_MAX ? -1 : a.w);
+}
+__device__ __forceinline__ int inone(const int &a) { return a == INT_MAX ? -1 : a; }
+__device__ __forceinline__ void iatomic_min(int32_t *p, const int4 &a) {
+    atomicMin(p, a.x); atomicMin(p + 1, a.y); atomicMin(p + 2, a.z); atomicMin(p + 3, a.w);
+}
+__device__ __forceinline__ void iatomic_min(int32_t *p, const int &a) { atomicMin(p, a); }
+template <int V> struct IVec;
+template <> struct IVec<4> { using type = int4; };
+template <> struct IVec<1> { using type = int; };
+
+template <int V, int L, int K, bool FULL>
+__global__ __launch_bounds__(kBlock) void gspmm_arg_kernel(const SpmmArgs a) {
+    using vec = typename Vec<V>::type;
+    using ivec = typename IVec<V>::type;
+    constexpr int FT = V * L * K;
+    constexpr int G = 64 / L;
+    constexpr int U = (K >= 2) ? 2 : 4;
+    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
+    __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int tile = a.tile_base + (int)(blockIdx.x % (unsigned)a.n_ftiles);
+    const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_ftiles) * kWavesPerBlock + wave;
+    if (item_id >= a.n_items) return;
+    const Item it = a.items[item_id];
+    const int g = lane / L, li = lane % L;
+    const int rt = tile / a.sub_per_tile, st = tile % a.sub_per_tile;
+    const int f_end = (rt + 1) * a.tile_w;
+    const int f_lo = rt * a.tile_w + st * FT + li * V;
+    bool on[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
+    const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
+    const int64_t voff = (int64_t)((rt * a.tile_w + st * FT) / a.head_len) * a.head_stride;
+    const int64_t F = a.F;
+    int2 *edge = s_edge[wave];
+    int2 regs[4];
+    vec target[K];
+    ivec acc[K];
+
+    // `first` = stored position of staged element 0
+    auto walk = [&](int b, int e, int first) {
+        for (int s0 = b; s0 < e; s0 += G * U) {
+            int2 cw[U];
+            bool ok[U];
+            vec xv[U][K];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int j = s0 + u * G + g;
+                ok[u] = j < e;
+                cw[u] = edge[ok[u] ? j : e - 1];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    if (FULL || on[k])
+                        xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<false>(a.x, lane_bytes, F, cw[u].x) + k * L * V);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    if ((FULL || on[k]) && ok[u])
+                        acc[k] = imatch(vscale(__int_as_float(cw[u].y), xv[u][k]), target[k], first + s0 + u * G + g, acc[k]);
+        }
+    };
+    auto begin_row = [&](int64_t row) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            acc[k] = isplat(ivec(), INT_MAX);
+            if (FULL || on[k]) target[k] = *reinterpret_cast<const vec *>(a.out + row * F + f_lo + k * L * V);
+        }
+    };
+    auto combine = [&]() {
+#pragma unroll
+        for (int off = L; off < 64; off <<= 1)
+#pragma unroll
+            for (int k = 0; k < K; ++k) acc[k] = imin4(acc[k], ishfl_xor(acc[k], off));
+    };
+
+    if (it.info < -1) {
+        const int nrows = -it.info;
+        if (it.len > 0) {
+            stage_load(a.indices, a.vals, it.start, it.len, lane, 1u, a.vstride, voff, regs);
+            stage_store(edge, lane, regs);
+        }
+        s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        wave_lds_sync();
+        int b = 0;
+        for (int q = 0; q < nrows; ++q) {
+            const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
+            begin_row(it.row + q);
+            walk(b, e, it.start);
+            combine();
+            if (g == 0) {
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    if (FULL || on[k])
+                        *reinterpret_cast<ivec *>(a.arg + (int64_t)(it.row + q) * F + f_lo + k * L * V) = inone(acc[k]);
+            }
+            b = e;
+        }
+        return;
+    }
+    begin_row(it.row);
+    for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
+        const int n = min(fg::kItemEdges, it.len - base);
+        wave_lds_sync();
+        stage_load(a.indices, a.vals, (int64_t)it.start + base, n, lane, 1u, a.vstride, voff, regs);
+        stage_store(edge, lane, regs);
+        wave_lds_sync();
+        walk(0, n, it.start + base);
+    }
+    combine();
+    if (g == 0) {
+        int32_t *dst = a.arg + (int64_t)it.row * F + f_lo;
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            if (FULL || on[k]) {
+                if (it.info < 0) *reinterpret_cast<ivec *>(dst + k * L * V) = inone(acc[k]);
+                else iatomic_min(dst + k * L * V, acc[k]);       // a piece: the row's other pieces add theirs
+            }
+    }
+}
+
+// arg rows of split rows start at INT_MAX so that their pieces can take the minimum.
+__global__ __launch_bounds__(256) void gspmm_arg_init_kernel(const Fixup *fixups, int64_t n_fixups, int32_t *arg, int F) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_fixups * F) return;
+    arg[(int64_t)fixups[t / F].row * F + t % F] = INT_MAX;
+}
+
+template <int V, int L, int K>
+void launch_arg_vlk(bool full, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+    if (full) hipLaunchKernelGGL((gspmm_arg_kernel<V, L, K, true>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((gspmm_arg_kernel<V, L, K, false>), grid, dim3(kBlock), 0, st, a);
+}
+
+template <int V>
+int launch_arg_v(int L, int K, bool full, dim3 grid, hipStream_t st, const SpmmArgs &a) {
+    if (K == 1) {
+        switch (L) {
+            case 4: launch_arg_vlk<V, 4, 1>(full, grid, st, a); return FG_OK;
+            case 8: launch_arg_vlk<V, 8, 1>(full, grid, st, a); return FG_OK;
+            case 16: launch_arg_vlk<V, 16, 1>(full, grid, st, a); return FG_OK;
+            case 32: launch_arg_vlk<V, 32, 1>(full, grid, st, a); return FG_OK;
+            case 64: launch_arg_vlk<V, 64, 1>(full, grid, st, a); return FG_OK;
+        }
+    } else if (L == 64 && K == 2) { launch_arg_vlk<V, 64, 2>(full, grid, st, a); return FG_OK; }
+    else if (L == 64 && K == 4) { launch_arg_vlk<V, 64, 4>(full, grid, st, a); return FG_OK; }
+    return FG_ERR_SHAPE;
+}
+
 // out[row, :] (+)= sum of the row's pieces, in piece order.  One lane per V columns.
 template <int V>
 __global__ __launch_bounds__(256) void spmm_fixup_kernel(const Fixup *fixups, int64_t n_fixups,
@@ -691,8 +871,10 @@ int launch_ext_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs 
 // head_major) and every kernel tile must lie inside one head.  vals == nullptr with allow_no_vals: every weight is 1.
 int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
              const float *x, float *out, int F, int T, void *stream, int heads = 1,
-             int reduce = FG_REDUCE_SUM, bool allow_no_vals = false, bool head_major = false) {
+             int reduce = FG_REDUCE_SUM, bool allow_no_vals = false, bool head_major = false,
+             int32_t *arg_out = nullptr) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (arg_out && reduce == FG_REDUCE_SUM) return fail(FG_ERR_ARG, "positions of the selected elements exist for max / min only");
     if (int drc = fg::check_device(pl)) return drc;
     if (pl->n_dst == 0) return FG_OK;
     if (!out || !pos || (pl->nnz > 0 && (!idx || (!vals && !allow_no_vals) || !x)))
@@ -702,7 +884,7 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
     if (reduce != FG_REDUCE_SUM && pl->num_col_partitions != 1)
         return fail(FG_ERR_ARG, "max / min aggregation needs a plan with one column partition");
     if (heads < 1 || F % heads != 0) return fail(FG_ERR_SHAPE, "feature length %d is not divisible by %d heads", F, heads);
-    const bool aligned16 = (((uintptr_t)x | (uintptr_t)out) & 15) == 0;
+    const bool aligned16 = (((uintptr_t)x | (uintptr_t)out | (uintptr_t)arg_out) & 15) == 0;
     int hpt = 1;
     if (heads > 1) {
         // A kernel tile holds whole heads or lies inside one: 64 floats when the head length divides
@@ -785,6 +967,27 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
             }
         }
     }
+    if (arg_out) {
+        // second sweep over the same items: which element equals the extreme that was just written
+        SpmmArgs a;
+        a.items = pl->items_dev; a.n_items = pl->n_items; a.pos = pos; a.indices = idx; a.vals = vals;
+        a.x = x; a.out = out; a.partial = nullptr; a.arg = arg_out;
+        a.F = F; a.tile_w = c.tile_w; a.sub_per_tile = c.sub_per_tile; a.n_ftiles = c.n_ftiles; a.tile_base = 0;
+        a.accumulate = 0; a.heads = heads; a.head_len = F / heads;
+        a.vstride = head_major ? 1 : heads; a.head_stride = head_major ? pl->nnz : 1;
+        if (pl->n_fixups > 0) {
+            const int64_t threads = pl->n_fixups * (int64_t)F;
+            hipLaunchKernelGGL(gspmm_arg_init_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
+                               pl->fixups_dev, pl->n_fixups, arg_out, F);
+        }
+        const int64_t blocks = ((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock) * c.n_ftiles;
+        if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
+        if (blocks > 0) {
+            rc = (c.V == 4) ? launch_arg_v<4>(c.L, c.K, c.full, dim3((unsigned)blocks), st, a)
+                            : launch_arg_v<1>(c.L, c.K, c.full, dim3((unsigned)blocks), st, a);
+            if (rc != FG_OK) return fail(FG_ERR_SHAPE, "no arg kernel for V=%d L=%d K=%d", c.V, c.L, c.K);
+        }
+    }
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;
 }
@@ -828,6 +1031,14 @@ extern "C" int fg_gspmm_f32(const fg_spmm_plan *plan, const int32_t *pos_dev, co
                             int vals_head_major, int reduce, int num_feat_partitions, void *stream) {
     return spmm_run(plan, pos_dev, idx_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream, heads,
                     reduce, /*allow_no_vals=*/true, vals_head_major != 0);
+}
+
+extern "C" int fg_gspmm_arg_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev, const int32_t *indices_dev,
+                                const float *vals_dev, const float *x_dev, float *out_dev, int32_t *arg_dev, int F,
+                                int heads, int vals_head_major, int reduce, int num_feat_partitions, void *stream) {
+    if (!arg_dev) return fail(FG_ERR_ARG, "fg_gspmm_arg_f32: arg_dev is null");
+    return spmm_run(plan, indptr_dev, indices_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream, heads,
+                    reduce, /*allow_no_vals=*/true, vals_head_major != 0, arg_dev);
 }
 
 namespace {

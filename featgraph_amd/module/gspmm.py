@@ -26,13 +26,18 @@ class GSpMMhip(VanillaSpMMhip):
     SrcFeat is (num_cols, F) or (num_cols, H, D); with H > 1 the weights are (nnz, H) and must
     be passed to run() as a second input, in the adjacency's CSR edge order.
     Rows without edges give 0 for every reduce.
+    'return_arg': True (max / min only) also fills self.arg_tvm, int32 of out's shape: the position, in
+    the adjacency's CSR edge order, of the edge whose message was selected (-1 for rows without edges).
     """
-    _compute_keys = ('num_feat_partitions', 'reduce', 'msg')
+    _compute_keys = ('num_feat_partitions', 'reduce', 'msg', 'return_arg')
 
     def build(self, input_placeholders, compute_args, schedule_args):
         compute_args = dict(compute_args)
         reduce = compute_args.pop('reduce', 'sum')
         msg = compute_args.pop('msg', 'u_mul_e')
+        return_arg = bool(compute_args.pop('return_arg', False))
+        if return_arg and reduce not in ('max', 'min'):
+            raise ValueError("return_arg is defined for reduce='max' / 'min' only")
         if reduce not in _REDUCE:
             raise ValueError("reduce must be one of %s" % sorted(_REDUCE))
         if msg not in ('u_mul_e', 'copy_u'):
@@ -65,6 +70,7 @@ class GSpMMhip(VanillaSpMMhip):
         self._reduce, self._msg, self._weights_at_run, self._notes = reduce, msg, weights_at_run, notes
         self._active = self._glayout(P)
         self._func = _lib.lib().fg_gspmm_f32
+        self._return_arg = return_arg
         self._inv_deg_edge = None
         self._w_head_major = None
         if reduce == 'mean':
@@ -72,6 +78,7 @@ class GSpMMhip(VanillaSpMMhip):
             inv = np.where(deg > 0, 1.0 / np.maximum(deg, 1), 0).astype(np.float32)
             self._inv_deg_edge = common.to_device_f32(np.repeat(inv, np.diff(self._adj_indptr)), self._ctx)
         self.out_tvm = torch.zeros((self._num_rows,) + tuple(src_ph.shape[1:]), dtype=torch.float32, device=self._ctx)
+        self.arg_tvm = torch.full(self.out_tvm.shape, -1, dtype=torch.int32, device=self._ctx) if return_arg else None
 
     def _glayout(self, P):
         """Layout for P source partitions plus, for P > 1, each DDS element's CSR position (so that
@@ -118,6 +125,12 @@ class GSpMMhip(VanillaSpMMhip):
         w, head_major = self._weights(weights)
         heads = w.shape[0] if head_major else 1
         self._w_keepalive = w
+        if self._return_arg:
+            _lib.check(_lib.lib().fg_gspmm_arg_f32(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']),
+                                                   _lib.dev_ptr(w), _lib.dev_ptr(src_feat), _lib.dev_ptr(self.out_tvm),
+                                                   _lib.dev_ptr(self.arg_tvm), self._feat_len, heads, head_major,
+                                                   _REDUCE[self._reduce], self._num_feat_partitions, common.stream_ptr()))
+            return
         _lib.check(self._func(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(w),
                               _lib.dev_ptr(src_feat), _lib.dev_ptr(self.out_tvm), self._feat_len, heads, head_major,
                               _REDUCE[self._reduce], self._num_feat_partitions, common.stream_ptr()))

@@ -27,6 +27,9 @@
  *       README.md:9-11 points to ("generalized SpMM") but the snapshot holds no code, test or
  *       vector for it.  Pinned by numpy maximum/minimum.reduceat closed forms, by reduce == sum
  *       with H == 1 equalling orc_spmm_csr_rowwise bit-exactly, and by brute force on tiny inputs.
+ *   orc_gspmm_arg
+ *       PARITY UNPINNED by the reference (no such operator).  Pinned by numpy argmax / argmin over the
+ *       gathered messages on inputs with many ties, and by its values equalling orc_gspmm's.
  *   orc_edge_softmax, orc_edge_softmax_backward
  *       PARITY UNPINNED by the reference: the snapshot has no attention / softmax operator at all.
  *       Pinned by scipy.special.softmax per row in float64, rows summing to 1, invariance under a
@@ -164,6 +167,34 @@ int orc_gspmm(int64_t n_dst, int F, int H, const int32_t *indptr, const int32_t 
                 else if (k == b) o[f] = m;
                 else if (reduce == 1) o[f] = m > o[f] ? m : o[f];
                 else o[f] = m < o[f] ? m : o[f];
+            }
+        }
+    }
+    return ORC_OK;
+}
+
+/*
+ * orc_gspmm for max (reduce 1) / min (reduce 2) that also reports the selected element.  NOT IN THE
+ * REFERENCE (parity unpinned, see the header): arg[v, f] = stored position of the first element of
+ * row v whose message equals the extreme, -1 for a row without elements.  Pinned by numpy argmax /
+ * argmin over the gathered messages (first occurrence on ties).
+ */
+int orc_gspmm_arg(int64_t n_dst, int F, int H, const int32_t *indptr, const int32_t *indices,
+                  const float *vals, const float *x, float *out, int32_t *arg, int reduce, int nthreads) {
+    if (F < 1 || H < 1 || F % H != 0 || reduce < 1 || reduce > 2 || nthreads < 1) return ORC_EARG;
+    const int D = F / H;
+#pragma omp parallel for num_threads(nthreads) schedule(dynamic, 64)
+    for (int64_t row = 0; row < n_dst; ++row) {
+        float *o = out + row * F;
+        int32_t *a = arg + row * F;
+        const int32_t b = indptr[row], e = indptr[row + 1];
+        for (int f = 0; f < F; ++f) { o[f] = 0.0f; a[f] = -1; }
+        for (int32_t k = b; k < e; ++k) {
+            const float *xr = x + (int64_t)indices[k] * F;
+            for (int f = 0; f < F; ++f) {
+                const float w = vals ? vals[(int64_t)k * H + f / D] : 1.0f;
+                const float m = w * xr[f];
+                if (k == b || (reduce == 1 ? m > o[f] : m < o[f])) { o[f] = m; a[f] = k; }
             }
         }
     }

@@ -52,6 +52,7 @@ def lib():
         L.orc_spmm_csr_rowwise.argtypes = [_i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int]
         L.orc_spmm_dds_x86.argtypes = [_i64, _i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int]
         L.orc_gspmm.argtypes = [_i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int]
+        L.orc_gspmm_arg.argtypes = [_i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _i32p, _int, _int]
         L.orc_edge_softmax.argtypes = [_i64, _int, _i32p, _f32p, _f32p, _int]
         L.orc_edge_softmax_backward.argtypes = [_i64, _int, _i32p, _f32p, _f32p, _f32p, _int]
         L.orc_sddmm_x86.argtypes = [_i64, _i64, _i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int, _int]
@@ -142,6 +143,28 @@ def gspmm(indptr, indices, vals, x, reduce="sum", nthreads=1):
     _check(lib().orc_gspmm(n_dst, F, H, _p(indptr, _i32p), _p(indices, _i32p), vp, _p(x2, _f32p),
                            _p(out, _f32p), REDUCE[reduce], nthreads), "gspmm")
     return out.reshape((n_dst,) + shape[1:])
+
+
+def gspmm_arg(indptr, indices, vals, x, reduce="max", nthreads=1):
+    """gspmm for max / min plus the stored position of the selected element per output (first
+    occurrence on ties, -1 for rows without elements).  Not in the reference."""
+    indptr = _c(indptr, np.int32); indices = _c(indices, np.int32)
+    x = _c(x, np.float32)
+    shape = x.shape
+    H = shape[1] if x.ndim == 3 else 1
+    x2 = x.reshape(shape[0], -1)
+    F = x2.shape[1]
+    vp = None
+    if vals is not None:
+        vals = _c(vals, np.float32).reshape(indices.shape[0], -1)
+        assert vals.shape[1] == H
+        vp = _p(vals, _f32p)
+    n_dst = indptr.shape[0] - 1
+    out = np.empty((n_dst, F), dtype=np.float32)
+    arg = np.empty((n_dst, F), dtype=np.int32)
+    _check(lib().orc_gspmm_arg(n_dst, F, H, _p(indptr, _i32p), _p(indices, _i32p), vp, _p(x2, _f32p),
+                               _p(out, _f32p), _p(arg, _i32p), REDUCE[reduce], nthreads), "gspmm_arg")
+    return out.reshape((n_dst,) + shape[1:]), arg.reshape((n_dst,) + shape[1:])
 
 
 def edge_softmax(indptr, x, nthreads=1):

@@ -45,3 +45,38 @@ def test_spmm_sddmm_gradients(shape, feat_len):
     assert torch.allclose(s.double(), s64, rtol=1e-4, atol=1e-4)
     assert torch.allclose(x.grad.double(), x64.grad, rtol=1e-4, atol=1e-4)
     assert torch.allclose(d.grad.double(), d64.grad, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("reduce", ["sum", "mean", "max", "min"])
+def test_aggregate_gradients(reduce):
+    """Graph.aggregate against a dense masked reduction in float64 (continuous random data: no ties)."""
+    import torch
+    from featgraph_amd.autograd import Graph
+    rng = np.random.default_rng(4)
+    n_dst, n_src, F = 70, 90, 24
+    adj = sp.random(n_dst, n_src, density=0.12, format="csr", random_state=rng).astype("float32").tolil()
+    adj[[3, 40], :] = 0                                   # rows without edges
+    adj = adj.tocsr(); adj.eliminate_zeros(); adj.sort_indices()
+    g = Graph(adj)
+    gen = torch.Generator(device="cuda"); gen.manual_seed(1)
+    x = torch.randn((n_src, F), generator=gen, device="cuda", requires_grad=True)
+    up = torch.randn((n_dst, F), generator=gen, device="cuda")
+    y = g.aggregate(x, reduce)
+    (y * up).sum().backward()
+
+    mask = torch.from_numpy((adj.toarray() != 0)).cuda()
+    x64 = x.detach().double().requires_grad_()
+    big = x64[None, :, :].expand(n_dst, -1, -1)
+    has = mask.any(1)
+    if reduce in ("sum", "mean"):
+        y64 = (mask[:, :, None] * big).sum(1)
+        if reduce == "mean":
+            y64 = y64 / mask.sum(1).clamp(min=1)[:, None]
+    else:
+        fill = float("-inf") if reduce == "max" else float("inf")
+        masked = torch.where(mask[:, :, None], big, torch.full_like(big, fill))
+        y64 = masked.max(1).values if reduce == "max" else masked.min(1).values
+        y64 = torch.where(has[:, None], y64, torch.zeros_like(y64))
+    (y64 * up.double()).sum().backward()
+    assert torch.allclose(y.double(), y64, rtol=1e-4, atol=1e-5)
+    assert torch.allclose(x.grad.double(), x64.grad, rtol=1e-4, atol=1e-5)

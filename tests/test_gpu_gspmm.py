@@ -153,3 +153,27 @@ def test_gsddmm_elementwise(torch_cuda, op, feat_len):
         else:
             expect = {"add": s + d, "sub": s - d, "mul": s * d}[op]
             assert out.shape == expect.shape and np.array_equal(out, expect)
+
+
+@pytest.mark.parametrize("reduce", ["max", "min"])
+@pytest.mark.parametrize("feat_len", [1, 4, 7, 32, 64, 100, 256, 512])
+def test_selected_elements(torch_cuda, oracle, reduce, feat_len):
+    """return_arg: the stored position of the edge that gave each output, exact against the oracle
+    (first occurrence on ties; few distinct values so that ties are frequent; a split hub row)."""
+    from featgraph_amd.module import GSpMMhip, placeholder
+    torch = torch_cuda
+    rng = np.random.default_rng(feat_len + (reduce == "min"))
+    adj = _graph(rng)
+    adj.data = rng.integers(-2, 3, size=adj.nnz).astype("float32")
+    x = rng.integers(-3, 4, size=(3000, feat_len)).astype("float32")
+    for msg in ("u_mul_e", "copy_u"):
+        m = GSpMMhip(adj)
+        m.build([placeholder(x.shape)], {'reduce': reduce, 'msg': msg, 'return_arg': True}, {})
+        out = m.run([torch.from_numpy(x).cuda()]).cpu().numpy()
+        arg = m.arg_tvm.cpu().numpy()
+        ref_out, ref_arg = oracle.gspmm_arg(adj.indptr, adj.indices, adj.data if msg == "u_mul_e" else None, x, reduce, 2)
+        assert np.array_equal(out, ref_out), (reduce, msg, feat_len)
+        assert np.array_equal(arg, ref_arg), (reduce, msg, feat_len)
+        assert (arg[np.diff(adj.indptr) == 0] == -1).all()
+    with pytest.raises(ValueError):
+        GSpMMhip(adj).build([placeholder(x.shape)], {'reduce': 'sum', 'return_arg': True}, {})

@@ -353,3 +353,25 @@ def test_edge_softmax_backward_closed_forms(oracle):
     # the gradient of each row sums to zero per head (softmax is shift-invariant)
     rows = indptr[:-1][np.diff(indptr) > 0]
     np.testing.assert_allclose(np.add.reduceat(got.astype(np.float64), rows, axis=0), 0.0, atol=1e-6)
+
+
+def test_gspmm_arg_closed_form(oracle):
+    """Selected elements of max / min aggregation against numpy argmax / argmin over the gathered
+    messages (both return the first occurrence), with repeated values so that ties occur."""
+    rng = np.random.default_rng(21)
+    adj = _rand_csr(rng, 40, 60, 0.2).tolil()
+    adj[[0, 17], :] = 0
+    adj = adj.tocsr().astype("float32"); adj.eliminate_zeros(); adj.sort_indices()
+    adj.data = rng.integers(-2, 3, size=adj.nnz).astype("float32")          # few distinct weights
+    x = rng.integers(-3, 4, size=(60, 6)).astype("float32")                  # few distinct values: many ties
+    for reduce, pick in (("max", np.argmax), ("min", np.argmin)):
+        out, arg = oracle.gspmm_arg(adj.indptr, adj.indices, adj.data, x, reduce)
+        assert np.array_equal(out, oracle.gspmm(adj.indptr, adj.indices, adj.data, x, reduce))
+        for r in range(40):
+            b, e = adj.indptr[r], adj.indptr[r + 1]
+            if e == b:
+                assert (arg[r] == -1).all() and (out[r] == 0).all()
+                continue
+            msgs = adj.data[b:e, None] * x[adj.indices[b:e]]
+            assert np.array_equal(arg[r], b + pick(msgs, axis=0))
+            assert np.array_equal(out[r], msgs[arg[r] - b, np.arange(6)])
