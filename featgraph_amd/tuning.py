@@ -42,7 +42,8 @@ def _partitions(n_src, row_bytes, nnz, n_rows, slice_bytes, min_segment):
 def choose_spmm(n_dst, n_src, nnz, feat_len):
     """(num_col_partitions, num_feat_partitions) for an SpMM of this size."""
     t = feature_tiles(feat_len)
-    row_bytes = 4 * feat_len / min(t, 8) if t > 1 else 4 * feat_len
+    # more than 8 tiles are launched 8 at a time, so an XCD never holds more than one tile's slice
+    row_bytes = 4 * feat_len / t if t > 1 else 4 * feat_len
     p = _partitions(n_src, row_bytes, nnz, n_dst, SPMM_SLICE_BYTES, min_segment=24)
     if p == 1 and feat_len <= 256:
         # rows too short to partition: nothing is reused through the L2 anyway, and whole rows per
