@@ -33,7 +33,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # Fabric-side bytes (rocprofv3 FETCH_SIZE x2 + WRITE_SIZE, scaled by the X copy of the same run) moved
-# by all launches of the named kernel in one operator call, at the default tiling; from
+# by all launches of the named kernel in one operator call, at the default tiling (the JSON reports
+# them per launch as `traffic` and per operator as `op_traffic`); from
 # profiles/bench_powerlaw233k_f512_rocprofv3.txt.  Other configurations have no measurement: null.
 MEASURED_TRAFFIC = {
     ("spmm", "powerlaw-233k", 512, 8, 8): 72.5e9,      # 8 x spmm_items_kernel (+ fix-ups)
@@ -229,10 +230,15 @@ def main():
     dom = "spmm" if t_spmm >= t_sddmm else "sddmm"
     key = (dom, args.workload, F, ops[dom].get("num_col_partitions", ops[dom].get("num_src_partitions")),
            ops[dom].get("num_feat_partitions", ops[dom].get("num_feat_tiles")))
-    traffic = MEASURED_TRAFFIC.get(key)
+    op_traffic = MEASURED_TRAFFIC.get(key)
+    n_launch = ops[dom]["launches"]
+    b_dom = b_spmm if dom == "spmm" else b_sddmm
+    # per launch of the gather kernel: algorithmic bytes / launches over op time / launches -- the same
+    # ratio as for the whole operator; `traffic` is the measured fabric-side bytes of one such launch
     roofline = {"bound": "hbm", "kernel": ops[dom]["kernel"], "achieved": round(ops[dom]["hbm_gbs"], 2),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ops[dom]["hbm_gbs"] / HBM_PEAK_GBS, 5),
-                "traffic": traffic, "algorithmic_bytes": int(b_spmm if dom == "spmm" else b_sddmm),
+                "traffic": (round(op_traffic / n_launch) if op_traffic else None), "op_traffic": op_traffic,
+                "algorithmic_bytes_per_launch": int(b_dom / n_launch), "algorithmic_bytes": int(b_dom),
                 "launches": ops[dom]["launches"], "kernels": ops[dom]["kernels"], "op_ms": round(ops[dom]["ms"], 4),
                 "avg_launch_ms": round(ops[dom]["ms"] / ops[dom]["launches"], 4)}
 
