@@ -135,8 +135,7 @@ def gspmm(indptr, indices, vals, x, reduce="sum", nthreads=1):
     F = x2.shape[1]
     vp = None
     if vals is not None:
-        vals = _c(vals, np.float32).reshape(indices.shape[0], -1)
-        assert vals.shape[1] == H
+        vals = _c(vals, np.float32).reshape(indices.shape[0], H)
         vp = _p(vals, _f32p)
     n_dst = indptr.shape[0] - 1
     out = np.empty((n_dst, F), dtype=np.float32)
@@ -156,8 +155,7 @@ def gspmm_arg(indptr, indices, vals, x, reduce="max", nthreads=1):
     F = x2.shape[1]
     vp = None
     if vals is not None:
-        vals = _c(vals, np.float32).reshape(indices.shape[0], -1)
-        assert vals.shape[1] == H
+        vals = _c(vals, np.float32).reshape(indices.shape[0], H)
         vp = _p(vals, _f32p)
     n_dst = indptr.shape[0] - 1
     out = np.empty((n_dst, F), dtype=np.float32)

@@ -1,0 +1,112 @@
+"""Seeded random sweep over graph shapes, densities, feature lengths, partition and tile counts:
+every case is compared with the CPU oracle / float64 closed forms.  The point is breadth -- kernel
+variants and boundary conditions that the hand-picked cases may not reach."""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+from helpers import RTOL, ATOL, assert_sum_close, spmm_mass, sddmm_mass
+
+pytestmark = pytest.mark.gpu
+
+FEATS = [1, 2, 3, 4, 5, 8, 12, 16, 20, 31, 32, 48, 64, 65, 96, 100, 128, 160, 192, 256, 257, 320, 384, 512, 768, 1024]
+
+
+def _random_graph(rng):
+    n_rows = int(rng.integers(1, 400))
+    n_cols = int(rng.integers(1, 400))
+    density = float(rng.choice([0.0, 0.002, 0.02, 0.1, 0.5, 1.0]))
+    a = sp.random(n_rows, n_cols, density=density, format="csr", random_state=rng,
+                  data_rvs=lambda k: rng.standard_normal(k)).astype("float32")
+    if rng.random() < 0.5 and n_cols > 4:                      # a long row, split into pieces at threshold 1024
+        a = a.tolil()
+        r = int(rng.integers(0, n_rows))
+        a[r, :] = rng.standard_normal(n_cols).astype("float32")
+        a = a.tocsr().astype("float32")
+    a.eliminate_zeros(); a.sort_indices()
+    return a
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_spmm(oracle, seed):
+    import torch
+    from featgraph_amd.module import VanillaSpMMhip, placeholder
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(20):
+        adj = _random_graph(rng)
+        F = int(rng.choice(FEATS))
+        P = int(rng.choice([1, 1, 2, 3, 5, 8]))
+        divisors = [t for t in (1, 2, 4, 8, 16) if F % t == 0]
+        T = int(rng.choice([0] + divisors))
+        x = rng.standard_normal((adj.shape[1], F)).astype("float32")
+        m = VanillaSpMMhip(adj, P)
+        m.build([placeholder(x.shape)], {'num_feat_partitions': T}, {'num_src_partitions': None})
+        m.out_tvm.fill_(float("nan"))
+        out = m.run([torch.from_numpy(x).cuda()]).cpu().numpy()
+        what = "seed %d case %d: %s nnz %d F=%d P=%d T=%d" % (seed, case, adj.shape, adj.nnz, F, P, T)
+        assert np.isfinite(out).all(), what
+        assert_sum_close(out, oracle.spmm_f64(adj, x), spmm_mass(adj, x), what)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_sddmm(oracle, seed):
+    import torch
+    from featgraph_amd.module import VanillaSDDMMhip, MultiHeadSDDMMhip, placeholder
+    rng = np.random.default_rng(2000 + seed)
+    for case in range(20):
+        adj = _random_graph(rng)
+        coo = adj.tocoo()
+        if rng.random() < 0.5:
+            H, D = 1, int(rng.choice(FEATS))
+        else:
+            H, D = int(rng.choice([2, 3, 4, 8, 16])), int(rng.choice([4, 8, 12, 16, 32, 64, 128]))
+        shp = (H, D) if H > 1 else (D,)
+        src = rng.standard_normal((adj.shape[1],) + shp).astype("float32")
+        dst = rng.standard_normal((adj.shape[0],) + shp).astype("float32")
+        order = str(rng.choice(["auto", "csr", "coo", "tiled"]))
+        sched = {'order': order}
+        F = H * D
+        if order == "tiled":
+            tiles = [t for t in (1, 2, 4, 8) if F % t == 0 and (F // t) in (16, 32, 64, 128, 256)
+                     and (H == 1 or (F // t) % D == 0 or D == (F // t))]
+            if not tiles or (H > 1 and (D % 4 != 0 or D < 8 or (D & (D - 1)) != 0)):
+                sched = {'order': 'auto'}
+            else:
+                sched.update({'num_src_partitions': int(rng.choice([1, 2, 3, 8])), 'num_feat_tiles': int(rng.choice(tiles))})
+        m = (MultiHeadSDDMMhip if H > 1 else VanillaSDDMMhip)(coo if rng.random() < 0.5 else adj)
+        m.build([placeholder(src.shape), placeholder(dst.shape)], {}, sched)
+        m.out_tvm.fill_(float("nan"))
+        out = m.run([torch.from_numpy(src).cuda(), torch.from_numpy(dst).cuda()]).cpu().numpy()
+        what = "seed %d case %d: %s nnz %d H=%d D=%d %s" % (seed, case, adj.shape, adj.nnz, H, D, sched)
+        assert np.isfinite(out).all(), what
+        ref = oracle.sddmm_multihead_f64(coo.row, coo.col, src, dst) if H > 1 else oracle.sddmm_f64(coo.row, coo.col, src, dst)
+        assert_sum_close(out, ref, sddmm_mass(coo.row, coo.col, src, dst), what)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_softmax_and_aggregation(oracle, seed):
+    import torch
+    from featgraph_amd.module import EdgeSoftmaxhip, GSpMMhip, placeholder
+    rng = np.random.default_rng(3000 + seed)
+    for case in range(20):
+        adj = _random_graph(rng)
+        H = int(rng.choice([1, 2, 3, 4, 5, 8, 16, 64]))
+        shape = (adj.nnz,) if H == 1 else (adj.nnz, H)
+        s = (rng.standard_normal(shape) * 3).astype("float32")
+        sm = EdgeSoftmaxhip(adj)
+        sm.build([placeholder(shape)])
+        a = sm.run([torch.from_numpy(s).cuda()]).cpu().numpy()
+        what = "seed %d case %d: %s nnz %d H=%d" % (seed, case, adj.shape, adj.nnz, H)
+        np.testing.assert_allclose(a, oracle.edge_softmax_f64(adj.indptr, s), rtol=RTOL, atol=ATOL, err_msg=what)
+        g = rng.standard_normal(shape).astype("float32")
+        dx = sm.backward(torch.from_numpy(a).cuda(), torch.from_numpy(g).cuda()).cpu().numpy()
+        np.testing.assert_allclose(dx, oracle.edge_softmax_backward(adj.indptr, a, g), rtol=1e-3, atol=2e-5, err_msg=what)
+        F = int(rng.choice([1, 4, 7, 32, 100, 256]))
+        x = rng.integers(-3, 4, size=(adj.shape[1], F)).astype("float32")
+        red = str(rng.choice(["max", "min"]))
+        gm = GSpMMhip(adj)
+        gm.build([placeholder(x.shape)], {'reduce': red, 'return_arg': True}, {})
+        out = gm.run([torch.from_numpy(x).cuda()]).cpu().numpy()
+        ref_out, ref_arg = oracle.gspmm_arg(adj.indptr, adj.indices, adj.data, x, red)
+        assert np.array_equal(out, ref_out), what
+        assert np.array_equal(gm.arg_tvm.cpu().numpy(), ref_arg), what
