@@ -264,6 +264,7 @@ struct SddmmTiledArgs {
     const float *src;         // partition p's first src row is src + p * src_stride
     int64_t src_stride;
     int first_part, conc, n_parts;   // this launch works on partitions [first_part, first_part + conc)
+    int tile_base;                   // ... and on tiles [tile_base, tile_base + n_tiles)
     const float *dst;
     float *out;               // out (direct mode) or partial (tile-sum mode)
     int64_t out_edge_stride;  // floats between consecutive edges in out
@@ -382,7 +383,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     // every XCD works on one tile of one partition
     const unsigned per = (unsigned)(a.n_tiles * a.conc);
     const int slot = (int)(blockIdx.x % per);
-    const int tile = slot % a.n_tiles;
+    const int tile = a.tile_base + slot % a.n_tiles;
     const int part = a.first_part + slot / a.n_tiles;
     if (part >= a.n_parts) return;
     const int64_t i0 = a.item_off[part];
@@ -843,16 +844,22 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
     const int conc = (T < 8 && 8 % T == 0) ? std::max(1, std::min(8 / T, P)) : 1;
     a.conc = conc;
     const bool off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
+    // More than 8 tiles: 8 per launch (one per XCD), as for SpMM.
+    const int per_launch = (T > 8 && T % 8 == 0) ? 8 : T;
+    a.n_tiles = per_launch;
     for (int p0 = 0; p0 < P; p0 += conc) {
         int64_t most = 0;
         for (int p = p0; p < std::min(P, p0 + conc); ++p) most = std::max(most, pl->item_off[p + 1] - pl->item_off[p]);
         if (most == 0) continue;
         a.first_part = p0;
-        const int64_t blocks = ((most + kWavesPerBlock - 1) / kWavesPerBlock) * T * conc;
+        const int64_t blocks = ((most + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch * conc;
         if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
-        const bool ok = (tile_sum || staged) ? launch_tiled_l<false>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a)
-                                             : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
-        if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);
+        for (int tb = 0; tb < T; tb += per_launch) {
+            a.tile_base = tb;
+            const bool ok = (tile_sum || staged) ? launch_tiled_l<false>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a)
+                                                 : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
+            if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);
+        }
     }
     if (tile_sum) {
         if ((uintptr_t)edge_pos_dev & 15) return fail(FG_ERR_ARG, "edge_pos must be 16-byte aligned");
