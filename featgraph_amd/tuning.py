@@ -42,6 +42,9 @@ def _partitions(n_src, row_bytes, nnz, n_rows, slice_bytes, min_segment):
 def choose_spmm(n_dst, n_src, nnz, feat_len):
     """(num_col_partitions, num_feat_partitions) for an SpMM of this size."""
     t = feature_tiles(feat_len)
+    if feat_len >= 2048 and feat_len % 128 == 0:
+        # rows of 8 KB and more: 128-float tiles (measured at F=2048: 57.0 ms against 68.7 ms with 64-float tiles)
+        t = feat_len // 128
     # more than 8 tiles are launched 8 at a time, so an XCD never holds more than one tile's slice
     row_bytes = 4 * feat_len / t if t > 1 else 4 * feat_len
     p = _partitions(n_src, row_bytes, nnz, n_dst, SPMM_SLICE_BYTES, min_segment=24)
