@@ -103,8 +103,7 @@ __device__ __forceinline__ void edge_heads(const typename Vec<V>::type (&s)[K], 
 
 // Dot products of the staged edges [0, n) of `edge` (x = column id, y = row id); results go to
 // out[j * H + head] for staged edge j.  The G lane groups take edges g, g+G, ...; U steps' src
-// loads are issued back to back.  A group keeps the dst row it fetched last and skips the
-// fetch while the row id repeats.  Per-head results are collected in registers -- the lane
+// loads are issued back to back.  Per-head results are collected in registers -- the lane
 // whose position in its head segment equals the step number (mod RW) keeps that step's value
 // -- and written out every RW steps as one dense run of RW*G*H floats.
 template <int V, int L, int K, int RW, int KH, bool FULL>
@@ -116,36 +115,33 @@ __device__ __forceinline__ void sddmm_staged(const int2 *edge, int n, int g, int
     constexpr int G = S::G, H = S::H, NH = S::NH;
     constexpr int U = (K >= 2) ? 2 : 4;
     const int seg_pos = li % RW, head0 = li / RW;
+    (void)held_row;
     float res[NH];
 #pragma unroll
     for (int kk = 0; kk < NH; ++kk) res[kk] = 0.f;
     const int nsteps = (n + G - 1) / G;
     for (int s0 = 0; s0 < nsteps; s0 += U) {
         int2 rc[U];
-        bool live[U];
-        vec sv[U][K];
+        vec sv[U][K], dw[U][K];
+        // no load sits under a branch: a group without an edge in this step re-reads the last edge
+        // (its result is not stored), and both operands are fetched for every edge -- when the row
+        // repeats, the destination row comes from the cache
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int j = (s0 + u) * G + g;
-            live[u] = j < n;
-            rc[u] = live[u] ? edge[j] : make_int2(0, -1);
-        }
+        for (int u = 0; u < U; ++u) rc[u] = edge[min((s0 + u) * G + g, n - 1)];
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int k = 0; k < K; ++k)
-                if (live[u] && (FULL || on[k]))
+                if (FULL || on[k]) {
                     sv[u][k] = *reinterpret_cast<const vec *>(sb + (int64_t)rc[u].x * F + k * L * V);
+                    dw[u][k] = *reinterpret_cast<const vec *>(db + (int64_t)rc[u].y * F + k * L * V);
+                }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int step = s0 + u;
             if (step < nsteps) {                       // uniform
-                if (live[u] && rc[u].y != held_row) {
 #pragma unroll
-                    for (int k = 0; k < K; ++k)
-                        if (FULL || on[k]) dv[k] = *reinterpret_cast<const vec *>(db + (int64_t)rc[u].y * F + k * L * V);
-                    held_row = rc[u].y;
-                }
+                for (int k = 0; k < K; ++k) dv[k] = dw[u][k];
                 float q[NH];
                 edge_heads<V, L, K, RW, KH, FULL>(sv[u], dv, on, q);
                 if ((step % RW) == seg_pos) {
