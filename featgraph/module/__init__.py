@@ -1,3 +1,4 @@
 from featgraph_amd.module import (VanillaSpMMhip, VanillaSpMMx86, VanillaSpMMcuda,
                                   VanillaSDDMMhip, VanillaSDDMMx86, VanillaSDDMMcuda,
-                                  MultiHeadSDDMMhip, GSpMMhip, GSDDMMhip, EdgeSoftmaxhip, placeholder)
+                                  MultiHeadSDDMMhip, GSpMMhip, GSDDMMhip, EdgeSoftmaxhip,
+                                  EdgeSoftmaxSpMMhip, placeholder)

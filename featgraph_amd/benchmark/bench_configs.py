@@ -18,7 +18,7 @@ import torch
 from .. import synthetic
 from ..module import common
 from ..module import (VanillaSpMMhip, VanillaSDDMMhip, MultiHeadSDDMMhip, GSpMMhip, EdgeSoftmaxhip,
-                      placeholder)
+                      EdgeSoftmaxSpMMhip, placeholder)
 
 HBM_PEAK_GBS = 8000.0
 
@@ -67,7 +67,17 @@ def run_attention_steps(name, adj, softmax_heads, head_shapes):
         _line(name, "spmm_per_head_weights", {"heads": H, "head_len": D, "partitions": m._active['P'],
                                               "tiles": m._num_feat_partitions}, t, nnz, H * D,
               4 * (n + 1) + 4 * nnz + 4 * nnz * H + 8 * n * H * D)
-        del m, x, w
+        del m
+        # the same aggregation from raw scores, without a stored softmax
+        gen.manual_seed(4)
+        sc = torch.randn((nnz, H), generator=gen, device="cuda")
+        f = EdgeSoftmaxSpMMhip(adj)
+        f.build([placeholder((nnz, H)), placeholder((n, H, D))], {}, {})
+        t = f.measure_average_time([sc, x], 5)
+        _line(name, "edge_softmax_spmm_fused", {"heads": H, "head_len": D, "partitions": f._agg._active['P'],
+                                                "tiles": f._agg._num_feat_partitions}, t, nnz, H * D,
+              4 * (n + 1) + 4 * nnz + 4 * nnz * H + 8 * n * H * D)
+        del f, x, w, sc
 
 
 def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):

@@ -354,6 +354,61 @@ __global__ __launch_bounds__(256) void edge_softmax_merge_kernel(const Fixup *fi
     for (int p = 0; p < fx.n_pieces; ++p) s[(int64_t)p * H] = make_float2(m, sum);
 }
 
+// ---- statistics only, and the fused normalise-and-relayout step ------------------------------------
+//
+// For attention without a stored softmax: row_stats[v, h] = (max, sum of exp(x - max)) over row v, then
+// edge_softmax_head_major_kernel writes exp(x - max) / sum straight into the head-major, traversal-ordered
+// weight array that the per-head SpMM streams -- the [nnz, H] softmax array is never written or re-read.
+
+template <bool LANEHEAD>
+__global__ __launch_bounds__(kBlock) void edge_softmax_stats_kernel(const SoftmaxArgs a, float2 *row_stats) {
+    const int lane = threadIdx.x & 63;
+    const int64_t item_id = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (item_id >= a.n_items) return;         // uniform per wavefront; no workgroup barriers below
+    const Item it = a.items[item_id];
+    if (it.len == 0) return;
+    if (it.info >= 0) {                       // a piece: its statistics go to the plan's scratch, merged later
+        run_together<false, LANEHEAD, true, false>(a, it.start, it.len, lane, it.info);
+        return;
+    }
+    SoftmaxArgs rows = a;
+    rows.stats = row_stats;                   // whole rows write their own entry, slot = row
+    const int nrows = -it.info;
+    const int ends = a.indptr[it.row + min(lane, nrows - 1) + 1];
+    int b = it.start;
+    for (int q = 0; q < nrows; ++q) {
+        const int e = __shfl(ends, q);
+        if (e > b) run_together<false, LANEHEAD, true, false>(rows, b, e - b, lane, it.row + q);
+        b = e;
+    }
+}
+
+// Merges the pieces of every split row and writes the row's entry of row_stats.
+__global__ __launch_bounds__(256) void edge_softmax_stats_merge_kernel(const Fixup *fixups, int64_t n_fixups,
+                                                                       const float2 *stats, float2 *row_stats, int H) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_fixups * H) return;
+    const Fixup fx = fixups[t / H];
+    const int h = (int)(t % H);
+    const float2 *s = stats + (int64_t)fx.slot0 * H + h;
+    float m = s[0].x, sum = 0.f;
+    for (int p = 1; p < fx.n_pieces; ++p) m = fmaxf(m, s[(int64_t)p * H].x);
+    for (int p = 0; p < fx.n_pieces; ++p) sum += s[(int64_t)p * H].y * __expf(s[(int64_t)p * H].x - m);
+    row_stats[(int64_t)fx.row * H + h] = make_float2(m, sum);
+}
+
+// dst[h, e'] = exp(x[pos[e'], h] - max) / sum with the statistics of the row of stored element pos[e'].
+__global__ __launch_bounds__(256) void edge_softmax_head_major_kernel(const float *x, const float2 *row_stats,
+                                                                      const int32_t *edge_row, const int32_t *pos,
+                                                                      int64_t n, int H, float *dst) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    const int64_t at = pos ? (int64_t)pos[e] : e;
+    const float *xs = x + at * H;
+    const float2 *st = row_stats + (int64_t)edge_row[at] * H;
+    for (int h = 0; h < H; ++h) dst[(int64_t)h * n + e] = __expf(xs[h] - st[h].x) / st[h].y;
+}
+
 template <bool BWD, bool LANEHEAD>
 void launch_both(const fg_spmm_plan *pl, const SoftmaxArgs &a, hipStream_t st) {
     const dim3 grid((unsigned)((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock));
@@ -396,6 +451,49 @@ int softmax_run(const fg_spmm_plan *pl, const int32_t *indptr, const float *x, c
 extern "C" int fg_edge_softmax_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev, const float *scores_dev,
                                    float *out_dev, int heads, void *stream) {
     return softmax_run(plan, indptr_dev, scores_dev, nullptr, out_dev, heads, stream, false);
+}
+
+extern "C" int fg_edge_softmax_stats_f32(const fg_spmm_plan *pl, const int32_t *indptr_dev, const float *scores_dev,
+                                         float *row_stats_dev, int heads, void *stream) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
+    if (pl->num_col_partitions != 1) return fail(FG_ERR_ARG, "edge softmax needs a plan with one column partition");
+    if (heads < 1) return fail(FG_ERR_SHAPE, "number of heads must be positive, got %d", heads);
+    if (pl->nnz == 0 || pl->n_items == 0) return FG_OK;
+    if (!indptr_dev || !scores_dev || !row_stats_dev) return fail(FG_ERR_ARG, "null device pointer");
+    if (((uintptr_t)row_stats_dev & 7) != 0) return fail(FG_ERR_ARG, "row_stats must be 8-byte aligned");
+    int rc = fg::ensure_partial(pl, (size_t)2 * (size_t)heads);
+    if (rc != FG_OK) return rc;
+    SoftmaxArgs a;
+    a.items = pl->items_dev; a.n_items = pl->n_items; a.indptr = indptr_dev;
+    a.x = scores_dev; a.g = nullptr; a.y = nullptr; a.stats = reinterpret_cast<float2 *>(pl->partial_dev); a.H = heads;
+    hipStream_t st = (hipStream_t)stream;
+    float2 *row_stats = reinterpret_cast<float2 *>(row_stats_dev);
+    const dim3 grid((unsigned)((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock));
+    if (heads <= 64 && (heads & (heads - 1)) == 0) hipLaunchKernelGGL(edge_softmax_stats_kernel<true>, grid, dim3(kBlock), 0, st, a, row_stats);
+    else hipLaunchKernelGGL(edge_softmax_stats_kernel<false>, grid, dim3(kBlock), 0, st, a, row_stats);
+    if (pl->n_fixups > 0) {
+        const int64_t threads = pl->n_fixups * heads;
+        hipLaunchKernelGGL(edge_softmax_stats_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
+                           pl->fixups_dev, pl->n_fixups, a.stats, row_stats, heads);
+    }
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
+}
+
+extern "C" int fg_edge_softmax_head_major_f32(const float *scores_dev, const float *row_stats_dev,
+                                              const int32_t *edge_row_dev, const int32_t *edge_pos_dev, int64_t n_edges,
+                                              int heads, float *dst_dev, void *stream) {
+    if (n_edges < 0 || heads < 1) return fail(FG_ERR_ARG, "fg_edge_softmax_head_major_f32: bad size");
+    if (n_edges == 0) return FG_OK;
+    if (!scores_dev || !row_stats_dev || !edge_row_dev || !dst_dev) return fail(FG_ERR_ARG, "null device pointer");
+    const int64_t blocks = (n_edges + 255) / 256;
+    if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "too many edges for one grid");
+    hipLaunchKernelGGL(edge_softmax_head_major_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       scores_dev, reinterpret_cast<const float2 *>(row_stats_dev), edge_row_dev, edge_pos_dev, n_edges,
+                       heads, dst_dev);
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
 }
 
 extern "C" int fg_edge_softmax_backward_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev,

@@ -110,3 +110,84 @@ class EdgeSoftmaxhip(object):
     @property
     def target(self):
         return self._target
+
+
+class EdgeSoftmaxSpMMhip(object):
+    """Attention aggregation without a stored softmax:
+
+        out[v, h, :] = sum over the edges e into v of softmax_v(Scores)[e, h] * SrcFeat[col e, h, :]
+
+    Scores is (nnz,) or (nnz, H) in the adjacency's CSR edge order, SrcFeat (num_cols, F) or
+    (num_cols, H, D).  Three launches: the rows' (max, sum of exp) per head, a pass that writes
+    exp(score - max) / sum directly in the order and layout the per-head weighted SpMM streams, and that
+    SpMM; the normalised [nnz, H] array of EdgeSoftmaxhip is never written or read back.  The reference
+    has neither operator; conventions as in its modules (python/featgraph/module/spmm.py:81-161).
+    """
+
+    def __init__(self, adj_scipy):
+        from .gspmm import GSpMMhip
+        self._agg = GSpMMhip(adj_scipy)
+        self._ctx = self._agg.ctx
+        self._target = self._agg.target
+        indptr = self._agg._adj_indptr
+        self._nnz = int(indptr[-1])
+        self._num_rows = self._agg._num_rows
+        rows = np.repeat(np.arange(self._num_rows, dtype=np.int32), np.diff(indptr))
+        self._edge_row = common.to_device_i32(rows, self._ctx)
+        self._placeholders = None
+        self.out_tvm = None
+
+    def build(self, input_placeholders, compute_args=None, schedule_args=None):
+        """input_placeholders: [Scores, SrcFeat]; schedule_args as for GSpMMhip ('num_src_partitions')."""
+        common.take_args(compute_args or {}, ('num_feat_partitions',), "compute_func")
+        if len(input_placeholders) != 2:
+            raise ValueError("takes two inputs (Scores, SrcFeat), got %d" % len(input_placeholders))
+        s_ph, x_ph = input_placeholders
+        heads = x_ph.shape[1] if len(x_ph.shape) == 3 else 1
+        want = ((self._nnz,), (self._nnz, 1)) if heads == 1 else ((self._nnz, heads),)
+        if tuple(s_ph.shape) not in want:
+            raise ValueError("Scores must have shape %s, got %s" % (want[-1], s_ph.shape))
+        w_shape = (self._nnz,) if heads == 1 else (self._nnz, heads)
+        self._agg.build([x_ph, common.placeholder(w_shape)], dict(compute_args or {}), dict(schedule_args or {}))
+        self._heads = heads
+        self._placeholders = [s_ph, x_ph]
+        self._row_stats = torch.zeros((self._num_rows, heads, 2), dtype=torch.float32, device=self._ctx)
+        self._weights = torch.empty((heads, self._nnz), dtype=torch.float32, device=self._ctx)
+        self.out_tvm = self._agg.out_tvm
+
+    def _launch(self, scores, x):
+        agg, L, s = self._agg, _lib.lib(), common.stream_ptr()
+        csr = agg._layouts[1]
+        lay = agg._active
+        _lib.check(L.fg_edge_softmax_stats_f32(csr['plan'], _lib.dev_ptr(csr['pos']), _lib.dev_ptr(scores),
+                                               _lib.dev_ptr(self._row_stats), self._heads, s))
+        pos = lay['edge_pos32'] if lay['P'] > 1 else None
+        _lib.check(L.fg_edge_softmax_head_major_f32(_lib.dev_ptr(scores), _lib.dev_ptr(self._row_stats),
+                                                    _lib.dev_ptr(self._edge_row), _lib.dev_ptr(pos), self._nnz,
+                                                    self._heads, _lib.dev_ptr(self._weights), s))
+        _lib.check(L.fg_gspmm_f32(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']),
+                                  _lib.dev_ptr(self._weights), _lib.dev_ptr(x), _lib.dev_ptr(self.out_tvm),
+                                  agg._feat_len, self._heads, 1, 0, agg._num_feat_partitions, s))
+
+    def run(self, input_tvm_ndarrays):
+        """[Scores, SrcFeat] -> self.out_tvm (the same tensor on every call); nothing is synchronised."""
+        if self._placeholders is None:
+            raise RuntimeError("call build() before run()")
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        self._launch(input_tvm_ndarrays[0], input_tvm_ndarrays[1])
+        return self.out_tvm
+
+    def measure_average_time(self, input_tvm_ndarrays, num_runs):
+        if self._placeholders is None:
+            raise RuntimeError("call build() before measure_average_time()")
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        s, x = input_tvm_ndarrays
+        return common.timed_mean_seconds(lambda: self._launch(s, x), num_runs)
+
+    @property
+    def ctx(self):
+        return self._ctx
+
+    @property
+    def target(self):
+        return self._target

@@ -172,3 +172,33 @@ def test_attention_chain_gradients(torch_cuda):
     assert torch.allclose(out.double(), out64, rtol=1e-4, atol=1e-4)
     for got, ref in ((q.grad, q64.grad), (k.grad, k64.grad), (v.grad, v64.grad)):
         assert torch.allclose(got.double(), ref, rtol=1e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("H,D,P", [(1, 32, None), (1, 100, 2), (4, 16, None), (4, 64, 3), (8, 8, None), (2, 128, 'auto'), (3, 32, None)])
+def test_fused_softmax_spmm(torch_cuda, oracle, H, D, P):
+    """EdgeSoftmaxSpMMhip (statistics + normalise-into-SpMM-layout + SpMM) against float64:
+    softmax per row and head (scipy), then the weighted sum per head."""
+    from featgraph_amd.module import EdgeSoftmaxSpMMhip, placeholder
+    from helpers import assert_sum_close
+    torch = torch_cuda
+    rng = np.random.default_rng(H * 100 + D)
+    adj = _ragged(rng, "hub")
+    n_rows, n_cols = adj.shape
+    nnz = adj.nnz
+    s_shape = (nnz,) if H == 1 else (nnz, H)
+    x_shape = (n_cols, D) if H == 1 else (n_cols, H, D)
+    s = (rng.standard_normal(s_shape) * 3).astype("float32")
+    x = rng.standard_normal(x_shape).astype("float32")
+    m = EdgeSoftmaxSpMMhip(adj)
+    m.build([placeholder(s_shape), placeholder(x_shape)], {}, {'num_src_partitions': P})
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([torch.from_numpy(s).cuda(), torch.from_numpy(x).cuda()]).cpu().numpy().reshape(n_rows, H, D)
+    a64 = oracle.edge_softmax_f64(adj.indptr, s).reshape(nnz, H)
+    x3 = x.reshape(n_cols, H, D).astype(np.float64)
+    ref = np.zeros((n_rows, H, D)); mass = np.zeros((n_rows, H, D))
+    for h in range(H):
+        ah = sp.csr_matrix((a64[:, h], adj.indices, adj.indptr), shape=adj.shape)
+        ref[:, h] = ah.dot(x3[:, h]); mass[:, h] = ah.dot(np.abs(x3[:, h]))
+    assert np.isfinite(out).all()
+    assert_sum_close(out, ref, mass, "H=%d D=%d P=%s" % (H, D, P))
+    assert (out[np.diff(adj.indptr) == 0] == 0).all()
