@@ -13,6 +13,7 @@
 #include <algorithm>
 
 #include "fg_common.h"
+#include "fg_device.h"
 
 using fg::fail;
 using fg::Item;
@@ -369,7 +370,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     constexpr int G = 64 / L;
     constexpr int U = (RW < 8 ? RW : 8) / (K >= 2 ? 2 : 1) > 0 ? (RW < 8 ? RW : 8) / (K >= 2 ? 2 : 1) : 1;
     static_assert(U <= kTilePad, "unclamped reads must stay inside the padded staging row");
-    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges + kTilePad];     // x = column word, y = edge_pos
+    __shared__ __align__(16) int2 s_edge[kWavesPerBlock][fg::kItemEdges + kTilePad];     // x = column word, y = edge_pos
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
     __shared__ int32_t s_next[kWavesPerBlock];
 
@@ -400,15 +401,16 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     float4 dv[K];
 
     auto stage = [&](int64_t base, int n) {
-        int2 r[4];
+        // lane l holds edges 4l .. 4l + 3 (past the end: the last edge again)
+        int32_t c[4], at[4] = {0, 0, 0, 0};
+        fg::load_four(a.col + base, n, lane, 1, c);
+        if (SCATTER) fg::load_four(a.edge_pos + base, n, lane, 1, at);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int t = min(lane + 64 * i, n - 1);
-            r[i] = make_int2((int)((uint32_t)a.col[base + t] * scale), SCATTER ? a.edge_pos[base + t] : 0);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) edge[lane + 64 * i] = r[i];
-        if (lane < kTilePad) edge[fg::kItemEdges + lane] = r[3];
+        for (int i = 0; i < 4; ++i) c[i] = (int)((uint32_t)c[i] * scale);
+        int4 *e4 = reinterpret_cast<int4 *>(edge);
+        e4[2 * lane] = make_int4(c[0], at[0], c[1], at[1]);
+        e4[2 * lane + 1] = make_int4(c[2], at[2], c[3], at[3]);
+        if (lane < kTilePad) edge[fg::kItemEdges + lane] = make_int2(c[3], at[3]);
     };
     auto load_dst = [&](int64_t row) {
 #pragma unroll

@@ -15,6 +15,7 @@
 #include <string>
 
 #include "fg_common.h"
+#include "fg_device.h"
 
 using fg::fail;
 using fg::Fixup;
@@ -177,22 +178,24 @@ __device__ __forceinline__ void finish_row(typename Vec<V>::type (&acc)[K], cons
     }
 }
 
-// Loads elements [base, base + min(n, 256)) of (indices, vals) into registers, 4 per lane; lanes
-// past the end re-read the last element so that no load is conditional.  n >= 1.
+// Loads elements [base, base + min(n, 256)) of (indices, vals) into registers, lane l holding
+// elements 4l .. 4l + 3.  n >= 1.
 // `scale` turns a column id into the staged word: the row's byte size (OFF32) or 1.  The weight of
 // element t is vals[t * vstride + voff] (one weight per head), or 1 when there are no weights.
 __device__ __forceinline__ void stage_load(const int32_t *indices, const float *vals, int64_t base, int n,
                                            int lane, uint32_t scale, int vstride, int64_t voff, int2 (&r)[4]) {
+    int32_t c[4];
+    float w[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    fg::load_four(indices + base, n, lane, 1, c);
+    if (vals) fg::load_four(vals + base * vstride + voff, n, lane, vstride, w);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int t = min(lane + 64 * i, n - 1);
-        const float w = vals ? vals[(base + t) * vstride + voff] : 1.0f;
-        r[i] = make_int2((int)((uint32_t)indices[base + t] * scale), __float_as_int(w));
-    }
+    for (int i = 0; i < 4; ++i) r[i] = make_int2((int)((uint32_t)c[i] * scale), __float_as_int(w[i]));
 }
+// Writes the staged words to the wavefront's staging row (16-byte aligned), two elements per store.
 __device__ __forceinline__ void stage_store(int2 *edge, int lane, const int2 (&r)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) edge[lane + 64 * i] = r[i];
+    int4 *e4 = reinterpret_cast<int4 *>(edge);
+    e4[2 * lane] = make_int4(r[0].x, r[0].y, r[1].x, r[1].y);
+    e4[2 * lane + 1] = make_int4(r[2].x, r[2].y, r[3].x, r[3].y);
     if (lane < kPad) edge[fg::kItemEdges + lane] = r[3];      // a valid element: slots past the end stay loadable
 }
 
@@ -201,19 +204,20 @@ template <int HPT>
 __device__ __forceinline__ void stage_load_w(const float *vals, int64_t base, int n, int lane, int vstride,
                                              int64_t voff, int64_t hstride, float (&w)[HPT][4]) {
 #pragma unroll
-    for (int h = 0; h < HPT; ++h)
+    for (int h = 0; h < HPT; ++h) {
+        if (vals) {
+            fg::load_four(vals + base * vstride + voff + h * hstride, n, lane, vstride, w[h]);
+        } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int t = min(lane + 64 * i, n - 1);
-            w[h][i] = vals ? vals[(base + t) * vstride + voff + h * hstride] : 1.0f;
+            for (int i = 0; i < 4; ++i) w[h][i] = 1.0f;
         }
+    }
 }
 template <int HPT, int ROW>
 __device__ __forceinline__ void stage_store_w(float (*rows)[ROW], int lane, const float (&w)[HPT][4]) {
 #pragma unroll
     for (int h = 0; h < HPT; ++h) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) rows[h][lane + 64 * i] = w[h][i];
+        *reinterpret_cast<float4 *>(&rows[h][4 * lane]) = make_float4(w[h][0], w[h][1], w[h][2], w[h][3]);
         if (lane < kPad) rows[h][fg::kItemEdges + lane] = w[h][3];
     }
 }
@@ -223,19 +227,19 @@ __device__ __forceinline__ void stage_store_w(float (*rows)[ROW], int lane, cons
 // OFF32: X spans less than 4 GiB, rows are addressed by 32-bit byte offsets; HPT: heads (with
 // their own weights) per kernel tile, each covered by L / HPT lanes.
 template <int V, int L, int K, bool FULL, bool ACC, bool OFF32, int HPT = 1>
-__global__ __launch_bounds__(kBlock) void spmm_items_kernel(const SpmmArgs a) {
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void spmm_items_kernel(const SpmmArgs a) {
     using vec = typename Vec<V>::type;
     static_assert(fg::kItemEdges == 256, "stage_load/stage_store move 4 x 64 elements");
     constexpr int FT = V * L * K;          // floats per kernel tile
     constexpr int G = 64 / L;              // lane groups per wavefront
-    constexpr int U = (K >= 2) ? 2 : (L <= 8 ? 8 : 4);   // steps whose loads are issued back to back
+    constexpr int U = (K >= 2) ? 2 : 4;   // steps whose loads are issued back to back
     static_assert(U <= kPad, "reads past a row's end must stay inside the padded staging row");
     // kPad extra slots: the lane-group-per-row walk may read up to U - 1 slots past a row's end
-    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
+    __shared__ __align__(16) int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
     __shared__ int32_t s_next[kWavesPerBlock];
     constexpr int kWRow = HPT > 1 ? fg::kItemEdges + kPad : 1;
-    __shared__ float s_w[kWavesPerBlock][HPT][kWRow];
+    __shared__ __align__(16) float s_w[kWavesPerBlock][HPT][kWRow];
     static_assert(HPT == 1 || (L % HPT == 0 && K == 1 && FULL), "heads of a tile split its lanes evenly");
 
     const int lane = threadIdx.x & 63;
@@ -444,7 +448,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_extreme_kernel(const SpmmArgs a)
     constexpr int FT = V * L * K;
     constexpr int G = 64 / L;
     constexpr int U = (K >= 2) ? 2 : 4;
-    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
+    __shared__ __align__(16) int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
 
     const int lane = threadIdx.x & 63;
@@ -602,7 +606,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_arg_kernel(const SpmmArgs a) {
     constexpr int FT = V * L * K;
     constexpr int G = 64 / L;
     constexpr int U = (K >= 2) ? 2 : 4;
-    __shared__ int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
+    __shared__ __align__(16) int2 s_edge[kWavesPerBlock][fg::kItemEdges + kPad];
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
 
     const int lane = threadIdx.x & 63;
