@@ -227,7 +227,7 @@ __device__ __forceinline__ void stage_store_w(float (*rows)[ROW], int lane, cons
 // OFF32: X spans less than 4 GiB, rows are addressed by 32-bit byte offsets; HPT: heads (with
 // their own weights) per kernel tile, each covered by L / HPT lanes.
 template <int V, int L, int K, bool FULL, bool ACC, bool OFF32, int HPT = 1>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void spmm_items_kernel(const SpmmArgs a) {
+__device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
     using vec = typename Vec<V>::type;
     static_assert(fg::kItemEdges == 256, "stage_load/stage_store move 4 x 64 elements");
     constexpr int FT = V * L * K;          // floats per kernel tile
@@ -418,6 +418,19 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
         gather_rows<V, L, K, FULL, U, OFF32, HPT>(edge, wrow, 0, n, g, a.x, lane_bytes, F, on, acc);
     }
     finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
+}
+
+// The kernels proper.  One load per lane and source row (K == 1) fits 64 registers without spilling
+// and is held to 8 wavefronts per SIMD; wider rows per lane and tiles of several heads keep the
+// compiler's own register budget.
+template <int V, int L, int K, bool FULL, bool ACC, bool OFF32>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void spmm_items_kernel(const SpmmArgs a) {
+    static_assert(K == 1, "wider rows use spmm_items_wide_kernel");
+    spmm_items_body<V, L, K, FULL, ACC, OFF32, 1>(a);
+}
+template <int V, int L, int K, bool FULL, bool ACC, bool OFF32, int HPT>
+__global__ __launch_bounds__(kBlock) void spmm_items_wide_kernel(const SpmmArgs a) {
+    spmm_items_body<V, L, K, FULL, ACC, OFF32, HPT>(a);
 }
 
 // ---- max / min aggregation ------------------------------------------------------------------------
@@ -794,19 +807,24 @@ int choose_config(int F, int T, bool aligned16, SpmmConfig *c) {
 
 template <int V, int L, int K, bool FULL, bool ACC>
 void launch_off(bool off32, dim3 grid, hipStream_t st, const SpmmArgs &a) {
-    if (off32) hipLaunchKernelGGL((spmm_items_kernel<V, L, K, FULL, ACC, true>), grid, dim3(kBlock), 0, st, a);
-    else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, FULL, ACC, false>), grid, dim3(kBlock), 0, st, a);
+    if constexpr (K == 1) {
+        if (off32) hipLaunchKernelGGL((spmm_items_kernel<V, L, K, FULL, ACC, true>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((spmm_items_kernel<V, L, K, FULL, ACC, false>), grid, dim3(kBlock), 0, st, a);
+    } else {
+        if (off32) hipLaunchKernelGGL((spmm_items_wide_kernel<V, L, K, FULL, ACC, true, 1>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((spmm_items_wide_kernel<V, L, K, FULL, ACC, false, 1>), grid, dim3(kBlock), 0, st, a);
+    }
 }
 
 // tiles of HPT heads: 128-bit lanes, one load per lane, no masking
 template <int L, int HPT>
 void launch_hpt(bool off32, dim3 grid, hipStream_t st, const SpmmArgs &a) {
     if (a.accumulate) {
-        if (off32) hipLaunchKernelGGL((spmm_items_kernel<4, L, 1, true, true, true, HPT>), grid, dim3(kBlock), 0, st, a);
-        else hipLaunchKernelGGL((spmm_items_kernel<4, L, 1, true, true, false, HPT>), grid, dim3(kBlock), 0, st, a);
+        if (off32) hipLaunchKernelGGL((spmm_items_wide_kernel<4, L, 1, true, true, true, HPT>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((spmm_items_wide_kernel<4, L, 1, true, true, false, HPT>), grid, dim3(kBlock), 0, st, a);
     } else {
-        if (off32) hipLaunchKernelGGL((spmm_items_kernel<4, L, 1, true, false, true, HPT>), grid, dim3(kBlock), 0, st, a);
-        else hipLaunchKernelGGL((spmm_items_kernel<4, L, 1, true, false, false, HPT>), grid, dim3(kBlock), 0, st, a);
+        if (off32) hipLaunchKernelGGL((spmm_items_wide_kernel<4, L, 1, true, false, true, HPT>), grid, dim3(kBlock), 0, st, a);
+        else hipLaunchKernelGGL((spmm_items_wide_kernel<4, L, 1, true, false, false, HPT>), grid, dim3(kBlock), 0, st, a);
     }
 }
 
@@ -1006,9 +1024,10 @@ std::string spmm_launch_text(const fg_spmm_plan *pl, int F, int T) {
     const int64_t per_part = pl->item_off.size() > 1 ? pl->item_off[1] - pl->item_off[0] : 0;
     snprintf(b, sizeof(b),
              "  feature length   : %d, %d requested tile(s) of %d, %d kernel tile(s) of %d floats\n"
-             "  kernel           : spmm_items_kernel<V=%d, L=%d, K=%d, FULL=%d, ACC=pass>0>; %d element(s) per step\n"
+             "  kernel           : %s<V=%d, L=%d, K=%d, FULL=%d, ACC=pass>0>; %d element(s) per step\n"
              "  launch           : %d pass(es); first pass grid %lld x block %d; fixup rows %lld\n",
-             F, c.n_ftiles / c.sub_per_tile, c.tile_w, c.n_ftiles, c.V * c.L * c.K, c.V, c.L, c.K,
+             F, c.n_ftiles / c.sub_per_tile, c.tile_w, c.n_ftiles, c.V * c.L * c.K,
+             c.K == 1 ? "spmm_items_kernel" : "spmm_items_wide_kernel", c.V, c.L, c.K,
              (int)c.full, 64 / c.L, pl->num_col_partitions,
              (long long)(((per_part + kWavesPerBlock - 1) / kWavesPerBlock) * c.n_ftiles), kBlock,
              (long long)pl->n_fixups);
