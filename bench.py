@@ -207,6 +207,11 @@ def main():
         conc = min(8 // T, P) if (T < 8 and 8 % T == 0) else 1
         return (P + conc - 1) // conc
 
+    def copies(n_tiles):
+        """Launches of the kernel that makes the tile-by-tile copy of the gathered operand (the library's
+        default rule: 4 or more feature tiles, 16 MB or more, 32-bit offsets)."""
+        return 1 if (n_tiles >= 4 and (16 << 20) <= 4 * n * F < (1 << 32)) else 0
+
     flops_op = 2.0 * nnz * F
     b_spmm = spmm_bytes(n, n, nnz, F)
     b_sddmm = sddmm_bytes(n, nnz, F, 1, csr=True)
@@ -214,13 +219,15 @@ def main():
         "spmm": {"ms": t_spmm, "gflops": flops_op / t_spmm / 1e6, "compulsory_gb": b_spmm / 1e9,
                  "hbm_gbs": b_spmm / t_spmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_spmm / 1e6,
                  "kernel": "spmm_items_kernel", "launches": spmm._active['P'],
-                 "kernels": {"spmm_items_kernel": spmm._active['P'], "spmm_fixup_kernel": spmm._active['P']},
+                 "kernels": {"tile_major_kernel": copies(spmm._num_feat_partitions or 1),
+                             "spmm_items_kernel": spmm._active['P'], "spmm_fixup_kernel": spmm._active['P']},
                  "num_col_partitions": spmm._active['P'], "num_feat_partitions": spmm._num_feat_partitions},
         "sddmm": {"ms": t_sddmm, "gflops": flops_op / t_sddmm / 1e6, "compulsory_gb": b_sddmm / 1e9,
                   "hbm_gbs": b_sddmm / t_sddmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_sddmm / 1e6,
                   "kernel": "sddmm_tiled_kernel" if sddmm._tiled else "sddmm_csr_kernel",
                   "launches": sddmm_launches(),
-                  "kernels": ({"sddmm_tiled_kernel": sddmm_launches(), "sddmm_tile_sum_kernel": 1}
+                  "kernels": ({"tile_major_kernel": copies(sddmm._tiled[1]), "sddmm_tiled_kernel": sddmm_launches(),
+                               "sddmm_tile_sum_kernel": 1}
                               if sddmm._tiled else {"sddmm_csr_kernel": 1}),
                   "num_src_partitions": sddmm._tiled[0]['P'] if sddmm._tiled else 1,
                   "num_feat_tiles": sddmm._tiled[1] if sddmm._tiled else 1},

@@ -52,6 +52,7 @@ struct fg_spmm_plan {
     int split_threshold = 0;
     int item_edges = 0;              // element budget of a multi-row item
     bool wide_offsets = false;       // never use 32-bit byte offsets into the feature matrices
+    int tile_major = 0;              // fg_plan_opts.tile_major
     int device = 0;
     // per partition: [item_begin, item_end) and [fixup_begin, fixup_end)
     std::vector<int64_t> item_off, fixup_off;
@@ -62,6 +63,9 @@ struct fg_spmm_plan {
     // partial sums of split rows; grown on demand to max_slots_in_partition * F floats
     mutable float *partial_dev = nullptr;
     mutable size_t partial_floats = 0;
+    // tile-by-tile copy of the source features of the call in progress; grown on demand
+    mutable float *tiled_dev = nullptr;
+    mutable size_t tiled_floats = 0;
     // statistics for fg_spmm_plan_describe
     int64_t max_len = 0, n_empty = 0, n_split_rows = 0, n_multi_items = 0;
 };
@@ -70,6 +74,13 @@ namespace fg {
 // Makes plan->partial_dev hold at least floats_per_piece floats for every piece of split rows of
 // one partition (grown on demand, never shrunk).
 int ensure_partial(const fg_spmm_plan *plan, size_t floats_per_piece);
+// Whether a call with n_tiles feature tiles over a source matrix of x_bytes gathers from a
+// tile-by-tile copy (the plan's tile_major option; the kernel-side conditions are the caller's).
+bool wants_tile_major(const fg_spmm_plan *plan, int n_tiles, uint64_t x_bytes);
+// plan->tiled_dev[(t * n_rows + r) * tile + i] = x[r * F + t * tile + i] for the F / tile tiles of
+// an [n_rows, F] matrix (F and tile multiples of 4, x 16-byte aligned, fewer than 2^32 floats),
+// on `stream`.  The buffer is grown on demand and never shrunk.
+int make_tile_major(const fg_spmm_plan *plan, const float *x, int64_t n_rows, int F, int tile, void *stream);
 // FG_OK when the calling thread's current device is the one the plan was created on.
 int check_device(const fg_spmm_plan *plan);
 }  // namespace fg

@@ -59,6 +59,11 @@ struct SpmmArgs {
     const int32_t *indices;
     const float *vals;
     const float *x;        // already offset to the partition's first source row
+    // Sum kernels, 32-bit offsets only.  Bytes between consecutive source rows, and, when the
+    // kernel tiles of x are stored one after the other ([tile][row][tile floats]), the bytes from
+    // one tile's block to the next; 0: rows of F floats that hold all tiles.
+    uint32_t x_row_bytes;
+    uint32_t x_tile_bytes;
     float *out;
     float *partial;
     int F;                 // row stride of x / out in floats
@@ -256,8 +261,9 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
     bool on[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
-    const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
-    const uint32_t scale = OFF32 ? (uint32_t)a.F * 4u : 1u;
+    const uint32_t lane_bytes = (OFF32 && a.x_tile_bytes) ? (uint32_t)tile * a.x_tile_bytes + (uint32_t)(li * V) * 4u
+                                                          : (uint32_t)f_lo * 4u;
+    const uint32_t scale = OFF32 ? a.x_row_bytes : 1u;
     const int64_t voff = (int64_t)((rt * a.tile_w + st * FT) / a.head_len) * a.head_stride;     // head of this kernel tile
     const int64_t F = a.F;
     int2 *edge = s_edge[wave];
@@ -889,6 +895,12 @@ int launch_ext_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs 
     return fail(FG_ERR_SHAPE, "no max/min kernel for V=%d L=%d K=%d", V, c.L, c.K);
 }
 
+// Whether the sum kernels of this configuration gather from a tile-by-tile copy of X.
+bool gathers_tile_major(const fg_spmm_plan *pl, const SpmmConfig &c, int F) {
+    return c.off32 && c.V == 4 && c.K == 1 && c.full && c.sub_per_tile == 1 && pl->nnz > 0 &&
+           fg::wants_tile_major(pl, c.n_ftiles, (uint64_t)pl->n_src * (uint64_t)F * 4u);
+}
+
 // reduce: FG_REDUCE_SUM / MAX / MIN.  heads > 1: vals is [nnz, heads] (or [heads, nnz] when
 // head_major) and every kernel tile must lie inside one head.  vals == nullptr with allow_no_vals: every weight is 1.
 int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
@@ -943,6 +955,14 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
+    // With several feature tiles an XCD gathers one tile's 256 bytes (or less) out of every source
+    // row, F * 4 bytes apart.  Gathered from a copy that stores each tile's slices back to back, the
+    // same working set is cached markedly better (232,965-node graph, 8 partitions: 13.5 -> 11.9 ms
+    // at F=512, 6.8 -> 6.1 ms at F=256, before the 0.25 / 0.13 ms that the copy takes); the sums
+    // are the same, in the same order.
+    const int ft = c.V * c.L * c.K;
+    const bool tiled = reduce == FG_REDUCE_SUM && gathers_tile_major(pl, c, F);
+    if (tiled && (rc = fg::make_tile_major(pl, x, pl->n_src, F, ft, stream)) != FG_OK) return rc;
     for (int p = 0; p < P; ++p) {
         const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
         if (i1 > i0) {
@@ -950,7 +970,9 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
             a.items = pl->items_dev + i0; a.n_items = i1 - i0;
             a.pos = pos + (int64_t)p * (pl->n_dst + 1);
             a.indices = idx; a.vals = vals;
-            a.x = x + (int64_t)p * width * F;
+            a.x = tiled ? pl->tiled_dev + (int64_t)p * width * ft : x + (int64_t)p * width * F;
+            a.x_row_bytes = (uint32_t)(tiled ? ft : F) * 4u;
+            a.x_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * ft * 4u) : 0u;
             a.out = out; a.partial = pl->partial_dev;
             a.F = F; a.tile_w = c.tile_w; a.sub_per_tile = c.sub_per_tile;
             a.heads = heads; a.head_len = F / heads;
@@ -1031,7 +1053,11 @@ std::string spmm_launch_text(const fg_spmm_plan *pl, int F, int T) {
              (int)c.full, 64 / c.L, pl->num_col_partitions,
              (long long)(((per_part + kWavesPerBlock - 1) / kWavesPerBlock) * c.n_ftiles), kBlock,
              (long long)pl->n_fixups);
-    return b;
+    std::string text = b;
+    c.off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
+    text += gathers_tile_major(pl, c, F) ? "  source features  : gathered from a tile-by-tile copy made at the start of every call\n"
+                                         : "  source features  : gathered from the caller's row-major matrix\n";
+    return text;
 }
 }  // namespace fg
 

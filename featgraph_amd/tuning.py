@@ -60,10 +60,18 @@ def choose_sddmm(n_rows, n_cols, nnz, heads, head_len):
     kernels should be used (small feature matrices, or a shape the tiled kernel does not take)."""
     feat_len = heads * head_len
     tile = None
-    # 256 floats or more per edge: 128-float tiles halve the per-tile partial sums (or hold two heads), and
-    # with fewer than 8 tiles the kernel runs 8 / tiles partitions per launch, so the slice an XCD holds
-    # stays the same (232,965-node graph: 15.0 -> 14.5 ms at F=512; H=8, D=64: 18.2 -> 16.7 ms)
-    order = (128, 64, 256, 32, 16) if feat_len >= 256 else (64, 128, 256, 32, 16)
+    # One result per edge: 64-float tiles.  With 4 or more tiles the kernel gathers from a tile-by-tile
+    # copy of the source features, and 8 partitions of 64-float tiles then beat 16 partitions of
+    # 128-float tiles (232,965-node graph: 13.7 against 13.8 ms at F=512, 6.8 against 7.3 ms at F=256).
+    # Several heads: a tile's results are scattered per edge, so wider tiles (more heads per write) win
+    # (H=8, D=32: 8.8 ms with 128-float tiles, 9.3 ms with 64; H=8, D=64: 16.0 against 16.8 ms) unless
+    # that leaves fewer than 4 tiles of whole 64-float heads (H=4, D=64: 7.7 ms, 7.3 ms with 64-float tiles).
+    if heads == 1:
+        order = (64, 128, 256, 32, 16)
+    elif feat_len >= 256 and not (head_len >= 64 and feat_len // 128 < 4):
+        order = (128, 64, 256, 32, 16)
+    else:
+        order = (64, 128, 256, 32, 16)
     for cand in order:
         if feat_len % cand != 0:
             continue
@@ -75,7 +83,7 @@ def choose_sddmm(n_rows, n_cols, nnz, heads, head_len):
     if tile is None:
         return None
     t = feat_len // tile
-    row_bytes = 4 * feat_len / min(t, 8)
+    row_bytes = 4 * feat_len / t          # more than 8 tiles are launched 8 at a time: one tile's slice per XCD
     if n_cols * row_bytes <= SDDMM_SLICE_BYTES:
         return None
     p = _partitions(n_cols, row_bytes, nnz, n_rows, SDDMM_SLICE_BYTES, min_segment=24)

@@ -170,8 +170,12 @@ def test_default_tilings():
     assert tuning.choose_spmm(n, n, nnz, 512) == (8, 8)
     assert tuning.choose_spmm(n, n, nnz, 128) == (8, 2)
     assert tuning.choose_spmm(2450000, 2450000, 61903880, 128) == (1, 1)     # rows too short to partition
-    assert tuning.choose_sddmm(n, n, nnz, 1, 512) == (16, 4)
+    assert tuning.choose_sddmm(n, n, nnz, 1, 512) == (8, 8)
+    assert tuning.choose_sddmm(n, n, nnz, 1, 256) == (8, 4)
+    assert tuning.choose_sddmm(n, n, nnz, 1, 1024) == (8, 16)
     assert tuning.choose_sddmm(n, n, nnz, 8, 64) == (16, 4)
+    assert tuning.choose_sddmm(n, n, nnz, 4, 64) == (8, 4)
+    assert tuning.choose_sddmm(n, n, nnz, 8, 32) == (16, 2)
     assert tuning.choose_sddmm(n, n, nnz, 4, 32) == (8, 2)
     assert tuning.choose_sddmm(10000, 10000, 170000, 1, 32) is None           # fits the caches: plain kernels
     for F in (32, 64, 128, 256, 512):
