@@ -37,8 +37,8 @@ HBM_PEAK_GBS = 8000.0
 # them per launch as `traffic` and per operator as `op_traffic`); from
 # profiles/bench_powerlaw233k_f512_rocprofv3.txt.  Other configurations have no measurement: null.
 MEASURED_TRAFFIC = {
-    ("spmm", "powerlaw-233k", 512, 8, 8): 72.4e9,      # 8 x spmm_items_kernel (+ fix-ups)
-    ("sddmm", "powerlaw-233k", 512, 16, 4): 79.1e9,    # 8 x sddmm_tiled_kernel (tile sum: +2.9e9)
+    ("spmm", "powerlaw-233k", 512, 8, 8): 72.4e9,      # 8 x spmm_items_kernel + fix-ups (copy: +0.95e9)
+    ("sddmm", "powerlaw-233k", 512, 8, 8): 70.9e9,     # 8 x sddmm_tiled_kernel (copy: +0.95e9, tile sum: +4.7e9)
 }
 METRIC = "SpMM/SDDMM GFLOP/s + achieved HBM GB/s (% roofline), 233k-node graph, feat 512"
 
