@@ -209,8 +209,8 @@ def main():
 
     def copies(n_tiles):
         """Launches of the kernel that makes the tile-by-tile copy of the gathered operand (the library's
-        default rule: 4 or more feature tiles, 16 MB or more, 32-bit offsets)."""
-        return 1 if (n_tiles >= 4 and (16 << 20) <= 4 * n * F < (1 << 32)) else 0
+        default rule: 4 or more feature tiles, 64 MB or more, 32-bit offsets)."""
+        return 1 if (n_tiles >= 4 and (64 << 20) <= 4 * n * F < (1 << 32)) else 0
 
     flops_op = 2.0 * nnz * F
     b_spmm = spmm_bytes(n, n, nnz, F)

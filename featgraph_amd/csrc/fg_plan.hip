@@ -149,9 +149,9 @@ namespace fg {
 bool wants_tile_major(const fg_spmm_plan *pl, int n_tiles, uint64_t x_bytes) {
     if (pl->tile_major == 2 || n_tiles < 2) return false;
     if (pl->tile_major == 1) return true;
-    // Measured on the 232,965-node graph: nothing at 2 tiles, 10-12 % at 4 and 8 tiles; a matrix
-    // that fits the L2s has nothing to gain.
-    return n_tiles >= 4 && x_bytes >= (16ull << 20);
+    // Measured on the 232,965-node graph (238 / 477 MB): nothing at 2 tiles, 10-12 % at 4 and 8 tiles;
+    // on a 23,296-node graph (47 MB, mostly cache-resident) the copy only costs its own time.
+    return n_tiles >= 4 && x_bytes >= (64ull << 20);
 }
 int make_tile_major(const fg_spmm_plan *pl, const float *x, int64_t n_rows, int F, int tile, void *stream) {
     const uint64_t floats = (uint64_t)n_rows * (uint64_t)F;
