@@ -59,7 +59,7 @@ struct SpmmArgs {
     const int32_t *indices;
     const float *vals;
     const float *x;        // already offset to the partition's first source row
-    // Sum kernels, 32-bit offsets only.  Bytes between consecutive source rows, and, when the
+    // Sum, max and min kernels, 32-bit offsets only.  Bytes between consecutive source rows, and, when the
     // kernel tiles of x are stored one after the other ([tile][row][tile floats]), the bytes from
     // one tile's block to the next; 0: rows of F floats that hold all tiles.
     uint32_t x_row_bytes;
@@ -483,8 +483,9 @@ __global__ __launch_bounds__(kBlock) void gspmm_extreme_kernel(const SpmmArgs a)
     bool on[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) on[k] = FULL || (f_lo + k * L * V < f_end);
-    const uint32_t lane_bytes = (uint32_t)f_lo * 4u;
-    const uint32_t scale = OFF32 ? (uint32_t)a.F * 4u : 1u;
+    const uint32_t lane_bytes = (OFF32 && a.x_tile_bytes) ? (uint32_t)tile * a.x_tile_bytes + (uint32_t)(li * V) * 4u
+                                                          : (uint32_t)f_lo * 4u;
+    const uint32_t scale = OFF32 ? a.x_row_bytes : 1u;
     const int64_t voff = (int64_t)((rt * a.tile_w + st * FT) / a.head_len) * a.head_stride;
     const int64_t F = a.F;
     int2 *edge = s_edge[wave];
@@ -895,7 +896,7 @@ int launch_ext_v(const SpmmConfig &c, dim3 grid, hipStream_t st, const SpmmArgs 
     return fail(FG_ERR_SHAPE, "no max/min kernel for V=%d L=%d K=%d", V, c.L, c.K);
 }
 
-// Whether the sum kernels of this configuration gather from a tile-by-tile copy of X.
+// Whether the sum / max / min kernels of this configuration gather from a tile-by-tile copy of X.
 bool gathers_tile_major(const fg_spmm_plan *pl, const SpmmConfig &c, int F) {
     return c.off32 && c.V == 4 && c.K == 1 && c.full && c.sub_per_tile == 1 && pl->nnz > 0 &&
            fg::wants_tile_major(pl, c.n_ftiles, (uint64_t)pl->n_src * (uint64_t)F * 4u);
@@ -961,7 +962,7 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
     // at F=512, 6.8 -> 6.1 ms at F=256, before the 0.25 / 0.13 ms that the copy takes); the sums
     // are the same, in the same order.
     const int ft = c.V * c.L * c.K;
-    const bool tiled = reduce == FG_REDUCE_SUM && gathers_tile_major(pl, c, F);
+    const bool tiled = gathers_tile_major(pl, c, F);
     if (tiled && (rc = fg::make_tile_major(pl, x, pl->n_src, F, ft, stream)) != FG_OK) return rc;
     for (int p = 0; p < P; ++p) {
         const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];

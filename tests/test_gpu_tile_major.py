@@ -111,3 +111,30 @@ def test_sddmm_copy_equals_row_major(oracle, monkeypatch, H, D, P, T):
     coo = adj.tocoo()
     want = oracle.sddmm_multihead_f64(coo.row, coo.col, src, dst) if H > 1 else oracle.sddmm_f64(coo.row, coo.col, src, dst)
     assert_sum_close(tiled, want, sddmm_mass(coo.row, coo.col, src, dst), "H=%d D=%d" % (H, D))
+
+
+@pytest.mark.parametrize("reduce", ["max", "min"])
+@pytest.mark.parametrize("feat_len", [128, 256, 512])
+def test_extreme_aggregation_copy_equals_row_major(oracle, monkeypatch, reduce, feat_len):
+    """max / min gather from the copy too; the positions of the selected elements are found by a second
+    sweep over the caller's matrix and must still match."""
+    import torch
+    from featgraph_amd import _lib
+    from featgraph_amd.module import GSpMMhip, placeholder
+    rng = np.random.default_rng(feat_len)
+    adj = _graph(rng)
+    x = rng.standard_normal((adj.shape[1], feat_len)).astype("float32")
+
+    def run():
+        m = GSpMMhip(adj)
+        m.build([placeholder(x.shape)], {'reduce': reduce, 'msg': 'u_mul_e', 'return_arg': True}, {})
+        out = m.run([torch.from_numpy(x).cuda()]).cpu().numpy().copy()
+        return out, m.arg_tvm.cpu().numpy().copy()
+
+    monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(tile_major=2))
+    plain, plain_arg = run()
+    monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(tile_major=1))
+    tiled, tiled_arg = run()
+    assert np.array_equal(plain, tiled) and np.array_equal(plain_arg, tiled_arg)
+    ref_out, ref_arg = oracle.gspmm_arg(adj.indptr, adj.indices, adj.data, x, reduce, 2)
+    assert np.array_equal(tiled, ref_out) and np.array_equal(tiled_arg, ref_arg)
