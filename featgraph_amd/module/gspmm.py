@@ -73,6 +73,7 @@ class GSpMMhip(VanillaSpMMhip):
         self._return_arg = return_arg
         self._inv_deg_edge = None
         self._w_head_major = None
+        self._w_static = None
         if reduce == 'mean':
             deg = np.diff(self._adj_indptr).astype(np.float32)
             inv = np.where(deg > 0, 1.0 / np.maximum(deg, 1), 0).astype(np.float32)
@@ -97,6 +98,8 @@ class GSpMMhip(VanillaSpMMhip):
         One weight per edge: a 1-D array in element order.  One weight per edge and head: the
         library's relayout kernel writes them head-major (each head contiguous) in element order."""
         lay = self._active
+        if given is None and self._w_static is not None:
+            return self._w_static          # the adjacency's own values: laid out once per build
         if self._msg == 'copy_u':
             w = None
         elif given is not None:
@@ -109,6 +112,14 @@ class GSpMMhip(VanillaSpMMhip):
             w = self._inv_deg_edge.reshape(-1, 1) if w is None else w * self._inv_deg_edge.reshape(-1, 1)
         if w is None:
             return None, 0
+        if given is None:
+            self._w_static = self._weights_in_layout(w, lay)
+            if self._w_static[0] is self._w_head_major:
+                self._w_head_major = None          # kept; weights given to later runs get a buffer of their own
+            return self._w_static
+        return self._weights_in_layout(w, lay)
+
+    def _weights_in_layout(self, w, lay):
         if w.shape[1] > 1 or lay['P'] > 1:
             w = w.contiguous()
             if self._w_head_major is None or self._w_head_major.shape != (w.shape[1], w.shape[0]):

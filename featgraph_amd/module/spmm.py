@@ -137,6 +137,10 @@ class SpMMbase(object):
                 T = auto_t
             if P > 1:
                 notes.append("%d source-column partitions chosen for the L2 size" % P)
+        elif T == 0 and tuning.feature_tiles(feat_len) > 1:
+            # the caller fixed the partitions but not the tiles: 64-float tiles across the XCDs
+            # (tiling changes which workgroup computes a column, not the sums)
+            T = tuning.feature_tiles(feat_len)
         return ph, feat_len, int(T), P, notes
 
     def build(self, input_placeholders, compute_args, schedule_args):
