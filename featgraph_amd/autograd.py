@@ -36,13 +36,7 @@ class Graph(object):
         self._tr = scipy.sparse.csr_matrix((np.ones(csr.nnz, np.float32), tr.indices.astype(np.int32),
                                             tr.indptr.astype(np.int32)), shape=tr.shape)
         self._tr_pos_host = (tr.data - 1).astype(np.int64)      # transposed edge order -> CSR position
-        self._tr_pos = None
         self._mods = {}
-
-    def _tr_perm(self, device):
-        if self._tr_pos is None or self._tr_pos.device != device:
-            self._tr_pos = torch.from_numpy(self._tr_pos_host).to(device)
-        return self._tr_pos
 
     def _spmm_mod(self, transposed, tail, w_heads):
         key = ('spmm', transposed, tail, w_heads)
@@ -51,6 +45,8 @@ class Graph(object):
             m = GSpMMhip(adj)
             w_shape = (self.nnz,) if w_heads == 0 else (self.nnz, w_heads)
             m.build([placeholder((adj.shape[1],) + tail), placeholder(w_shape)], {}, {})
+            if transposed:
+                m.set_weight_order(self._tr_pos_host)      # weights arrive in this graph's CSR edge order
             self._mods[key] = m
         return self._mods[key]
 
@@ -77,8 +73,6 @@ class Graph(object):
             raise ValueError("with x of shape (n, H, D) the weights must be (nnz, H)")
         if x.dim() == 2 and w.dim() != 1:
             raise ValueError("with x of shape (n, F) the weights must be (nnz,)")
-        if transposed:
-            w = w.index_select(0, self._tr_perm(w.device))
         mod = self._spmm_mod(transposed, tuple(x.shape[1:]), 0 if w.dim() == 1 else w.shape[1])
         return mod.run([x, w.contiguous()]).clone()
 

@@ -109,6 +109,8 @@ class GSpMMhip(VanillaSpMMhip):
             if w is None:
                 w = common.to_device_f32(self._adj_scipy_csr.data, self._ctx).reshape(-1, 1)
         if self._inv_deg_edge is not None:
+            if given is not None and getattr(self, '_weight_perm', None) is not None:
+                raise ValueError("reduce='mean' with weights in another edge order is not supported")
             w = self._inv_deg_edge.reshape(-1, 1) if w is None else w * self._inv_deg_edge.reshape(-1, 1)
         if w is None:
             return None, 0
@@ -117,14 +119,40 @@ class GSpMMhip(VanillaSpMMhip):
             if self._w_static[0] is self._w_head_major:
                 self._w_head_major = None          # kept; weights given to later runs get a buffer of their own
             return self._w_static
-        return self._weights_in_layout(w, lay)
+        return self._weights_in_layout(w, lay, given=True)
 
-    def _weights_in_layout(self, w, lay):
-        if w.shape[1] > 1 or lay['P'] > 1:
+    def set_weight_order(self, position_of_edge):
+        """Weights given to run() are stored in another edge order: position_of_edge[i] is where the
+        weight of this adjacency's i-th edge (CSR order) lies in the given array (int array of nnz entries,
+        or None for CSR order).  The library's relayout kernel follows it; no separate permutation pass."""
+        if position_of_edge is None:
+            self._weight_perm = None
+        else:
+            perm = torch.as_tensor(position_of_edge, device=self._ctx).to(torch.int32).contiguous()
+            if perm.shape != (self._adj_indices.shape[0],):
+                raise ValueError("position_of_edge must have nnz = %d entries" % self._adj_indices.shape[0])
+            self._weight_perm = perm
+        self._perm_pos = {}
+
+    def _given_pos(self, lay):
+        """Element of the active layout -> position in the array given to run() (None: identity)."""
+        perm = getattr(self, '_weight_perm', None)
+        pos = lay['edge_pos32'] if lay['P'] > 1 else None
+        if perm is None:
+            return pos
+        if pos is None:
+            return perm
+        cache = self.__dict__.setdefault('_perm_pos', {})
+        if lay['P'] not in cache:
+            cache[lay['P']] = perm[pos.long()].contiguous()
+        return cache[lay['P']]
+
+    def _weights_in_layout(self, w, lay, given=False):
+        pos = self._given_pos(lay) if given else (lay['edge_pos32'] if lay['P'] > 1 else None)
+        if w.shape[1] > 1 or pos is not None:
             w = w.contiguous()
             if self._w_head_major is None or self._w_head_major.shape != (w.shape[1], w.shape[0]):
                 self._w_head_major = torch.empty((w.shape[1], w.shape[0]), dtype=torch.float32, device=self._ctx)
-            pos = lay['edge_pos32'] if lay['P'] > 1 else None
             _lib.check(_lib.lib().fg_edge_values_head_major_f32(_lib.dev_ptr(w), _lib.dev_ptr(pos), w.shape[0],
                                                                 w.shape[1], _lib.dev_ptr(self._w_head_major),
                                                                 common.stream_ptr()))
