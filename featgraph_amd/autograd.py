@@ -74,10 +74,10 @@ class Graph(object):
         if x.dim() == 2 and w.dim() != 1:
             raise ValueError("with x of shape (n, F) the weights must be (nnz,)")
         mod = self._spmm_mod(transposed, tuple(x.shape[1:]), 0 if w.dim() == 1 else w.shape[1])
-        return mod.run([x, w.contiguous()]).clone()
+        return _fresh_run(mod, [x, w.contiguous()])
 
     def _sddmm_raw(self, src, dst):
-        return self._sddmm_mod(tuple(src.shape[1:])).run([src.contiguous(), dst.contiguous()]).clone()
+        return _fresh_run(self._sddmm_mod(tuple(src.shape[1:])), [src.contiguous(), dst.contiguous()])
 
     def spmm(self, x, w):
         """y[v,:] = sum_e w[e] x[col e,:]; x (num_cols, F) with w (nnz,), or x (num_cols, H, D) with
@@ -121,6 +121,13 @@ class Graph(object):
         return _EdgeSoftmax.apply(self, scores)
 
 
+def _fresh_run(mod, inputs):
+    """run() into a tensor of the caller's own: the module's output buffer (every element of which a run
+    overwrites) is replaced first, so nothing has to be copied out of it."""
+    mod.out_tvm = torch.empty_like(mod.out_tvm)
+    return mod.run(inputs)
+
+
 class _SpMM(torch.autograd.Function):
     @staticmethod
     def forward(ctx, g, x, w):
@@ -157,14 +164,16 @@ class _EdgeSoftmax(torch.autograd.Function):
     @staticmethod
     def forward(ctx, g, scores):
         ctx.g = g
-        a = g._softmax_mod(tuple(scores.shape)).run([scores.contiguous()]).clone()
+        a = _fresh_run(g._softmax_mod(tuple(scores.shape)), [scores.contiguous()])
         ctx.save_for_backward(a)
         return a
 
     @staticmethod
     def backward(ctx, da):
         (a,) = ctx.saved_tensors
-        return None, ctx.g._softmax_mod(tuple(a.shape)).backward(a, da.contiguous()).clone()
+        mod = ctx.g._softmax_mod(tuple(a.shape))
+        mod.grad_tvm = torch.empty_like(a)          # handed to the caller; the module takes a new one next time
+        return None, mod.backward(a, da.contiguous())
 
 
 class _Aggregate(torch.autograd.Function):
