@@ -1,4 +1,4 @@
 from featgraph_amd.module import (VanillaSpMMhip, VanillaSpMMx86, VanillaSpMMcuda,
                                   VanillaSDDMMhip, VanillaSDDMMx86, VanillaSDDMMcuda,
                                   MultiHeadSDDMMhip, GSpMMhip, GSDDMMhip, EdgeSoftmaxhip,
-                                  EdgeSoftmaxSpMMhip, placeholder)
+                                  EdgeSoftmaxSpMMhip, GraphAttentionhip, placeholder)

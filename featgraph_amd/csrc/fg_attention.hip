@@ -1,0 +1,331 @@
+// Dot-product attention over the edges of a graph, in one sweep per source-column partition:
+//
+//   s[e, h]   = scale * <K[col e, h, :], Q[row e, h, :]>
+//   a[e, h]   = softmax of s[., h] over the edges of row(e)
+//   out[v, h, :] = sum over the edges e of row v of a[e, h] * V[col e, h, :]
+//
+// i.e. multi-head SDDMM, edge softmax and per-head weighted SpMM without ever storing the [nnz, H]
+// scores: every lane group keeps a running maximum, a running sum of exponentials and the running
+// weighted sum of its row (rescaled whenever the maximum grows), and source-column partitions are
+// merged the same way through `out` and a small [n_dst, H, 2] state array.  Not in the reference (no
+// attention operator exists there); the result is defined by the composition of the three operators.
+//
+// Layout of the work: one head (16, 32 or 64 floats) per kernel tile, the tile index fastest in the
+// workgroup id so that every XCD gathers one head's slices of K and V; items, staging and the
+// tile-by-tile copies of the gathered operands are those of the SpMM kernels.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "fg_common.h"
+#include "fg_device.h"
+
+using fg::fail;
+using fg::Item;
+
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = 64 * kWavesPerBlock;
+constexpr int kPad = 8;
+constexpr int kU = 4;                  // elements per lane group whose gathers are issued back to back
+
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over the L (4, 8 or 16) consecutive lanes of a lane group; every lane of the group gets it.
+template <int L>
+__device__ __forceinline__ float group_sum(float v) {
+    v += dpp_move<0xB1>(v);                  // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);                  // quad_perm [2,3,0,1]
+    if (L >= 8) v += dpp_move<0x141>(v);     // row_half_mirror
+    if (L >= 16) v += dpp_move<0x140>(v);    // row_mirror
+    return v;
+}
+
+struct AttnArgs {
+    const Item *items;
+    int64_t n_items;
+    const int32_t *pos;       // this partition's row boundaries
+    const int32_t *indices;   // partition-local column ids
+    const float *q;           // [n_dst, F]
+    const float *k, *v;       // offset to the partition's first source row
+    uint32_t kv_row_bytes;    // bytes between consecutive rows of k / v
+    uint32_t kv_tile_bytes;   // k / v stored head by head: bytes from one head's block to the next; 0: rows of F floats
+    float *out;               // [n_dst, F]: running weighted sums (divided by the sum of exponentials at the end)
+    float *state;             // [n_dst, H, 2]: running maximum and sum of exponentials
+    int F, H;
+    int n_heads, head_base;   // heads of this launch
+    float scale;
+};
+
+// Running softmax-weighted sum of one lane group: maximum, sum of exponentials, weighted sum.
+struct Running {
+    float m, l;
+    float4 acc;
+};
+
+__device__ __forceinline__ Running running_empty() { return {-INFINITY, 0.f, make_float4(0.f, 0.f, 0.f, 0.f)}; }
+
+// r <- r and s merged (both relative to their own maxima).
+__device__ __forceinline__ void running_merge(Running &r, const Running &s) {
+    const float m = fmaxf(r.m, s.m);
+    if (m == -INFINITY) return;               // both empty
+    const float fr = __expf(r.m - m), fs = __expf(s.m - m);      // exp(-inf) = 0 for the empty side
+    r.acc.x = r.acc.x * fr + s.acc.x * fs; r.acc.y = r.acc.y * fr + s.acc.y * fs;
+    r.acc.z = r.acc.z * fr + s.acc.z * fs; r.acc.w = r.acc.w * fr + s.acc.w * fs;
+    r.l = r.l * fr + s.l * fs;
+    r.m = m;
+}
+
+// NU steps of one row for this lane group: staged elements s0 + g, s0 + g + G, ...; every step but the
+// last lies wholly below e, and in the last one (unless ALLVALID) a group whose element would be e or
+// beyond re-reads element e - 1 and gives it no weight.  All 2 * NU gathers are issued before the first
+// is used.
+template <int L, int NU, bool ALLVALID>
+__device__ __forceinline__ void walk_batch(const int32_t *cols, int s0, int e, int g, const float *k, const float *v,
+                                           uint32_t lane_bytes, const float4 &q, float scale, Running &r) {
+    constexpr int G = 64 / L;
+    const bool last_valid = ALLVALID || s0 + (NU - 1) * G + g < e;
+    int c[NU];
+#pragma unroll
+    for (int u = 0; u < NU; ++u) c[u] = cols[(u < NU - 1 || last_valid) ? s0 + u * G + g : e - 1];
+    float4 kk[NU], vv[NU];
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        kk[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(k) + ((uint32_t)c[u] + lane_bytes));
+        vv[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(v) + ((uint32_t)c[u] + lane_bytes));
+    }
+    float s[NU];
+    float m = r.m;
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        const float d = kk[u].x * q.x + kk[u].y * q.y + kk[u].z * q.z + kk[u].w * q.w;
+        const float t = group_sum<L>(d) * scale;      // every lane takes part in the cross-lane sum
+        s[u] = (u < NU - 1 || last_valid) ? t : -INFINITY;
+        m = fmaxf(m, s[u]);
+    }
+    if (m == -INFINITY) return;             // nothing finite so far (uniform inside a lane group)
+    const float f = __expf(r.m - m);
+    r.acc.x *= f; r.acc.y *= f; r.acc.z *= f; r.acc.w *= f;
+    r.l *= f;
+    r.m = m;
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        const float p = __expf(s[u] - m);
+        r.l += p;
+        r.acc.x += p * vv[u].x; r.acc.y += p * vv[u].y; r.acc.z += p * vv[u].z; r.acc.w += p * vv[u].w;
+    }
+}
+
+// Staged elements [b, e) of one row, shared by the G lane groups; the last batch is issued with exactly
+// the steps it has left.
+template <int L>
+__device__ __forceinline__ void walk(const int32_t *cols, int b, int e, int g, const float *k, const float *v,
+                                     uint32_t lane_bytes, const float4 &q, float scale, Running &r) {
+    constexpr int G = 64 / L;
+    int s0 = b;
+    for (; s0 + G * kU <= e; s0 += G * kU) walk_batch<L, kU, true>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+    if (s0 >= e) return;
+    const int nu = (e - s0 + G - 1) / G;    // uniform: 1 .. kU
+    static_assert(kU == 4, "the tail below lists the step counts");
+    if (nu == 1) walk_batch<L, 1, false>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+    else if (nu == 2) walk_batch<L, 2, false>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+    else if (nu == 3) walk_batch<L, 3, false>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+    else walk_batch<L, 4, false>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+}
+
+// What the earlier partitions left for a row (read before the row's gathers are issued).
+template <bool FIRST>
+__device__ __forceinline__ Running load_state(const float *out_row, const float *state_row) {
+    Running old = running_empty();
+    if (!FIRST) {
+        old.m = state_row[0]; old.l = state_row[1];
+        old.acc = *reinterpret_cast<const float4 *>(out_row);
+    }
+    return old;
+}
+
+// Merges the lane groups' running sums (every group ends with the row's), then, in later passes, the
+// row's state from the earlier partitions, and stores the row.
+template <int L, bool FIRST>
+__device__ __forceinline__ void finish_row(Running r, const Running &old, int g, int li, float *out_row, float *state_row) {
+#pragma unroll
+    for (int off = L; off < 64; off <<= 1) {
+        Running o;
+        o.m = __shfl_xor(r.m, off); o.l = __shfl_xor(r.l, off);
+        o.acc = make_float4(__shfl_xor(r.acc.x, off), __shfl_xor(r.acc.y, off), __shfl_xor(r.acc.z, off), __shfl_xor(r.acc.w, off));
+        running_merge(r, o);
+    }
+    if (g != 0) return;
+    if (!FIRST) running_merge(r, old);
+    *reinterpret_cast<float4 *>(out_row) = r.acc;
+    if (li == 0) { state_row[0] = r.m; state_row[1] = r.l; }
+}
+
+// L lanes x 128 bits cover one head.  FIRST: the first partition's pass writes every row's state; later
+// passes merge into it and skip rows without elements in their partition.
+template <int L, bool FIRST>
+__global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs a) {
+    constexpr int G = 64 / L, D = 4 * L;
+    __shared__ __align__(16) int32_t s_col[kWavesPerBlock][fg::kItemEdges + kPad];
+    __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int head = a.head_base + (int)(blockIdx.x % (unsigned)a.n_heads);
+    const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_heads) * kWavesPerBlock + wave;
+    if (item_id >= a.n_items) return;
+    const Item it = a.items[item_id];
+    const int g = lane / L, li = lane % L;
+    const int f_lo = head * D + li * 4;
+    const uint32_t lane_bytes = a.kv_tile_bytes ? (uint32_t)head * a.kv_tile_bytes + (uint32_t)li * 16u : (uint32_t)f_lo * 4u;
+    const int64_t F = a.F;
+    int32_t *cols = s_col[wave];
+
+    auto stage = [&](int64_t base, int n) {
+        int32_t c[4];
+        fg::load_four(a.indices + base, n, lane, 1, c);
+        *reinterpret_cast<int4 *>(cols + 4 * lane) = make_int4((int)((uint32_t)c[0] * a.kv_row_bytes), (int)((uint32_t)c[1] * a.kv_row_bytes),
+                                                               (int)((uint32_t)c[2] * a.kv_row_bytes), (int)((uint32_t)c[3] * a.kv_row_bytes));
+        if (lane < kPad) cols[fg::kItemEdges + lane] = (int)((uint32_t)c[3] * a.kv_row_bytes);
+    };
+    auto out_row = [&](int64_t row) { return a.out + row * F + f_lo; };
+    auto state_row = [&](int64_t row) { return a.state + (row * a.H + head) * 2; };
+
+    if (it.info < -1) {
+        // several whole rows, at most 256 elements: staged once
+        const int nrows = -it.info;
+        // The rows of Q (and, in later passes, the rows' earlier sums) are read once here, one word per row
+        // and 128 bytes, while the column ids are on their way: loads return in order, so a row fetched
+        // from memory when it is needed would hold up every gather behind it.
+        float touched = 0.f;
+        constexpr int kLines = (D * 4 + 127) / 128;
+        static_assert(fg::kItemRows * kLines <= 128, "two touches per lane cover an item's rows");
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int t = lane + 64 * i;
+            const int64_t at = (int64_t)(it.row + min(t / kLines, nrows - 1)) * F + head * D + min((t % kLines) * 32, D - 1);
+            touched += a.q[at];
+            if (!FIRST) touched += a.out[at];
+        }
+        if (it.len > 0) stage(it.start, it.len);
+        s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        wave_lds_sync();
+        asm volatile("" ::"v"(touched));      // keeps the loads
+        int b = 0;
+        for (int r = 0; r < nrows; ++r) {
+            const int e = __builtin_amdgcn_readfirstlane(s_end[wave][r]);
+            if (e > b || FIRST) {
+                const float4 q = *reinterpret_cast<const float4 *>(a.q + (int64_t)(it.row + r) * F + f_lo);
+                const Running old = load_state<FIRST>(out_row(it.row + r), state_row(it.row + r));
+                Running run = running_empty();
+                walk<L>(cols, b, e, g, a.k, a.v, lane_bytes, q, a.scale, run);
+                finish_row<L, FIRST>(run, old, g, li, out_row(it.row + r), state_row(it.row + r));
+            }
+            b = e;
+        }
+        return;
+    }
+    // one row of any length: 256 elements at a time
+    const float4 q = *reinterpret_cast<const float4 *>(a.q + (int64_t)it.row * F + f_lo);
+    const Running old = load_state<FIRST>(out_row(it.row), state_row(it.row));
+    Running run = running_empty();
+    for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
+        const int n = min(fg::kItemEdges, it.len - base);
+        wave_lds_sync();
+        stage((int64_t)it.start + base, n);
+        wave_lds_sync();
+        walk<L>(cols, 0, n, g, a.k, a.v, lane_bytes, q, a.scale, run);
+    }
+    if (it.len > 0 || FIRST) finish_row<L, FIRST>(run, old, g, li, out_row(it.row), state_row(it.row));
+}
+
+// out[v, h, :] /= state[v, h].sum (rows without edges: 0).
+__global__ __launch_bounds__(256) void attention_finish_kernel(float4 *out, const float *state, uint32_t n_words,
+                                                               uint32_t row_words, uint32_t head_words, int H) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= n_words) return;
+    const uint32_t r = i / row_words, h = (i - r * row_words) / head_words;
+    const float l = state[((uint64_t)r * H + h) * 2 + 1];
+    float4 o = out[i];
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    o.x *= inv; o.y *= inv; o.z *= inv; o.w *= inv;
+    out[i] = l > 0.f ? o : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+template <int L>
+void launch(bool first, dim3 grid, hipStream_t st, const AttnArgs &a) {
+    if (first) hipLaunchKernelGGL((attention_items_kernel<L, true>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((attention_items_kernel<L, false>), grid, dim3(kBlock), 0, st, a);
+}
+
+}  // namespace
+
+extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
+                                      const float *q_dev, const float *k_dev, const float *v_dev, float *out_dev,
+                                      int heads, int head_len, float scale, void *stream) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
+    if (heads < 1 || !(head_len == 16 || head_len == 32 || head_len == 64))
+        return fail(FG_ERR_SHAPE, "attention takes heads of 16, 32 or 64 floats, got %d heads of %d", heads, head_len);
+    if (pl->n_fixups > 0)
+        return fail(FG_ERR_ARG, "attention needs a plan without split rows (fg_plan_opts.split_threshold = INT32_MAX)");
+    if (pl->n_dst == 0) return FG_OK;
+    if (!pos_dev || !q_dev || !out_dev || (pl->nnz > 0 && (!idx_dev || !k_dev || !v_dev)))
+        return fail(FG_ERR_ARG, "null device pointer");
+    if ((((uintptr_t)q_dev | (uintptr_t)k_dev | (uintptr_t)v_dev | (uintptr_t)out_dev) & 15) != 0)
+        return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
+    const int F = heads * head_len;
+    if ((uint64_t)pl->n_src * (uint64_t)F * 4u >= (1ull << 32) || (uint64_t)pl->n_dst * (uint64_t)F >= (1ull << 32))
+        return fail(FG_ERR_SHAPE, "attention operands of 4 GiB and more are not supported");
+    int rc = fg::ensure_scratch(pl, (size_t)pl->n_dst * heads * 2);
+    if (rc != FG_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const int P = pl->num_col_partitions;
+    const int64_t width = (pl->n_src + P - 1) / P;
+    // K and V head by head, as the SpMM kernels gather X tile by tile
+    const bool tiled = pl->nnz > 0 && fg::wants_tile_major(pl, heads, (uint64_t)pl->n_src * (uint64_t)F * 4u);
+    const float *k = k_dev, *v = v_dev;
+    if (tiled) {
+        if ((rc = fg::make_tile_major(pl, k_dev, pl->n_src, F, head_len, stream, 0, 2)) != FG_OK) return rc;
+        if ((rc = fg::make_tile_major(pl, v_dev, pl->n_src, F, head_len, stream, 1, 2)) != FG_OK) return rc;
+        k = pl->tiled_dev; v = pl->tiled_dev + (size_t)pl->n_src * F;
+    }
+    const int row_floats = tiled ? head_len : F;
+    for (int p = 0; p < P; ++p) {
+        const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
+        if (i1 == i0) continue;
+        AttnArgs a;
+        a.items = pl->items_dev + i0; a.n_items = i1 - i0;
+        a.pos = pos_dev + (int64_t)p * (pl->n_dst + 1);
+        a.indices = idx_dev; a.q = q_dev;
+        a.k = k + (int64_t)p * width * row_floats; a.v = v + (int64_t)p * width * row_floats;
+        a.kv_row_bytes = (uint32_t)row_floats * 4u;
+        a.kv_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * head_len * 4u) : 0u;
+        a.out = out_dev; a.state = pl->partial_dev; a.F = F; a.H = heads; a.scale = scale;
+        const int per_launch = (heads > 8 && heads % 8 == 0) ? 8 : heads;
+        for (int hb = 0; hb < heads; hb += per_launch) {
+            a.n_heads = per_launch; a.head_base = hb;
+            const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
+            if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
+            const dim3 grid((unsigned)blocks);
+            if (head_len == 64) launch<16>(p == 0, grid, st, a);
+            else if (head_len == 32) launch<8>(p == 0, grid, st, a);
+            else launch<4>(p == 0, grid, st, a);
+        }
+    }
+    const uint32_t n_words = (uint32_t)((uint64_t)pl->n_dst * F / 4);
+    hipLaunchKernelGGL(attention_finish_kernel, dim3((n_words + 255u) / 256u), dim3(256), 0, st,
+                       reinterpret_cast<float4 *>(out_dev), pl->partial_dev, n_words, (uint32_t)(F / 4),
+                       (uint32_t)(head_len / 4), heads);
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
+}

@@ -80,7 +80,12 @@ bool wants_tile_major(const fg_spmm_plan *plan, int n_tiles, uint64_t x_bytes);
 // plan->tiled_dev[(t * n_rows + r) * tile + i] = x[r * F + t * tile + i] for the F / tile tiles of
 // an [n_rows, F] matrix (F and tile multiples of 4, x 16-byte aligned, fewer than 2^32 floats),
 // on `stream`.  The buffer is grown on demand and never shrunk.
-int make_tile_major(const fg_spmm_plan *plan, const float *x, int64_t n_rows, int F, int tile, void *stream);
+// With n_slots > 1 the buffer holds that many copies of this size one after the other and the call fills
+// copy `slot` (fill slot 0 first: growing the buffer discards what it held).
+int make_tile_major(const fg_spmm_plan *plan, const float *x, int64_t n_rows, int F, int tile, void *stream,
+                    int slot = 0, int n_slots = 1);
+// Makes plan->partial_dev hold at least `floats` floats (grown on demand, never shrunk).
+int ensure_scratch(const fg_spmm_plan *plan, size_t floats);
 // FG_OK when the calling thread's current device is the one the plan was created on.
 int check_device(const fg_spmm_plan *plan);
 }  // namespace fg

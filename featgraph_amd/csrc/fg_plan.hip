@@ -153,20 +153,21 @@ bool wants_tile_major(const fg_spmm_plan *pl, int n_tiles, uint64_t x_bytes) {
     // on a 23,296-node graph (47 MB, mostly cache-resident) the copy only costs its own time.
     return n_tiles >= 4 && x_bytes >= (64ull << 20);
 }
-int make_tile_major(const fg_spmm_plan *pl, const float *x, int64_t n_rows, int F, int tile, void *stream) {
+int make_tile_major(const fg_spmm_plan *pl, const float *x, int64_t n_rows, int F, int tile, void *stream, int slot, int n_slots) {
     const uint64_t floats = (uint64_t)n_rows * (uint64_t)F;
+    if (slot < 0 || slot >= n_slots) return fail(FG_ERR_ARG, "tile-major copy: slot %d of %d", slot, n_slots);
     if (F % 4 != 0 || tile % 4 != 0 || F % tile != 0 || floats >= (1ull << 32) || ((uintptr_t)x & 15) != 0)
         return fail(FG_ERR_SHAPE, "tile-major copy of a %lld x %d matrix in tiles of %d floats", (long long)n_rows, F, tile);
-    if (floats > pl->tiled_floats) {
+    if (floats * (uint64_t)n_slots > pl->tiled_floats) {
         if (pl->tiled_dev) FG_HIP_TRY(hipFree(pl->tiled_dev));
         pl->tiled_dev = nullptr; pl->tiled_floats = 0;
-        FG_HIP_TRY(hipMalloc((void **)&pl->tiled_dev, floats * sizeof(float)));
-        pl->tiled_floats = floats;
+        FG_HIP_TRY(hipMalloc((void **)&pl->tiled_dev, floats * n_slots * sizeof(float)));
+        pl->tiled_floats = floats * n_slots;
     }
     const uint32_t n_words = (uint32_t)(floats / 4);
     if (n_words == 0) return FG_OK;
     hipLaunchKernelGGL(tile_major_kernel, dim3((n_words + 255u) / 256u), dim3(256), 0, (hipStream_t)stream,
-                       reinterpret_cast<const float4 *>(x), reinterpret_cast<float4 *>(pl->tiled_dev),
+                       reinterpret_cast<const float4 *>(x), reinterpret_cast<float4 *>(pl->tiled_dev + floats * slot),
                        (uint32_t)n_rows, (uint32_t)(F / 4), (uint32_t)(tile / 4), n_words);
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;
@@ -178,14 +179,16 @@ int check_device(const fg_spmm_plan *pl) {
         return fail(FG_ERR_ARG, "the plan lives on device %d but the current device is %d", pl->device, dev);
     return FG_OK;
 }
-int ensure_partial(const fg_spmm_plan *pl, size_t floats_per_piece) {
-    const size_t need = (size_t)pl->max_slots_in_partition * floats_per_piece;
+int ensure_scratch(const fg_spmm_plan *pl, size_t need) {
     if (need <= pl->partial_floats) return FG_OK;
     if (pl->partial_dev) FG_HIP_TRY(hipFree(pl->partial_dev));
     pl->partial_dev = nullptr; pl->partial_floats = 0;
     FG_HIP_TRY(hipMalloc((void **)&pl->partial_dev, need * sizeof(float)));
     pl->partial_floats = need;
     return FG_OK;
+}
+int ensure_partial(const fg_spmm_plan *pl, size_t floats_per_piece) {
+    return ensure_scratch(pl, (size_t)pl->max_slots_in_partition * floats_per_piece);
 }
 // Declared in fg_spmm.hip: text of the launch the SpMM entry points would use.
 std::string spmm_launch_text(const fg_spmm_plan *plan, int F, int num_feat_partitions);

@@ -767,17 +767,6 @@ extern "C" int fg_sddmm_csr_f32(const fg_spmm_plan *plan, const int32_t *indptr_
                      out_dev, H, D, stream);
 }
 
-namespace {
-int ensure_floats(const fg_spmm_plan *pl, size_t need) {
-    if (need <= pl->partial_floats) return FG_OK;
-    if (pl->partial_dev) FG_HIP_TRY(hipFree(pl->partial_dev));
-    pl->partial_dev = nullptr; pl->partial_floats = 0;
-    FG_HIP_TRY(hipMalloc((void **)&pl->partial_dev, need * sizeof(float)));
-    pl->partial_floats = need;
-    return FG_OK;
-}
-}  // namespace
-
 extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_dev, const int32_t *s1_idx_dev,
                                 const int32_t *edge_pos_dev, const float *src_dev, const float *dst_dev,
                                 float *out_dev, int H, int D, int num_feat_partitions, void *stream) {
@@ -826,11 +815,11 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
     const bool staged = !tile_sum && hpt == 1 && H >= 4 && T > 1;
     if (tile_sum) {
         const int64_t stride = (pl->nnz + 3) & ~(int64_t)3;
-        int rc = ensure_floats(pl, (size_t)T * (size_t)stride);
+        int rc = fg::ensure_scratch(pl, (size_t)T * (size_t)stride);
         if (rc != FG_OK) return rc;
         a.out = pl->partial_dev; a.out_edge_stride = 1; a.out_tile_stride = stride;
     } else if (staged) {
-        int rc = ensure_floats(pl, (size_t)H * (size_t)pl->nnz);
+        int rc = fg::ensure_scratch(pl, (size_t)H * (size_t)pl->nnz);
         if (rc != FG_OK) return rc;
         a.out = pl->partial_dev; a.out_edge_stride = hpt; a.out_tile_stride = pl->nnz * hpt;
     } else {

@@ -3,3 +3,4 @@ from .sddmm import VanillaSDDMMhip, VanillaSDDMMx86, VanillaSDDMMcuda, MultiHead
 from .gspmm import GSpMMhip
 from .common import placeholder
 from .softmax import EdgeSoftmaxhip, EdgeSoftmaxSpMMhip
+from .attention import GraphAttentionhip

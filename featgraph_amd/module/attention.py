@@ -1,0 +1,130 @@
+"""Dot-product attention over a graph's edges in one operator: multi-head SDDMM, edge softmax and per-head
+weighted SpMM without the [nnz, H] scores ever being stored.  The reference has no such operator; the
+class follows the build()/run() conventions of its modules (python/featgraph/module/spmm.py:81-161)."""
+import ctypes
+
+import numpy as np
+import torch
+
+from .. import _lib
+from .. import tuning
+from ..util import util_convert_csr_to_dds
+from . import common
+
+_INT32_MAX = 2 ** 31 - 1
+
+
+class GraphAttentionhip(object):
+    """out[v, h, :] = sum over the edges e into v of softmax_v(scale * <K[col e, h, :], Q[v, h, :]>) * V[col e, h, :]
+
+    Q is (num_rows, H, D), K and V are (num_cols, H, D), D in {16, 32, 64}; rows without edges give 0.
+    compute_args: 'scale' (default 1 / sqrt(D)).  schedule_args: 'num_src_partitions': 'auto' (default: chosen
+    for the L2 size, as for SpMM) | int | None (plain CSR).
+    Equal, within rounding, to MultiHeadSDDMMhip -> EdgeSoftmaxhip -> GSpMMhip with per-head weights.
+    """
+
+    def __init__(self, adj_scipy):
+        csr = adj_scipy.tocsr() if adj_scipy.format != 'csr' else adj_scipy
+        self._num_rows, self._num_cols = csr.shape
+        self._target = 'rocm'
+        self._ctx = common.device()
+        self._indptr = np.ascontiguousarray(csr.indptr, dtype=np.int32)
+        self._indices = np.ascontiguousarray(csr.indices, dtype=np.int32)
+        _lib.check(_lib.lib().fg_check_csr_host(self._num_rows, self._num_cols, _lib.host_ptr(self._indptr),
+                                                _lib.host_ptr(self._indices)))
+        self._csr = csr
+        self._layouts = {}
+        self._placeholders = None
+        self.out_tvm = None
+
+    def _layout(self, P):
+        """Device arrays and a plan without split rows for P source-column partitions (built once per P)."""
+        if P in self._layouts:
+            return self._layouts[P]
+        if P > 1:
+            pos, idx, _ = util_convert_csr_to_dds(self._csr, P)
+        else:
+            pos, idx = self._indptr, self._indices
+        lay = {'P': P, 'pos': common.to_device_i32(pos, self._ctx), 'idx': common.to_device_i32(idx, self._ctx),
+               'plan': ctypes.c_void_p()}
+        base = _lib.plan_opts
+        opts = _lib.FgPlanOpts(split_threshold=_INT32_MAX, item_edges=base.item_edges if base is not None else 0,
+                               wide_offsets=0, tile_major=base.tile_major if base is not None else 0)
+        with torch.cuda.device(self._ctx):
+            _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(np.ascontiguousarray(pos, dtype=np.int32)),
+                                                      self._num_rows, self._num_cols, P, ctypes.byref(opts),
+                                                      ctypes.byref(lay['plan'])))
+        self._layouts[P] = lay
+        return lay
+
+    def __del__(self):
+        for lay in getattr(self, "_layouts", {}).values():
+            plan = lay.get('plan')
+            if plan is not None and plan.value:
+                try:
+                    _lib.lib().fg_spmm_plan_destroy(plan)
+                except Exception:
+                    pass
+                lay['plan'] = None
+
+    def build(self, input_placeholders, compute_args=None, schedule_args=None):
+        """input_placeholders: [Q (num_rows, H, D), K (num_cols, H, D), V (num_cols, H, D)]."""
+        compute_args = common.take_args(compute_args or {}, ('scale',), "compute_func")
+        schedule_args = common.take_args(schedule_args or {}, ('num_src_partitions',), "schedule_func")
+        if len(input_placeholders) != 3:
+            raise ValueError("attention takes three inputs (Q, K, V), got %d" % len(input_placeholders))
+        q_ph, k_ph, v_ph = input_placeholders
+        if len(q_ph.shape) != 3 or q_ph.shape[0] != self._num_rows:
+            raise ValueError("Q must be (num_rows=%d, H, D), got %s" % (self._num_rows, q_ph.shape))
+        heads, head_len = int(q_ph.shape[1]), int(q_ph.shape[2])
+        for name, ph in (("K", k_ph), ("V", v_ph)):
+            if tuple(ph.shape) != (self._num_cols, heads, head_len):
+                raise ValueError("%s must be (num_cols=%d, %d, %d), got %s" % (name, self._num_cols, heads, head_len, ph.shape))
+        if head_len not in (16, 32, 64):
+            raise ValueError("heads of 16, 32 or 64 floats, got %d" % head_len)
+        src_parts = schedule_args.get('num_src_partitions', 'auto')
+        if src_parts is None:
+            P = 1
+        elif src_parts == 'auto':
+            # one head per XCD, and that XCD's L2 holds the head's slices of both K and V
+            P = tuning._partitions(self._num_cols, 2 * 4 * head_len, self._indices.shape[0], self._num_rows,
+                                   tuning.SPMM_SLICE_BYTES, min_segment=24)
+        else:
+            P = int(src_parts)
+            if P < 1:
+                raise ValueError("num_src_partitions must be >= 1")
+        self._heads, self._head_len = heads, head_len
+        self._scale = float(compute_args.get('scale', 1.0 / np.sqrt(head_len)))
+        self._active = self._layout(P)
+        self._placeholders = [q_ph, k_ph, v_ph]
+        self.out_tvm = torch.zeros((self._num_rows, heads, head_len), dtype=torch.float32, device=self._ctx)
+
+    def _launch(self, q, k, v):
+        lay = self._active
+        _lib.check(_lib.lib().fg_graph_attention_f32(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']),
+                                                     _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v),
+                                                     _lib.dev_ptr(self.out_tvm), self._heads, self._head_len,
+                                                     ctypes.c_float(self._scale), common.stream_ptr()))
+
+    def run(self, input_tvm_ndarrays):
+        """[Q, K, V] -> self.out_tvm (the same tensor on every call); nothing is synchronised."""
+        if self._placeholders is None:
+            raise RuntimeError("call build() before run()")
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        self._launch(*input_tvm_ndarrays)
+        return self.out_tvm
+
+    def measure_average_time(self, input_tvm_ndarrays, num_runs):
+        if self._placeholders is None:
+            raise RuntimeError("call build() before measure_average_time()")
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        q, k, v = input_tvm_ndarrays
+        return common.timed_mean_seconds(lambda: self._launch(q, k, v), num_runs)
+
+    @property
+    def ctx(self):
+        return self._ctx
+
+    @property
+    def target(self):
+        return self._target

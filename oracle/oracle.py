@@ -294,3 +294,21 @@ def edge_softmax_f64(indptr, x):
         if e > b:
             out[b:e] = scipy.special.softmax(x64[b:e], axis=0)
     return out
+
+
+def graph_attention_f64(indptr, indices, q, k, v, scale):
+    """out[r, h, :] = sum_e softmax_e(scale * <k[col e, h, :], q[r, h, :]>) * v[col e, h, :] in float64:
+    the composition of sddmm_multihead_f64, edge_softmax_f64 and a per-head weighted sum, row by row.
+    No attention operator exists in the reference (parity unpinned); pinned by that composition."""
+    q64, k64, v64 = (np.asarray(a, dtype=np.float64) for a in (q, k, v))
+    out = np.zeros_like(q64)
+    import scipy.special
+    for r in range(len(indptr) - 1):
+        b, e = int(indptr[r]), int(indptr[r + 1])
+        if e == b:
+            continue
+        cols = indices[b:e]
+        s = scale * np.einsum("ehd,hd->eh", k64[cols], q64[r])
+        a = scipy.special.softmax(s, axis=0)
+        out[r] = np.einsum("eh,ehd->hd", a, v64[cols])
+    return out

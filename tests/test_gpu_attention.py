@@ -1,0 +1,123 @@
+"""Graph attention in one operator (multi-head SDDMM + edge softmax + per-head weighted SpMM without stored
+scores) against the float64 composition of the three, and against the three GPU operators chained."""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph(rng, n_rows=300, n_cols=700, long_len=650, density=0.03):
+    a = sp.random(n_rows, n_cols, density=density, format="csr", random_state=rng,
+                  data_rvs=lambda k: np.ones(k)).astype("float32").tolil()
+    a[[0, n_rows // 2], :] = 0                                   # rows without edges
+    a[7, rng.choice(n_cols, size=long_len, replace=False)] = 1   # a long row (several staging rounds)
+    a = a.tocsr().astype("float32"); a.eliminate_zeros(); a.sort_indices()
+    return a
+
+
+def _run(adj, q, k, v, P, scale=None):
+    import torch
+    from featgraph_amd.module import GraphAttentionhip, placeholder
+    m = GraphAttentionhip(adj)
+    m.build([placeholder(q.shape), placeholder(k.shape), placeholder(v.shape)],
+            {} if scale is None else {'scale': scale}, {'num_src_partitions': P})
+    m.out_tvm.fill_(float("nan"))
+    return m.run([torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()]).cpu().numpy().copy()
+
+
+@pytest.mark.parametrize("H,D", [(1, 64), (4, 64), (8, 64), (16, 64), (4, 32), (8, 16), (3, 64), (10, 32)])
+@pytest.mark.parametrize("P", [None, 2, 5])
+def test_against_float64_composition(oracle, H, D, P):
+    rng = np.random.default_rng(H * 100 + D + (P or 0))
+    adj = _graph(rng)
+    q = rng.standard_normal((adj.shape[0], H, D)).astype("float32")
+    k = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    v = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    out = _run(adj, q, k, v, P)
+    ref = oracle.graph_attention_f64(adj.indptr, adj.indices, q, k, v, 1.0 / np.sqrt(D))
+    assert np.isfinite(out).all()
+    assert (out[np.diff(adj.indptr) == 0] == 0).all()
+    np.testing.assert_allclose(out, ref, rtol=1e-4, atol=2e-5)
+
+
+def test_large_scores_do_not_overflow(oracle):
+    """Scores in the thousands: the running maximum keeps every exponential at or below 1."""
+    rng = np.random.default_rng(11)
+    adj = _graph(rng)
+    H, D = 4, 64
+    q = (30 * rng.standard_normal((adj.shape[0], H, D))).astype("float32")
+    k = (30 * rng.standard_normal((adj.shape[1], H, D))).astype("float32")
+    v = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    out = _run(adj, q, k, v, 3, scale=1.0)
+    ref = oracle.graph_attention_f64(adj.indptr, adj.indices, q, k, v, 1.0)
+    assert np.isfinite(out).all()
+    np.testing.assert_allclose(out, ref, rtol=1e-3, atol=1e-4)
+
+
+def test_uniform_scores_give_the_mean(oracle):
+    """K = 0: every edge weighs the same and the result is the mean of the neighbours' V."""
+    rng = np.random.default_rng(12)
+    adj = _graph(rng)
+    H, D = 2, 32
+    q = rng.standard_normal((adj.shape[0], H, D)).astype("float32")
+    k = np.zeros((adj.shape[1], H, D), np.float32)
+    v = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    out = _run(adj, q, k, v, 2)
+    deg = np.diff(adj.indptr)
+    mean = np.asarray(adj.astype(np.float64).dot(v.reshape(v.shape[0], -1).astype(np.float64)))
+    mean[deg > 0] /= deg[deg > 0, None]
+    np.testing.assert_allclose(out.reshape(mean.shape), mean, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("tile_major", [1, 2])
+def test_equals_the_three_operators_chained(monkeypatch, tile_major):
+    import torch
+    from featgraph_amd import _lib
+    from featgraph_amd.autograd import Graph
+    monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(tile_major=tile_major))
+    rng = np.random.default_rng(13)
+    adj = _graph(rng, 500, 900, 800, 0.05)
+    H, D = 8, 64
+    q = rng.standard_normal((adj.shape[0], H, D)).astype("float32")
+    k = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    v = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    out = _run(adj, q, k, v, 4)
+    g = Graph(adj)
+    s = g.sddmm(torch.from_numpy(k).cuda(), torch.from_numpy(q).cuda()) * (1.0 / np.sqrt(D))
+    chained = g.spmm(torch.from_numpy(v).cuda(), g.edge_softmax(s)).cpu().numpy()
+    np.testing.assert_allclose(out, chained, rtol=2e-4, atol=5e-5)
+
+
+def test_repeatable_and_shapes_are_checked():
+    import torch
+    from featgraph_amd.module import GraphAttentionhip, placeholder
+    rng = np.random.default_rng(14)
+    adj = _graph(rng)
+    H, D = 4, 64
+    q = rng.standard_normal((adj.shape[0], H, D)).astype("float32")
+    k = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    v = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    a = _run(adj, q, k, v, 3)
+    b = _run(adj, q, k, v, 3)
+    assert np.array_equal(a, b)
+    m = GraphAttentionhip(adj)
+    with pytest.raises(ValueError):
+        m.build([placeholder((adj.shape[0], H, 48)), placeholder((adj.shape[1], H, 48)), placeholder((adj.shape[1], H, 48))])
+    with pytest.raises(ValueError):
+        m.build([placeholder(q.shape), placeholder(k.shape), placeholder((adj.shape[1], H, 32))])
+    with pytest.raises(RuntimeError):
+        GraphAttentionhip(adj).run([torch.from_numpy(q).cuda()] * 3)
+
+
+def test_empty_graph_and_empty_partition():
+    adj = sp.csr_matrix((50, 40), dtype=np.float32)
+    rng = np.random.default_rng(15)
+    q = rng.standard_normal((50, 2, 64)).astype("float32")
+    k = rng.standard_normal((40, 2, 64)).astype("float32")
+    out = _run(adj, q, k, k, 2)
+    assert (out == 0).all()
+    # all edges in the last partition's columns
+    adj = sp.csr_matrix((np.ones(3, np.float32), (np.array([1, 1, 4]), np.array([38, 39, 39]))), shape=(50, 40))
+    out = _run(adj, q, k, k, 4)
+    assert np.isfinite(out).all() and (out[0] == 0).all() and np.allclose(out[4], k[39], atol=1e-6)
