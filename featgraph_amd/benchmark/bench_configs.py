@@ -18,7 +18,7 @@ import torch
 from .. import synthetic
 from ..module import common
 from ..module import (VanillaSpMMhip, VanillaSDDMMhip, MultiHeadSDDMMhip, GSpMMhip, EdgeSoftmaxhip,
-                      EdgeSoftmaxSpMMhip, placeholder)
+                      EdgeSoftmaxSpMMhip, GraphAttentionhip, placeholder)
 
 HBM_PEAK_GBS = 8000.0
 
@@ -77,7 +77,18 @@ def run_attention_steps(name, adj, softmax_heads, head_shapes):
         _line(name, "edge_softmax_spmm_fused", {"heads": H, "head_len": D, "partitions": f._agg._active['P'],
                                                 "tiles": f._agg._num_feat_partitions}, t, nnz, H * D,
               4 * (n + 1) + 4 * nnz + 4 * nnz * H + 8 * n * H * D)
-        del f, x, w, sc
+        del f, w, sc
+        # scores, softmax and aggregation in one operator (no [nnz, H] array at all)
+        gen.manual_seed(5)
+        q = torch.randn((n, H, D), generator=gen, device="cuda")
+        k = torch.randn((n, H, D), generator=gen, device="cuda")
+        g = GraphAttentionhip(adj)
+        g.build([placeholder((n, H, D))] * 3, {}, {})
+        t = g.measure_average_time([q, k, x], 5)
+        # byte model: indices once, Q, K, V and the output once; flops: two gathered operands per edge
+        _line(name, "graph_attention", {"heads": H, "head_len": D, "partitions": g._active['P']}, t, nnz, 2 * H * D,
+              4 * (n + 1) + 4 * nnz + 16 * n * H * D)
+        del g, q, k, x
 
 
 def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):

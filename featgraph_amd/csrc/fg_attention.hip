@@ -143,6 +143,41 @@ __device__ __forceinline__ void walk(const int32_t *cols, int b, int e, int g, c
     else walk_batch<L, 4, false>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
 }
 
+// kU consecutive staged elements j .. j + kU - 1 of this lane group's own row (those below e count; the
+// slots behind them hold later rows' elements or the padding: loadable, given no weight).
+template <int L>
+__device__ __forceinline__ void own_batch(const int32_t *cols, int j, int e, const float *k, const float *v,
+                                          uint32_t lane_bytes, const float4 &q, float scale, Running &r) {
+    int c[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) c[u] = cols[j + u];
+    float4 kk[kU], vv[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+        kk[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(k) + ((uint32_t)c[u] + lane_bytes));
+        vv[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(v) + ((uint32_t)c[u] + lane_bytes));
+    }
+    float s[kU];
+    float m = r.m;
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+        const float d = kk[u].x * q.x + kk[u].y * q.y + kk[u].z * q.z + kk[u].w * q.w;
+        const float t = group_sum<L>(d) * scale;
+        s[u] = (j + u < e) ? t : -INFINITY;
+        m = fmaxf(m, s[u]);
+    }
+    const float f = __expf(r.m - m);          // j < e: at least one finite score, so m is finite
+    r.acc.x *= f; r.acc.y *= f; r.acc.z *= f; r.acc.w *= f;
+    r.l *= f;
+    r.m = m;
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+        const float p = __expf(s[u] - m);
+        r.l += p;
+        r.acc.x += p * vv[u].x; r.acc.y += p * vv[u].y; r.acc.z += p * vv[u].z; r.acc.w += p * vv[u].w;
+    }
+}
+
 // What the earlier partitions left for a row (read before the row's gathers are issued).
 template <bool FIRST>
 __device__ __forceinline__ Running load_state(const float *out_row, const float *state_row) {
@@ -178,6 +213,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
     constexpr int G = 64 / L, D = 4 * L;
     __shared__ __align__(16) int32_t s_col[kWavesPerBlock][fg::kItemEdges + kPad];
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
+    __shared__ int32_t s_next[kWavesPerBlock];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int head = a.head_base + (int)(blockIdx.x % (unsigned)a.n_heads);
@@ -218,8 +254,49 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
         }
         if (it.len > 0) stage(it.start, it.len);
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        if (lane == 0) s_next[wave] = 0;
         wave_lds_sync();
         asm volatile("" ::"v"(touched));      // keeps the loads
+        if (nrows >= 2 * G && it.len <= nrows * 2 * kU) {
+            // Many rows of a few elements: every lane group takes rows of its own (next free row from a
+            // counter in LDS), walks the row's elements kU at a time and stores the row itself, so G rows are
+            // in flight per wavefront and nothing crosses lane groups.  (Rows of 30 elements are faster
+            // shared: 26.7 against 27.6 ms at H=8, D=64 on the 232,965-node graph with 16 partitions.)
+            int r = -1, j = 0, e = 0;
+            bool done = false, live = false;
+            float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
+            Running run = running_empty(), old = running_empty();
+            for (;;) {
+                if (!done && j >= e) {
+                    if (live) {                      // the row this group just finished
+                        if (!FIRST) running_merge(run, old);
+                        *reinterpret_cast<float4 *>(out_row(it.row + r)) = run.acc;
+                        if (li == 0) { float *st = state_row(it.row + r); st[0] = run.m; st[1] = run.l; }
+                    }
+                    int rn = 0;
+                    if (li == 0) rn = atomicAdd(&s_next[wave], 1);
+                    r = __shfl(rn, g * L);
+                    if (r >= nrows) {
+                        done = true;
+                    } else {
+                        j = r ? s_end[wave][r - 1] : 0;
+                        e = s_end[wave][r];
+                        live = FIRST || e > j;
+                        if (live) {
+                            q = *reinterpret_cast<const float4 *>(a.q + (int64_t)(it.row + r) * F + f_lo);
+                            old = load_state<FIRST>(out_row(it.row + r), state_row(it.row + r));
+                            run = running_empty();
+                        }
+                    }
+                }
+                if (__all(done)) break;
+                if (!done && j < e) {
+                    own_batch<L>(cols, j, e, a.k, a.v, lane_bytes, q, a.scale, run);
+                    j += kU;
+                }
+            }
+            return;
+        }
         int b = 0;
         for (int r = 0; r < nrows; ++r) {
             const int e = __builtin_amdgcn_readfirstlane(s_end[wave][r]);
