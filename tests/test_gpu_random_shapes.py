@@ -117,3 +117,30 @@ def test_random_softmax_and_aggregation(oracle, seed):
         ref_out, ref_arg = oracle.gspmm_arg(adj.indptr, adj.indices, adj.data, x, red)
         assert np.array_equal(out, ref_out), what
         assert np.array_equal(gm.arg_tvm.cpu().numpy(), ref_arg), what
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_attention(oracle, monkeypatch, seed):
+    import torch
+    from featgraph_amd import _lib
+    from featgraph_amd.module import GraphAttentionhip, placeholder
+    if seed % 2:
+        monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(tile_major=1))
+    rng = np.random.default_rng(4000 + seed)
+    for case in range(10):
+        adj = _random_graph(rng)
+        H = int(rng.choice([1, 2, 3, 4, 8, 9, 16]))
+        D = int(rng.choice([16, 32, 64]))
+        P = rng.choice([None, 1, 2, 3, 7])
+        P = None if P is None else int(P)
+        q = rng.standard_normal((adj.shape[0], H, D)).astype("float32")
+        k = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+        v = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+        m = GraphAttentionhip(adj)
+        m.build([placeholder(q.shape), placeholder(k.shape), placeholder(v.shape)], {}, {'num_src_partitions': P})
+        m.out_tvm.fill_(float("nan"))
+        out = m.run([torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()]).cpu().numpy()
+        what = "seed %d case %d: %s nnz %d H=%d D=%d P=%s" % (seed, case, adj.shape, adj.nnz, H, D, P)
+        ref = oracle.graph_attention_f64(adj.indptr, adj.indices, q, k, v, 1.0 / np.sqrt(D))
+        assert np.isfinite(out).all(), what
+        np.testing.assert_allclose(out, ref, rtol=1e-4, atol=2e-5, err_msg=what)
