@@ -121,3 +121,36 @@ def test_empty_graph_and_empty_partition():
     adj = sp.csr_matrix((np.ones(3, np.float32), (np.array([1, 1, 4]), np.array([38, 39, 39]))), shape=(50, 40))
     out = _run(adj, q, k, k, 4)
     assert np.isfinite(out).all() and (out[0] == 0).all() and np.allclose(out[4], k[39], atol=1e-6)
+
+
+def test_full_size_graph(oracle):
+    """232,965 nodes / 114.77M edges, H=4, D=64 (the tile-by-tile copies of K and V are in use at this size):
+    sampled rows against float64, and K = 0 against the mean aggregation of the SpMM path."""
+    import torch
+    from featgraph_amd import synthetic
+    from featgraph_amd.module import GraphAttentionhip, GSpMMhip, placeholder
+    indptr, indices = synthetic.make_workload("powerlaw-233k")
+    n, nnz = indptr.shape[0] - 1, int(indptr[-1])
+    adj = sp.csr_matrix((np.ones(nnz, np.float32), indices, indptr), shape=(n, n))
+    H, D = 4, 64
+    gen = torch.Generator(device="cuda"); gen.manual_seed(3)
+    q, k, v = (torch.randn((n, H, D), generator=gen, device="cuda") for _ in range(3))
+    m = GraphAttentionhip(adj)
+    m.build([placeholder((n, H, D))] * 3, {}, {})
+    out = m.run([q, k, v]).cpu().numpy().copy()
+    assert np.isfinite(out).all()
+    deg = np.diff(indptr)
+    rows = np.unique(np.concatenate([[0, n - 1, int(deg.argmax()), int(deg.argmin())],
+                                     np.random.default_rng(0).integers(0, n, 60)]))
+    qh, kh, vh = q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy()
+    sub_ptr = np.concatenate([[0], np.cumsum(deg[rows])]).astype(np.int64)
+    sub_idx = np.concatenate([indices[indptr[r]:indptr[r + 1]] for r in rows])
+    ref = oracle.graph_attention_f64(sub_ptr, sub_idx, qh[rows], kh, vh, 1.0 / np.sqrt(D))
+    np.testing.assert_allclose(out[rows], ref, rtol=1e-4, atol=2e-5)
+    # uniform scores: the neighbours' mean
+    got = m.run([q, torch.zeros_like(k), v]).reshape(n, H * D).clone()
+    agg = GSpMMhip(adj)
+    agg.build([placeholder((n, H * D))], {'reduce': 'mean', 'msg': 'copy_u'}, {})
+    want = agg.run([v.reshape(n, H * D)])
+    err = (got - want).abs().max().item()
+    assert err < 2e-5, err
