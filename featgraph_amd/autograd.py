@@ -13,7 +13,8 @@ import numpy as np
 import scipy.sparse
 import torch
 
-from .module import EdgeSoftmaxhip, GSpMMhip, MultiHeadSDDMMhip, VanillaSDDMMhip, placeholder
+from .module import (EdgeSoftmaxhip, GraphAttentionhip, GSpMMhip, MultiHeadSDDMMhip, VanillaSDDMMhip,
+                     placeholder)
 
 
 class Graph(object):
@@ -115,6 +116,24 @@ class Graph(object):
             self._ones = torch.ones(self.nnz, device=device)
             self._cols = torch.from_numpy(self._csr.indices.astype(np.int64)).to(device)
         return self._inv_deg
+
+    def attention(self, q, k, v, scale=None):
+        """out[r, h, :] = sum over the edges e into r of softmax_r(scale * <k[col e, h, :], q[r, h, :]>) * v[col e, h, :];
+        q (num_rows, H, D), k and v (num_cols, H, D), scale 1 / sqrt(D) unless given.  Without gradients
+        (inference) and with D in {16, 32, 64} this is one operator that stores no scores; otherwise the
+        differentiable chain sddmm -> edge_softmax -> spmm."""
+        if scale is None:
+            scale = 1.0 / float(q.shape[-1]) ** 0.5
+        needs_grad = torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)
+        if not needs_grad and q.dim() == 3 and q.shape[-1] in (16, 32, 64):
+            key = ('attention', tuple(q.shape[1:]), float(scale))
+            if key not in self._mods:
+                m = GraphAttentionhip(self._csr)
+                m.build([placeholder(tuple(q.shape)), placeholder(tuple(k.shape)), placeholder(tuple(v.shape))],
+                        {'scale': float(scale)}, {})
+                self._mods[key] = m
+            return _fresh_run(self._mods[key], [q.contiguous(), k.contiguous(), v.contiguous()])
+        return self.spmm(v, self.edge_softmax(self.sddmm(k, q) * scale))
 
     def edge_softmax(self, scores):
         """Softmax of scores, (nnz,) or (nnz, H), over the edges of each destination row, per head."""

@@ -80,3 +80,36 @@ def test_aggregate_gradients(reduce):
     (y64 * up.double()).sum().backward()
     assert torch.allclose(y.double(), y64, rtol=1e-4, atol=1e-5)
     assert torch.allclose(x.grad.double(), x64.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_attention_with_and_without_gradients():
+    """Graph.attention: one operator under no_grad, the differentiable chain otherwise; same values, and the
+    chain's gradients match float64 torch autograd."""
+    import torch
+    from featgraph_amd.autograd import Graph
+    rng = np.random.default_rng(21)
+    adj = sp.random(120, 150, density=0.08, format="csr", random_state=rng).astype("float32")
+    adj.sort_indices()
+    g = Graph(adj)
+    H, D = 4, 32
+    q = torch.from_numpy(rng.standard_normal((120, H, D)).astype("float32")).cuda().requires_grad_()
+    k = torch.from_numpy(rng.standard_normal((150, H, D)).astype("float32")).cuda().requires_grad_()
+    v = torch.from_numpy(rng.standard_normal((150, H, D)).astype("float32")).cuda().requires_grad_()
+    with torch.no_grad():
+        fused = g.attention(q, k, v)
+    chained = g.attention(q, k, v)
+    assert chained.requires_grad and not fused.requires_grad
+    np.testing.assert_allclose(fused.cpu().numpy(), chained.detach().cpu().numpy(), rtol=2e-4, atol=2e-5)
+    chained.square().sum().backward()
+    # float64 reference on the dense masked form
+    coo = adj.tocoo()
+    mask = torch.zeros((120, 150), dtype=torch.bool); mask[coo.row, coo.col] = True
+    q64, k64, v64 = (t.detach().cpu().double().requires_grad_() for t in (q, k, v))
+    s = torch.einsum("rhd,chd->hrc", q64, k64) / D ** 0.5
+    s = s.masked_fill(~mask, float("-inf"))
+    a = torch.nan_to_num(torch.softmax(s, dim=-1), nan=0.0)
+    ref = torch.einsum("hrc,chd->rhd", a, v64)
+    np.testing.assert_allclose(chained.detach().cpu().numpy(), ref.detach().numpy(), rtol=1e-4, atol=2e-5)
+    ref.square().sum().backward()
+    for got, want in ((q.grad, q64.grad), (k.grad, k64.grad), (v.grad, v64.grad)):
+        np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=1e-3, atol=1e-4)
