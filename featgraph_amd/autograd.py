@@ -119,21 +119,24 @@ class Graph(object):
 
     def attention(self, q, k, v, scale=None):
         """out[r, h, :] = sum over the edges e into r of softmax_r(scale * <k[col e, h, :], q[r, h, :]>) * v[col e, h, :];
-        q (num_rows, H, D), k and v (num_cols, H, D), scale 1 / sqrt(D) unless given.  Without gradients
-        (inference) and with D in {16, 32, 64} this is one operator that stores no scores; otherwise the
-        differentiable chain sddmm -> edge_softmax -> spmm."""
+        q (num_rows, H, D), k and v (num_cols, H, D), scale 1 / sqrt(D) unless given.  With D in {16, 32, 64}
+        this is one operator that stores no scores, and its backward pass forms them again (two sweeps, one
+        of them over the transposed adjacency); otherwise the differentiable chain sddmm -> edge_softmax ->
+        spmm."""
         if scale is None:
             scale = 1.0 / float(q.shape[-1]) ** 0.5
-        needs_grad = torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)
-        if not needs_grad and q.dim() == 3 and q.shape[-1] in (16, 32, 64):
-            key = ('attention', tuple(q.shape[1:]), float(scale))
-            if key not in self._mods:
-                m = GraphAttentionhip(self._csr)
-                m.build([placeholder(tuple(q.shape)), placeholder(tuple(k.shape)), placeholder(tuple(v.shape))],
-                        {'scale': float(scale)}, {})
-                self._mods[key] = m
-            return _fresh_run(self._mods[key], [q.contiguous(), k.contiguous(), v.contiguous()])
+        if q.dim() == 3 and q.shape[-1] in (16, 32, 64):
+            return _Attention.apply(self, q, k, v, float(scale))
         return self.spmm(v, self.edge_softmax(self.sddmm(k, q) * scale))
+
+    def _attention_mod(self, q, k, v, scale):
+        key = ('attention', tuple(q.shape[1:]), scale)
+        if key not in self._mods:
+            m = GraphAttentionhip(self._csr)
+            m.build([placeholder(tuple(q.shape)), placeholder(tuple(k.shape)), placeholder(tuple(v.shape))],
+                    {'scale': scale}, {})
+            self._mods[key] = m
+        return self._mods[key]
 
     def edge_softmax(self, scores):
         """Softmax of scores, (nnz,) or (nnz, H), over the edges of each destination row, per head."""
@@ -177,6 +180,24 @@ class _SDDMM(torch.autograd.Function):
         dsrc = g._spmm_raw(dst, ds, transposed=True) if ctx.needs_input_grad[1] else None
         ddst = g._spmm_raw(src, ds) if ctx.needs_input_grad[2] else None
         return None, dsrc, ddst
+
+
+class _Attention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, g, q, k, v, scale):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        mod = g._attention_mod(q, k, v, scale)
+        mod.state_tvm = torch.empty_like(mod.state_tvm)        # handed to backward with the output
+        out = _fresh_run(mod, [q, k, v])
+        ctx.g, ctx.scale = g, scale
+        ctx.save_for_backward(q, k, v, out, mod.state_tvm)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, state = ctx.saved_tensors
+        dq, dk, dv = ctx.g._attention_mod(q, k, v, ctx.scale).backward(q, k, v, out, state, dout.contiguous())
+        return None, dq, dk, dv, None
 
 
 class _EdgeSoftmax(torch.autograd.Function):

@@ -1,8 +1,11 @@
-"""One attention layer, forward and backward, through the autograd layer: scores = SDDMM(K, Q) per head,
-softmax over each destination's edges, out = per-head weighted SpMM of V; the backward pass is three
-per-head SpMMs (two of them on the transposed graph), one multi-head SDDMM and the softmax gradient.
+"""One attention layer, forward and backward, through the autograd layer.
 
-    python -m featgraph_amd.benchmark.bench_attention_step [--workload powerlaw-233k] [--heads 8] [--head-len 64]
+Default: Graph.attention, one operator forward (no stored scores) and two sweeps backward (one over the
+adjacency for dQ, one over its transpose for dK and dV).  With --chain: scores = SDDMM(K, Q) per head, softmax
+over each destination's edges, out = per-head weighted SpMM of V, whose backward pass is three per-head SpMMs
+(two of them on the transposed graph), one multi-head SDDMM and the softmax gradient.
+
+    python -m featgraph_amd.benchmark.bench_attention_step [--workload powerlaw-233k] [--heads 8] [--head-len 64] [--chain]
 
 Prints one JSON line with the mean times (HIP events on the launch stream) of the steps after the first."""
 import argparse
@@ -22,6 +25,7 @@ def main():
     ap.add_argument("--heads", type=int, default=8)
     ap.add_argument("--head-len", type=int, default=64)
     ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--chain", action="store_true", help="the three operators instead of the single one")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("bench_attention_step needs a GPU")
@@ -40,9 +44,13 @@ def main():
     times = []
     for step in range(args.steps + 1):
         e = [mark()]
-        s = g.sddmm(k, q); e.append(mark())
-        a = g.edge_softmax(s * (1.0 / D ** 0.5)); e.append(mark())
-        out = g.spmm(v, a); e.append(mark())
+        if args.chain:
+            s = g.sddmm(k, q); e.append(mark())
+            a = g.edge_softmax(s * (1.0 / D ** 0.5)); e.append(mark())
+            out = g.spmm(v, a); e.append(mark())
+        else:
+            e += [e[0], e[0]]
+            out = g.attention(q, k, v); e.append(mark())
         loss = out.square().mean()
         loss.backward(); e.append(mark())
         torch.cuda.synchronize()
@@ -50,10 +58,14 @@ def main():
             times.append([e[i].elapsed_time(e[i + 1]) for i in range(4)])
         q.grad = k.grad = v.grad = None
     t = np.mean(np.array(times), axis=0)
-    print(json.dumps({"workload": args.workload, "nodes": n, "edges": nnz, "heads": H, "head_len": D,
-                      "sddmm_ms": round(float(t[0]), 3), "edge_softmax_ms": round(float(t[1]), 3),
-                      "spmm_ms": round(float(t[2]), 3), "loss_and_backward_ms": round(float(t[3]), 3),
-                      "step_ms": round(float(t.sum()), 3), "steps": args.steps}))
+    line = {"workload": args.workload, "nodes": n, "edges": nnz, "heads": H, "head_len": D,
+            "operators": "sddmm + edge_softmax + spmm" if args.chain else "attention"}
+    if args.chain:
+        line.update(sddmm_ms=round(float(t[0]), 3), edge_softmax_ms=round(float(t[1]), 3), spmm_ms=round(float(t[2]), 3))
+    else:
+        line.update(attention_ms=round(float(t[2]), 3))
+    line.update(loss_and_backward_ms=round(float(t[3]), 3), step_ms=round(float(t.sum()), 3), steps=args.steps)
+    print(json.dumps(line))
 
 
 if __name__ == "__main__":

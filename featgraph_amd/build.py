@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libfeatgraph_hip.so")
 
-SOURCES = ["fg_host.cpp", "fg_plan.hip", "fg_spmm.hip", "fg_sddmm.hip", "fg_softmax.hip", "fg_attention.hip"]
+SOURCES = ["fg_host.cpp", "fg_plan.hip", "fg_spmm.hip", "fg_sddmm.hip", "fg_softmax.hip", "fg_attention.hip", "fg_attention_bwd.hip"]
 
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 instructions.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=fast",

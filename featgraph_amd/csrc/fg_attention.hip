@@ -348,7 +348,7 @@ void launch(bool first, dim3 grid, hipStream_t st, const AttnArgs &a) {
 
 extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
                                       const float *q_dev, const float *k_dev, const float *v_dev, float *out_dev,
-                                      int heads, int head_len, float scale, void *stream) {
+                                      float *row_state_dev, int heads, int head_len, float scale, void *stream) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (int drc = fg::check_device(pl)) return drc;
     if (heads < 1 || !(head_len == 16 || head_len == 32 || head_len == 64))
@@ -363,8 +363,11 @@ extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos
     const int F = heads * head_len;
     if ((uint64_t)pl->n_src * (uint64_t)F * 4u >= (1ull << 32) || (uint64_t)pl->n_dst * (uint64_t)F >= (1ull << 32))
         return fail(FG_ERR_SHAPE, "attention operands of 4 GiB and more are not supported");
-    int rc = fg::ensure_scratch(pl, (size_t)pl->n_dst * heads * 2);
-    if (rc != FG_OK) return rc;
+    int rc = FG_OK;
+    if (!row_state_dev) {
+        if ((rc = fg::ensure_scratch(pl, (size_t)pl->n_dst * heads * 2)) != FG_OK) return rc;
+        row_state_dev = pl->partial_dev;
+    }
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
@@ -387,7 +390,7 @@ extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos
         a.k = k + (int64_t)p * width * row_floats; a.v = v + (int64_t)p * width * row_floats;
         a.kv_row_bytes = (uint32_t)row_floats * 4u;
         a.kv_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * head_len * 4u) : 0u;
-        a.out = out_dev; a.state = pl->partial_dev; a.F = F; a.H = heads; a.scale = scale;
+        a.out = out_dev; a.state = row_state_dev; a.F = F; a.H = heads; a.scale = scale;
         const int per_launch = (heads > 8 && heads % 8 == 0) ? 8 : heads;
         for (int hb = 0; hb < heads; hb += per_launch) {
             a.n_heads = per_launch; a.head_base = hb;
@@ -401,7 +404,7 @@ extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos
     }
     const uint32_t n_words = (uint32_t)((uint64_t)pl->n_dst * F / 4);
     hipLaunchKernelGGL(attention_finish_kernel, dim3((n_words + 255u) / 256u), dim3(256), 0, st,
-                       reinterpret_cast<float4 *>(out_dev), pl->partial_dev, n_words, (uint32_t)(F / 4),
+                       reinterpret_cast<float4 *>(out_dev), row_state_dev, n_words, (uint32_t)(F / 4),
                        (uint32_t)(head_len / 4), heads);
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;

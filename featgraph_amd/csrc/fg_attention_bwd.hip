@@ -1,0 +1,369 @@
+// Gradients of the graph attention operator (fg_attention.hip), without any [nnz, H] array.
+//
+// With s[e, h] = scale * <K[c, h, :], Q[r, h, :]>, a[e, h] = exp(s - m[r, h]) / l[r, h] (m, l: the row's
+// maximum and sum of exponentials, kept by the forward pass) and out[r, h, :] = sum_e a * V[c, h, :]:
+//
+//   da[e, h] = <dout[r, h, :], V[c, h, :]>
+//   ds[e, h] = a * (da - delta[r, h]),   delta[r, h] = sum_e a * da = <dout[r, h, :], out[r, h, :]>
+//   dQ[r]   += scale * ds * K[c]          (a sum over the row's edges: the forward pass's traversal)
+//   dV[c]   += a * dout[r],  dK[c] += scale * ds * Q[r]      (sums over a column's edges: the same
+//                                                            traversal of the transposed adjacency)
+//
+// Both kernels form s again from Q and K, read (m + log l, delta) per row and head, and gather two
+// operands per edge, as the forward pass does.  Not in the reference.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <type_traits>
+
+#include "fg_common.h"
+#include "fg_device.h"
+
+using fg::fail;
+using fg::Item;
+
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = 64 * kWavesPerBlock;
+constexpr int kPad = 8;
+constexpr int kU = 4;                  // elements per lane group whose gathers are issued back to back
+
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over the L (4, 8 or 16) consecutive lanes of a lane group; every lane of the group gets it.
+template <int L>
+__device__ __forceinline__ float group_sum(float v) {
+    v += dpp_move<0xB1>(v);                  // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);                  // quad_perm [2,3,0,1]
+    if (L >= 8) v += dpp_move<0x141>(v);     // row_half_mirror
+    if (L >= 16) v += dpp_move<0x140>(v);    // row_mirror
+    return v;
+}
+
+__device__ __forceinline__ float dot4(const float4 &a, const float4 &b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
+__device__ __forceinline__ void fma4(float4 &acc, float w, const float4 &x) {
+    acc.x += w * x.x; acc.y += w * x.y; acc.z += w * x.z; acc.w += w * x.w;
+}
+__device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ __forceinline__ void shfl_add(float4 &a, int off) {
+    a.x += __shfl_xor(a.x, off); a.y += __shfl_xor(a.y, off); a.z += __shfl_xor(a.z, off); a.w += __shfl_xor(a.w, off);
+}
+
+// One traversal serves both kernels.  The "own" side is the row of the traversed matrix, the "far" side is
+// what its elements point at:
+//   BY_COLUMN == false (adjacency, rows = destinations): own = (Q[r], dout[r], coef[r]), far = (K[c], V[c]);
+//     result A = dQ[r].
+//   BY_COLUMN == true (transposed adjacency, rows = sources): own = (K[c], V[c]), far = (Q[r], dout[r],
+//     coef[r]); results A = dK[c], B = dV[c].
+struct BwdArgs {
+    const Item *items;
+    int64_t n_items;
+    const int32_t *pos;
+    const int32_t *indices;   // partition-local ids of the far side
+    const float *own0, *own1; // [n_own, F]: (Q, dout) or (K, V)
+    const float *far0, *far1; // offset to the partition's first far row: (K, V) or (Q, dout)
+    uint32_t far_row_bytes, far_tile_bytes;
+    const float *coef;        // [n_dst, H, 2]: (m + log l, delta); BY_COLUMN: offset to the partition's first far row
+    float *res0, *res1;       // [n_own, F]: dQ, or dK and dV
+    int F, H;
+    int n_heads, head_base;
+    int accumulate;
+    float scale;
+};
+
+template <int L, bool BY_COLUMN, bool ACC>
+__global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArgs a) {
+    constexpr int G = 64 / L, D = 4 * L;
+    // x = far row's byte offset, y = far row's offset into coef (bytes; BY_COLUMN only)
+    __shared__ __align__(16) int2 s_far[kWavesPerBlock][fg::kItemEdges + kPad];
+    __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int head = a.head_base + (int)(blockIdx.x % (unsigned)a.n_heads);
+    const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_heads) * kWavesPerBlock + wave;
+    if (item_id >= a.n_items) return;
+    const Item it = a.items[item_id];
+    const int g = lane / L, li = lane % L;
+    const int f_lo = head * D + li * 4;
+    const uint32_t lane_bytes = a.far_tile_bytes ? (uint32_t)head * a.far_tile_bytes + (uint32_t)li * 16u : (uint32_t)f_lo * 4u;
+    const int64_t F = a.F;
+    int2 *far = s_far[wave];
+    const uint32_t coef_row_bytes = (uint32_t)a.H * 8u;
+
+    auto stage = [&](int64_t base, int n) {
+        int32_t c[4];
+        fg::load_four(a.indices + base, n, lane, 1, c);
+        int4 *f4 = reinterpret_cast<int4 *>(far);
+        f4[2 * lane] = make_int4((int)((uint32_t)c[0] * a.far_row_bytes), (int)((uint32_t)c[0] * coef_row_bytes),
+                                 (int)((uint32_t)c[1] * a.far_row_bytes), (int)((uint32_t)c[1] * coef_row_bytes));
+        f4[2 * lane + 1] = make_int4((int)((uint32_t)c[2] * a.far_row_bytes), (int)((uint32_t)c[2] * coef_row_bytes),
+                                     (int)((uint32_t)c[3] * a.far_row_bytes), (int)((uint32_t)c[3] * coef_row_bytes));
+        if (lane < kPad) far[fg::kItemEdges + lane] = make_int2((int)((uint32_t)c[3] * a.far_row_bytes), (int)((uint32_t)c[3] * coef_row_bytes));
+    };
+
+    // NU steps of one row for this lane group (elements s0 + g, s0 + g + G, ...; only the last step may have
+    // groups without an element, which re-read element e - 1 and give it no weight).
+    auto batch = [&](auto nu_tag, auto allvalid_tag, int s0, int e, const float4 &o0, const float4 &o1, float c1, float delta,
+                     float4 &accA, float4 &accB) {
+        constexpr int NU = decltype(nu_tag)::value;
+        constexpr bool ALLVALID = decltype(allvalid_tag)::value;
+        const bool last_valid = ALLVALID || s0 + (NU - 1) * G + g < e;
+        int2 w[NU];
+#pragma unroll
+        for (int u = 0; u < NU; ++u) w[u] = far[(u < NU - 1 || last_valid) ? s0 + u * G + g : e - 1];
+        float4 f0[NU], f1[NU];
+        float2 cf[NU];
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+            f0[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far0) + ((uint32_t)w[u].x + lane_bytes));
+            f1[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far1) + ((uint32_t)w[u].x + lane_bytes));
+            if (BY_COLUMN)
+                cf[u] = *reinterpret_cast<const float2 *>(reinterpret_cast<const char *>(a.coef) + ((uint32_t)w[u].y + (uint32_t)head * 8u));
+        }
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+            // rows: o0 = Q[r], o1 = dout[r], f0 = K[c], f1 = V[c];  columns: o0 = K[c], o1 = V[c], f0 = Q[r], f1 = dout[r]
+            const float s = group_sum<L>(dot4(f0[u], o0)) * a.scale;
+            const float da = group_sum<L>(dot4(f1[u], o1));
+            const float cc = BY_COLUMN ? cf[u].x : c1, dd = BY_COLUMN ? cf[u].y : delta;
+            float p = __expf(s - cc);                       // the softmax value; cc = +inf for rows without edges
+            if (!(u < NU - 1 || last_valid)) p = 0.f;
+            const float ds = p * (da - dd);
+            if (BY_COLUMN) { fma4(accA, ds, f0[u]); fma4(accB, p, f1[u]); }     // dK += ds * Q[r], dV += a * dout[r]
+            else fma4(accA, ds, f0[u]);                                         // dQ += ds * K[c]
+        }
+    };
+    auto walk = [&](int b, int e, const float4 &o0, const float4 &o1, float c1, float delta, float4 &accA, float4 &accB) {
+        using std::integral_constant;
+        int s0 = b;
+        for (; s0 + G * kU <= e; s0 += G * kU)
+            batch(integral_constant<int, kU>(), integral_constant<bool, true>(), s0, e, o0, o1, c1, delta, accA, accB);
+        if (s0 >= e) return;
+        const int nu = (e - s0 + G - 1) / G;
+        static_assert(kU == 4, "the tail below lists the step counts");
+        if (nu == 1) batch(integral_constant<int, 1>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB);
+        else if (nu == 2) batch(integral_constant<int, 2>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB);
+        else if (nu == 3) batch(integral_constant<int, 3>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB);
+        else batch(integral_constant<int, 4>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB);
+    };
+    // sums the lane groups' parts, scales what carries the score's scale, and stores (ACC: adds to) the row
+    auto finish = [&](int64_t row, float4 accA, float4 accB, const float4 &oldA, const float4 &oldB) {
+#pragma unroll
+        for (int off = L; off < 64; off <<= 1) {
+            shfl_add(accA, off);
+            if (BY_COLUMN) shfl_add(accB, off);
+        }
+        if (g != 0) return;
+        accA.x *= a.scale; accA.y *= a.scale; accA.z *= a.scale; accA.w *= a.scale;
+        if (ACC) { accA.x += oldA.x; accA.y += oldA.y; accA.z += oldA.z; accA.w += oldA.w; }
+        *reinterpret_cast<float4 *>(a.res0 + row * F + f_lo) = accA;
+        if (BY_COLUMN) {
+            if (ACC) { accB.x += oldB.x; accB.y += oldB.y; accB.z += oldB.z; accB.w += oldB.w; }
+            *reinterpret_cast<float4 *>(a.res1 + row * F + f_lo) = accB;
+        }
+    };
+    auto row_inputs = [&](int64_t row, float4 &o0, float4 &o1, float &c1, float &delta, float4 &oldA, float4 &oldB) {
+        o0 = *reinterpret_cast<const float4 *>(a.own0 + row * F + f_lo);
+        o1 = *reinterpret_cast<const float4 *>(a.own1 + row * F + f_lo);
+        c1 = 0.f; delta = 0.f;
+        if (!BY_COLUMN) {
+            const float2 cf = *reinterpret_cast<const float2 *>(a.coef + (row * a.H + head) * 2);
+            c1 = cf.x; delta = cf.y;
+        }
+        oldA = zero4(); oldB = zero4();
+        if (ACC) {
+            oldA = *reinterpret_cast<const float4 *>(a.res0 + row * F + f_lo);
+            if (BY_COLUMN) oldB = *reinterpret_cast<const float4 *>(a.res1 + row * F + f_lo);
+        }
+    };
+
+    float4 o0, o1, oldA, oldB;
+    float c1, delta;
+    if (it.info < -1) {
+        const int nrows = -it.info;
+        // own rows read once while the ids are on their way (loads return in order)
+        float touched = 0.f;
+        constexpr int kLines = (D * 4 + 127) / 128;
+        static_assert(fg::kItemRows * kLines <= 128, "two touches per lane cover an item's rows");
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int t = lane + 64 * i;
+            const int64_t at = (int64_t)(it.row + min(t / kLines, nrows - 1)) * F + head * D + min((t % kLines) * 32, D - 1);
+            touched += a.own0[at] + a.own1[at];
+            if (ACC) touched += a.res0[at] + (BY_COLUMN ? a.res1[at] : 0.f);
+        }
+        if (it.len > 0) stage(it.start, it.len);
+        s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        wave_lds_sync();
+        asm volatile("" ::"v"(touched));      // keeps the loads
+        int b = 0;
+        for (int r = 0; r < nrows; ++r) {
+            const int e = __builtin_amdgcn_readfirstlane(s_end[wave][r]);
+            if (e > b || !ACC) {
+                row_inputs(it.row + r, o0, o1, c1, delta, oldA, oldB);
+                float4 accA = zero4(), accB = zero4();
+                walk(b, e, o0, o1, c1, delta, accA, accB);
+                finish(it.row + r, accA, accB, oldA, oldB);
+            }
+            b = e;
+        }
+        return;
+    }
+    // one row of any length: 256 elements at a time
+    row_inputs(it.row, o0, o1, c1, delta, oldA, oldB);
+    float4 accA = zero4(), accB = zero4();
+    for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
+        const int n = min(fg::kItemEdges, it.len - base);
+        wave_lds_sync();
+        stage((int64_t)it.start + base, n);
+        wave_lds_sync();
+        walk(0, n, o0, o1, c1, delta, accA, accB);
+    }
+    if (it.len > 0 || !ACC) finish(it.row, accA, accB, oldA, oldB);
+}
+
+// coef[r, h] = (m + log l, <dout[r, h, :], out[r, h, :]>); rows without edges (l == 0): (+inf, 0), so that
+// every softmax value formed from them is 0.  One lane group of head_len / 4 lanes per (row, head).
+template <int L>
+__global__ __launch_bounds__(256) void attention_coef_kernel(const float *out, const float *dout, const float *state,
+                                                             float *coef, int64_t n_pairs) {
+    const int64_t pair = ((int64_t)blockIdx.x * 256 + threadIdx.x) / L;
+    const int li = threadIdx.x % L;
+    const bool on = pair < n_pairs;
+    const int64_t at = (on ? pair : 0) * (4 * L) + li * 4;
+    const float4 o = *reinterpret_cast<const float4 *>(out + at), d = *reinterpret_cast<const float4 *>(dout + at);
+    const float delta = group_sum<L>(dot4(o, d));
+    if (on && li == 0) {
+        const float m = state[pair * 2], l = state[pair * 2 + 1];
+        coef[pair * 2] = l > 0.f ? m + __logf(l) : INFINITY;
+        coef[pair * 2 + 1] = l > 0.f ? delta : 0.f;
+    }
+}
+
+template <int L, bool BY_COLUMN>
+void launch(bool acc, dim3 grid, hipStream_t st, const BwdArgs &a) {
+    if (acc) hipLaunchKernelGGL((attention_backward_kernel<L, BY_COLUMN, true>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((attention_backward_kernel<L, BY_COLUMN, false>), grid, dim3(kBlock), 0, st, a);
+}
+
+int check_common(const fg_spmm_plan *pl, int heads, int head_len, int64_t n_far_rows) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
+    if (heads < 1 || !(head_len == 16 || head_len == 32 || head_len == 64))
+        return fail(FG_ERR_SHAPE, "attention takes heads of 16, 32 or 64 floats, got %d heads of %d", heads, head_len);
+    if (pl->n_fixups > 0)
+        return fail(FG_ERR_ARG, "attention needs a plan without split rows (fg_plan_opts.split_threshold = INT32_MAX)");
+    const uint64_t F = (uint64_t)heads * head_len;
+    if ((uint64_t)n_far_rows * F * 4u >= (1ull << 32) || (uint64_t)pl->n_dst * F >= (1ull << 32) ||
+        (uint64_t)n_far_rows * heads * 8u >= (1ull << 32))
+        return fail(FG_ERR_SHAPE, "attention operands of 4 GiB and more are not supported");
+    return FG_OK;
+}
+
+// The passes over the source-column partitions of `pl`; far0 / far1 are gathered through its column ids.
+template <bool BY_COLUMN>
+int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev, const float *own0,
+                 const float *own1, const float *far0_dev, const float *far1_dev, const float *coef_dev,
+                 float *res0, float *res1, int heads, int head_len, float scale, void *stream) {
+    const int F = heads * head_len;
+    hipStream_t st = (hipStream_t)stream;
+    const int P = pl->num_col_partitions;
+    const int64_t width = (pl->n_src + P - 1) / P;
+    int rc = FG_OK;
+    const bool tiled = pl->nnz > 0 && fg::wants_tile_major(pl, heads, (uint64_t)pl->n_src * (uint64_t)F * 4u);
+    const float *far0 = far0_dev, *far1 = far1_dev;
+    if (tiled) {
+        if ((rc = fg::make_tile_major(pl, far0_dev, pl->n_src, F, head_len, stream, 0, 2)) != FG_OK) return rc;
+        if ((rc = fg::make_tile_major(pl, far1_dev, pl->n_src, F, head_len, stream, 1, 2)) != FG_OK) return rc;
+        far0 = pl->tiled_dev; far1 = pl->tiled_dev + (size_t)pl->n_src * F;
+    }
+    const int row_floats = tiled ? head_len : F;
+    for (int p = 0; p < P; ++p) {
+        const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
+        if (i1 == i0) continue;
+        BwdArgs a;
+        a.items = pl->items_dev + i0; a.n_items = i1 - i0;
+        a.pos = pos_dev + (int64_t)p * (pl->n_dst + 1);
+        a.indices = idx_dev;
+        a.own0 = own0; a.own1 = own1;
+        a.far0 = far0 + (int64_t)p * width * row_floats; a.far1 = far1 + (int64_t)p * width * row_floats;
+        a.far_row_bytes = (uint32_t)row_floats * 4u;
+        a.far_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * head_len * 4u) : 0u;
+        a.coef = BY_COLUMN ? coef_dev + (int64_t)p * width * heads * 2 : coef_dev;
+        a.res0 = res0; a.res1 = res1; a.F = F; a.H = heads; a.scale = scale; a.accumulate = p > 0;
+        const int per_launch = (heads > 8 && heads % 8 == 0) ? 8 : heads;
+        for (int hb = 0; hb < heads; hb += per_launch) {
+            a.n_heads = per_launch; a.head_base = hb;
+            const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
+            if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
+            const dim3 grid((unsigned)blocks);
+            if (head_len == 64) launch<16, BY_COLUMN>(p > 0, grid, st, a);
+            else if (head_len == 32) launch<8, BY_COLUMN>(p > 0, grid, st, a);
+            else launch<4, BY_COLUMN>(p > 0, grid, st, a);
+        }
+    }
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
+}
+
+}  // namespace
+
+extern "C" int fg_graph_attention_coef_f32(const float *out_dev, const float *dout_dev, const float *row_state_dev,
+                                           float *row_coef_dev, int64_t n_dst, int heads, int head_len, void *stream) {
+    if (n_dst < 0 || heads < 1 || !(head_len == 16 || head_len == 32 || head_len == 64))
+        return fail(FG_ERR_SHAPE, "attention takes heads of 16, 32 or 64 floats, got %d heads of %d", heads, head_len);
+    if (n_dst == 0) return FG_OK;
+    if (!out_dev || !dout_dev || !row_state_dev || !row_coef_dev) return fail(FG_ERR_ARG, "null device pointer");
+    if ((((uintptr_t)out_dev | (uintptr_t)dout_dev) & 15) != 0) return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
+    const int64_t n_pairs = n_dst * heads;
+    const int L = head_len / 4;
+    const int64_t threads = n_pairs * L;
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    hipStream_t st = (hipStream_t)stream;
+    if (L == 16) hipLaunchKernelGGL(attention_coef_kernel<16>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs);
+    else if (L == 8) hipLaunchKernelGGL(attention_coef_kernel<8>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs);
+    else hipLaunchKernelGGL(attention_coef_kernel<4>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs);
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
+}
+
+extern "C" int fg_graph_attention_backward_q_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
+                                                 const float *q_dev, const float *k_dev, const float *v_dev,
+                                                 const float *dout_dev, const float *row_coef_dev, float *dq_dev,
+                                                 int heads, int head_len, float scale, void *stream) {
+    if (pl == nullptr) return fail(FG_ERR_ARG, "plan is null");
+    if (int rc = check_common(pl, heads, head_len, pl->n_src)) return rc;
+    if (pl->n_dst == 0) return FG_OK;
+    if (!pos_dev || !q_dev || !dout_dev || !row_coef_dev || !dq_dev || (pl->nnz > 0 && (!idx_dev || !k_dev || !v_dev)))
+        return fail(FG_ERR_ARG, "null device pointer");
+    if ((((uintptr_t)q_dev | (uintptr_t)k_dev | (uintptr_t)v_dev | (uintptr_t)dout_dev | (uintptr_t)dq_dev) & 15) != 0)
+        return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
+    return run_backward<false>(pl, pos_dev, idx_dev, q_dev, dout_dev, k_dev, v_dev, row_coef_dev, dq_dev, nullptr,
+                               heads, head_len, scale, stream);
+}
+
+extern "C" int fg_graph_attention_backward_kv_f32(const fg_spmm_plan *pl, const int32_t *pos_t_dev, const int32_t *idx_t_dev,
+                                                  const float *q_dev, const float *dout_dev, const float *k_dev,
+                                                  const float *v_dev, const float *row_coef_dev, float *dk_dev,
+                                                  float *dv_dev, int heads, int head_len, float scale, void *stream) {
+    if (pl == nullptr) return fail(FG_ERR_ARG, "plan is null");
+    if (int rc = check_common(pl, heads, head_len, pl->n_src)) return rc;
+    if (pl->n_dst == 0) return FG_OK;
+    if (!pos_t_dev || !k_dev || !v_dev || !dk_dev || !dv_dev || (pl->nnz > 0 && (!idx_t_dev || !q_dev || !dout_dev || !row_coef_dev)))
+        return fail(FG_ERR_ARG, "null device pointer");
+    if ((((uintptr_t)q_dev | (uintptr_t)k_dev | (uintptr_t)v_dev | (uintptr_t)dout_dev | (uintptr_t)dk_dev | (uintptr_t)dv_dev) & 15) != 0 ||
+        ((uintptr_t)row_coef_dev & 7) != 0)
+        return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
+    return run_backward<true>(pl, pos_t_dev, idx_t_dev, k_dev, v_dev, q_dev, dout_dev, row_coef_dev, dk_dev, dv_dev,
+                              heads, head_len, scale, stream);
+}

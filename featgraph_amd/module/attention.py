@@ -19,7 +19,8 @@ class GraphAttentionhip(object):
 
     Q is (num_rows, H, D), K and V are (num_cols, H, D), D in {16, 32, 64}; rows without edges give 0.
     compute_args: 'scale' (default 1 / sqrt(D)).  schedule_args: 'num_src_partitions': 'auto' (default: chosen
-    for the L2 size, as for SpMM) | int | None (plain CSR).
+    for the L2 size, as for SpMM) | int | None (plain CSR); 'num_dst_partitions': the same for the transposed
+    adjacency that backward() sweeps.
     Equal, within rounding, to MultiHeadSDDMMhip -> EdgeSoftmaxhip -> GSpMMhip with per-head weights.
     """
 
@@ -70,7 +71,7 @@ class GraphAttentionhip(object):
     def build(self, input_placeholders, compute_args=None, schedule_args=None):
         """input_placeholders: [Q (num_rows, H, D), K (num_cols, H, D), V (num_cols, H, D)]."""
         compute_args = common.take_args(compute_args or {}, ('scale',), "compute_func")
-        schedule_args = common.take_args(schedule_args or {}, ('num_src_partitions',), "schedule_func")
+        schedule_args = common.take_args(schedule_args or {}, ('num_src_partitions', 'num_dst_partitions'), "schedule_func")
         if len(input_placeholders) != 3:
             raise ValueError("attention takes three inputs (Q, K, V), got %d" % len(input_placeholders))
         q_ph, k_ph, v_ph = input_placeholders
@@ -94,16 +95,22 @@ class GraphAttentionhip(object):
             if P < 1:
                 raise ValueError("num_src_partitions must be >= 1")
         self._heads, self._head_len = heads, head_len
+        t_parts = schedule_args.get('num_dst_partitions')       # backward(): partitions of the transposed adjacency
+        self._t_parts = None if t_parts in (None, 'auto') else int(t_parts)
         self._scale = float(compute_args.get('scale', 1.0 / np.sqrt(head_len)))
         self._active = self._layout(P)
         self._placeholders = [q_ph, k_ph, v_ph]
         self.out_tvm = torch.zeros((self._num_rows, heads, head_len), dtype=torch.float32, device=self._ctx)
+        # every row's maximum score and sum of exponentials, per head: what backward() starts from
+        self.state_tvm = torch.zeros((self._num_rows, heads, 2), dtype=torch.float32, device=self._ctx)
+        self._coef = None
 
     def _launch(self, q, k, v):
         lay = self._active
         _lib.check(_lib.lib().fg_graph_attention_f32(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']),
                                                      _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v),
-                                                     _lib.dev_ptr(self.out_tvm), self._heads, self._head_len,
+                                                     _lib.dev_ptr(self.out_tvm), _lib.dev_ptr(self.state_tvm),
+                                                     self._heads, self._head_len,
                                                      ctypes.c_float(self._scale), common.stream_ptr()))
 
     def run(self, input_tvm_ndarrays):
@@ -113,6 +120,61 @@ class GraphAttentionhip(object):
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         self._launch(*input_tvm_ndarrays)
         return self.out_tvm
+
+    def _layout_t(self, P):
+        """The transposed adjacency (rows = sources) with P partitions over the destinations."""
+        key = ('t', P)
+        if key in self._layouts:
+            return self._layouts[key]
+        tr = self._csr.T.tocsr()
+        tr.sort_indices()
+        if P > 1:
+            pos, idx, _ = util_convert_csr_to_dds(tr, P)
+        else:
+            pos, idx = tr.indptr, tr.indices
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        lay = {'P': P, 'pos': common.to_device_i32(pos, self._ctx),
+               'idx': common.to_device_i32(np.ascontiguousarray(idx, dtype=np.int32), self._ctx), 'plan': ctypes.c_void_p()}
+        base = _lib.plan_opts
+        opts = _lib.FgPlanOpts(split_threshold=_INT32_MAX, item_edges=base.item_edges if base is not None else 0,
+                               wide_offsets=0, tile_major=base.tile_major if base is not None else 0)
+        with torch.cuda.device(self._ctx):
+            _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(pos), self._num_cols, self._num_rows, P,
+                                                      ctypes.byref(opts), ctypes.byref(lay['plan'])))
+        self._layouts[key] = lay
+        return lay
+
+    def backward(self, q, k, v, out, state, grad_out):
+        """(dQ, dK, dV) for dL/d(out) = grad_out, given the inputs, the output and the row state
+        (out_tvm / state_tvm as they were after run() on these inputs).  The scores are formed again from Q
+        and K; dQ comes from a sweep like the forward pass, dK and dV from the same sweep over the
+        transposed adjacency.  Returns new tensors."""
+        if self._placeholders is None:
+            raise RuntimeError("call build() before backward()")
+        common.check_inputs([q, k, v], self._placeholders, self._ctx)
+        common.check_inputs([out, grad_out], [self._placeholders[0]] * 2, self._ctx)
+        L, s = _lib.lib(), common.stream_ptr()
+        coef = torch.empty_like(state)
+        _lib.check(L.fg_graph_attention_coef_f32(_lib.dev_ptr(out), _lib.dev_ptr(grad_out), _lib.dev_ptr(state),
+                                                 _lib.dev_ptr(coef), self._num_rows, self._heads, self._head_len, s))
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        lay = self._active
+        _lib.check(L.fg_graph_attention_backward_q_f32(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']),
+                                                       _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v),
+                                                       _lib.dev_ptr(grad_out), _lib.dev_ptr(coef), _lib.dev_ptr(dq),
+                                                       self._heads, self._head_len, ctypes.c_float(self._scale), s))
+        # partitions over the destinations, sized like the forward pass's over the sources
+        Pt = 1 if lay['P'] == 1 else max(1, tuning._partitions(self._num_rows, 2 * 4 * self._head_len,
+                                                               self._indices.shape[0], self._num_cols,
+                                                               tuning.SPMM_SLICE_BYTES, min_segment=24))
+        lt = self._layout_t(Pt if self._t_parts is None else self._t_parts)
+        _lib.check(L.fg_graph_attention_backward_kv_f32(lt['plan'], _lib.dev_ptr(lt['pos']), _lib.dev_ptr(lt['idx']),
+                                                        _lib.dev_ptr(q), _lib.dev_ptr(grad_out), _lib.dev_ptr(k),
+                                                        _lib.dev_ptr(v), _lib.dev_ptr(coef), _lib.dev_ptr(dk),
+                                                        _lib.dev_ptr(dv), self._heads, self._head_len,
+                                                        ctypes.c_float(self._scale), s))
+        self._coef = coef
+        return dq, dk, dv
 
     def measure_average_time(self, input_tvm_ndarrays, num_runs):
         if self._placeholders is None:

@@ -154,3 +154,50 @@ def test_full_size_graph(oracle):
     want = agg.run([v.reshape(n, H * D)])
     err = (got - want).abs().max().item()
     assert err < 2e-5, err
+
+
+def _dense_reference(adj, q, k, v, scale, dout):
+    """out and (dq, dk, dv) for sum(out * dout) by float64 torch autograd on the dense masked form."""
+    import torch
+    coo = adj.tocoo()
+    mask = torch.zeros(adj.shape, dtype=torch.bool)
+    mask[coo.row, coo.col] = True
+    q64, k64, v64 = (torch.from_numpy(t).double().requires_grad_() for t in (q, k, v))
+    s = torch.einsum("rhd,chd->hrc", q64, k64) * scale
+    a = torch.nan_to_num(torch.softmax(s.masked_fill(~mask, float("-inf")), dim=-1), nan=0.0)
+    out = torch.einsum("hrc,chd->rhd", a, v64)
+    (out * torch.from_numpy(dout).double()).sum().backward()
+    return out.detach().numpy(), q64.grad.numpy(), k64.grad.numpy(), v64.grad.numpy()
+
+
+@pytest.mark.parametrize("H,D,P,Pt", [(1, 64, None, None), (4, 64, 2, 3), (8, 64, 3, 2), (4, 32, 2, 2), (8, 16, 5, 4),
+                                      (3, 64, 1, 4), (16, 32, 4, 1)])
+@pytest.mark.parametrize("tile_major", [0, 1])
+def test_gradients_against_float64(monkeypatch, H, D, P, Pt, tile_major):
+    import torch
+    from featgraph_amd import _lib
+    from featgraph_amd.module import GraphAttentionhip, placeholder
+    if tile_major:
+        monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(tile_major=1))
+    rng = np.random.default_rng(H * 1000 + D * 10 + (P or 0))
+    adj = _graph(rng, 200, 260, 250, 0.05)
+    q = rng.standard_normal((adj.shape[0], H, D)).astype("float32")
+    k = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    v = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    dout = rng.standard_normal(q.shape).astype("float32")
+    m = GraphAttentionhip(adj)
+    m.build([placeholder(q.shape), placeholder(k.shape), placeholder(v.shape)], {},
+            {'num_src_partitions': P, 'num_dst_partitions': Pt})
+    qd, kd, vd, dd = (torch.from_numpy(t).cuda() for t in (q, k, v, dout))
+    out = m.run([qd, kd, vd])
+    dq, dk, dv = m.backward(qd, kd, vd, out, m.state_tvm, dd)
+    ref_out, ref_dq, ref_dk, ref_dv = _dense_reference(adj, q, k, v, 1.0 / np.sqrt(D), dout)
+    np.testing.assert_allclose(out.cpu().numpy(), ref_out, rtol=1e-4, atol=2e-5)
+    for got, want, name in ((dq, ref_dq, "dq"), (dk, ref_dk, "dk"), (dv, ref_dv, "dv")):
+        got = got.cpu().numpy()
+        assert np.isfinite(got).all(), name
+        np.testing.assert_allclose(got, want, rtol=1e-3, atol=1e-4, err_msg=name)
+    # rows / columns without edges get zero gradients
+    assert (dq.cpu().numpy()[np.diff(adj.indptr) == 0] == 0).all()
+    no_in = np.diff(adj.T.tocsr().indptr) == 0
+    assert (dk.cpu().numpy()[no_in] == 0).all() and (dv.cpu().numpy()[no_in] == 0).all()
