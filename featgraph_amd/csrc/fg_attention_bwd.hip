@@ -73,7 +73,8 @@ struct BwdArgs {
     const float *own0, *own1; // [n_own, F]: (Q, dout) or (K, V)
     const float *far0, *far1; // offset to the partition's first far row: (K, V) or (Q, dout)
     uint32_t far_row_bytes, far_tile_bytes;
-    const float *coef;        // [n_dst, H, 2]: (m + log l, delta); BY_COLUMN: offset to the partition's first far row
+    const float *coef;        // [H, n_dst, 2]: (m + log l, delta), head by head; BY_COLUMN: offset to the partition's first far row
+    int64_t coef_head_floats; // floats from one head's block of coef to the next (2 * n_dst)
     float *res0, *res1;       // [n_own, F]: dQ, or dK and dV
     int F, H;
     int n_heads, head_base;
@@ -98,7 +99,8 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
     const uint32_t lane_bytes = a.far_tile_bytes ? (uint32_t)head * a.far_tile_bytes + (uint32_t)li * 16u : (uint32_t)f_lo * 4u;
     const int64_t F = a.F;
     int2 *far = s_far[wave];
-    const uint32_t coef_row_bytes = (uint32_t)a.H * 8u;
+    constexpr uint32_t coef_row_bytes = 8u;
+    const float *coef_head = a.coef + (int64_t)head * a.coef_head_floats;
 
     auto stage = [&](int64_t base, int n) {
         int32_t c[4];
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
             f0[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far0) + ((uint32_t)w[u].x + lane_bytes));
             f1[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far1) + ((uint32_t)w[u].x + lane_bytes));
             if (BY_COLUMN)
-                cf[u] = *reinterpret_cast<const float2 *>(reinterpret_cast<const char *>(a.coef) + ((uint32_t)w[u].y + (uint32_t)head * 8u));
+                cf[u] = *reinterpret_cast<const float2 *>(reinterpret_cast<const char *>(coef_head) + (uint32_t)w[u].y);
         }
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
@@ -177,7 +179,7 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
         o1 = *reinterpret_cast<const float4 *>(a.own1 + row * F + f_lo);
         c1 = 0.f; delta = 0.f;
         if (!BY_COLUMN) {
-            const float2 cf = *reinterpret_cast<const float2 *>(a.coef + (row * a.H + head) * 2);
+            const float2 cf = *reinterpret_cast<const float2 *>(coef_head + row * 2);
             c1 = cf.x; delta = cf.y;
         }
         oldA = zero4(); oldB = zero4();
@@ -232,11 +234,12 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
     if (it.len > 0 || !ACC) finish(it.row, accA, accB, oldA, oldB);
 }
 
-// coef[r, h] = (m + log l, <dout[r, h, :], out[r, h, :]>); rows without edges (l == 0): (+inf, 0), so that
+// coef[h, r] = (m + log l, <dout[r, h, :], out[r, h, :]>), head by head so that the gathers of one head stay
+// inside 8 * n_dst bytes; rows without edges (l == 0): (+inf, 0), so that
 // every softmax value formed from them is 0.  One lane group of head_len / 4 lanes per (row, head).
 template <int L>
 __global__ __launch_bounds__(256) void attention_coef_kernel(const float *out, const float *dout, const float *state,
-                                                             float *coef, int64_t n_pairs) {
+                                                             float *coef, int64_t n_pairs, int64_t n_rows, int H) {
     const int64_t pair = ((int64_t)blockIdx.x * 256 + threadIdx.x) / L;
     const int li = threadIdx.x % L;
     const bool on = pair < n_pairs;
@@ -245,8 +248,10 @@ __global__ __launch_bounds__(256) void attention_coef_kernel(const float *out, c
     const float delta = group_sum<L>(dot4(o, d));
     if (on && li == 0) {
         const float m = state[pair * 2], l = state[pair * 2 + 1];
-        coef[pair * 2] = l > 0.f ? m + __logf(l) : INFINITY;
-        coef[pair * 2 + 1] = l > 0.f ? delta : 0.f;
+        const int64_t r = pair / H, h = pair - r * H;
+        float *c = coef + (h * n_rows + r) * 2;                 // head by head
+        c[0] = l > 0.f ? m + __logf(l) : INFINITY;
+        c[1] = l > 0.f ? delta : 0.f;
     }
 }
 
@@ -265,7 +270,7 @@ int check_common(const fg_spmm_plan *pl, int heads, int head_len, int64_t n_far_
         return fail(FG_ERR_ARG, "attention needs a plan without split rows (fg_plan_opts.split_threshold = INT32_MAX)");
     const uint64_t F = (uint64_t)heads * head_len;
     if ((uint64_t)n_far_rows * F * 4u >= (1ull << 32) || (uint64_t)pl->n_dst * F >= (1ull << 32) ||
-        (uint64_t)n_far_rows * heads * 8u >= (1ull << 32))
+        (uint64_t)n_far_rows * 8u >= (1ull << 32))
         return fail(FG_ERR_SHAPE, "attention operands of 4 GiB and more are not supported");
     return FG_OK;
 }
@@ -299,7 +304,8 @@ int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *
         a.far0 = far0 + (int64_t)p * width * row_floats; a.far1 = far1 + (int64_t)p * width * row_floats;
         a.far_row_bytes = (uint32_t)row_floats * 4u;
         a.far_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * head_len * 4u) : 0u;
-        a.coef = BY_COLUMN ? coef_dev + (int64_t)p * width * heads * 2 : coef_dev;
+        a.coef = BY_COLUMN ? coef_dev + (int64_t)p * width * 2 : coef_dev;
+        a.coef_head_floats = 2 * (BY_COLUMN ? pl->n_src : pl->n_dst);
         a.res0 = res0; a.res1 = res1; a.F = F; a.H = heads; a.scale = scale; a.accumulate = p > 0;
         const int per_launch = (heads > 8 && heads % 8 == 0) ? 8 : heads;
         for (int hb = 0; hb < heads; hb += per_launch) {
@@ -330,9 +336,9 @@ extern "C" int fg_graph_attention_coef_f32(const float *out_dev, const float *do
     const int64_t threads = n_pairs * L;
     const dim3 grid((unsigned)((threads + 255) / 256));
     hipStream_t st = (hipStream_t)stream;
-    if (L == 16) hipLaunchKernelGGL(attention_coef_kernel<16>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs);
-    else if (L == 8) hipLaunchKernelGGL(attention_coef_kernel<8>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs);
-    else hipLaunchKernelGGL(attention_coef_kernel<4>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs);
+    if (L == 16) hipLaunchKernelGGL(attention_coef_kernel<16>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs, n_dst, heads);
+    else if (L == 8) hipLaunchKernelGGL(attention_coef_kernel<8>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs, n_dst, heads);
+    else hipLaunchKernelGGL(attention_coef_kernel<4>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs, n_dst, heads);
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;
 }
