@@ -83,8 +83,7 @@ def test_aggregate_gradients(reduce):
 
 
 def test_attention_with_and_without_gradients():
-    """Graph.attention: one operator under no_grad, the differentiable chain otherwise; same values, and the
-    chain's gradients match float64 torch autograd."""
+    """Graph.attention with and without gradients: same values, and the gradients match float64 torch autograd."""
     import torch
     from featgraph_amd.autograd import Graph
     rng = np.random.default_rng(21)
