@@ -21,6 +21,8 @@
 
 using fg::fail;
 using fg::Item;
+using fg::group_sum;
+using fg::wave_lds_sync;
 
 namespace {
 
@@ -28,27 +30,6 @@ constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = 64 * kWavesPerBlock;
 constexpr int kPad = 8;
 constexpr int kU = 4;                  // elements per lane group whose gathers are issued back to back
-
-__device__ __forceinline__ void wave_lds_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-
-// Sum over the L (4, 8 or 16) consecutive lanes of a lane group; every lane of the group gets it.
-template <int L>
-__device__ __forceinline__ float group_sum(float v) {
-    v += dpp_move<0xB1>(v);                  // quad_perm [1,0,3,2]
-    v += dpp_move<0x4E>(v);                  // quad_perm [2,3,0,1]
-    if (L >= 8) v += dpp_move<0x141>(v);     // row_half_mirror
-    if (L >= 16) v += dpp_move<0x140>(v);    // row_mirror
-    return v;
-}
 
 __device__ __forceinline__ float dot4(const float4 &a, const float4 &b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
 __device__ __forceinline__ void fma4(float4 &acc, float w, const float4 &x) {

@@ -30,4 +30,29 @@ __device__ __forceinline__ void load_four(const T *p, int n, int lane, int strid
     }
 }
 
+// Orders this wavefront's LDS writes before its later LDS reads (and the reverse); for staging buffers
+// that are private to one wavefront, so no workgroup barrier is involved.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// v from another lane of the same 16-lane row, chosen by a DPP control word (no LDS traffic).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over the L (4, 8 or 16) consecutive lanes of a lane group; every lane of the group gets it.
+template <int L>
+__device__ __forceinline__ float group_sum(float v) {
+    static_assert(L == 4 || L == 8 || L == 16, "lane groups inside one 16-lane row");
+    v += dpp_move<0xB1>(v);                  // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);                  // quad_perm [2,3,0,1]
+    if (L >= 8) v += dpp_move<0x141>(v);     // row_half_mirror
+    if (L >= 16) v += dpp_move<0x140>(v);    // row_mirror
+    return v;
+}
+
 }  // namespace fg

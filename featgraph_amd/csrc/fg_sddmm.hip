@@ -17,6 +17,8 @@
 
 using fg::fail;
 using fg::Item;
+using fg::dpp_move;
+using fg::wave_lds_sync;
 
 namespace {
 
@@ -34,18 +36,6 @@ __device__ __forceinline__ float vdot(const float4 &a, const float4 &b) {
 }
 __device__ __forceinline__ float vdot(const float &a, const float &b) { return a * b; }
 __device__ __forceinline__ float4 vzero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
-
-__device__ __forceinline__ void wave_lds_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// v from another lane of the same 16-lane row, chosen by a DPP control word (no LDS traffic).
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
 
 // Sum over the RW consecutive lanes of a head segment; every lane of the segment gets it.
 // Inside a 16-lane row the butterfly runs on DPP moves: swap neighbours, swap pairs, mirror

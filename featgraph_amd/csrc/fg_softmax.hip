@@ -15,24 +15,18 @@
 #include <cmath>
 
 #include "fg_common.h"
+#include "fg_device.h"
 
 using fg::fail;
 using fg::Fixup;
 using fg::Item;
+using fg::wave_lds_sync;
 
 namespace {
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = 64 * kWavesPerBlock;
 constexpr int kStage = 1024;          // floats of a multi-row item staged in LDS per wavefront
-
-// Orders this wavefront's LDS writes before its later LDS reads (and the reverse); the staging
-// buffers are private to one wavefront, so no workgroup barrier is involved.
-__device__ __forceinline__ void wave_lds_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 
 struct SoftmaxArgs {
     const Item *items;

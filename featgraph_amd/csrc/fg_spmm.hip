@@ -20,6 +20,7 @@
 using fg::fail;
 using fg::Fixup;
 using fg::Item;
+using fg::wave_lds_sync;
 
 namespace {
 
@@ -43,14 +44,6 @@ __device__ __forceinline__ float4 vshfl_xor(const float4 &a, int off) {
     return make_float4(__shfl_xor(a.x, off), __shfl_xor(a.y, off), __shfl_xor(a.z, off), __shfl_xor(a.w, off));
 }
 __device__ __forceinline__ float vshfl_xor(const float &a, int off) { return __shfl_xor(a, off); }
-
-// Orders this wavefront's LDS writes before its later LDS reads (and the reverse); the
-// staging buffers are private to one wavefront, so no workgroup barrier is involved.
-__device__ __forceinline__ void wave_lds_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 
 struct SpmmArgs {
     const Item *items;
