@@ -58,6 +58,7 @@ SIGNATURES = {
     "fg_edge_softmax_stats_f32": (_int, [_vp, _vp, _vp, _vp, _int, _vp]),
     "fg_edge_softmax_head_major_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _vp, _vp]),
     "fg_graph_attention_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),
+    "fg_graph_attention_additive_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),
     "fg_graph_attention_coef_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "fg_graph_attention_backward_q_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),
     "fg_graph_attention_backward_kv_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),

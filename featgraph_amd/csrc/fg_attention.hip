@@ -46,6 +46,10 @@ struct AttnArgs {
     int F, H;
     int n_heads, head_base;   // heads of this launch
     float scale;
+    // additive scores: q = er [H, n_dst] and k = el [H, n_src] (k offset to the partition's first source), one
+    // scalar per vertex and head; floats from one head's block to the next; negative slope of the leaky ReLU
+    int64_t q_head_floats, k_head_floats;
+    float slope;
 };
 
 // Running softmax-weighted sum of one lane group: maximum, sum of exponentials, weighted sum.
@@ -67,31 +71,44 @@ __device__ __forceinline__ void running_merge(Running &r, const Running &s) {
     r.m = m;
 }
 
-// NU steps of one row for this lane group: staged elements s0 + g, s0 + g + G, ...; every step but the
-// last lies wholly below e, and in the last one (unless ALLVALID) a group whose element would be e or
-// beyond re-reads element e - 1 and gives it no weight.  All 2 * NU gathers are issued before the first
-// is used.
-template <int L, int NU, bool ALLVALID>
-__device__ __forceinline__ void walk_batch(const int32_t *cols, int s0, int e, int g, const float *k, const float *v,
-                                           uint32_t lane_bytes, const float4 &q, float scale, Running &r) {
-    constexpr int G = 64 / L;
-    const bool last_valid = ALLVALID || s0 + (NU - 1) * G + g < e;
-    int c[NU];
-#pragma unroll
-    for (int u = 0; u < NU; ++u) c[u] = cols[(u < NU - 1 || last_valid) ? s0 + u * G + g : e - 1];
+// What is staged per element: the byte offset of its row in K / V, and, for additive scores, the byte
+// offset of its scalar as well.
+template <bool ADD> struct Staged;
+template <> struct Staged<false> { using type = int32_t; };
+template <> struct Staged<true> { using type = int2; };
+__device__ __forceinline__ uint32_t slice_off(int32_t c) { return (uint32_t)c; }
+__device__ __forceinline__ uint32_t slice_off(const int2 &c) { return (uint32_t)c.x; }
+__device__ __forceinline__ uint32_t scalar_off(int32_t) { return 0u; }
+__device__ __forceinline__ uint32_t scalar_off(const int2 &c) { return (uint32_t)c.y; }
+
+// NU elements of one row, those with valid[u] counted: all gathers are issued before the first is used,
+// then the scores and the running update.
+//   ADD == false: score = scale * <K[c, h, :], q>  (k: the K slices, this lane's 16 bytes at lane_bytes);
+//   ADD == true : score = leaky_relu(k[c] + q.x) with negative slope `scale`  (k: one scalar per source and head).
+template <int L, int NU, bool ADD, typename S>
+__device__ __forceinline__ void update(const S (&c)[NU], const bool (&valid)[NU], const float *k, const float *v,
+                                       uint32_t lane_bytes, const float4 &q, float scale, Running &r) {
     float4 kk[NU], vv[NU];
+    float ev[NU];
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
-        kk[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(k) + ((uint32_t)c[u] + lane_bytes));
-        vv[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(v) + ((uint32_t)c[u] + lane_bytes));
+        if constexpr (ADD) ev[u] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(k) + scalar_off(c[u]));
+        else kk[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(k) + (slice_off(c[u]) + lane_bytes));
+        vv[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(v) + (slice_off(c[u]) + lane_bytes));
     }
     float s[NU];
     float m = r.m;
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
-        const float d = kk[u].x * q.x + kk[u].y * q.y + kk[u].z * q.z + kk[u].w * q.w;
-        const float t = group_sum<L>(d) * scale;      // every lane takes part in the cross-lane sum
-        s[u] = (u < NU - 1 || last_valid) ? t : -INFINITY;
+        float t;
+        if constexpr (ADD) {
+            const float z = ev[u] + q.x;
+            t = z > 0.f ? z : z * scale;
+        } else {
+            const float d = kk[u].x * q.x + kk[u].y * q.y + kk[u].z * q.z + kk[u].w * q.w;
+            t = group_sum<L>(d) * scale;                // every lane takes part in the cross-lane sum
+        }
+        s[u] = valid[u] ? t : -INFINITY;
         m = fmaxf(m, s[u]);
     }
     if (m == -INFINITY) return;             // nothing finite so far (uniform inside a lane group)
@@ -107,56 +124,54 @@ __device__ __forceinline__ void walk_batch(const int32_t *cols, int s0, int e, i
     }
 }
 
+// NU steps of one row for this lane group: staged elements s0 + g, s0 + g + G, ...; every step but the
+// last lies wholly below e, and in the last one (unless ALLVALID) a group whose element would be e or
+// beyond re-reads element e - 1 and gives it no weight.
+template <int L, int NU, bool ALLVALID, bool ADD, typename S>
+__device__ __forceinline__ void walk_batch(const S *cols, int s0, int e, int g, const float *k, const float *v,
+                                           uint32_t lane_bytes, const float4 &q, float scale, Running &r) {
+    constexpr int G = 64 / L;
+    const bool last_valid = ALLVALID || s0 + (NU - 1) * G + g < e;
+    S c[NU];
+    bool valid[NU];
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        valid[u] = u < NU - 1 || last_valid;
+        c[u] = cols[valid[u] ? s0 + u * G + g : e - 1];
+    }
+    update<L, NU, ADD>(c, valid, k, v, lane_bytes, q, scale, r);
+}
+
 // Staged elements [b, e) of one row, shared by the G lane groups; the last batch is issued with exactly
 // the steps it has left.
-template <int L>
-__device__ __forceinline__ void walk(const int32_t *cols, int b, int e, int g, const float *k, const float *v,
+template <int L, bool ADD, typename S>
+__device__ __forceinline__ void walk(const S *cols, int b, int e, int g, const float *k, const float *v,
                                      uint32_t lane_bytes, const float4 &q, float scale, Running &r) {
     constexpr int G = 64 / L;
     int s0 = b;
-    for (; s0 + G * kU <= e; s0 += G * kU) walk_batch<L, kU, true>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+    for (; s0 + G * kU <= e; s0 += G * kU) walk_batch<L, kU, true, ADD>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
     if (s0 >= e) return;
     const int nu = (e - s0 + G - 1) / G;    // uniform: 1 .. kU
     static_assert(kU == 4, "the tail below lists the step counts");
-    if (nu == 1) walk_batch<L, 1, false>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
-    else if (nu == 2) walk_batch<L, 2, false>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
-    else if (nu == 3) walk_batch<L, 3, false>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
-    else walk_batch<L, 4, false>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+    if (nu == 1) walk_batch<L, 1, false, ADD>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+    else if (nu == 2) walk_batch<L, 2, false, ADD>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+    else if (nu == 3) walk_batch<L, 3, false, ADD>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
+    else walk_batch<L, 4, false, ADD>(cols, s0, e, g, k, v, lane_bytes, q, scale, r);
 }
 
 // kU consecutive staged elements j .. j + kU - 1 of this lane group's own row (those below e count; the
 // slots behind them hold later rows' elements or the padding: loadable, given no weight).
-template <int L>
-__device__ __forceinline__ void own_batch(const int32_t *cols, int j, int e, const float *k, const float *v,
+template <int L, bool ADD, typename S>
+__device__ __forceinline__ void own_batch(const S *cols, int j, int e, const float *k, const float *v,
                                           uint32_t lane_bytes, const float4 &q, float scale, Running &r) {
-    int c[kU];
-#pragma unroll
-    for (int u = 0; u < kU; ++u) c[u] = cols[j + u];
-    float4 kk[kU], vv[kU];
+    S c[kU];
+    bool valid[kU];
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
-        kk[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(k) + ((uint32_t)c[u] + lane_bytes));
-        vv[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(v) + ((uint32_t)c[u] + lane_bytes));
+        c[u] = cols[j + u];
+        valid[u] = j + u < e;
     }
-    float s[kU];
-    float m = r.m;
-#pragma unroll
-    for (int u = 0; u < kU; ++u) {
-        const float d = kk[u].x * q.x + kk[u].y * q.y + kk[u].z * q.z + kk[u].w * q.w;
-        const float t = group_sum<L>(d) * scale;
-        s[u] = (j + u < e) ? t : -INFINITY;
-        m = fmaxf(m, s[u]);
-    }
-    const float f = __expf(r.m - m);          // j < e: at least one finite score, so m is finite
-    r.acc.x *= f; r.acc.y *= f; r.acc.z *= f; r.acc.w *= f;
-    r.l *= f;
-    r.m = m;
-#pragma unroll
-    for (int u = 0; u < kU; ++u) {
-        const float p = __expf(s[u] - m);
-        r.l += p;
-        r.acc.x += p * vv[u].x; r.acc.y += p * vv[u].y; r.acc.z += p * vv[u].z; r.acc.w += p * vv[u].w;
-    }
+    update<L, kU, ADD>(c, valid, k, v, lane_bytes, q, scale, r);
 }
 
 // What the earlier partitions left for a row (read before the row's gathers are issued).
@@ -189,10 +204,13 @@ __device__ __forceinline__ void finish_row(Running r, const Running &old, int g,
 
 // L lanes x 128 bits cover one head.  FIRST: the first partition's pass writes every row's state; later
 // passes merge into it and skip rows without elements in their partition.
-template <int L, bool FIRST>
+// ADD: scores are leaky_relu(el[col e, h] + er[row e, h]) (a.k = el and a.q = er, one scalar per vertex and head,
+// head by head) instead of scaled dot products of K and Q slices.
+template <int L, bool FIRST, bool ADD>
 __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs a) {
     constexpr int G = 64 / L, D = 4 * L;
-    __shared__ __align__(16) int32_t s_col[kWavesPerBlock][fg::kItemEdges + kPad];
+    using S = typename Staged<ADD>::type;
+    __shared__ __align__(16) S s_col[kWavesPerBlock][fg::kItemEdges + kPad];
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
     __shared__ int32_t s_next[kWavesPerBlock];
 
@@ -205,14 +223,32 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
     const int f_lo = head * D + li * 4;
     const uint32_t lane_bytes = a.kv_tile_bytes ? (uint32_t)head * a.kv_tile_bytes + (uint32_t)li * 16u : (uint32_t)f_lo * 4u;
     const int64_t F = a.F;
-    int32_t *cols = s_col[wave];
+    S *cols = s_col[wave];
+    // ADD: this head's scalars; the score's second parameter is the negative slope
+    const float *kptr = ADD ? a.k + (int64_t)head * a.k_head_floats : a.k;
+    const float *q_head = a.q + (int64_t)head * a.q_head_floats;
+    const float sparam = ADD ? a.slope : a.scale;
 
     auto stage = [&](int64_t base, int n) {
         int32_t c[4];
         fg::load_four(a.indices + base, n, lane, 1, c);
-        *reinterpret_cast<int4 *>(cols + 4 * lane) = make_int4((int)((uint32_t)c[0] * a.kv_row_bytes), (int)((uint32_t)c[1] * a.kv_row_bytes),
-                                                               (int)((uint32_t)c[2] * a.kv_row_bytes), (int)((uint32_t)c[3] * a.kv_row_bytes));
-        if (lane < kPad) cols[fg::kItemEdges + lane] = (int)((uint32_t)c[3] * a.kv_row_bytes);
+        uint32_t b[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) b[i] = (uint32_t)c[i] * a.kv_row_bytes;
+        if constexpr (ADD) {
+            int4 *c4 = reinterpret_cast<int4 *>(cols);
+            c4[2 * lane] = make_int4((int)b[0], c[0] * 4, (int)b[1], c[1] * 4);
+            c4[2 * lane + 1] = make_int4((int)b[2], c[2] * 4, (int)b[3], c[3] * 4);
+            if (lane < kPad) cols[fg::kItemEdges + lane] = make_int2((int)b[3], c[3] * 4);
+        } else {
+            *reinterpret_cast<int4 *>(cols + 4 * lane) = make_int4((int)b[0], (int)b[1], (int)b[2], (int)b[3]);
+            if (lane < kPad) cols[fg::kItemEdges + lane] = (int)b[3];
+        }
+    };
+    // the row's own operand: its slice of Q, or (ADD) its scalar in .x
+    auto own_q = [&](int64_t row) {
+        if constexpr (ADD) return make_float4(q_head[row], 0.f, 0.f, 0.f);
+        else return *reinterpret_cast<const float4 *>(a.q + row * F + f_lo);
     };
     auto out_row = [&](int64_t row) { return a.out + row * F + f_lo; };
     auto state_row = [&](int64_t row) { return a.state + (row * a.H + head) * 2; };
@@ -230,7 +266,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
         for (int i = 0; i < 2; ++i) {
             const int t = lane + 64 * i;
             const int64_t at = (int64_t)(it.row + min(t / kLines, nrows - 1)) * F + head * D + min((t % kLines) * 32, D - 1);
-            touched += a.q[at];
+            if (!ADD) touched += a.q[at];
             if (!FIRST) touched += a.out[at];
         }
         if (it.len > 0) stage(it.start, it.len);
@@ -264,7 +300,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
                         e = s_end[wave][r];
                         live = FIRST || e > j;
                         if (live) {
-                            q = *reinterpret_cast<const float4 *>(a.q + (int64_t)(it.row + r) * F + f_lo);
+                            q = own_q(it.row + r);
                             old = load_state<FIRST>(out_row(it.row + r), state_row(it.row + r));
                             run = running_empty();
                         }
@@ -272,7 +308,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
                 }
                 if (__all(done)) break;
                 if (!done && j < e) {
-                    own_batch<L>(cols, j, e, a.k, a.v, lane_bytes, q, a.scale, run);
+                    own_batch<L, ADD>(cols, j, e, kptr, a.v, lane_bytes, q, sparam, run);
                     j += kU;
                 }
             }
@@ -282,10 +318,10 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
         for (int r = 0; r < nrows; ++r) {
             const int e = __builtin_amdgcn_readfirstlane(s_end[wave][r]);
             if (e > b || FIRST) {
-                const float4 q = *reinterpret_cast<const float4 *>(a.q + (int64_t)(it.row + r) * F + f_lo);
+                const float4 q = own_q(it.row + r);
                 const Running old = load_state<FIRST>(out_row(it.row + r), state_row(it.row + r));
                 Running run = running_empty();
-                walk<L>(cols, b, e, g, a.k, a.v, lane_bytes, q, a.scale, run);
+                walk<L, ADD>(cols, b, e, g, kptr, a.v, lane_bytes, q, sparam, run);
                 finish_row<L, FIRST>(run, old, g, li, out_row(it.row + r), state_row(it.row + r));
             }
             b = e;
@@ -293,7 +329,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
         return;
     }
     // one row of any length: 256 elements at a time
-    const float4 q = *reinterpret_cast<const float4 *>(a.q + (int64_t)it.row * F + f_lo);
+    const float4 q = own_q(it.row);
     const Running old = load_state<FIRST>(out_row(it.row), state_row(it.row));
     Running run = running_empty();
     for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
@@ -301,7 +337,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
         wave_lds_sync();
         stage((int64_t)it.start + base, n);
         wave_lds_sync();
-        walk<L>(cols, 0, n, g, a.k, a.v, lane_bytes, q, a.scale, run);
+        walk<L, ADD>(cols, 0, n, g, kptr, a.v, lane_bytes, q, sparam, run);
     }
     if (it.len > 0 || FIRST) finish_row<L, FIRST>(run, old, g, li, out_row(it.row), state_row(it.row));
 }
@@ -319,17 +355,18 @@ __global__ __launch_bounds__(256) void attention_finish_kernel(float4 *out, cons
     out[i] = l > 0.f ? o : make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
-template <int L>
+template <int L, bool ADD>
 void launch(bool first, dim3 grid, hipStream_t st, const AttnArgs &a) {
-    if (first) hipLaunchKernelGGL((attention_items_kernel<L, true>), grid, dim3(kBlock), 0, st, a);
-    else hipLaunchKernelGGL((attention_items_kernel<L, false>), grid, dim3(kBlock), 0, st, a);
+    if (first) hipLaunchKernelGGL((attention_items_kernel<L, true, ADD>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((attention_items_kernel<L, false, ADD>), grid, dim3(kBlock), 0, st, a);
 }
 
-}  // namespace
-
-extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
-                                      const float *q_dev, const float *k_dev, const float *v_dev, float *out_dev,
-                                      float *row_state_dev, int heads, int head_len, float scale, void *stream) {
+// The passes over the source partitions.  ADD == false: q / k are the [n, F] operands of the dot products and
+// `param` their scale; ADD == true: q = er [H, n_dst], k = el [H, n_src] and `param` the leaky ReLU's slope.
+template <bool ADD>
+int run_forward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev, const float *q_dev,
+                const float *k_dev, const float *v_dev, float *out_dev, float *row_state_dev, int heads,
+                int head_len, float param, void *stream) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (int drc = fg::check_device(pl)) return drc;
     if (heads < 1 || !(head_len == 16 || head_len == 32 || head_len == 64))
@@ -339,7 +376,7 @@ extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos
     if (pl->n_dst == 0) return FG_OK;
     if (!pos_dev || !q_dev || !out_dev || (pl->nnz > 0 && (!idx_dev || !k_dev || !v_dev)))
         return fail(FG_ERR_ARG, "null device pointer");
-    if ((((uintptr_t)q_dev | (uintptr_t)k_dev | (uintptr_t)v_dev | (uintptr_t)out_dev) & 15) != 0)
+    if ((((uintptr_t)v_dev | (uintptr_t)out_dev | (ADD ? 0 : ((uintptr_t)q_dev | (uintptr_t)k_dev))) & 15) != 0)
         return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
     const int F = heads * head_len;
     if ((uint64_t)pl->n_src * (uint64_t)F * 4u >= (1ull << 32) || (uint64_t)pl->n_dst * (uint64_t)F >= (1ull << 32))
@@ -352,13 +389,17 @@ extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
-    // K and V head by head, as the SpMM kernels gather X tile by tile
+    // the gathered [n_src, F] operands head by head, as the SpMM kernels gather X tile by tile
     const bool tiled = pl->nnz > 0 && fg::wants_tile_major(pl, heads, (uint64_t)pl->n_src * (uint64_t)F * 4u);
     const float *k = k_dev, *v = v_dev;
     if (tiled) {
-        if ((rc = fg::make_tile_major(pl, k_dev, pl->n_src, F, head_len, stream, 0, 2)) != FG_OK) return rc;
-        if ((rc = fg::make_tile_major(pl, v_dev, pl->n_src, F, head_len, stream, 1, 2)) != FG_OK) return rc;
-        k = pl->tiled_dev; v = pl->tiled_dev + (size_t)pl->n_src * F;
+        const int slots = ADD ? 1 : 2;
+        if ((rc = fg::make_tile_major(pl, v_dev, pl->n_src, F, head_len, stream, 0, slots)) != FG_OK) return rc;
+        v = pl->tiled_dev;
+        if (!ADD) {
+            if ((rc = fg::make_tile_major(pl, k_dev, pl->n_src, F, head_len, stream, 1, slots)) != FG_OK) return rc;
+            k = pl->tiled_dev + (size_t)pl->n_src * F;
+        }
     }
     const int row_floats = tiled ? head_len : F;
     for (int p = 0; p < P; ++p) {
@@ -368,19 +409,21 @@ extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos
         a.items = pl->items_dev + i0; a.n_items = i1 - i0;
         a.pos = pos_dev + (int64_t)p * (pl->n_dst + 1);
         a.indices = idx_dev; a.q = q_dev;
-        a.k = k + (int64_t)p * width * row_floats; a.v = v + (int64_t)p * width * row_floats;
+        a.k = ADD ? k + (int64_t)p * width : k + (int64_t)p * width * row_floats;
+        a.v = v + (int64_t)p * width * row_floats;
         a.kv_row_bytes = (uint32_t)row_floats * 4u;
         a.kv_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * head_len * 4u) : 0u;
-        a.out = out_dev; a.state = row_state_dev; a.F = F; a.H = heads; a.scale = scale;
+        a.out = out_dev; a.state = row_state_dev; a.F = F; a.H = heads; a.scale = param; a.slope = param;
+        a.q_head_floats = ADD ? pl->n_dst : 0; a.k_head_floats = ADD ? pl->n_src : 0;
         const int per_launch = (heads > 8 && heads % 8 == 0) ? 8 : heads;
         for (int hb = 0; hb < heads; hb += per_launch) {
             a.n_heads = per_launch; a.head_base = hb;
             const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
             if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
             const dim3 grid((unsigned)blocks);
-            if (head_len == 64) launch<16>(p == 0, grid, st, a);
-            else if (head_len == 32) launch<8>(p == 0, grid, st, a);
-            else launch<4>(p == 0, grid, st, a);
+            if (head_len == 64) launch<16, ADD>(p == 0, grid, st, a);
+            else if (head_len == 32) launch<8, ADD>(p == 0, grid, st, a);
+            else launch<4, ADD>(p == 0, grid, st, a);
         }
     }
     const uint32_t n_words = (uint32_t)((uint64_t)pl->n_dst * F / 4);
@@ -389,4 +432,20 @@ extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos
                        (uint32_t)(head_len / 4), heads);
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;
+}
+
+}  // namespace
+
+extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
+                                      const float *q_dev, const float *k_dev, const float *v_dev, float *out_dev,
+                                      float *row_state_dev, int heads, int head_len, float scale, void *stream) {
+    return run_forward<false>(pl, pos_dev, idx_dev, q_dev, k_dev, v_dev, out_dev, row_state_dev, heads, head_len, scale, stream);
+}
+
+extern "C" int fg_graph_attention_additive_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
+                                               const float *er_dev, const float *el_dev, const float *v_dev,
+                                               float *out_dev, float *row_state_dev, int heads, int head_len,
+                                               float negative_slope, void *stream) {
+    return run_forward<true>(pl, pos_dev, idx_dev, er_dev, el_dev, v_dev, out_dev, row_state_dev, heads, head_len,
+                             negative_slope, stream);
 }

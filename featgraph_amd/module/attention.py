@@ -18,7 +18,9 @@ class GraphAttentionhip(object):
     """out[v, h, :] = sum over the edges e into v of softmax_v(scale * <K[col e, h, :], Q[v, h, :]>) * V[col e, h, :]
 
     Q is (num_rows, H, D), K and V are (num_cols, H, D), D in {16, 32, 64}; rows without edges give 0.
-    compute_args: 'scale' (default 1 / sqrt(D)).  schedule_args: 'num_src_partitions': 'auto' (default: chosen
+    compute_args: 'scale' (default 1 / sqrt(D)); 'scores': 'dot' (default) | 'additive' -- the attention of GAT
+    layers, scores leaky_relu(El[col e, h] + Er[v, h]) with 'negative_slope' (default 0.2); the inputs are then
+    [Er (num_rows, H), El (num_cols, H), V (num_cols, H, D)].  schedule_args: 'num_src_partitions': 'auto' (default: chosen
     for the L2 size, as for SpMM) | int | None (plain CSR); 'num_dst_partitions': the same for the transposed
     adjacency that backward() sweeps.
     Equal, within rounding, to MultiHeadSDDMMhip -> EdgeSoftmaxhip -> GSpMMhip with per-head weights.
@@ -70,7 +72,12 @@ class GraphAttentionhip(object):
 
     def build(self, input_placeholders, compute_args=None, schedule_args=None):
         """input_placeholders: [Q (num_rows, H, D), K (num_cols, H, D), V (num_cols, H, D)]."""
-        compute_args = common.take_args(compute_args or {}, ('scale',), "compute_func")
+        compute_args = common.take_args(compute_args or {}, ('scale', 'scores', 'negative_slope'), "compute_func")
+        self._additive = compute_args.get('scores', 'dot') == 'additive'
+        if compute_args.get('scores', 'dot') not in ('dot', 'additive'):
+            raise ValueError("scores must be 'dot' or 'additive'")
+        if self._additive:
+            return self._build_additive(input_placeholders, compute_args, schedule_args)
         schedule_args = common.take_args(schedule_args or {}, ('num_src_partitions', 'num_dst_partitions'), "schedule_func")
         if len(input_placeholders) != 3:
             raise ValueError("attention takes three inputs (Q, K, V), got %d" % len(input_placeholders))
@@ -83,17 +90,7 @@ class GraphAttentionhip(object):
                 raise ValueError("%s must be (num_cols=%d, %d, %d), got %s" % (name, self._num_cols, heads, head_len, ph.shape))
         if head_len not in (16, 32, 64):
             raise ValueError("heads of 16, 32 or 64 floats, got %d" % head_len)
-        src_parts = schedule_args.get('num_src_partitions', 'auto')
-        if src_parts is None:
-            P = 1
-        elif src_parts == 'auto':
-            # one head per XCD, and that XCD's L2 holds the head's slices of both K and V
-            P = tuning._partitions(self._num_cols, 2 * 4 * head_len, self._indices.shape[0], self._num_rows,
-                                   tuning.SPMM_SLICE_BYTES, min_segment=24)
-        else:
-            P = int(src_parts)
-            if P < 1:
-                raise ValueError("num_src_partitions must be >= 1")
+        P = self._partitions(schedule_args, 2 * 4 * head_len)
         self._heads, self._head_len = heads, head_len
         t_parts = schedule_args.get('num_dst_partitions')       # backward(): partitions of the transposed adjacency
         self._t_parts = None if t_parts in (None, 'auto') else int(t_parts)
@@ -105,7 +102,53 @@ class GraphAttentionhip(object):
         self.state_tvm = torch.zeros((self._num_rows, heads, 2), dtype=torch.float32, device=self._ctx)
         self._coef = None
 
+    def _partitions(self, schedule_args, slice_row_bytes):
+        """Source partitions: one head per XCD, whose L2 holds the head's slices of the gathered operands."""
+        src_parts = schedule_args.get('num_src_partitions', 'auto')
+        if src_parts is None:
+            return 1
+        if src_parts == 'auto':
+            return tuning._partitions(self._num_cols, slice_row_bytes, self._indices.shape[0], self._num_rows,
+                                      tuning.SPMM_SLICE_BYTES, min_segment=24)
+        if int(src_parts) < 1:
+            raise ValueError("num_src_partitions must be >= 1")
+        return int(src_parts)
+
+    def _build_additive(self, input_placeholders, compute_args, schedule_args):
+        schedule_args = common.take_args(schedule_args or {}, ('num_src_partitions', 'num_dst_partitions'), "schedule_func")
+        if len(input_placeholders) != 3:
+            raise ValueError("additive attention takes three inputs (Er, El, V), got %d" % len(input_placeholders))
+        er_ph, el_ph, v_ph = input_placeholders
+        if len(v_ph.shape) != 3 or v_ph.shape[0] != self._num_cols:
+            raise ValueError("V must be (num_cols=%d, H, D), got %s" % (self._num_cols, v_ph.shape))
+        heads, head_len = int(v_ph.shape[1]), int(v_ph.shape[2])
+        if tuple(er_ph.shape) != (self._num_rows, heads) or tuple(el_ph.shape) != (self._num_cols, heads):
+            raise ValueError("Er must be (num_rows=%d, %d) and El (num_cols=%d, %d), got %s and %s"
+                             % (self._num_rows, heads, self._num_cols, heads, er_ph.shape, el_ph.shape))
+        if head_len not in (16, 32, 64):
+            raise ValueError("heads of 16, 32 or 64 floats, got %d" % head_len)
+        self._heads, self._head_len = heads, head_len
+        self._slope = float(compute_args.get('negative_slope', 0.2))
+        self._scale = 1.0
+        t_parts = schedule_args.get('num_dst_partitions')
+        self._t_parts = None if t_parts in (None, 'auto') else int(t_parts)
+        self._active = self._layout(self._partitions(schedule_args, 4 * head_len))
+        self._placeholders = [er_ph, el_ph, v_ph]
+        self.out_tvm = torch.zeros((self._num_rows, heads, head_len), dtype=torch.float32, device=self._ctx)
+        self.state_tvm = torch.zeros((self._num_rows, heads, 2), dtype=torch.float32, device=self._ctx)
+        self._coef = None
+
+    def _launch_additive(self, er, el, v):
+        lay = self._active
+        self._er_t, self._el_t = er.t().contiguous(), el.t().contiguous()      # head by head
+        _lib.check(_lib.lib().fg_graph_attention_additive_f32(
+            lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(self._er_t),
+            _lib.dev_ptr(self._el_t), _lib.dev_ptr(v), _lib.dev_ptr(self.out_tvm), _lib.dev_ptr(self.state_tvm),
+            self._heads, self._head_len, ctypes.c_float(self._slope), common.stream_ptr()))
+
     def _launch(self, q, k, v):
+        if self._additive:
+            return self._launch_additive(q, k, v)
         lay = self._active
         _lib.check(_lib.lib().fg_graph_attention_f32(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']),
                                                      _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v),

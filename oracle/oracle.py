@@ -312,3 +312,20 @@ def graph_attention_f64(indptr, indices, q, k, v, scale):
         a = scipy.special.softmax(s, axis=0)
         out[r] = np.einsum("eh,ehd->hd", a, v64[cols])
     return out
+
+
+def graph_attention_additive_f64(indptr, indices, er, el, v, negative_slope):
+    """out[r, h, :] = sum_e softmax_e(leaky_relu(el[col e, h] + er[r, h])) * v[col e, h, :] in float64 (the
+    attention of a GAT layer; er is [n_dst, H], el [n_src, H]).  No counterpart in the reference."""
+    import scipy.special
+    er64, el64, v64 = (np.asarray(a, dtype=np.float64) for a in (er, el, v))
+    out = np.zeros((len(indptr) - 1,) + v64.shape[1:], dtype=np.float64)
+    for r in range(len(indptr) - 1):
+        b, e = int(indptr[r]), int(indptr[r + 1])
+        if e == b:
+            continue
+        cols = indices[b:e]
+        z = el64[cols] + er64[r]
+        a = scipy.special.softmax(np.where(z > 0, z, negative_slope * z), axis=0)
+        out[r] = np.einsum("eh,ehd->hd", a, v64[cols])
+    return out

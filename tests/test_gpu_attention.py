@@ -201,3 +201,23 @@ def test_gradients_against_float64(monkeypatch, H, D, P, Pt, tile_major):
     assert (dq.cpu().numpy()[np.diff(adj.indptr) == 0] == 0).all()
     no_in = np.diff(adj.T.tocsr().indptr) == 0
     assert (dk.cpu().numpy()[no_in] == 0).all() and (dv.cpu().numpy()[no_in] == 0).all()
+
+
+@pytest.mark.parametrize("H,D,P", [(1, 64, None), (4, 64, 3), (8, 32, 2), (8, 16, 5), (3, 64, 1)])
+def test_additive_scores_against_float64(oracle, H, D, P):
+    """The attention of GAT layers: leaky_relu(El[col] + Er[row]) as scores."""
+    import torch
+    from featgraph_amd.module import GraphAttentionhip, placeholder
+    rng = np.random.default_rng(H * 7 + D + (P or 0))
+    adj = _graph(rng)
+    er = rng.standard_normal((adj.shape[0], H)).astype("float32")
+    el = (3 * rng.standard_normal((adj.shape[1], H))).astype("float32")
+    v = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    m = GraphAttentionhip(adj)
+    m.build([placeholder(er.shape), placeholder(el.shape), placeholder(v.shape)],
+            {'scores': 'additive', 'negative_slope': 0.2}, {'num_src_partitions': P})
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([torch.from_numpy(er).cuda(), torch.from_numpy(el).cuda(), torch.from_numpy(v).cuda()]).cpu().numpy()
+    ref = oracle.graph_attention_additive_f64(adj.indptr, adj.indices, er, el, v, 0.2)
+    assert np.isfinite(out).all() and (out[np.diff(adj.indptr) == 0] == 0).all()
+    np.testing.assert_allclose(out, ref, rtol=1e-4, atol=2e-5)
