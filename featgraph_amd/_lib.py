@@ -62,6 +62,9 @@ SIGNATURES = {
     "fg_graph_attention_coef_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "fg_graph_attention_backward_q_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),
     "fg_graph_attention_backward_kv_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),
+    "fg_graph_attention_additive_coef_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
+    "fg_graph_attention_additive_backward_er_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),
+    "fg_graph_attention_additive_backward_elv_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),
     "fg_synth_powerlaw_csr": (_int, [_i64, _vp, _vp, _vp, ctypes.c_uint64, _int, _vp, _vp]),
 }
 

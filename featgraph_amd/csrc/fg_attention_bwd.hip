@@ -61,9 +61,18 @@ struct BwdArgs {
     int n_heads, head_base;
     int accumulate;
     float scale;
+    // Additive scores leaky_relu(el[c] + er[r]) (ADD): no far0 / own0 slices; instead
+    //   rows:    far_s = el [H, n_src] (4 bytes per element), coef holds (m + log l, delta, er[r], 0) per row;
+    //   columns: own_s = el [H, n_src], far_s = that 16-byte coef of the destinations;
+    // res_s = d_er (rows) or d_el (columns), [H, n_own]; all head by head, *_head_floats apart.
+    const float *own_s, *far_s;
+    float *res_s;
+    int64_t own_s_head_floats, far_s_head_floats;
+    uint32_t far_s_bytes;     // bytes per far element in far_s (4 or 16)
+    float slope;
 };
 
-template <int L, bool BY_COLUMN, bool ACC>
+template <int L, bool BY_COLUMN, bool ACC, bool ADD>
 __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArgs a) {
     constexpr int G = 64 / L, D = 4 * L;
     // x = far row's byte offset, y = far row's offset into coef (bytes; BY_COLUMN only)
@@ -80,8 +89,11 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
     const uint32_t lane_bytes = a.far_tile_bytes ? (uint32_t)head * a.far_tile_bytes + (uint32_t)li * 16u : (uint32_t)f_lo * 4u;
     const int64_t F = a.F;
     int2 *far = s_far[wave];
-    constexpr uint32_t coef_row_bytes = 8u;
+    const uint32_t coef_row_bytes = ADD ? a.far_s_bytes : 8u;       // second staged word: the far element's scalar data
     const float *coef_head = a.coef + (int64_t)head * a.coef_head_floats;
+    const float *far_s_head = ADD ? a.far_s + (int64_t)head * a.far_s_head_floats : nullptr;
+    const float *own_s_head = (ADD && BY_COLUMN) ? a.own_s + (int64_t)head * a.own_s_head_floats : nullptr;
+    float *res_s_head = ADD ? a.res_s + (int64_t)head * a.own_s_head_floats : nullptr;
 
     auto stage = [&](int64_t base, int n) {
         int32_t c[4];
@@ -97,81 +109,115 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
     // NU steps of one row for this lane group (elements s0 + g, s0 + g + G, ...; only the last step may have
     // groups without an element, which re-read element e - 1 and give it no weight).
     auto batch = [&](auto nu_tag, auto allvalid_tag, int s0, int e, const float4 &o0, const float4 &o1, float c1, float delta,
-                     float4 &accA, float4 &accB) {
+                     float4 &accA, float4 &accB, float &accS) {
         constexpr int NU = decltype(nu_tag)::value;
         constexpr bool ALLVALID = decltype(allvalid_tag)::value;
         const bool last_valid = ALLVALID || s0 + (NU - 1) * G + g < e;
         int2 w[NU];
 #pragma unroll
         for (int u = 0; u < NU; ++u) w[u] = far[(u < NU - 1 || last_valid) ? s0 + u * G + g : e - 1];
-        float4 f0[NU], f1[NU];
+        float4 f0[NU], f1[NU], cf4[NU];
         float2 cf[NU];
+        float ev[NU];
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
-            f0[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far0) + ((uint32_t)w[u].x + lane_bytes));
+            if constexpr (!ADD) f0[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far0) + ((uint32_t)w[u].x + lane_bytes));
             f1[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far1) + ((uint32_t)w[u].x + lane_bytes));
-            if (BY_COLUMN)
+            if constexpr (ADD) {
+                if (BY_COLUMN) cf4[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(far_s_head) + (uint32_t)w[u].y);
+                else ev[u] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(far_s_head) + (uint32_t)w[u].y);
+            } else if (BY_COLUMN) {
                 cf[u] = *reinterpret_cast<const float2 *>(reinterpret_cast<const char *>(coef_head) + (uint32_t)w[u].y);
+            }
         }
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
             // rows: o0 = Q[r], o1 = dout[r], f0 = K[c], f1 = V[c];  columns: o0 = K[c], o1 = V[c], f0 = Q[r], f1 = dout[r]
-            const float s = group_sum<L>(dot4(f0[u], o0)) * a.scale;
+            // ADD: o0.x = the own scalar (er[r] | el[c]) and the far one comes from ev (el[c]) | cf4.z (er[r])
+            float s, gate = 1.f;
+            if constexpr (ADD) {
+                const float z = o0.x + (BY_COLUMN ? cf4[u].z : ev[u]);
+                gate = z > 0.f ? 1.f : a.slope;
+                s = z * gate;
+            } else {
+                s = group_sum<L>(dot4(f0[u], o0)) * a.scale;
+            }
             const float da = group_sum<L>(dot4(f1[u], o1));
-            const float cc = BY_COLUMN ? cf[u].x : c1, dd = BY_COLUMN ? cf[u].y : delta;
+            const float cc = BY_COLUMN ? (ADD ? cf4[u].x : cf[u].x) : c1, dd = BY_COLUMN ? (ADD ? cf4[u].y : cf[u].y) : delta;
             float p = __expf(s - cc);                       // the softmax value; cc = +inf for rows without edges
             if (!(u < NU - 1 || last_valid)) p = 0.f;
             const float ds = p * (da - dd);
-            if (BY_COLUMN) { fma4(accA, ds, f0[u]); fma4(accB, p, f1[u]); }     // dK += ds * Q[r], dV += a * dout[r]
-            else fma4(accA, ds, f0[u]);                                         // dQ += ds * K[c]
+            if constexpr (ADD) {
+                accS += ds * gate;                                                  // d_er[r] | d_el[c]
+                if (BY_COLUMN) fma4(accB, p, f1[u]);                                // dV += a * dout[r]
+            } else {
+                if (BY_COLUMN) { fma4(accA, ds, f0[u]); fma4(accB, p, f1[u]); }     // dK += ds * Q[r], dV += a * dout[r]
+                else fma4(accA, ds, f0[u]);                                         // dQ += ds * K[c]
+            }
         }
     };
-    auto walk = [&](int b, int e, const float4 &o0, const float4 &o1, float c1, float delta, float4 &accA, float4 &accB) {
+    auto walk = [&](int b, int e, const float4 &o0, const float4 &o1, float c1, float delta, float4 &accA, float4 &accB, float &accS) {
         using std::integral_constant;
         int s0 = b;
         for (; s0 + G * kU <= e; s0 += G * kU)
-            batch(integral_constant<int, kU>(), integral_constant<bool, true>(), s0, e, o0, o1, c1, delta, accA, accB);
+            batch(integral_constant<int, kU>(), integral_constant<bool, true>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
         if (s0 >= e) return;
         const int nu = (e - s0 + G - 1) / G;
         static_assert(kU == 4, "the tail below lists the step counts");
-        if (nu == 1) batch(integral_constant<int, 1>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB);
-        else if (nu == 2) batch(integral_constant<int, 2>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB);
-        else if (nu == 3) batch(integral_constant<int, 3>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB);
-        else batch(integral_constant<int, 4>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB);
+        if (nu == 1) batch(integral_constant<int, 1>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
+        else if (nu == 2) batch(integral_constant<int, 2>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
+        else if (nu == 3) batch(integral_constant<int, 3>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
+        else batch(integral_constant<int, 4>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
     };
     // sums the lane groups' parts, scales what carries the score's scale, and stores (ACC: adds to) the row
-    auto finish = [&](int64_t row, float4 accA, float4 accB, const float4 &oldA, const float4 &oldB) {
+    auto finish = [&](int64_t row, float4 accA, float4 accB, float accS, const float4 &oldA, const float4 &oldB, float oldS) {
 #pragma unroll
         for (int off = L; off < 64; off <<= 1) {
-            shfl_add(accA, off);
+            if (!ADD) shfl_add(accA, off);
             if (BY_COLUMN) shfl_add(accB, off);
+            if (ADD) accS += __shfl_xor(accS, off);
         }
         if (g != 0) return;
-        accA.x *= a.scale; accA.y *= a.scale; accA.z *= a.scale; accA.w *= a.scale;
-        if (ACC) { accA.x += oldA.x; accA.y += oldA.y; accA.z += oldA.z; accA.w += oldA.w; }
-        *reinterpret_cast<float4 *>(a.res0 + row * F + f_lo) = accA;
+        if constexpr (ADD) {
+            if (li == 0) res_s_head[row] = ACC ? accS + oldS : accS;
+        } else {
+            accA.x *= a.scale; accA.y *= a.scale; accA.z *= a.scale; accA.w *= a.scale;
+            if (ACC) { accA.x += oldA.x; accA.y += oldA.y; accA.z += oldA.z; accA.w += oldA.w; }
+            *reinterpret_cast<float4 *>(a.res0 + row * F + f_lo) = accA;
+        }
         if (BY_COLUMN) {
             if (ACC) { accB.x += oldB.x; accB.y += oldB.y; accB.z += oldB.z; accB.w += oldB.w; }
             *reinterpret_cast<float4 *>(a.res1 + row * F + f_lo) = accB;
         }
     };
-    auto row_inputs = [&](int64_t row, float4 &o0, float4 &o1, float &c1, float &delta, float4 &oldA, float4 &oldB) {
-        o0 = *reinterpret_cast<const float4 *>(a.own0 + row * F + f_lo);
+    auto row_inputs = [&](int64_t row, float4 &o0, float4 &o1, float &c1, float &delta, float4 &oldA, float4 &oldB, float &oldS) {
         o1 = *reinterpret_cast<const float4 *>(a.own1 + row * F + f_lo);
         c1 = 0.f; delta = 0.f;
-        if (!BY_COLUMN) {
-            const float2 cf = *reinterpret_cast<const float2 *>(coef_head + row * 2);
-            c1 = cf.x; delta = cf.y;
+        if constexpr (ADD) {
+            if (BY_COLUMN) {
+                o0 = make_float4(own_s_head[row], 0.f, 0.f, 0.f);
+            } else {
+                const float4 cf = *reinterpret_cast<const float4 *>(coef_head + row * 4);
+                c1 = cf.x; delta = cf.y;
+                o0 = make_float4(cf.z, 0.f, 0.f, 0.f);
+            }
+        } else {
+            o0 = *reinterpret_cast<const float4 *>(a.own0 + row * F + f_lo);
+            if (!BY_COLUMN) {
+                const float2 cf = *reinterpret_cast<const float2 *>(coef_head + row * 2);
+                c1 = cf.x; delta = cf.y;
+            }
         }
-        oldA = zero4(); oldB = zero4();
+        oldA = zero4(); oldB = zero4(); oldS = 0.f;
         if (ACC) {
-            oldA = *reinterpret_cast<const float4 *>(a.res0 + row * F + f_lo);
+            if (ADD) oldS = res_s_head[row];
+            else oldA = *reinterpret_cast<const float4 *>(a.res0 + row * F + f_lo);
             if (BY_COLUMN) oldB = *reinterpret_cast<const float4 *>(a.res1 + row * F + f_lo);
         }
     };
 
     float4 o0, o1, oldA, oldB;
-    float c1, delta;
+    float c1, delta, oldS;
     if (it.info < -1) {
         const int nrows = -it.info;
         // own rows read once while the ids are on their way (loads return in order)
@@ -182,8 +228,10 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
         for (int i = 0; i < 2; ++i) {
             const int t = lane + 64 * i;
             const int64_t at = (int64_t)(it.row + min(t / kLines, nrows - 1)) * F + head * D + min((t % kLines) * 32, D - 1);
-            touched += a.own0[at] + a.own1[at];
-            if (ACC) touched += a.res0[at] + (BY_COLUMN ? a.res1[at] : 0.f);
+            touched += a.own1[at];
+            if (!ADD) touched += a.own0[at];
+            if (ACC && !ADD) touched += a.res0[at];
+            if (ACC && BY_COLUMN) touched += a.res1[at];
         }
         if (it.len > 0) stage(it.start, it.len);
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
@@ -193,26 +241,28 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
         for (int r = 0; r < nrows; ++r) {
             const int e = __builtin_amdgcn_readfirstlane(s_end[wave][r]);
             if (e > b || !ACC) {
-                row_inputs(it.row + r, o0, o1, c1, delta, oldA, oldB);
+                row_inputs(it.row + r, o0, o1, c1, delta, oldA, oldB, oldS);
                 float4 accA = zero4(), accB = zero4();
-                walk(b, e, o0, o1, c1, delta, accA, accB);
-                finish(it.row + r, accA, accB, oldA, oldB);
+                float accS = 0.f;
+                walk(b, e, o0, o1, c1, delta, accA, accB, accS);
+                finish(it.row + r, accA, accB, accS, oldA, oldB, oldS);
             }
             b = e;
         }
         return;
     }
     // one row of any length: 256 elements at a time
-    row_inputs(it.row, o0, o1, c1, delta, oldA, oldB);
+    row_inputs(it.row, o0, o1, c1, delta, oldA, oldB, oldS);
     float4 accA = zero4(), accB = zero4();
+    float accS = 0.f;
     for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
         const int n = min(fg::kItemEdges, it.len - base);
         wave_lds_sync();
         stage((int64_t)it.start + base, n);
         wave_lds_sync();
-        walk(0, n, o0, o1, c1, delta, accA, accB);
+        walk(0, n, o0, o1, c1, delta, accA, accB, accS);
     }
-    if (it.len > 0 || !ACC) finish(it.row, accA, accB, oldA, oldB);
+    if (it.len > 0 || !ACC) finish(it.row, accA, accB, accS, oldA, oldB, oldS);
 }
 
 // coef[h, r] = (m + log l, <dout[r, h, :], out[r, h, :]>), head by head so that the gathers of one head stay
@@ -220,7 +270,8 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
 // every softmax value formed from them is 0.  One lane group of head_len / 4 lanes per (row, head).
 template <int L>
 __global__ __launch_bounds__(256) void attention_coef_kernel(const float *out, const float *dout, const float *state,
-                                                             float *coef, int64_t n_pairs, int64_t n_rows, int H) {
+                                                             const float *er, float *coef, int64_t n_pairs,
+                                                             int64_t n_rows, int H) {
     const int64_t pair = ((int64_t)blockIdx.x * 256 + threadIdx.x) / L;
     const int li = threadIdx.x % L;
     const bool on = pair < n_pairs;
@@ -230,16 +281,20 @@ __global__ __launch_bounds__(256) void attention_coef_kernel(const float *out, c
     if (on && li == 0) {
         const float m = state[pair * 2], l = state[pair * 2 + 1];
         const int64_t r = pair / H, h = pair - r * H;
-        float *c = coef + (h * n_rows + r) * 2;                 // head by head
-        c[0] = l > 0.f ? m + __logf(l) : INFINITY;
-        c[1] = l > 0.f ? delta : 0.f;
+        const float c1 = l > 0.f ? m + __logf(l) : INFINITY, dl = l > 0.f ? delta : 0.f;
+        if (er) {       // additive scores: the row's own scalar rides along, 16 bytes per row and head
+            *reinterpret_cast<float4 *>(coef + (h * n_rows + r) * 4) = make_float4(c1, dl, er[h * n_rows + r], 0.f);
+        } else {
+            float *c = coef + (h * n_rows + r) * 2;             // head by head
+            c[0] = c1; c[1] = dl;
+        }
     }
 }
 
-template <int L, bool BY_COLUMN>
+template <int L, bool BY_COLUMN, bool ADD>
 void launch(bool acc, dim3 grid, hipStream_t st, const BwdArgs &a) {
-    if (acc) hipLaunchKernelGGL((attention_backward_kernel<L, BY_COLUMN, true>), grid, dim3(kBlock), 0, st, a);
-    else hipLaunchKernelGGL((attention_backward_kernel<L, BY_COLUMN, false>), grid, dim3(kBlock), 0, st, a);
+    if (acc) hipLaunchKernelGGL((attention_backward_kernel<L, BY_COLUMN, true, ADD>), grid, dim3(kBlock), 0, st, a);
+    else hipLaunchKernelGGL((attention_backward_kernel<L, BY_COLUMN, false, ADD>), grid, dim3(kBlock), 0, st, a);
 }
 
 int check_common(const fg_spmm_plan *pl, int heads, int head_len, int64_t n_far_rows) {
@@ -257,10 +312,13 @@ int check_common(const fg_spmm_plan *pl, int heads, int head_len, int64_t n_far_
 }
 
 // The passes over the source-column partitions of `pl`; far0 / far1 are gathered through its column ids.
-template <bool BY_COLUMN>
+// ADD (additive scores): far0 / own0 are not used; own_s / far_s / res_s as described at BwdArgs, coef_dev is
+// the 16-byte form.
+template <bool BY_COLUMN, bool ADD>
 int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev, const float *own0,
                  const float *own1, const float *far0_dev, const float *far1_dev, const float *coef_dev,
-                 float *res0, float *res1, int heads, int head_len, float scale, void *stream) {
+                 float *res0, float *res1, int heads, int head_len, float param, void *stream,
+                 const float *own_s = nullptr, const float *far_s = nullptr, float *res_s = nullptr) {
     const int F = heads * head_len;
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
@@ -269,11 +327,16 @@ int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *
     const bool tiled = pl->nnz > 0 && fg::wants_tile_major(pl, heads, (uint64_t)pl->n_src * (uint64_t)F * 4u);
     const float *far0 = far0_dev, *far1 = far1_dev;
     if (tiled) {
-        if ((rc = fg::make_tile_major(pl, far0_dev, pl->n_src, F, head_len, stream, 0, 2)) != FG_OK) return rc;
-        if ((rc = fg::make_tile_major(pl, far1_dev, pl->n_src, F, head_len, stream, 1, 2)) != FG_OK) return rc;
-        far0 = pl->tiled_dev; far1 = pl->tiled_dev + (size_t)pl->n_src * F;
+        const int slots = ADD ? 1 : 2;
+        if ((rc = fg::make_tile_major(pl, far1_dev, pl->n_src, F, head_len, stream, 0, slots)) != FG_OK) return rc;
+        far1 = pl->tiled_dev;
+        if (!ADD) {
+            if ((rc = fg::make_tile_major(pl, far0_dev, pl->n_src, F, head_len, stream, 1, slots)) != FG_OK) return rc;
+            far0 = pl->tiled_dev + (size_t)pl->n_src * F;
+        }
     }
     const int row_floats = tiled ? head_len : F;
+    const int far_s_floats = BY_COLUMN ? 4 : 1;          // ADD: floats per far element in far_s
     for (int p = 0; p < P; ++p) {
         const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
         if (i1 == i0) continue;
@@ -282,23 +345,51 @@ int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *
         a.pos = pos_dev + (int64_t)p * (pl->n_dst + 1);
         a.indices = idx_dev;
         a.own0 = own0; a.own1 = own1;
-        a.far0 = far0 + (int64_t)p * width * row_floats; a.far1 = far1 + (int64_t)p * width * row_floats;
+        a.far0 = ADD ? nullptr : far0 + (int64_t)p * width * row_floats; a.far1 = far1 + (int64_t)p * width * row_floats;
         a.far_row_bytes = (uint32_t)row_floats * 4u;
         a.far_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * head_len * 4u) : 0u;
-        a.coef = BY_COLUMN ? coef_dev + (int64_t)p * width * 2 : coef_dev;
-        a.coef_head_floats = 2 * (BY_COLUMN ? pl->n_src : pl->n_dst);
-        a.res0 = res0; a.res1 = res1; a.F = F; a.H = heads; a.scale = scale; a.accumulate = p > 0;
+        if (ADD) {
+            a.coef = coef_dev; a.coef_head_floats = 4 * pl->n_dst;       // rows only: the own rows' 16-byte coef
+            a.own_s = own_s; a.own_s_head_floats = pl->n_dst; a.res_s = res_s;
+            a.far_s = far_s + (int64_t)p * width * far_s_floats; a.far_s_head_floats = (int64_t)far_s_floats * pl->n_src;
+            a.far_s_bytes = 4u * far_s_floats;
+        } else {
+            a.coef = BY_COLUMN ? coef_dev + (int64_t)p * width * 2 : coef_dev;
+            a.coef_head_floats = 2 * (BY_COLUMN ? pl->n_src : pl->n_dst);
+            a.own_s = a.far_s = nullptr; a.res_s = nullptr; a.own_s_head_floats = a.far_s_head_floats = 0; a.far_s_bytes = 0;
+        }
+        a.res0 = res0; a.res1 = res1; a.F = F; a.H = heads; a.scale = param; a.slope = param; a.accumulate = p > 0;
         const int per_launch = (heads > 8 && heads % 8 == 0) ? 8 : heads;
         for (int hb = 0; hb < heads; hb += per_launch) {
             a.n_heads = per_launch; a.head_base = hb;
             const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
             if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
             const dim3 grid((unsigned)blocks);
-            if (head_len == 64) launch<16, BY_COLUMN>(p > 0, grid, st, a);
-            else if (head_len == 32) launch<8, BY_COLUMN>(p > 0, grid, st, a);
-            else launch<4, BY_COLUMN>(p > 0, grid, st, a);
+            if (head_len == 64) launch<16, BY_COLUMN, ADD>(p > 0, grid, st, a);
+            else if (head_len == 32) launch<8, BY_COLUMN, ADD>(p > 0, grid, st, a);
+            else launch<4, BY_COLUMN, ADD>(p > 0, grid, st, a);
         }
     }
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
+}
+
+int run_coef(const float *out_dev, const float *dout_dev, const float *row_state_dev, const float *er_dev,
+             float *row_coef_dev, int64_t n_dst, int heads, int head_len, void *stream) {
+    if (n_dst < 0 || heads < 1 || !(head_len == 16 || head_len == 32 || head_len == 64))
+        return fail(FG_ERR_SHAPE, "attention takes heads of 16, 32 or 64 floats, got %d heads of %d", heads, head_len);
+    if (n_dst == 0) return FG_OK;
+    if (!out_dev || !dout_dev || !row_state_dev || !row_coef_dev) return fail(FG_ERR_ARG, "null device pointer");
+    if ((((uintptr_t)out_dev | (uintptr_t)dout_dev | (uintptr_t)row_coef_dev) & 15) != 0)
+        return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
+    const int64_t n_pairs = n_dst * heads;
+    const int L = head_len / 4;
+    const int64_t threads = n_pairs * L;
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    hipStream_t st = (hipStream_t)stream;
+    if (L == 16) hipLaunchKernelGGL(attention_coef_kernel<16>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, er_dev, row_coef_dev, n_pairs, n_dst, heads);
+    else if (L == 8) hipLaunchKernelGGL(attention_coef_kernel<8>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, er_dev, row_coef_dev, n_pairs, n_dst, heads);
+    else hipLaunchKernelGGL(attention_coef_kernel<4>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, er_dev, row_coef_dev, n_pairs, n_dst, heads);
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;
 }
@@ -307,21 +398,7 @@ int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *
 
 extern "C" int fg_graph_attention_coef_f32(const float *out_dev, const float *dout_dev, const float *row_state_dev,
                                            float *row_coef_dev, int64_t n_dst, int heads, int head_len, void *stream) {
-    if (n_dst < 0 || heads < 1 || !(head_len == 16 || head_len == 32 || head_len == 64))
-        return fail(FG_ERR_SHAPE, "attention takes heads of 16, 32 or 64 floats, got %d heads of %d", heads, head_len);
-    if (n_dst == 0) return FG_OK;
-    if (!out_dev || !dout_dev || !row_state_dev || !row_coef_dev) return fail(FG_ERR_ARG, "null device pointer");
-    if ((((uintptr_t)out_dev | (uintptr_t)dout_dev) & 15) != 0) return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
-    const int64_t n_pairs = n_dst * heads;
-    const int L = head_len / 4;
-    const int64_t threads = n_pairs * L;
-    const dim3 grid((unsigned)((threads + 255) / 256));
-    hipStream_t st = (hipStream_t)stream;
-    if (L == 16) hipLaunchKernelGGL(attention_coef_kernel<16>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs, n_dst, heads);
-    else if (L == 8) hipLaunchKernelGGL(attention_coef_kernel<8>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs, n_dst, heads);
-    else hipLaunchKernelGGL(attention_coef_kernel<4>, grid, dim3(256), 0, st, out_dev, dout_dev, row_state_dev, row_coef_dev, n_pairs, n_dst, heads);
-    FG_HIP_TRY(hipGetLastError());
-    return FG_OK;
+    return run_coef(out_dev, dout_dev, row_state_dev, nullptr, row_coef_dev, n_dst, heads, head_len, stream);
 }
 
 extern "C" int fg_graph_attention_backward_q_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
@@ -335,7 +412,7 @@ extern "C" int fg_graph_attention_backward_q_f32(const fg_spmm_plan *pl, const i
         return fail(FG_ERR_ARG, "null device pointer");
     if ((((uintptr_t)q_dev | (uintptr_t)k_dev | (uintptr_t)v_dev | (uintptr_t)dout_dev | (uintptr_t)dq_dev) & 15) != 0)
         return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
-    return run_backward<false>(pl, pos_dev, idx_dev, q_dev, dout_dev, k_dev, v_dev, row_coef_dev, dq_dev, nullptr,
+    return run_backward<false, false>(pl, pos_dev, idx_dev, q_dev, dout_dev, k_dev, v_dev, row_coef_dev, dq_dev, nullptr,
                                heads, head_len, scale, stream);
 }
 
@@ -351,6 +428,46 @@ extern "C" int fg_graph_attention_backward_kv_f32(const fg_spmm_plan *pl, const 
     if ((((uintptr_t)q_dev | (uintptr_t)k_dev | (uintptr_t)v_dev | (uintptr_t)dout_dev | (uintptr_t)dk_dev | (uintptr_t)dv_dev) & 15) != 0 ||
         ((uintptr_t)row_coef_dev & 7) != 0)
         return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
-    return run_backward<true>(pl, pos_t_dev, idx_t_dev, k_dev, v_dev, q_dev, dout_dev, row_coef_dev, dk_dev, dv_dev,
+    return run_backward<true, false>(pl, pos_t_dev, idx_t_dev, k_dev, v_dev, q_dev, dout_dev, row_coef_dev, dk_dev, dv_dev,
                               heads, head_len, scale, stream);
+}
+
+extern "C" int fg_graph_attention_additive_coef_f32(const float *out_dev, const float *dout_dev, const float *row_state_dev,
+                                                    const float *er_dev, float *row_coef_dev, int64_t n_dst, int heads,
+                                                    int head_len, void *stream) {
+    if (!er_dev) return fail(FG_ERR_ARG, "null device pointer");
+    return run_coef(out_dev, dout_dev, row_state_dev, er_dev, row_coef_dev, n_dst, heads, head_len, stream);
+}
+
+extern "C" int fg_graph_attention_additive_backward_er_f32(const fg_spmm_plan *pl, const int32_t *pos_dev,
+                                                           const int32_t *idx_dev, const float *el_dev, const float *v_dev,
+                                                           const float *dout_dev, const float *row_coef_dev,
+                                                           float *der_dev, int heads, int head_len,
+                                                           float negative_slope, void *stream) {
+    if (pl == nullptr) return fail(FG_ERR_ARG, "plan is null");
+    if (int rc = check_common(pl, heads, head_len, pl->n_src)) return rc;
+    if (pl->n_dst == 0) return FG_OK;
+    if (!pos_dev || !dout_dev || !row_coef_dev || !der_dev || (pl->nnz > 0 && (!idx_dev || !el_dev || !v_dev)))
+        return fail(FG_ERR_ARG, "null device pointer");
+    if ((((uintptr_t)v_dev | (uintptr_t)dout_dev | (uintptr_t)row_coef_dev) & 15) != 0)
+        return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
+    return run_backward<false, true>(pl, pos_dev, idx_dev, nullptr, dout_dev, nullptr, v_dev, row_coef_dev, nullptr, nullptr,
+                                     heads, head_len, negative_slope, stream, nullptr, el_dev, der_dev);
+}
+
+extern "C" int fg_graph_attention_additive_backward_elv_f32(const fg_spmm_plan *pl, const int32_t *pos_t_dev,
+                                                            const int32_t *idx_t_dev, const float *dout_dev,
+                                                            const float *el_dev, const float *v_dev,
+                                                            const float *row_coef_dev, float *del_dev, float *dv_dev,
+                                                            int heads, int head_len, float negative_slope, void *stream) {
+    if (pl == nullptr) return fail(FG_ERR_ARG, "plan is null");
+    if (int rc = check_common(pl, heads, head_len, pl->n_src)) return rc;
+    if ((uint64_t)pl->n_src * 16u >= (1ull << 32)) return fail(FG_ERR_SHAPE, "attention operands of 4 GiB and more are not supported");
+    if (pl->n_dst == 0) return FG_OK;
+    if (!pos_t_dev || !el_dev || !v_dev || !del_dev || !dv_dev || (pl->nnz > 0 && (!idx_t_dev || !dout_dev || !row_coef_dev)))
+        return fail(FG_ERR_ARG, "null device pointer");
+    if ((((uintptr_t)v_dev | (uintptr_t)dout_dev | (uintptr_t)dv_dev | (uintptr_t)row_coef_dev) & 15) != 0)
+        return fail(FG_ERR_ARG, "attention needs 16-byte aligned arrays");
+    return run_backward<true, true>(pl, pos_t_dev, idx_t_dev, nullptr, v_dev, nullptr, dout_dev, row_coef_dev, nullptr, dv_dev,
+                                    heads, head_len, negative_slope, stream, el_dev, row_coef_dev, del_dev);
 }

@@ -195,6 +195,8 @@ class GraphAttentionhip(object):
         if self._placeholders is None:
             raise RuntimeError("call build() before backward()")
         common.check_inputs([q, k, v], self._placeholders, self._ctx)
+        if self._additive:
+            return self._backward_additive(q, k, v, out, state, grad_out)
         common.check_inputs([out, grad_out], [self._placeholders[0]] * 2, self._ctx)
         L, s = _lib.lib(), common.stream_ptr()
         coef = torch.empty_like(state)
@@ -207,10 +209,7 @@ class GraphAttentionhip(object):
                                                        _lib.dev_ptr(grad_out), _lib.dev_ptr(coef), _lib.dev_ptr(dq),
                                                        self._heads, self._head_len, ctypes.c_float(self._scale), s))
         # partitions over the destinations, sized like the forward pass's over the sources
-        Pt = 1 if lay['P'] == 1 else max(1, tuning._partitions(self._num_rows, 2 * 4 * self._head_len,
-                                                               self._indices.shape[0], self._num_cols,
-                                                               tuning.SPMM_SLICE_BYTES, min_segment=24))
-        lt = self._layout_t(Pt if self._t_parts is None else self._t_parts)
+        lt = self._layout_t(self._dst_partitions(2 * 4 * self._head_len))
         _lib.check(L.fg_graph_attention_backward_kv_f32(lt['plan'], _lib.dev_ptr(lt['pos']), _lib.dev_ptr(lt['idx']),
                                                         _lib.dev_ptr(q), _lib.dev_ptr(grad_out), _lib.dev_ptr(k),
                                                         _lib.dev_ptr(v), _lib.dev_ptr(coef), _lib.dev_ptr(dk),
@@ -218,6 +217,39 @@ class GraphAttentionhip(object):
                                                         ctypes.c_float(self._scale), s))
         self._coef = coef
         return dq, dk, dv
+
+    def _dst_partitions(self, slice_row_bytes):
+        if self._t_parts is not None:
+            return self._t_parts
+        if self._active['P'] == 1:
+            return 1
+        return max(1, tuning._partitions(self._num_rows, slice_row_bytes, self._indices.shape[0], self._num_cols,
+                                         tuning.SPMM_SLICE_BYTES, min_segment=24))
+
+    def _backward_additive(self, er, el, v, out, state, grad_out):
+        """(dEr, dEl, dV) of the additive-score operator."""
+        out_ph = common.placeholder((self._num_rows, self._heads, self._head_len))
+        common.check_inputs([out, grad_out], [out_ph] * 2, self._ctx)
+        L, s = _lib.lib(), common.stream_ptr()
+        H, D = self._heads, self._head_len
+        er_t, el_t = er.t().contiguous(), el.t().contiguous()
+        coef = torch.empty((H, self._num_rows, 4), dtype=torch.float32, device=self._ctx)
+        _lib.check(L.fg_graph_attention_additive_coef_f32(_lib.dev_ptr(out), _lib.dev_ptr(grad_out), _lib.dev_ptr(state),
+                                                          _lib.dev_ptr(er_t), _lib.dev_ptr(coef), self._num_rows, H, D, s))
+        der_t = torch.empty_like(er_t)
+        del_t = torch.empty_like(el_t)
+        dv = torch.empty_like(v)
+        lay = self._active
+        _lib.check(L.fg_graph_attention_additive_backward_er_f32(
+            lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(el_t), _lib.dev_ptr(v),
+            _lib.dev_ptr(grad_out), _lib.dev_ptr(coef), _lib.dev_ptr(der_t), H, D, ctypes.c_float(self._slope), s))
+        lt = self._layout_t(self._dst_partitions(4 * D))
+        _lib.check(L.fg_graph_attention_additive_backward_elv_f32(
+            lt['plan'], _lib.dev_ptr(lt['pos']), _lib.dev_ptr(lt['idx']), _lib.dev_ptr(grad_out), _lib.dev_ptr(el_t),
+            _lib.dev_ptr(v), _lib.dev_ptr(coef), _lib.dev_ptr(del_t), _lib.dev_ptr(dv), H, D,
+            ctypes.c_float(self._slope), s))
+        self._coef = coef
+        return der_t.t().contiguous(), del_t.t().contiguous(), dv
 
     def measure_average_time(self, input_tvm_ndarrays, num_runs):
         if self._placeholders is None:

@@ -221,3 +221,39 @@ def test_additive_scores_against_float64(oracle, H, D, P):
     ref = oracle.graph_attention_additive_f64(adj.indptr, adj.indices, er, el, v, 0.2)
     assert np.isfinite(out).all() and (out[np.diff(adj.indptr) == 0] == 0).all()
     np.testing.assert_allclose(out, ref, rtol=1e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("H,D,P,Pt", [(1, 64, None, None), (4, 64, 2, 3), (8, 32, 3, 2), (8, 16, 5, 4), (3, 64, 1, 4)])
+@pytest.mark.parametrize("tile_major", [0, 1])
+def test_additive_gradients_against_float64(monkeypatch, H, D, P, Pt, tile_major):
+    import torch
+    from featgraph_amd import _lib
+    from featgraph_amd.module import GraphAttentionhip, placeholder
+    if tile_major:
+        monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(tile_major=1))
+    rng = np.random.default_rng(H * 1000 + D * 10 + (P or 0) + 5)
+    adj = _graph(rng, 200, 260, 250, 0.05)
+    er = rng.standard_normal((adj.shape[0], H)).astype("float32")
+    el = (2 * rng.standard_normal((adj.shape[1], H))).astype("float32")
+    v = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    dout = rng.standard_normal((adj.shape[0], H, D)).astype("float32")
+    m = GraphAttentionhip(adj)
+    m.build([placeholder(er.shape), placeholder(el.shape), placeholder(v.shape)], {'scores': 'additive', 'negative_slope': 0.2},
+            {'num_src_partitions': P, 'num_dst_partitions': Pt})
+    erd, eld, vd, dd = (torch.from_numpy(t).cuda() for t in (er, el, v, dout))
+    out = m.run([erd, eld, vd])
+    der, del_, dv = m.backward(erd, eld, vd, out, m.state_tvm, dd)
+    # float64 torch autograd on the dense masked form
+    coo = adj.tocoo()
+    mask = torch.zeros(adj.shape, dtype=torch.bool); mask[coo.row, coo.col] = True
+    er64, el64, v64 = (torch.from_numpy(t).double().requires_grad_() for t in (er, el, v))
+    z = er64.t()[:, :, None] + el64.t()[:, None, :]                      # [H, rows, cols]
+    s = torch.nn.functional.leaky_relu(z, 0.2).masked_fill(~mask, float("-inf"))
+    a = torch.nan_to_num(torch.softmax(s, dim=-1), nan=0.0)
+    ref = torch.einsum("hrc,chd->rhd", a, v64)
+    (ref * torch.from_numpy(dout).double()).sum().backward()
+    np.testing.assert_allclose(out.cpu().numpy(), ref.detach().numpy(), rtol=1e-4, atol=2e-5)
+    for got, want, name in ((der, er64.grad, "d_er"), (del_, el64.grad, "d_el"), (dv, v64.grad, "dv")):
+        got = got.cpu().numpy()
+        assert np.isfinite(got).all(), name
+        np.testing.assert_allclose(got, want.numpy(), rtol=1e-3, atol=1e-4, err_msg=name)
