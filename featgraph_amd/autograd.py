@@ -129,6 +129,22 @@ class Graph(object):
             return _Attention.apply(self, q, k, v, float(scale))
         return self.spmm(v, self.edge_softmax(self.sddmm(k, q) * scale))
 
+    def gat_attention(self, er, el, v, negative_slope=0.2):
+        """The attention of a GAT layer: out[r, h, :] = sum over the edges e into r of
+        softmax_r(leaky_relu(el[col e, h] + er[r, h])) * v[col e, h, :]; er (num_rows, H), el (num_cols, H),
+        v (num_cols, H, D) with D in {16, 32, 64}.  One operator forward, two sweeps backward; no per-edge
+        array is stored."""
+        return _GatAttention.apply(self, er, el, v, float(negative_slope))
+
+    def _gat_mod(self, er, el, v, slope):
+        key = ('gat', tuple(v.shape[1:]), slope)
+        if key not in self._mods:
+            m = GraphAttentionhip(self._csr)
+            m.build([placeholder(tuple(er.shape)), placeholder(tuple(el.shape)), placeholder(tuple(v.shape))],
+                    {'scores': 'additive', 'negative_slope': slope}, {})
+            self._mods[key] = m
+        return self._mods[key]
+
     def _attention_mod(self, q, k, v, scale):
         key = ('attention', tuple(q.shape[1:]), scale)
         if key not in self._mods:
@@ -198,6 +214,24 @@ class _Attention(torch.autograd.Function):
         q, k, v, out, state = ctx.saved_tensors
         dq, dk, dv = ctx.g._attention_mod(q, k, v, ctx.scale).backward(q, k, v, out, state, dout.contiguous())
         return None, dq, dk, dv, None
+
+
+class _GatAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, g, er, el, v, slope):
+        er, el, v = er.contiguous(), el.contiguous(), v.contiguous()
+        mod = g._gat_mod(er, el, v, slope)
+        mod.state_tvm = torch.empty_like(mod.state_tvm)
+        out = _fresh_run(mod, [er, el, v])
+        ctx.g, ctx.slope = g, slope
+        ctx.save_for_backward(er, el, v, out, mod.state_tvm)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        er, el, v, out, state = ctx.saved_tensors
+        der, del_, dv = ctx.g._gat_mod(er, el, v, ctx.slope).backward(er, el, v, out, state, dout.contiguous())
+        return None, der, del_, dv, None
 
 
 class _EdgeSoftmax(torch.autograd.Function):

@@ -112,3 +112,29 @@ def test_attention_with_and_without_gradients():
     ref.square().sum().backward()
     for got, want in ((q.grad, q64.grad), (k.grad, k64.grad), (v.grad, v64.grad)):
         np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=1e-3, atol=1e-4)
+
+
+def test_gat_attention_gradients():
+    """Graph.gat_attention (additive scores through a leaky ReLU) against float64 torch autograd."""
+    import torch
+    from featgraph_amd.autograd import Graph
+    rng = np.random.default_rng(22)
+    adj = sp.random(90, 140, density=0.1, format="csr", random_state=rng).astype("float32")
+    adj.sort_indices()
+    g = Graph(adj)
+    H, D = 4, 16
+    er = torch.from_numpy(rng.standard_normal((90, H)).astype("float32")).cuda().requires_grad_()
+    el = torch.from_numpy(rng.standard_normal((140, H)).astype("float32")).cuda().requires_grad_()
+    v = torch.from_numpy(rng.standard_normal((140, H, D)).astype("float32")).cuda().requires_grad_()
+    out = g.gat_attention(er, el, v, 0.1)
+    out.square().sum().backward()
+    coo = adj.tocoo()
+    mask = torch.zeros((90, 140), dtype=torch.bool); mask[coo.row, coo.col] = True
+    er64, el64, v64 = (t.detach().cpu().double().requires_grad_() for t in (er, el, v))
+    z = er64.t()[:, :, None] + el64.t()[:, None, :]
+    a = torch.nan_to_num(torch.softmax(torch.nn.functional.leaky_relu(z, 0.1).masked_fill(~mask, float("-inf")), dim=-1), nan=0.0)
+    ref = torch.einsum("hrc,chd->rhd", a, v64)
+    ref.square().sum().backward()
+    np.testing.assert_allclose(out.detach().cpu().numpy(), ref.detach().numpy(), rtol=1e-4, atol=2e-5)
+    for got, want in ((er.grad, er64.grad), (el.grad, el64.grad), (v.grad, v64.grad)):
+        np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=1e-3, atol=1e-4)
