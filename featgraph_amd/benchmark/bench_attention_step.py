@@ -5,7 +5,7 @@ adjacency for dQ, one over its transpose for dK and dV).  With --chain: scores =
 over each destination's edges, out = per-head weighted SpMM of V, whose backward pass is three per-head SpMMs
 (two of them on the transposed graph), one multi-head SDDMM and the softmax gradient.
 
-    python -m featgraph_amd.benchmark.bench_attention_step [--workload powerlaw-233k] [--heads 8] [--head-len 64] [--chain]
+    python -m featgraph_amd.benchmark.bench_attention_step [--workload powerlaw-233k] [--heads 8] [--head-len 64] [--chain | --additive]
 
 Prints one JSON line with the mean times (HIP events on the launch stream) of the steps after the first."""
 import argparse
@@ -26,6 +26,8 @@ def main():
     ap.add_argument("--head-len", type=int, default=64)
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--chain", action="store_true", help="the three operators instead of the single one")
+    ap.add_argument("--additive", action="store_true",
+                    help="the additive scores of a GAT layer, leaky_relu(el[col] + er[row]), instead of dot products")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("bench_attention_step needs a GPU")
@@ -35,6 +37,9 @@ def main():
     H, D = args.heads, args.head_len
     gen = torch.Generator(device="cuda"); gen.manual_seed(2)
     q, k, v = (torch.randn((n, H, D), generator=gen, device="cuda").requires_grad_() for _ in range(3))
+    er, el = (torch.randn((n, H), generator=gen, device="cuda").requires_grad_() for _ in range(2))
+    if args.additive and args.chain:
+        raise SystemExit("--additive times the single operator only")
 
     def mark():
         e = torch.cuda.Event(enable_timing=True)
@@ -50,16 +55,16 @@ def main():
             out = g.spmm(v, a); e.append(mark())
         else:
             e += [e[0], e[0]]
-            out = g.attention(q, k, v); e.append(mark())
+            out = g.gat_attention(er, el, v) if args.additive else g.attention(q, k, v); e.append(mark())
         loss = out.square().mean()
         loss.backward(); e.append(mark())
         torch.cuda.synchronize()
         if step > 0:                      # the first step builds the modules and allocates
             times.append([e[i].elapsed_time(e[i + 1]) for i in range(4)])
-        q.grad = k.grad = v.grad = None
+        q.grad = k.grad = v.grad = er.grad = el.grad = None
     t = np.mean(np.array(times), axis=0)
     line = {"workload": args.workload, "nodes": n, "edges": nnz, "heads": H, "head_len": D,
-            "operators": "sddmm + edge_softmax + spmm" if args.chain else "attention"}
+            "operators": "sddmm + edge_softmax + spmm" if args.chain else ("gat_attention" if args.additive else "attention")}
     if args.chain:
         line.update(sddmm_ms=round(float(t[0]), 3), edge_softmax_ms=round(float(t[1]), 3), spmm_ms=round(float(t[2]), 3))
     else:
