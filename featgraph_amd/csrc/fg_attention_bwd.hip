@@ -59,7 +59,6 @@ struct BwdArgs {
     float *res0, *res1;       // [n_own, F]: dQ, or dK and dV
     int F, H;
     int n_heads, head_base;
-    int accumulate;
     float scale;
     // Additive scores leaky_relu(el[c] + er[r]) (ADD): no far0 / own0 slices; instead
     //   rows:    far_s = el [H, n_src] (4 bytes per element), coef holds (m + log l, delta, er[r], 0) per row;
@@ -358,7 +357,7 @@ int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *
             a.coef_head_floats = 2 * (BY_COLUMN ? pl->n_src : pl->n_dst);
             a.own_s = a.far_s = nullptr; a.res_s = nullptr; a.own_s_head_floats = a.far_s_head_floats = 0; a.far_s_bytes = 0;
         }
-        a.res0 = res0; a.res1 = res1; a.F = F; a.H = heads; a.scale = param; a.slope = param; a.accumulate = p > 0;
+        a.res0 = res0; a.res1 = res1; a.F = F; a.H = heads; a.scale = param; a.slope = param;
         const int per_launch = (heads > 8 && heads % 8 == 0) ? 8 : heads;
         for (int hb = 0; hb < heads; hb += per_launch) {
             a.n_heads = per_launch; a.head_base = hb;
