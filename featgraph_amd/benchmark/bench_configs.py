@@ -88,7 +88,14 @@ def run_attention_steps(name, adj, softmax_heads, head_shapes):
         # byte model: indices once, Q, K, V and the output once; flops: two gathered operands per edge
         _line(name, "graph_attention", {"heads": H, "head_len": D, "partitions": g._active['P']}, t, nnz, 2 * H * D,
               4 * (n + 1) + 4 * nnz + 16 * n * H * D)
-        del g, q, k, x
+        # the same with the additive scores of GAT layers: only V is gathered
+        er = torch.randn((n, H), generator=gen, device="cuda")
+        el = torch.randn((n, H), generator=gen, device="cuda")
+        g.build([placeholder((n, H)), placeholder((n, H)), placeholder((n, H, D))], {'scores': 'additive'}, {})
+        t = g.measure_average_time([er, el, x], 5)
+        _line(name, "graph_attention_additive", {"heads": H, "head_len": D, "partitions": g._active['P']}, t, nnz, H * D,
+              4 * (n + 1) + 4 * nnz + 8 * n * H + 8 * n * H * D)
+        del g, q, k, x, er, el
 
 
 def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):
