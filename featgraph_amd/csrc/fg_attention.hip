@@ -71,20 +71,20 @@ __device__ __forceinline__ void running_merge(Running &r, const Running &s) {
     r.m = m;
 }
 
-// What is staged per element: the byte offset of its row in K / V, and, for additive scores, the byte
-// offset of its scalar as well.
+// What is staged per element: the byte offset of its row in K / V, and, for additive scores, its scalar
+// el[col, h] as well (gathered once per item, 64 elements per load, instead of once per step).
 template <bool ADD> struct Staged;
 template <> struct Staged<false> { using type = int32_t; };
 template <> struct Staged<true> { using type = int2; };
 __device__ __forceinline__ uint32_t slice_off(int32_t c) { return (uint32_t)c; }
 __device__ __forceinline__ uint32_t slice_off(const int2 &c) { return (uint32_t)c.x; }
-__device__ __forceinline__ uint32_t scalar_off(int32_t) { return 0u; }
-__device__ __forceinline__ uint32_t scalar_off(const int2 &c) { return (uint32_t)c.y; }
+__device__ __forceinline__ float staged_scalar(int32_t) { return 0.f; }
+__device__ __forceinline__ float staged_scalar(const int2 &c) { return __int_as_float(c.y); }
 
 // NU elements of one row, those with valid[u] counted: all gathers are issued before the first is used,
 // then the scores and the running update.
 //   ADD == false: score = scale * <K[c, h, :], q>  (k: the K slices, this lane's 16 bytes at lane_bytes);
-//   ADD == true : score = leaky_relu(k[c] + q.x) with negative slope `scale`  (k: one scalar per source and head).
+//   ADD == true : score = leaky_relu(el + q.x) with negative slope `scale`  (el: the element's staged scalar).
 template <int L, int NU, bool ADD, typename S>
 __device__ __forceinline__ void update(const S (&c)[NU], const bool (&valid)[NU], const float *k, const float *v,
                                        uint32_t lane_bytes, const float4 &q, float scale, Running &r) {
@@ -92,7 +92,7 @@ __device__ __forceinline__ void update(const S (&c)[NU], const bool (&valid)[NU]
     float ev[NU];
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
-        if constexpr (ADD) ev[u] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(k) + scalar_off(c[u]));
+        if constexpr (ADD) ev[u] = staged_scalar(c[u]);
         else kk[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(k) + (slice_off(c[u]) + lane_bytes));
         vv[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(v) + (slice_off(c[u]) + lane_bytes));
     }
@@ -236,10 +236,13 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
 #pragma unroll
         for (int i = 0; i < 4; ++i) b[i] = (uint32_t)c[i] * a.kv_row_bytes;
         if constexpr (ADD) {
+            int ev[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ev[i] = __float_as_int(kptr[c[i]]);
             int4 *c4 = reinterpret_cast<int4 *>(cols);
-            c4[2 * lane] = make_int4((int)b[0], c[0] * 4, (int)b[1], c[1] * 4);
-            c4[2 * lane + 1] = make_int4((int)b[2], c[2] * 4, (int)b[3], c[3] * 4);
-            if (lane < kPad) cols[fg::kItemEdges + lane] = make_int2((int)b[3], c[3] * 4);
+            c4[2 * lane] = make_int4((int)b[0], ev[0], (int)b[1], ev[1]);
+            c4[2 * lane + 1] = make_int4((int)b[2], ev[2], (int)b[3], ev[3]);
+            if (lane < kPad) cols[fg::kItemEdges + lane] = make_int2((int)b[3], ev[3]);
         } else {
             *reinterpret_cast<int4 *>(cols + 4 * lane) = make_int4((int)b[0], (int)b[1], (int)b[2], (int)b[3]);
             if (lane < kPad) cols[fg::kItemEdges + lane] = (int)b[3];

@@ -40,6 +40,17 @@ __device__ __forceinline__ void shfl_add(float4 &a, int off) {
     a.x += __shfl_xor(a.x, off); a.y += __shfl_xor(a.y, off); a.z += __shfl_xor(a.z, off); a.w += __shfl_xor(a.w, off);
 }
 
+// What is staged per element of a row: the byte offset of the far row's slices and, gathered once per item
+// (64 elements per load) rather than once per step, the far side's scalars:
+//   rows, dot products : nothing more                       rows, additive scores   : el[c, h]
+//   columns            : the destination's (m + log l, delta), and with additive scores its er[r, h]
+template <bool BY_COLUMN, bool ADD> struct FarStaged { using type = int4; };
+template <> struct FarStaged<false, false> { using type = int32_t; };
+template <> struct FarStaged<false, true> { using type = int2; };
+__device__ __forceinline__ uint32_t far_off(int32_t w) { return (uint32_t)w; }
+__device__ __forceinline__ uint32_t far_off(const int2 &w) { return (uint32_t)w.x; }
+__device__ __forceinline__ uint32_t far_off(const int4 &w) { return (uint32_t)w.x; }
+
 // One traversal serves both kernels.  The "own" side is the row of the traversed matrix, the "far" side is
 // what its elements point at:
 //   BY_COLUMN == false (adjacency, rows = destinations): own = (Q[r], dout[r], coef[r]), far = (K[c], V[c]);
@@ -67,15 +78,15 @@ struct BwdArgs {
     const float *own_s, *far_s;
     float *res_s;
     int64_t own_s_head_floats, far_s_head_floats;
-    uint32_t far_s_bytes;     // bytes per far element in far_s (4 or 16)
     float slope;
 };
 
 template <int L, bool BY_COLUMN, bool ACC, bool ADD>
 __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArgs a) {
     constexpr int G = 64 / L, D = 4 * L;
-    // x = far row's byte offset, y = far row's offset into coef (bytes; BY_COLUMN only)
-    __shared__ __align__(16) int2 s_far[kWavesPerBlock][fg::kItemEdges + kPad];
+    constexpr int KU = kU;   // (two steps in flight by column lower the registers from 95 to 74 and change no time)
+    using W = typename FarStaged<BY_COLUMN, ADD>::type;
+    __shared__ __align__(16) W s_far[kWavesPerBlock][fg::kItemEdges + kPad];
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -87,8 +98,7 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
     const int f_lo = head * D + li * 4;
     const uint32_t lane_bytes = a.far_tile_bytes ? (uint32_t)head * a.far_tile_bytes + (uint32_t)li * 16u : (uint32_t)f_lo * 4u;
     const int64_t F = a.F;
-    int2 *far = s_far[wave];
-    const uint32_t coef_row_bytes = ADD ? a.far_s_bytes : 8u;       // second staged word: the far element's scalar data
+    W *far = s_far[wave];
     const float *coef_head = a.coef + (int64_t)head * a.coef_head_floats;
     const float *far_s_head = ADD ? a.far_s + (int64_t)head * a.far_s_head_floats : nullptr;
     const float *own_s_head = (ADD && BY_COLUMN) ? a.own_s + (int64_t)head * a.own_s_head_floats : nullptr;
@@ -97,12 +107,25 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
     auto stage = [&](int64_t base, int n) {
         int32_t c[4];
         fg::load_four(a.indices + base, n, lane, 1, c);
-        int4 *f4 = reinterpret_cast<int4 *>(far);
-        f4[2 * lane] = make_int4((int)((uint32_t)c[0] * a.far_row_bytes), (int)((uint32_t)c[0] * coef_row_bytes),
-                                 (int)((uint32_t)c[1] * a.far_row_bytes), (int)((uint32_t)c[1] * coef_row_bytes));
-        f4[2 * lane + 1] = make_int4((int)((uint32_t)c[2] * a.far_row_bytes), (int)((uint32_t)c[2] * coef_row_bytes),
-                                     (int)((uint32_t)c[3] * a.far_row_bytes), (int)((uint32_t)c[3] * coef_row_bytes));
-        if (lane < kPad) far[fg::kItemEdges + lane] = make_int2((int)((uint32_t)c[3] * a.far_row_bytes), (int)((uint32_t)c[3] * coef_row_bytes));
+        W w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int off = (int)((uint32_t)c[i] * a.far_row_bytes);
+            if constexpr (BY_COLUMN && ADD) {
+                const float4 cf = *reinterpret_cast<const float4 *>(far_s_head + (int64_t)c[i] * 4);
+                w[i] = make_int4(off, __float_as_int(cf.x), __float_as_int(cf.y), __float_as_int(cf.z));
+            } else if constexpr (BY_COLUMN) {
+                const float2 cf = *reinterpret_cast<const float2 *>(coef_head + (int64_t)c[i] * 2);
+                w[i] = make_int4(off, __float_as_int(cf.x), __float_as_int(cf.y), 0);
+            } else if constexpr (ADD) {
+                w[i] = make_int2(off, __float_as_int(far_s_head[c[i]]));
+            } else {
+                w[i] = off;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) far[4 * lane + i] = w[i];
+        if (lane < kPad) far[fg::kItemEdges + lane] = w[3];
     };
 
     // NU steps of one row for this lane group (elements s0 + g, s0 + g + G, ...; only the last step may have
@@ -112,37 +135,32 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
         constexpr int NU = decltype(nu_tag)::value;
         constexpr bool ALLVALID = decltype(allvalid_tag)::value;
         const bool last_valid = ALLVALID || s0 + (NU - 1) * G + g < e;
-        int2 w[NU];
+        W w[NU];
 #pragma unroll
         for (int u = 0; u < NU; ++u) w[u] = far[(u < NU - 1 || last_valid) ? s0 + u * G + g : e - 1];
-        float4 f0[NU], f1[NU], cf4[NU];
-        float2 cf[NU];
-        float ev[NU];
+        float4 f0[NU], f1[NU];
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
-            if constexpr (!ADD) f0[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far0) + ((uint32_t)w[u].x + lane_bytes));
-            f1[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far1) + ((uint32_t)w[u].x + lane_bytes));
-            if constexpr (ADD) {
-                if (BY_COLUMN) cf4[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(far_s_head) + (uint32_t)w[u].y);
-                else ev[u] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(far_s_head) + (uint32_t)w[u].y);
-            } else if (BY_COLUMN) {
-                cf[u] = *reinterpret_cast<const float2 *>(reinterpret_cast<const char *>(coef_head) + (uint32_t)w[u].y);
-            }
+            if constexpr (!ADD) f0[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far0) + (far_off(w[u]) + lane_bytes));
+            f1[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(a.far1) + (far_off(w[u]) + lane_bytes));
         }
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
             // rows: o0 = Q[r], o1 = dout[r], f0 = K[c], f1 = V[c];  columns: o0 = K[c], o1 = V[c], f0 = Q[r], f1 = dout[r]
-            // ADD: o0.x = the own scalar (er[r] | el[c]) and the far one comes from ev (el[c]) | cf4.z (er[r])
-            float s, gate = 1.f;
+            // ADD: o0.x = the own scalar (er[r] | el[c]); the far one (el[c] | er[r]) was staged with the offsets
+            float s, gate = 1.f, cc = c1, dd = delta;
+            if constexpr (BY_COLUMN) { cc = __int_as_float(w[u].y); dd = __int_as_float(w[u].z); }
             if constexpr (ADD) {
-                const float z = o0.x + (BY_COLUMN ? cf4[u].z : ev[u]);
+                float far_scalar;
+                if constexpr (BY_COLUMN) far_scalar = __int_as_float(w[u].w);
+                else far_scalar = __int_as_float(w[u].y);
+                const float z = o0.x + far_scalar;
                 gate = z > 0.f ? 1.f : a.slope;
                 s = z * gate;
             } else {
                 s = group_sum<L>(dot4(f0[u], o0)) * a.scale;
             }
             const float da = group_sum<L>(dot4(f1[u], o1));
-            const float cc = BY_COLUMN ? (ADD ? cf4[u].x : cf[u].x) : c1, dd = BY_COLUMN ? (ADD ? cf4[u].y : cf[u].y) : delta;
             float p = __expf(s - cc);                       // the softmax value; cc = +inf for rows without edges
             if (!(u < NU - 1 || last_valid)) p = 0.f;
             const float ds = p * (da - dd);
@@ -158,13 +176,13 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
     auto walk = [&](int b, int e, const float4 &o0, const float4 &o1, float c1, float delta, float4 &accA, float4 &accB, float &accS) {
         using std::integral_constant;
         int s0 = b;
-        for (; s0 + G * kU <= e; s0 += G * kU)
-            batch(integral_constant<int, kU>(), integral_constant<bool, true>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
+        for (; s0 + G * KU <= e; s0 += G * KU)
+            batch(integral_constant<int, KU>(), integral_constant<bool, true>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
         if (s0 >= e) return;
         const int nu = (e - s0 + G - 1) / G;
-        static_assert(kU == 4, "the tail below lists the step counts");
+        static_assert(KU == 2 || KU == 4, "the tail below lists the step counts");
         if (nu == 1) batch(integral_constant<int, 1>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
-        else if (nu == 2) batch(integral_constant<int, 2>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
+        else if (KU == 2 || nu == 2) batch(integral_constant<int, 2>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
         else if (nu == 3) batch(integral_constant<int, 3>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
         else batch(integral_constant<int, 4>(), integral_constant<bool, false>(), s0, e, o0, o1, c1, delta, accA, accB, accS);
     };
@@ -351,11 +369,10 @@ int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *
             a.coef = coef_dev; a.coef_head_floats = 4 * pl->n_dst;       // rows only: the own rows' 16-byte coef
             a.own_s = own_s; a.own_s_head_floats = pl->n_dst; a.res_s = res_s;
             a.far_s = far_s + (int64_t)p * width * far_s_floats; a.far_s_head_floats = (int64_t)far_s_floats * pl->n_src;
-            a.far_s_bytes = 4u * far_s_floats;
         } else {
             a.coef = BY_COLUMN ? coef_dev + (int64_t)p * width * 2 : coef_dev;
             a.coef_head_floats = 2 * (BY_COLUMN ? pl->n_src : pl->n_dst);
-            a.own_s = a.far_s = nullptr; a.res_s = nullptr; a.own_s_head_floats = a.far_s_head_floats = 0; a.far_s_bytes = 0;
+            a.own_s = a.far_s = nullptr; a.res_s = nullptr; a.own_s_head_floats = a.far_s_head_floats = 0;
         }
         a.res0 = res0; a.res1 = res1; a.F = F; a.H = heads; a.scale = param; a.slope = param;
         const int per_launch = (heads > 8 && heads % 8 == 0) ? 8 : heads;
