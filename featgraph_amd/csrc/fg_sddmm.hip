@@ -831,7 +831,7 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
     // The gathers of an XCD touch one tile's slice of every src row, F * 4 bytes apart; from a copy
     // that stores each tile's slices back to back the same working set is cached better
     // (232,965-node graph, F=512: 14.5 -> 13.7 ms with 4 tiles x 16 partitions, 14.9 -> 13.5 ms with
-    // 8 x 8, before the 0.25 ms of the copy).  The destination rows gain nothing from it.
+    // 8 x 8, before the 0.15 ms of the copy).  The destination rows gain nothing from it.
     if (off32 && pl->nnz > 0 && ((uintptr_t)src_dev & 15) == 0 &&
         fg::wants_tile_major(pl, T, (uint64_t)pl->n_src * (uint64_t)F * 4u)) {
         int rc = fg::make_tile_major(pl, src_dev, pl->n_src, F, tile_w, stream);
