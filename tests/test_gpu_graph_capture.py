@@ -60,3 +60,51 @@ def test_spmm_sddmm_softmax_replay():
         assert torch.equal(g_a, e_a), "edge softmax replay %d differs from the eager run" % k
         ref = adj.astype(np.float64).dot(x.cpu().numpy().astype(np.float64))
         np.testing.assert_allclose(g_out.cpu().numpy(), ref, rtol=RTOL, atol=1e-4)
+
+
+@pytest.mark.parametrize("scores", ["dot", "additive"])
+def test_attention_replay(scores):
+    """Forward and gradient kernels of the attention operator recorded once and replayed on new inputs."""
+    import torch
+    from featgraph_amd.module import GraphAttentionhip, placeholder
+    rng = np.random.default_rng(5)
+    n_dst, n_src, H, D = 400, 600, 4, 32
+    adj = sp.random(n_dst, n_src, density=0.05, format="csr", random_state=rng).astype("float32").tolil()
+    adj[3, rng.choice(n_src, size=550, replace=False)] = 1.0
+    adj[5, :] = 0
+    adj = adj.tocsr().astype("float32"); adj.eliminate_zeros(); adj.sort_indices()
+    m = GraphAttentionhip(adj)
+    v = torch.zeros((n_src, H, D), device="cuda")
+    d = torch.zeros((n_dst, H, D), device="cuda")
+    if scores == "additive":
+        a = torch.zeros((n_dst, H), device="cuda"); b = torch.zeros((n_src, H), device="cuda")
+        m.build([placeholder(a.shape), placeholder(b.shape), placeholder(v.shape)], {'scores': 'additive'},
+                {'num_src_partitions': 3, 'num_dst_partitions': 2})
+    else:
+        a = torch.zeros((n_dst, H, D), device="cuda"); b = torch.zeros((n_src, H, D), device="cuda")
+        m.build([placeholder(a.shape), placeholder(b.shape), placeholder(v.shape)], {},
+                {'num_src_partitions': 3, 'num_dst_partitions': 2})
+
+    def step():
+        out = m.run([a, b, v])
+        return (out,) + tuple(m.backward(a, b, v, out, m.state_tvm, d))
+
+    step()                                                 # first call: plans' scratch is allocated here
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        recorded = step()
+    gen = torch.Generator(device="cuda")
+    for k in range(3):
+        gen.manual_seed(20 + k)
+        for t in (a, b, v, d):
+            t.copy_(torch.randn(t.shape, generator=gen, device="cuda"))
+        eager = tuple(t.clone() for t in step())
+        torch.cuda.synchronize()
+        for t in recorded:
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for i, (r, e) in enumerate(zip(recorded, eager)):
+            assert torch.isfinite(e).all()
+            assert torch.equal(r, e), "replay %d: result %d differs from the eager run" % (k, i)
