@@ -1,7 +1,10 @@
 """Seeded random sweep over graph shapes, densities, feature lengths, partition and tile counts:
 every case is compared with the CPU oracle / float64 closed forms.  The point is breadth -- kernel
 variants and boundary conditions that the hand-picked cases may not reach.  Half of the SpMM and SDDMM
-seeds run with the tile-by-tile copy of the gathered operand forced on."""
+seeds run with the tile-by-tile copy of the gathered operand forced on.  FG_TEST_SEED_BASE=<int> in the
+environment shifts every seed, for sweeps beyond the committed cases."""
+import os
+
 import numpy as np
 import pytest
 import scipy.sparse as sp
@@ -9,6 +12,8 @@ import scipy.sparse as sp
 from helpers import RTOL, ATOL, assert_sum_close, spmm_mass, sddmm_mass
 
 pytestmark = pytest.mark.gpu
+
+SEED_BASE = int(os.environ.get("FG_TEST_SEED_BASE", "0"))
 
 FEATS = [1, 2, 3, 4, 5, 8, 12, 16, 20, 31, 32, 48, 64, 65, 96, 100, 128, 160, 192, 256, 257, 320, 384, 512, 768, 1024]
 
@@ -35,7 +40,7 @@ def test_random_spmm(oracle, monkeypatch, seed):
     from featgraph_amd.module import VanillaSpMMhip, placeholder
     if seed % 2:        # odd seeds: gather from the tile-by-tile copy wherever the kernel allows it
         monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(tile_major=1))
-    rng = np.random.default_rng(1000 + seed)
+    rng = np.random.default_rng(SEED_BASE + 1000 + seed)
     for case in range(20):
         adj = _random_graph(rng)
         F = int(rng.choice(FEATS))
@@ -59,7 +64,7 @@ def test_random_sddmm(oracle, monkeypatch, seed):
     from featgraph_amd.module import VanillaSDDMMhip, MultiHeadSDDMMhip, placeholder
     if seed % 2:
         monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(tile_major=1))
-    rng = np.random.default_rng(2000 + seed)
+    rng = np.random.default_rng(SEED_BASE + 2000 + seed)
     for case in range(20):
         adj = _random_graph(rng)
         coo = adj.tocoo()
@@ -94,7 +99,7 @@ def test_random_sddmm(oracle, monkeypatch, seed):
 def test_random_softmax_and_aggregation(oracle, seed):
     import torch
     from featgraph_amd.module import EdgeSoftmaxhip, GSpMMhip, placeholder
-    rng = np.random.default_rng(3000 + seed)
+    rng = np.random.default_rng(SEED_BASE + 3000 + seed)
     for case in range(20):
         adj = _random_graph(rng)
         H = int(rng.choice([1, 2, 3, 4, 5, 8, 16, 64]))
@@ -126,7 +131,7 @@ def test_random_attention(oracle, monkeypatch, seed):
     from featgraph_amd.module import GraphAttentionhip, placeholder
     if seed % 2:
         monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(tile_major=1))
-    rng = np.random.default_rng(4000 + seed)
+    rng = np.random.default_rng(SEED_BASE + 4000 + seed)
     for case in range(10):
         adj = _random_graph(rng)
         H = int(rng.choice([1, 2, 3, 4, 8, 9, 16]))
