@@ -27,6 +27,7 @@ def _ragged(rng, kind):
     else:                                    # single-row items and split rows
         lens = rng.integers(0, 60, size=120)
         lens[7] = 300; lens[40] = 1024; lens[41] = 1025; lens[90] = 5000
+        lens[91] = 4096; lens[92] = 4097; lens[93] = 2049; lens[94] = 129     # either side of the workgroups' capacities at H = 8
     lens[::11] = 0
     lens[3] = 1
     indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
