@@ -375,3 +375,59 @@ def test_gspmm_arg_closed_form(oracle):
             msgs = adj.data[b:e, None] * x[adj.indices[b:e]]
             assert np.array_equal(arg[r], b + pick(msgs, axis=0))
             assert np.array_equal(out[r], msgs[arg[r] - b, np.arange(6)])
+
+
+# ---- attention in one operator: the dense masked form ---------------------------------
+
+def _dense_attention(adj, scores, v):
+    """softmax over each row's stored columns of a dense [H, n_dst, n_src] score array, times V, with torch in
+    float64; rows without stored columns give 0."""
+    import torch
+    mask = torch.from_numpy(adj.toarray() != 0)
+    s = torch.from_numpy(scores).masked_fill(~mask[None], float("-inf"))
+    a = torch.nan_to_num(torch.softmax(s, dim=2), nan=0.0)          # rows of -inf only: nan -> 0
+    return torch.einsum("hvu,uhd->vhd", a, torch.from_numpy(np.asarray(v, dtype=np.float64))).numpy()
+
+
+def test_graph_attention_dense_form(oracle):
+    rng = np.random.default_rng(21)
+    adj = _rand_csr(rng, 23, 31, 0.2)
+    adj = adj.tolil(); adj[4, :] = 0; adj[9, :] = 1; adj = adj.tocsr(); adj.eliminate_zeros(); adj.sort_indices()
+    H, D = 3, 8
+    q = rng.standard_normal((23, H, D)); k = rng.standard_normal((31, H, D)); v = rng.standard_normal((31, H, D))
+    scale = 0.37
+    got = oracle.graph_attention_f64(adj.indptr, adj.indices, q.astype("float32"), k.astype("float32"),
+                                     v.astype("float32"), scale)
+    f32 = lambda a: a.astype("float32").astype(np.float64)
+    ref = _dense_attention(adj, scale * np.einsum("vhd,uhd->hvu", f32(q), f32(k)), f32(v))
+    np.testing.assert_allclose(got, ref, rtol=1e-12, atol=1e-13)
+    assert (got[4] == 0).all()
+    # one stored column: the output is that column's V, whatever the scores
+    one = sp.csr_matrix((np.ones(1), ([0], [5])), shape=(1, 31))
+    np.testing.assert_allclose(oracle.graph_attention_f64(one.indptr, one.indices, q[:1], k, v, 5.0)[0], v[5], rtol=1e-14)
+    # swapping the roles of two heads permutes the output's heads (catches a head mixed into another)
+    perm = [2, 0, 1]
+    swapped = oracle.graph_attention_f64(adj.indptr, adj.indices, q[:, perm], k[:, perm], v[:, perm], scale)
+    np.testing.assert_allclose(swapped, oracle.graph_attention_f64(adj.indptr, adj.indices, q, k, v, scale)[:, perm], rtol=1e-13)
+
+
+def test_graph_attention_additive_dense_form(oracle):
+    rng = np.random.default_rng(22)
+    adj = _rand_csr(rng, 19, 27, 0.25)
+    adj = adj.tolil(); adj[2, :] = 0; adj = adj.tocsr(); adj.eliminate_zeros(); adj.sort_indices()
+    H, D = 4, 6
+    er = rng.standard_normal((19, H)); el = rng.standard_normal((27, H)); v = rng.standard_normal((27, H, D))
+    slope = 0.2
+    got = oracle.graph_attention_additive_f64(adj.indptr, adj.indices, er, el, v, slope)
+    z = el.T[:, None, :] + er.T[:, :, None]                          # [H, n_dst, n_src]
+    ref = _dense_attention(adj, np.maximum(z, 0) + slope * np.minimum(z, 0), v)
+    np.testing.assert_allclose(got, ref, rtol=1e-12, atol=1e-13)
+    assert (got[2] == 0).all()
+    # a shift of er moves every score of a row on the positive side by the same amount: nothing changes there
+    pos = oracle.graph_attention_additive_f64(adj.indptr, adj.indices, er + 50.0, np.abs(el), v, slope)
+    pos2 = oracle.graph_attention_additive_f64(adj.indptr, adj.indices, er + 70.0, np.abs(el), v, slope)
+    np.testing.assert_allclose(pos, pos2, rtol=1e-9)
+    # slope 1 makes the score el + er, and er cancels in the softmax
+    lin = oracle.graph_attention_additive_f64(adj.indptr, adj.indices, er, el, v, 1.0)
+    lin0 = oracle.graph_attention_additive_f64(adj.indptr, adj.indices, np.zeros_like(er), el, v, 1.0)
+    np.testing.assert_allclose(lin, lin0, rtol=1e-9, atol=1e-12)
