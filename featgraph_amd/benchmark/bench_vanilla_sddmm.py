@@ -16,11 +16,17 @@ from ..module import VanillaSDDMMhip, placeholder
 from .common import exp_range, load_adjacency, report
 
 
-def bench_vanilla_sddmm(adj_scipy_coo, feat_len, max_partitions=8, num_runs=5):
+def bench_vanilla_sddmm(adj_scipy_coo, feat_len, max_partitions=8, num_runs=5, src_feat=None, dst_feat=None,
+                        collect=None):
+    """Times every sweep point.  src_feat / dst_feat: the features to use (default: U[0,1) like the
+    reference, bench_vanilla_sddmm.py:31-32); collect: a list that receives (knobs, seconds, output in
+    the ORIGINAL stored edge order as a numpy array) per point, for callers that check the results."""
     num_rows, num_cols = adj_scipy_coo.shape
     nnz = adj_scipy_coo.nnz
-    src_feat = torch.rand((num_cols, feat_len), device="cuda", dtype=torch.float32)
-    dst_feat = torch.rand((num_rows, feat_len), device="cuda", dtype=torch.float32)
+    if src_feat is None:
+        src_feat = torch.rand((num_cols, feat_len), device="cuda", dtype=torch.float32)
+    if dst_feat is None:
+        dst_feat = torch.rand((num_rows, feat_len), device="cuda", dtype=torch.float32)
     bytes_model = 8 * nnz + 4 * (num_rows + num_cols) * feat_len + 4 * nnz
     phs = [placeholder((num_cols, feat_len)), placeholder((num_rows, feat_len))]
 
@@ -32,6 +38,11 @@ def bench_vanilla_sddmm(adj_scipy_coo, feat_len, max_partitions=8, num_runs=5):
             print("# skipped %s: %s" % (knobs, e))
             return
         report("sddmm", knobs, tcost, nnz, feat_len, bytes_model)
+        if collect is not None:
+            out = module.run([src_feat, dst_feat]).cpu().numpy().copy()
+            if module._edge_mapping is not None:
+                out = out[module.edge_mapping]
+            collect.append((knobs, tcost, out))
 
     module = VanillaSDDMMhip(adj_scipy_coo)
     run(module, {"order": "auto"}, {})

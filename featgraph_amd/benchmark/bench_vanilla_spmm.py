@@ -17,16 +17,22 @@ from ..module import VanillaSpMMhip, placeholder
 from .common import exp_range, load_adjacency, report
 
 
-def bench_vanilla_spmm(adj_scipy_csr, feat_len, max_col_partitions=32, num_runs=5):
+def bench_vanilla_spmm(adj_scipy_csr, feat_len, max_col_partitions=32, num_runs=5, src_feat=None, collect=None):
+    """Times every sweep point.  src_feat: the source features to use (default: U[0,1) like the
+    reference's np.random.random, bench_vanilla_spmm.py:29); collect: a list that receives
+    (knobs, seconds, output as a numpy array) per point, for callers that check the results."""
     num_rows, num_cols = adj_scipy_csr.shape
     nnz = adj_scipy_csr.nnz
-    src_feat = torch.rand((num_cols, feat_len), device="cuda", dtype=torch.float32)   # U[0,1) as the reference
+    if src_feat is None:
+        src_feat = torch.rand((num_cols, feat_len), device="cuda", dtype=torch.float32)
     bytes_model = 4 * (num_rows + 1) + 8 * nnz + 4 * num_cols * feat_len + 4 * num_rows * feat_len
 
     def run(module, knobs, compute_args, schedule_args):
         module.build([placeholder((num_cols, feat_len))], compute_args, schedule_args)
         tcost = module.measure_average_time([src_feat], num_runs)
         report("spmm", knobs, tcost, nnz, feat_len, bytes_model)
+        if collect is not None:
+            collect.append((knobs, tcost, module.run([src_feat]).cpu().numpy().copy()))
 
     module = VanillaSpMMhip(adj_scipy_csr)
     run(module, {"num_col_partitions": "auto", "num_feat_partitions": "auto"}, {}, {})

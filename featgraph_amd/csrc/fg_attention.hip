@@ -118,9 +118,12 @@ __device__ __forceinline__ void update(const S (&c)[NU], const bool (&valid)[NU]
     r.m = m;
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
-        const float p = __expf(s[u] - m);
+        const float p = __expf(s[u] - m);      // 0 for a slot without an element
         r.l += p;
-        r.acc.x += p * vv[u].x; r.acc.y += p * vv[u].y; r.acc.z += p * vv[u].z; r.acc.w += p * vv[u].w;
+        // such a slot's V slice (a re-read or a later row's element) is dropped by a select: a product
+        // with p = 0 would turn a non-finite row of V into NaN in rows that do not reference it
+        const float4 w = valid[u] ? vv[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+        r.acc.x += p * w.x; r.acc.y += p * w.y; r.acc.z += p * w.z; r.acc.w += p * w.w;
     }
 }
 
@@ -367,7 +370,7 @@ void launch(bool first, dim3 grid, hipStream_t st, const AttnArgs &a) {
 // The passes over the source partitions.  ADD == false: q / k are the [n, F] operands of the dot products and
 // `param` their scale; ADD == true: q = er [H, n_dst], k = el [H, n_src] and `param` the leaky ReLU's slope.
 template <bool ADD>
-int run_forward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev, const float *q_dev,
+int run_forward(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev, const float *q_dev,
                 const float *k_dev, const float *v_dev, float *out_dev, float *row_state_dev, int heads,
                 int head_len, float param, void *stream) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
@@ -384,16 +387,16 @@ int run_forward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *i
     const int F = heads * head_len;
     if ((uint64_t)pl->n_src * (uint64_t)F * 4u >= (1ull << 32) || (uint64_t)pl->n_dst * (uint64_t)F >= (1ull << 32))
         return fail(FG_ERR_SHAPE, "attention operands of 4 GiB and more are not supported");
-    int rc = FG_OK;
-    if (!row_state_dev) {
-        if ((rc = fg::ensure_scratch(pl, (size_t)pl->n_dst * heads * 2)) != FG_OK) return rc;
-        row_state_dev = pl->partial_dev;
-    }
+    fg::ScratchNeed need;
+    int rc = fg::attention_scratch_need(pl, heads, head_len, ADD, !row_state_dev, &need);
+    if (rc == FG_OK) rc = fg::ensure_scratch(pl, need, stream);
+    if (rc != FG_OK) return rc;
+    if (!row_state_dev) row_state_dev = pl->partial_dev;
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
     // the gathered [n_src, F] operands head by head, as the SpMM kernels gather X tile by tile
-    const bool tiled = pl->nnz > 0 && fg::wants_tile_major(pl, heads, (uint64_t)pl->n_src * (uint64_t)F * 4u);
+    const bool tiled = need.tiled > 0;
     const float *k = k_dev, *v = v_dev;
     if (tiled) {
         const int slots = ADD ? 1 : 2;
@@ -439,13 +442,29 @@ int run_forward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *i
 
 }  // namespace
 
-extern "C" int fg_graph_attention_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
+namespace fg {
+// The rows' (max, sum) state when the caller passes none, and the head-by-head copies of the gathered
+// operands (V, and K for dot-product scores); the gradient kernels need the same copies and no state.
+int attention_scratch_need(const fg_spmm_plan *pl, int heads, int head_len, bool additive, bool own_row_state,
+                           ScratchNeed *need) {
+    if (heads < 1 || !(head_len == 16 || head_len == 32 || head_len == 64))
+        return fail(FG_ERR_SHAPE, "attention takes heads of 16, 32 or 64 floats, got %d heads of %d", heads, head_len);
+    const uint64_t F = (uint64_t)heads * head_len;
+    need->partial = own_row_state ? (size_t)pl->n_dst * heads * 2 : 0;
+    need->tiled = 0;
+    if (pl->nnz > 0 && wants_tile_major(pl, heads, (uint64_t)pl->n_src * F * 4u))
+        need->tiled = (size_t)pl->n_src * F * (additive ? 1 : 2);
+    return FG_OK;
+}
+}  // namespace fg
+
+extern "C" int fg_graph_attention_f32(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
                                       const float *q_dev, const float *k_dev, const float *v_dev, float *out_dev,
                                       float *row_state_dev, int heads, int head_len, float scale, void *stream) {
     return run_forward<false>(pl, pos_dev, idx_dev, q_dev, k_dev, v_dev, out_dev, row_state_dev, heads, head_len, scale, stream);
 }
 
-extern "C" int fg_graph_attention_additive_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
+extern "C" int fg_graph_attention_additive_f32(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
                                                const float *er_dev, const float *el_dev, const float *v_dev,
                                                float *out_dev, float *row_state_dev, int heads, int head_len,
                                                float negative_slope, void *stream) {

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
     };
 
     // NU steps of one row for this lane group (elements s0 + g, s0 + g + G, ...; only the last step may have
-    // groups without an element, which re-read element e - 1 and give it no weight).
+    // groups without an element, which re-read element e - 1 and discard it).
     auto batch = [&](auto nu_tag, auto allvalid_tag, int s0, int e, const float4 &o0, const float4 &o1, float c1, float delta,
                      float4 &accA, float4 &accB, float &accS) {
         constexpr int NU = decltype(nu_tag)::value;
@@ -162,8 +162,14 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
             }
             const float da = group_sum<L>(dot4(f1[u], o1));
             float p = __expf(s - cc);                       // the softmax value; cc = +inf for rows without edges
-            if (!(u < NU - 1 || last_valid)) p = 0.f;
-            const float ds = p * (da - dd);
+            float ds = p * (da - dd);
+            if (!(u < NU - 1 || last_valid)) {
+                // a group without an element: nothing of what it re-read may reach the sums (selects, not
+                // products with zero, so that non-finite operands stay in the rows that reference them)
+                p = 0.f; ds = 0.f;
+                if constexpr (!ADD) f0[u] = zero4();
+                f1[u] = zero4();
+            }
             if constexpr (ADD) {
                 accS += ds * gate;                                                  // d_er[r] | d_el[c]
                 if (BY_COLUMN) fma4(accB, p, f1[u]);                                // dV += a * dout[r]
@@ -332,7 +338,7 @@ int check_common(const fg_spmm_plan *pl, int heads, int head_len, int64_t n_far_
 // ADD (additive scores): far0 / own0 are not used; own_s / far_s / res_s as described at BwdArgs, coef_dev is
 // the 16-byte form.
 template <bool BY_COLUMN, bool ADD>
-int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev, const float *own0,
+int run_backward(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev, const float *own0,
                  const float *own1, const float *far0_dev, const float *far1_dev, const float *coef_dev,
                  float *res0, float *res1, int heads, int head_len, float param, void *stream,
                  const float *own_s = nullptr, const float *far_s = nullptr, float *res_s = nullptr) {
@@ -340,8 +346,11 @@ int run_backward(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
-    int rc = FG_OK;
-    const bool tiled = pl->nnz > 0 && fg::wants_tile_major(pl, heads, (uint64_t)pl->n_src * (uint64_t)F * 4u);
+    fg::ScratchNeed need;
+    int rc = fg::attention_scratch_need(pl, heads, head_len, ADD, false, &need);
+    if (rc == FG_OK) rc = fg::ensure_scratch(pl, need, stream);
+    if (rc != FG_OK) return rc;
+    const bool tiled = need.tiled > 0;
     const float *far0 = far0_dev, *far1 = far1_dev;
     if (tiled) {
         const int slots = ADD ? 1 : 2;
@@ -417,7 +426,7 @@ extern "C" int fg_graph_attention_coef_f32(const float *out_dev, const float *do
     return run_coef(out_dev, dout_dev, row_state_dev, nullptr, row_coef_dev, n_dst, heads, head_len, stream);
 }
 
-extern "C" int fg_graph_attention_backward_q_f32(const fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
+extern "C" int fg_graph_attention_backward_q_f32(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev,
                                                  const float *q_dev, const float *k_dev, const float *v_dev,
                                                  const float *dout_dev, const float *row_coef_dev, float *dq_dev,
                                                  int heads, int head_len, float scale, void *stream) {
@@ -432,7 +441,7 @@ extern "C" int fg_graph_attention_backward_q_f32(const fg_spmm_plan *pl, const i
                                heads, head_len, scale, stream);
 }
 
-extern "C" int fg_graph_attention_backward_kv_f32(const fg_spmm_plan *pl, const int32_t *pos_t_dev, const int32_t *idx_t_dev,
+extern "C" int fg_graph_attention_backward_kv_f32(fg_spmm_plan *pl, const int32_t *pos_t_dev, const int32_t *idx_t_dev,
                                                   const float *q_dev, const float *dout_dev, const float *k_dev,
                                                   const float *v_dev, const float *row_coef_dev, float *dk_dev,
                                                   float *dv_dev, int heads, int head_len, float scale, void *stream) {
@@ -455,7 +464,7 @@ extern "C" int fg_graph_attention_additive_coef_f32(const float *out_dev, const 
     return run_coef(out_dev, dout_dev, row_state_dev, er_dev, row_coef_dev, n_dst, heads, head_len, stream);
 }
 
-extern "C" int fg_graph_attention_additive_backward_er_f32(const fg_spmm_plan *pl, const int32_t *pos_dev,
+extern "C" int fg_graph_attention_additive_backward_er_f32(fg_spmm_plan *pl, const int32_t *pos_dev,
                                                            const int32_t *idx_dev, const float *el_dev, const float *v_dev,
                                                            const float *dout_dev, const float *row_coef_dev,
                                                            float *der_dev, int heads, int head_len,
@@ -471,7 +480,7 @@ extern "C" int fg_graph_attention_additive_backward_er_f32(const fg_spmm_plan *p
                                      heads, head_len, negative_slope, stream, nullptr, el_dev, der_dev);
 }
 
-extern "C" int fg_graph_attention_additive_backward_elv_f32(const fg_spmm_plan *pl, const int32_t *pos_t_dev,
+extern "C" int fg_graph_attention_additive_backward_elv_f32(fg_spmm_plan *pl, const int32_t *pos_t_dev,
                                                             const int32_t *idx_t_dev, const float *dout_dev,
                                                             const float *el_dev, const float *v_dev,
                                                             const float *row_coef_dev, float *del_dev, float *dv_dev,

@@ -60,32 +60,46 @@ struct fg_spmm_plan {
     fg::Item *items_dev = nullptr;
     int64_t *item_off_dev = nullptr;     // item_off on the device (num_col_partitions + 1 entries)
     fg::Fixup *fixups_dev = nullptr;
-    // partial sums of split rows; grown on demand to max_slots_in_partition * F floats
-    mutable float *partial_dev = nullptr;
-    mutable size_t partial_floats = 0;
-    // tile-by-tile copy of the source features of the call in progress; grown on demand
-    mutable float *tiled_dev = nullptr;
-    mutable size_t tiled_floats = 0;
+    // Scratch that the operator calls fill and read (partial sums of split rows, per-tile partial scores,
+    // softmax statistics, attention row state); grown by fg_spmm_plan_reserve or by the first call that
+    // needs more, never shrunk.
+    float *partial_dev = nullptr;
+    size_t partial_floats = 0;
+    // tile-by-tile copy of the gathered operand(s) of the call in progress; grown the same way
+    float *tiled_dev = nullptr;
+    size_t tiled_floats = 0;
     // statistics for fg_spmm_plan_describe
     int64_t max_len = 0, n_empty = 0, n_split_rows = 0, n_multi_items = 0;
 };
 
 namespace fg {
-// Makes plan->partial_dev hold at least floats_per_piece floats for every piece of split rows of
-// one partition (grown on demand, never shrunk).
-int ensure_partial(const fg_spmm_plan *plan, size_t floats_per_piece);
+// Device scratch one operator call needs from its plan, in floats.
+struct ScratchNeed {
+    size_t partial = 0;   // plan->partial_dev
+    size_t tiled = 0;     // plan->tiled_dev
+};
+// Makes the plan's two scratch buffers hold at least `need` (grown on demand, never shrunk).  Growing
+// frees and allocates device memory, which synchronises the device and cannot be recorded: when `stream`
+// is being captured into a graph and a buffer is too small, nothing is changed and FG_ERR_ARG is returned
+// (reserve the scratch with fg_spmm_plan_reserve, or run the call once, before capturing).
+int ensure_scratch(fg_spmm_plan *plan, const ScratchNeed &need, void *stream);
 // Whether a call with n_tiles feature tiles over a source matrix of x_bytes gathers from a
 // tile-by-tile copy (the plan's tile_major option; the kernel-side conditions are the caller's).
 bool wants_tile_major(const fg_spmm_plan *plan, int n_tiles, uint64_t x_bytes);
 // plan->tiled_dev[(t * n_rows + r) * tile + i] = x[r * F + t * tile + i] for the F / tile tiles of
 // an [n_rows, F] matrix (F and tile multiples of 4, x 16-byte aligned, fewer than 2^32 floats),
-// on `stream`.  The buffer is grown on demand and never shrunk.
-// With n_slots > 1 the buffer holds that many copies of this size one after the other and the call fills
-// copy `slot` (fill slot 0 first: growing the buffer discards what it held).
+// on `stream`.  With n_slots > 1 the buffer holds that many copies of this size one after the other and
+// the call fills copy `slot`.  The buffer must already be large enough (ensure_scratch).
 int make_tile_major(const fg_spmm_plan *plan, const float *x, int64_t n_rows, int F, int tile, void *stream,
                     int slot = 0, int n_slots = 1);
-// Makes plan->partial_dev hold at least `floats` floats (grown on demand, never shrunk).
-int ensure_scratch(const fg_spmm_plan *plan, size_t floats);
 // FG_OK when the calling thread's current device is the one the plan was created on.
 int check_device(const fg_spmm_plan *plan);
+
+// What one call of each operator needs (the same functions size the buffers inside the calls).
+// Each returns FG_OK or the status the call itself would return for that shape.
+int spmm_scratch_need(const fg_spmm_plan *plan, int F, int heads, int reduce, int num_feat_partitions, ScratchNeed *need);
+int sddmm_dds_scratch_need(const fg_spmm_plan *plan, int H, int D, int num_feat_partitions, ScratchNeed *need);
+int softmax_scratch_need(const fg_spmm_plan *plan, int heads, ScratchNeed *need);
+int attention_scratch_need(const fg_spmm_plan *plan, int heads, int head_len, bool additive, bool own_row_state,
+                           ScratchNeed *need);
 }  // namespace fg

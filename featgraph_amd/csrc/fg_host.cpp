@@ -1,6 +1,7 @@
 // Host-side parts of libfeatgraph_hip.so: error reporting, graph partitioners, structural
 // checks and the seeded synthetic-graph generator.  No device code in this file.
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <numeric>
 #include <thread>
@@ -143,15 +144,15 @@ extern "C" int fg_partition_coo_2d(int64_t n_rows, int64_t n_cols, int64_t nnz,
         for (int64_t e = 0; e < nnz; ++e)
             byrow[cur[row[e]]++] = ((uint64_t)(uint32_t)col[e] << 32) | (uint32_t)(e + 1);
     }
-    bool dup = false;
+    std::atomic<bool> dup{false};     // set by any worker thread
     fg::parallel_ranges(n_rows, nt, [&](int, int64_t r0, int64_t r1) {
         for (int64_t r = r0; r < r1; ++r) {
             std::sort(byrow.begin() + rowptr[r], byrow.begin() + rowptr[r + 1]);
             for (int64_t k = rowptr[r] + 1; k < rowptr[r + 1]; ++k)
-                if ((byrow[k] >> 32) == (byrow[k - 1] >> 32)) dup = true;
+                if ((byrow[k] >> 32) == (byrow[k - 1] >> 32)) dup.store(true, std::memory_order_relaxed);
         }
     });
-    if (dup) return fail(FG_ERR_GRAPH, "duplicate (row, col) pairs: edge ids would be ambiguous");
+    if (dup.load()) return fail(FG_ERR_GRAPH, "duplicate (row, col) pairs: edge ids would be ambiguous");
 
     const int64_t rp = (n_rows + R - 1) / R, cp = (n_cols + C - 1) / C;
     const int64_t n_blocks = (int64_t)R * C;
@@ -229,15 +230,15 @@ extern "C" int fg_synth_powerlaw_csr(int64_t n, const int32_t *in_degree, const 
         }
         return FG_OK;
     }
-    bool bad = false;
+    std::atomic<bool> bad{false};     // set by any worker thread
     fg::parallel_ranges(n, nt, [&](int, int64_t v0, int64_t v1) {
         std::vector<int32_t> buf;
         for (int64_t v = v0; v < v1; ++v) {
             draw_row(v, n, in_degree[v], cdf, perm, seed, buf);
-            if ((int64_t)buf.size() != indptr[v + 1] - indptr[v]) { bad = true; continue; }
+            if ((int64_t)buf.size() != indptr[v + 1] - indptr[v]) { bad.store(true, std::memory_order_relaxed); continue; }
             std::copy(buf.begin(), buf.end(), indices + indptr[v]);
         }
     });
-    if (bad) return fail(FG_ERR_ARG, "fg_synth_powerlaw_csr: indptr does not match this seed");
+    if (bad.load()) return fail(FG_ERR_ARG, "fg_synth_powerlaw_csr: indptr does not match this seed");
     return FG_OK;
 }

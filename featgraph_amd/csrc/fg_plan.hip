@@ -158,12 +158,9 @@ int make_tile_major(const fg_spmm_plan *pl, const float *x, int64_t n_rows, int 
     if (slot < 0 || slot >= n_slots) return fail(FG_ERR_ARG, "tile-major copy: slot %d of %d", slot, n_slots);
     if (F % 4 != 0 || tile % 4 != 0 || F % tile != 0 || floats >= (1ull << 32) || ((uintptr_t)x & 15) != 0)
         return fail(FG_ERR_SHAPE, "tile-major copy of a %lld x %d matrix in tiles of %d floats", (long long)n_rows, F, tile);
-    if (floats * (uint64_t)n_slots > pl->tiled_floats) {
-        if (pl->tiled_dev) FG_HIP_TRY(hipFree(pl->tiled_dev));
-        pl->tiled_dev = nullptr; pl->tiled_floats = 0;
-        FG_HIP_TRY(hipMalloc((void **)&pl->tiled_dev, floats * n_slots * sizeof(float)));
-        pl->tiled_floats = floats * n_slots;
-    }
+    if (floats * (uint64_t)n_slots > pl->tiled_floats)
+        return fail(FG_ERR_ARG, "tile-major copy: the plan's buffer holds %zu floats, %llu needed", pl->tiled_floats,
+                    (unsigned long long)(floats * n_slots));
     const uint32_t n_words = (uint32_t)(floats / 4);
     if (n_words == 0) return FG_OK;
     hipLaunchKernelGGL(tile_major_kernel, dim3((n_words + 255u) / 256u), dim3(256), 0, (hipStream_t)stream,
@@ -179,19 +176,52 @@ int check_device(const fg_spmm_plan *pl) {
         return fail(FG_ERR_ARG, "the plan lives on device %d but the current device is %d", pl->device, dev);
     return FG_OK;
 }
-int ensure_scratch(const fg_spmm_plan *pl, size_t need) {
-    if (need <= pl->partial_floats) return FG_OK;
-    if (pl->partial_dev) FG_HIP_TRY(hipFree(pl->partial_dev));
-    pl->partial_dev = nullptr; pl->partial_floats = 0;
-    FG_HIP_TRY(hipMalloc((void **)&pl->partial_dev, need * sizeof(float)));
-    pl->partial_floats = need;
+namespace {
+int grow(float **buf, size_t *have, size_t need, void *stream, const char *what) {
+    if (need <= *have) return FG_OK;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    // (the NULL stream cannot be captured, and querying it while another stream is being captured would
+    // invalidate that capture)
+    if (stream && hipStreamIsCapturing((hipStream_t)stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+        return fail(FG_ERR_ARG, "the plan's %s holds %zu floats and this call needs %zu, but the stream is being captured: "
+                    "call fg_spmm_plan_reserve (or run the call once) before capturing", what, *have, need);
+    if (*buf) FG_HIP_TRY(hipFree(*buf));
+    *buf = nullptr; *have = 0;
+    if (hipMalloc((void **)buf, need * sizeof(float)) != hipSuccess) {
+        (void)hipGetLastError();
+        *buf = nullptr;
+        return fail(FG_ERR_NOMEM, "cannot allocate %zu bytes for the plan's %s", need * sizeof(float), what);
+    }
+    *have = need;
     return FG_OK;
 }
-int ensure_partial(const fg_spmm_plan *pl, size_t floats_per_piece) {
-    return ensure_scratch(pl, (size_t)pl->max_slots_in_partition * floats_per_piece);
+}  // namespace
+int ensure_scratch(fg_spmm_plan *pl, const ScratchNeed &need, void *stream) {
+    if (int rc = grow(&pl->partial_dev, &pl->partial_floats, need.partial, stream, "scratch buffer")) return rc;
+    return grow(&pl->tiled_dev, &pl->tiled_floats, need.tiled, stream, "tile-by-tile copy buffer");
 }
 // Declared in fg_spmm.hip: text of the launch the SpMM entry points would use.
 std::string spmm_launch_text(const fg_spmm_plan *plan, int F, int num_feat_partitions);
+}
+
+extern "C" int fg_spmm_plan_reserve(fg_spmm_plan *pl, int op, int heads, int head_len, int num_feat_partitions) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
+    if (heads < 1 || head_len < 1 || (int64_t)heads * head_len > INT32_MAX)
+        return fail(FG_ERR_SHAPE, "heads and head length must be positive, got %d x %d", heads, head_len);
+    fg::ScratchNeed need;
+    int rc;
+    switch (op) {
+        case FG_OP_SPMM_SUM: rc = fg::spmm_scratch_need(pl, heads * head_len, heads, FG_REDUCE_SUM, num_feat_partitions, &need); break;
+        case FG_OP_SPMM_EXTREME: rc = fg::spmm_scratch_need(pl, heads * head_len, heads, FG_REDUCE_MAX, num_feat_partitions, &need); break;
+        case FG_OP_SDDMM_DDS: rc = fg::sddmm_dds_scratch_need(pl, heads, head_len, num_feat_partitions, &need); break;
+        case FG_OP_EDGE_SOFTMAX: rc = fg::softmax_scratch_need(pl, heads, &need); break;
+        case FG_OP_ATTENTION: rc = fg::attention_scratch_need(pl, heads, head_len, false, true, &need); break;
+        case FG_OP_ATTENTION_ADDITIVE: rc = fg::attention_scratch_need(pl, heads, head_len, true, true, &need); break;
+        default: return fail(FG_ERR_ARG, "fg_spmm_plan_reserve: unknown operator %d", op);
+    }
+    if (rc != FG_OK) return rc;
+    return fg::ensure_scratch(pl, need, nullptr);
 }
 
 extern "C" int fg_spmm_plan_describe(const fg_spmm_plan *pl, int F, int T, char *buf, size_t buf_len) {

@@ -757,20 +757,23 @@ extern "C" int fg_sddmm_csr_f32(const fg_spmm_plan *plan, const int32_t *indptr_
                      out_dev, H, D, stream);
 }
 
-extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_dev, const int32_t *s1_idx_dev,
-                                const int32_t *edge_pos_dev, const float *src_dev, const float *dst_dev,
-                                float *out_dev, int H, int D, int num_feat_partitions, void *stream) {
-    if (!pl) return fail(FG_ERR_ARG, "plan is null");
-    if (int drc = fg::check_device(pl)) return drc;
+namespace {
+// How the tiled traversal covers H heads of D floats with T feature tiles.
+struct TiledShape {
+    int F, T, tile_w;
+    int L, K;          // tile = L lanes x K loads x 4 floats
+    int RW, KH;        // lanes per head inside a load / loads per head (0: head narrower than a load)
+    int hpt;           // whole heads per tile (1 when a head spans one or more tiles)
+    bool tile_sum;     // tiles hold partial sums of one head
+    bool staged;       // several heads, one per tile: results staged per tile, written per edge by a last kernel
+    bool off32, tile_major;
+};
+
+int resolve_tiled(const fg_spmm_plan *pl, int H, int D, int T, bool src_aligned16, TiledShape *ts) {
     if (H < 1 || D < 1) return fail(FG_ERR_SHAPE, "heads and head length must be positive, got H=%d D=%d", H, D);
-    if (pl->nnz == 0) return FG_OK;
-    if (!s1_pos_dev || !s1_idx_dev || !edge_pos_dev || !src_dev || !dst_dev || !out_dev)
-        return fail(FG_ERR_ARG, "null device pointer");
-    if ((((uintptr_t)src_dev | (uintptr_t)dst_dev) & 15) != 0) return fail(FG_ERR_ARG, "src/dst must be 16-byte aligned");
     const int64_t F64 = (int64_t)H * D;
     if (F64 > INT32_MAX) return fail(FG_ERR_SHAPE, "H*D too large");
     const int F = (int)F64;
-    const int T = num_feat_partitions;
     if (T < 1 || F % T != 0) return fail(FG_ERR_SHAPE, "feature length %d is not divisible by num_feat_partitions %d", F, T);
     const int tile_w = F / T;
     if (tile_w % 4 != 0 || tile_w > 256 || !is_pow2(tile_w / 4) || tile_w < 16)
@@ -780,8 +783,8 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
     const int K = tile_w >= 128 ? 2 : 1;
     const int L = tile_w / 4 / K;
     const int load_w = L * 4;     // floats covered by one load of the lane group
-    int RW, KH;                   // lanes per head inside a load / loads per head (0: head narrower than a load)
-    bool tile_sum;                // tiles hold partial sums of one head
+    int RW, KH;
+    bool tile_sum;
     if (D >= tile_w) {
         if (D % tile_w != 0) return fail(FG_ERR_SHAPE, "head length %d is not a multiple of the %d-float tile", D, tile_w);
         if (D > tile_w && H != 1) return fail(FG_ERR_SHAPE, "a head spanning several tiles needs H == 1");
@@ -793,24 +796,65 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
         else { RW = D / 4; KH = 0; }
         tile_sum = false;
     }
-    hipStream_t st = (hipStream_t)stream;
-    SddmmTiledArgs a;
-    a.col = s1_idx_dev; a.edge_pos = edge_pos_dev; a.dst = dst_dev; a.F = F; a.n_tiles = T;
+    ts->F = F; ts->T = T; ts->tile_w = tile_w; ts->L = L; ts->K = K; ts->RW = RW; ts->KH = KH;
+    ts->hpt = D >= tile_w ? 1 : tile_w / D;
+    ts->tile_sum = tile_sum;
     // Several heads: a tile's results, 4 or 8 bytes per edge, would land H floats apart in out.  They
     // are kept per tile in traversal order instead and a last kernel writes each edge's H results
     // as one run.
     // (Measured on the 232,965-node graph: 20.2 -> 18.4 ms at H=8, D=64; with several heads per tile the
     // direct writes are wider and staging them costs more than it saves.)
-    const int hpt = D >= tile_w ? 1 : tile_w / D;
-    const bool staged = !tile_sum && hpt == 1 && H >= 4 && T > 1;
+    ts->staged = !tile_sum && ts->hpt == 1 && H >= 4 && T > 1;
+    ts->off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
+    // The gathers of an XCD touch one tile's slice of every src row, F * 4 bytes apart; from a copy
+    // that stores each tile's slices back to back the same working set is cached better
+    // (232,965-node graph, F=512: 14.5 -> 13.7 ms with 4 tiles x 16 partitions, 14.9 -> 13.5 ms with
+    // 8 x 8, before the 0.15 ms of the copy).  The destination rows gain nothing from it.
+    ts->tile_major = ts->off32 && pl->nnz > 0 && src_aligned16 &&
+                     fg::wants_tile_major(pl, T, (uint64_t)pl->n_src * (uint64_t)F * 4u);
+    return FG_OK;
+}
+
+fg::ScratchNeed tiled_need(const fg_spmm_plan *pl, const TiledShape &ts, int H) {
+    fg::ScratchNeed need;
+    if (ts.tile_sum) need.partial = (size_t)ts.T * (size_t)((pl->nnz + 3) & ~(int64_t)3);
+    else if (ts.staged) need.partial = (size_t)H * (size_t)pl->nnz;
+    if (ts.tile_major) need.tiled = (size_t)pl->n_src * (size_t)ts.F;
+    return need;
+}
+}  // namespace
+
+namespace fg {
+int sddmm_dds_scratch_need(const fg_spmm_plan *pl, int H, int D, int T, ScratchNeed *need) {
+    TiledShape ts;
+    if (int rc = resolve_tiled(pl, H, D, T, true, &ts)) return rc;
+    *need = tiled_need(pl, ts, H);
+    return FG_OK;
+}
+}  // namespace fg
+
+extern "C" int fg_sddmm_dds_f32(fg_spmm_plan *pl, const int32_t *s1_pos_dev, const int32_t *s1_idx_dev,
+                                const int32_t *edge_pos_dev, const float *src_dev, const float *dst_dev,
+                                float *out_dev, int H, int D, int num_feat_partitions, void *stream) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
+    TiledShape ts;
+    int rc = resolve_tiled(pl, H, D, num_feat_partitions, (((uintptr_t)src_dev) & 15) == 0, &ts);
+    if (rc != FG_OK) return rc;
+    if (pl->nnz == 0) return FG_OK;
+    if (!s1_pos_dev || !s1_idx_dev || !edge_pos_dev || !src_dev || !dst_dev || !out_dev)
+        return fail(FG_ERR_ARG, "null device pointer");
+    if ((((uintptr_t)src_dev | (uintptr_t)dst_dev) & 15) != 0) return fail(FG_ERR_ARG, "src/dst must be 16-byte aligned");
+    if (ts.tile_sum && ((uintptr_t)edge_pos_dev & 15)) return fail(FG_ERR_ARG, "edge_pos must be 16-byte aligned");
+    if ((rc = fg::ensure_scratch(pl, tiled_need(pl, ts, H), stream)) != FG_OK) return rc;
+    const int F = ts.F, T = ts.T, tile_w = ts.tile_w, L = ts.L, K = ts.K, RW = ts.RW, KH = ts.KH, hpt = ts.hpt;
+    const bool tile_sum = ts.tile_sum, staged = ts.staged, off32 = ts.off32;
+    hipStream_t st = (hipStream_t)stream;
+    SddmmTiledArgs a;
+    a.col = s1_idx_dev; a.edge_pos = edge_pos_dev; a.dst = dst_dev; a.F = F; a.n_tiles = T;
     if (tile_sum) {
-        const int64_t stride = (pl->nnz + 3) & ~(int64_t)3;
-        int rc = fg::ensure_scratch(pl, (size_t)T * (size_t)stride);
-        if (rc != FG_OK) return rc;
-        a.out = pl->partial_dev; a.out_edge_stride = 1; a.out_tile_stride = stride;
+        a.out = pl->partial_dev; a.out_edge_stride = 1; a.out_tile_stride = (pl->nnz + 3) & ~(int64_t)3;
     } else if (staged) {
-        int rc = fg::ensure_scratch(pl, (size_t)H * (size_t)pl->nnz);
-        if (rc != FG_OK) return rc;
         a.out = pl->partial_dev; a.out_edge_stride = hpt; a.out_tile_stride = pl->nnz * hpt;
     } else {
         a.out = out_dev; a.out_edge_stride = H; a.out_tile_stride = tile_w / D;
@@ -827,15 +871,8 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
     // (232,965-node graph: 3.93 -> 3.71 ms at F=128, 7.89 -> 7.56 ms at F=256, 1.96 -> 1.82 ms at F=64.)
     const int conc = (T < 8 && 8 % T == 0) ? std::max(1, std::min(8 / T, P)) : 1;
     a.conc = conc;
-    const bool off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
-    // The gathers of an XCD touch one tile's slice of every src row, F * 4 bytes apart; from a copy
-    // that stores each tile's slices back to back the same working set is cached better
-    // (232,965-node graph, F=512: 14.5 -> 13.7 ms with 4 tiles x 16 partitions, 14.9 -> 13.5 ms with
-    // 8 x 8, before the 0.15 ms of the copy).  The destination rows gain nothing from it.
-    if (off32 && pl->nnz > 0 && ((uintptr_t)src_dev & 15) == 0 &&
-        fg::wants_tile_major(pl, T, (uint64_t)pl->n_src * (uint64_t)F * 4u)) {
-        int rc = fg::make_tile_major(pl, src_dev, pl->n_src, F, tile_w, stream);
-        if (rc != FG_OK) return rc;
+    if (ts.tile_major) {
+        if ((rc = fg::make_tile_major(pl, src_dev, pl->n_src, F, tile_w, stream)) != FG_OK) return rc;
         a.src = pl->tiled_dev; a.src_stride = width * tile_w;
         a.src_row_bytes = (uint32_t)tile_w * 4u; a.src_tile_bytes = (uint32_t)((uint64_t)pl->n_src * tile_w * 4u);
     }
@@ -857,7 +894,6 @@ extern "C" int fg_sddmm_dds_f32(const fg_spmm_plan *pl, const int32_t *s1_pos_de
         }
     }
     if (tile_sum) {
-        if ((uintptr_t)edge_pos_dev & 15) return fail(FG_ERR_ARG, "edge_pos must be 16-byte aligned");
         const unsigned blocks = (unsigned)((pl->nnz + 1023) / 1024);
         hipLaunchKernelGGL(sddmm_tile_sum_kernel, dim3(blocks), dim3(256), 0, st, pl->partial_dev, edge_pos_dev,
                            out_dev, pl->nnz, (pl->nnz + 3) & ~(int64_t)3, T);

@@ -417,7 +417,7 @@ void launch_both(const fg_spmm_plan *pl, const SoftmaxArgs &a, hipStream_t st) {
     }
 }
 
-int softmax_run(const fg_spmm_plan *pl, const int32_t *indptr, const float *x, const float *g, float *y,
+int softmax_run(fg_spmm_plan *pl, const int32_t *indptr, const float *x, const float *g, float *y,
                 int H, void *stream, bool bwd) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (int drc = fg::check_device(pl)) return drc;
@@ -427,7 +427,9 @@ int softmax_run(const fg_spmm_plan *pl, const int32_t *indptr, const float *x, c
     if (!indptr || !x || !y || (bwd && !g)) return fail(FG_ERR_ARG, "null device pointer");
     if ((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock > 0x7fffffffLL)
         return fail(FG_ERR_SHAPE, "too many work items for one grid");
-    int rc = fg::ensure_partial(pl, (size_t)2 * (size_t)H);
+    fg::ScratchNeed need;
+    int rc = fg::softmax_scratch_need(pl, H, &need);
+    if (rc == FG_OK) rc = fg::ensure_scratch(pl, need, stream);
     if (rc != FG_OK) return rc;
     SoftmaxArgs a;
     a.items = pl->items_dev; a.n_items = pl->n_items; a.indptr = indptr;
@@ -442,12 +444,22 @@ int softmax_run(const fg_spmm_plan *pl, const int32_t *indptr, const float *x, c
 
 }  // namespace
 
-extern "C" int fg_edge_softmax_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev, const float *scores_dev,
+namespace fg {
+// (max, sum) per head for every piece of a split row
+int softmax_scratch_need(const fg_spmm_plan *pl, int heads, ScratchNeed *need) {
+    if (heads < 1) return fail(FG_ERR_SHAPE, "number of heads must be positive, got %d", heads);
+    need->partial = (size_t)pl->max_slots_in_partition * 2 * (size_t)heads;
+    need->tiled = 0;
+    return FG_OK;
+}
+}  // namespace fg
+
+extern "C" int fg_edge_softmax_f32(fg_spmm_plan *plan, const int32_t *indptr_dev, const float *scores_dev,
                                    float *out_dev, int heads, void *stream) {
     return softmax_run(plan, indptr_dev, scores_dev, nullptr, out_dev, heads, stream, false);
 }
 
-extern "C" int fg_edge_softmax_stats_f32(const fg_spmm_plan *pl, const int32_t *indptr_dev, const float *scores_dev,
+extern "C" int fg_edge_softmax_stats_f32(fg_spmm_plan *pl, const int32_t *indptr_dev, const float *scores_dev,
                                          float *row_stats_dev, int heads, void *stream) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (int drc = fg::check_device(pl)) return drc;
@@ -456,7 +468,9 @@ extern "C" int fg_edge_softmax_stats_f32(const fg_spmm_plan *pl, const int32_t *
     if (pl->nnz == 0 || pl->n_items == 0) return FG_OK;
     if (!indptr_dev || !scores_dev || !row_stats_dev) return fail(FG_ERR_ARG, "null device pointer");
     if (((uintptr_t)row_stats_dev & 7) != 0) return fail(FG_ERR_ARG, "row_stats must be 8-byte aligned");
-    int rc = fg::ensure_partial(pl, (size_t)2 * (size_t)heads);
+    fg::ScratchNeed need;
+    int rc = fg::softmax_scratch_need(pl, heads, &need);
+    if (rc == FG_OK) rc = fg::ensure_scratch(pl, need, stream);
     if (rc != FG_OK) return rc;
     SoftmaxArgs a;
     a.items = pl->items_dev; a.n_items = pl->n_items; a.indptr = indptr_dev;
@@ -490,7 +504,7 @@ extern "C" int fg_edge_softmax_head_major_f32(const float *scores_dev, const flo
     return FG_OK;
 }
 
-extern "C" int fg_edge_softmax_backward_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev,
+extern "C" int fg_edge_softmax_backward_f32(fg_spmm_plan *plan, const int32_t *indptr_dev,
                                             const float *softmax_dev, const float *grad_softmax_dev,
                                             float *grad_scores_dev, int heads, void *stream) {
     return softmax_run(plan, indptr_dev, softmax_dev, grad_softmax_dev, grad_scores_dev, heads, stream, true);

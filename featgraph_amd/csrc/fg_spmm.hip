@@ -44,6 +44,11 @@ __device__ __forceinline__ float4 vshfl_xor(const float4 &a, int off) {
     return make_float4(__shfl_xor(a.x, off), __shfl_xor(a.y, off), __shfl_xor(a.z, off), __shfl_xor(a.w, off));
 }
 __device__ __forceinline__ float vshfl_xor(const float &a, int off) { return __shfl_xor(a, off); }
+// a where `keep`, else zeros
+__device__ __forceinline__ float4 vkeep(bool keep, const float4 &a) {
+    return make_float4(keep ? a.x : 0.f, keep ? a.y : 0.f, keep ? a.z : 0.f, keep ? a.w : 0.f);
+}
+__device__ __forceinline__ float vkeep(bool keep, const float &a) { return keep ? a : 0.f; }
 
 struct SpmmArgs {
     const Item *items;
@@ -85,7 +90,9 @@ __device__ __forceinline__ const float *row_ptr(const float *x, uint32_t lane_by
 
 // The last, partly filled batch of gather_rows: exactly `nu` steps (1 <= nu <= NU, uniform over
 // the wavefront), so that no step is spent re-reading the row's last element; inside the last
-// step a lane without an element still re-reads it with weight zero (no load under a branch).
+// step a lane without an element still re-reads it (no load under a branch) and replaces what it
+// loaded by zeros -- a select, not a product with weight zero, so that a non-finite source row
+// only ever reaches the rows that reference it.
 template <int V, int L, int K, bool FULL, int NU, bool OFF32, int HPT>
 __device__ __forceinline__ void gather_tail(int nu, const int2 *s_edge, const float *wrow, int s0, int e, int g,
                                             const float *x, uint32_t lane_bytes, int64_t F, const bool (&on)[K],
@@ -111,17 +118,21 @@ __device__ __forceinline__ void gather_tail(int nu, const int2 *s_edge, const fl
         for (int k = 0; k < K; ++k)
             if (FULL || on[k])
                 xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<OFF32>(x, lane_bytes, F, cw[u].x) + k * L * V);
+    const bool last_has = s0 + (NU - 1) * G + g < e;      // steps before the last are full
 #pragma unroll
     for (int u = 0; u < NU; ++u)
 #pragma unroll
         for (int k = 0; k < K; ++k)
-            if (FULL || on[k]) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
+            if (FULL || on[k]) {
+                if (u == NU - 1) xv[u][k] = vkeep(last_has, xv[u][k]);
+                vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
+            }
 }
 
 // Adds vals * X rows for the staged elements [b, e) of s_edge (x = staged column word, y =
 // weight bits) into acc.  The G lane groups take elements b+g, b+g+G, ...; U steps' loads are
 // issued back to back before the first use.  No load sits under a branch: in the last, partly
-// filled batch a lane without an element re-reads the row's last element with weight zero.
+// filled batch a lane without an element re-reads the row's last element and discards it.
 // HPT > 1: the kernel tile holds HPT heads and the lane's weight is wrow[slot] (its head's staged
 // weights) instead of the word staged next to the column.
 template <int V, int L, int K, bool FULL, int U, bool OFF32, int HPT>
@@ -363,8 +374,8 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
                 vec xv[U][K];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    // past the row's end this is a later row's element (or the padding): a valid
-                    // source row, given weight zero
+                    // past the row's end this is a later row's element (or the padding): a loadable
+                    // source row whose values are replaced by zeros below
                     cw[u] = edge[j + u];
                     if (HPT > 1) cw[u].y = __float_as_int(wrow[j + u]);
                     if (j + u >= e) cw[u].y = 0;
@@ -379,7 +390,11 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
                 for (int u = 0; u < U; ++u)
 #pragma unroll
                     for (int k = 0; k < K; ++k)
-                        if (FULL || on[k]) vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
+                        if (FULL || on[k]) {
+                            // u == 0 is always the row's own element (j < e)
+                            if (u > 0) xv[u][k] = vkeep(j + u < e, xv[u][k]);
+                            vfma(acc[k], __int_as_float(cw[u].y), xv[u][k]);
+                        }
                 j += U;
             }
         }
@@ -895,24 +910,15 @@ bool gathers_tile_major(const fg_spmm_plan *pl, const SpmmConfig &c, int F) {
            fg::wants_tile_major(pl, c.n_ftiles, (uint64_t)pl->n_src * (uint64_t)F * 4u);
 }
 
-// reduce: FG_REDUCE_SUM / MAX / MIN.  heads > 1: vals is [nnz, heads] (or [heads, nnz] when
-// head_major) and every kernel tile must lie inside one head.  vals == nullptr with allow_no_vals: every weight is 1.
-int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
-             const float *x, float *out, int F, int T, void *stream, int heads = 1,
-             int reduce = FG_REDUCE_SUM, bool allow_no_vals = false, bool head_major = false,
-             int32_t *arg_out = nullptr) {
-    if (!pl) return fail(FG_ERR_ARG, "plan is null");
-    if (arg_out && reduce == FG_REDUCE_SUM) return fail(FG_ERR_ARG, "positions of the selected elements exist for max / min only");
-    if (int drc = fg::check_device(pl)) return drc;
-    if (pl->n_dst == 0) return FG_OK;
-    if (!out || !pos || (pl->nnz > 0 && (!idx || (!vals && !allow_no_vals) || !x)))
-        return fail(FG_ERR_ARG, "null device pointer");
+// The kernel configuration of one call: feature length F in `heads` heads, T requested tiles (0 = choose).
+// heads > 1: every kernel tile must hold whole heads or lie inside one.
+int resolve_config(const fg_spmm_plan *pl, int F, int T, int heads, int reduce, bool aligned16, SpmmConfig *c) {
     if (reduce != FG_REDUCE_SUM && reduce != FG_REDUCE_MAX && reduce != FG_REDUCE_MIN)
         return fail(FG_ERR_ARG, "unknown reduce op %d", reduce);
     if (reduce != FG_REDUCE_SUM && pl->num_col_partitions != 1)
         return fail(FG_ERR_ARG, "max / min aggregation needs a plan with one column partition");
+    if (F < 1) return fail(FG_ERR_SHAPE, "feature length must be positive, got %d", F);
     if (heads < 1 || F % heads != 0) return fail(FG_ERR_SHAPE, "feature length %d is not divisible by %d heads", F, heads);
-    const bool aligned16 = (((uintptr_t)x | (uintptr_t)out | (uintptr_t)arg_out) & 15) == 0;
     int hpt = 1;
     if (heads > 1) {
         // A kernel tile holds whole heads or lies inside one: 64 floats when the head length divides
@@ -940,12 +946,37 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
                 return fail(FG_ERR_SHAPE, "no kernel for tiles of %d floats holding %d heads", tile, hpt);
         }
     }
-    SpmmConfig c;
-    int rc = choose_config(F, T, aligned16, &c);
+    int rc = choose_config(F, T, aligned16, c);
     if (rc != FG_OK) return rc;
-    c.hpt = hpt;
-    if ((rc = fg::ensure_partial(pl, (size_t)F)) != FG_OK) return rc;
-    c.off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
+    c->hpt = hpt;
+    c->off32 = !pl->wide_offsets && (uint64_t)pl->n_src * (uint64_t)F * 4u < (1ull << 32);
+    return FG_OK;
+}
+
+fg::ScratchNeed scratch_need(const fg_spmm_plan *pl, const SpmmConfig &c, int F) {
+    fg::ScratchNeed need;
+    need.partial = (size_t)pl->max_slots_in_partition * (size_t)F;      // one row of F floats per piece of a split row
+    if (gathers_tile_major(pl, c, F)) need.tiled = (size_t)pl->n_src * (size_t)F;
+    return need;
+}
+
+// reduce: FG_REDUCE_SUM / MAX / MIN.  heads > 1: vals is [nnz, heads] (or [heads, nnz] when
+// head_major).  vals == nullptr with allow_no_vals: every weight is 1.
+int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
+             const float *x, float *out, int F, int T, void *stream, int heads = 1,
+             int reduce = FG_REDUCE_SUM, bool allow_no_vals = false, bool head_major = false,
+             int32_t *arg_out = nullptr) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (arg_out && reduce == FG_REDUCE_SUM) return fail(FG_ERR_ARG, "positions of the selected elements exist for max / min only");
+    if (int drc = fg::check_device(pl)) return drc;
+    if (pl->n_dst == 0) return FG_OK;
+    if (!out || !pos || (pl->nnz > 0 && (!idx || (!vals && !allow_no_vals) || !x)))
+        return fail(FG_ERR_ARG, "null device pointer");
+    const bool aligned16 = (((uintptr_t)x | (uintptr_t)out | (uintptr_t)arg_out) & 15) == 0;
+    SpmmConfig c;
+    int rc = resolve_config(pl, F, T, heads, reduce, aligned16, &c);
+    if (rc != FG_OK) return rc;
+    if ((rc = fg::ensure_scratch(pl, scratch_need(pl, c, F), stream)) != FG_OK) return rc;
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
@@ -1033,6 +1064,12 @@ int spmm_run(const fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, con
 }  // namespace
 
 namespace fg {
+int spmm_scratch_need(const fg_spmm_plan *pl, int F, int heads, int reduce, int T, ScratchNeed *need) {
+    SpmmConfig c;
+    if (int rc = resolve_config(pl, F, T, heads, reduce, true, &c)) return rc;
+    *need = scratch_need(pl, c, F);
+    return FG_OK;
+}
 std::string spmm_launch_text(const fg_spmm_plan *pl, int F, int T) {
     SpmmConfig c;
     if (choose_config(F, T, true, &c) != FG_OK) return std::string("  launch           : ") + fg_last_error() + "\n";
@@ -1055,7 +1092,7 @@ std::string spmm_launch_text(const fg_spmm_plan *pl, int F, int T) {
 }
 }  // namespace fg
 
-extern "C" int fg_spmm_csr_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev,
+extern "C" int fg_spmm_csr_f32(fg_spmm_plan *plan, const int32_t *indptr_dev,
                                const int32_t *indices_dev, const float *vals_dev, const float *x_dev,
                                float *out_dev, int F, int num_feat_partitions, void *stream) {
     if (plan && plan->num_col_partitions != 1)
@@ -1063,20 +1100,20 @@ extern "C" int fg_spmm_csr_f32(const fg_spmm_plan *plan, const int32_t *indptr_d
     return spmm_run(plan, indptr_dev, indices_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
 }
 
-extern "C" int fg_spmm_dds_f32(const fg_spmm_plan *plan, const int32_t *s1_pos_dev,
+extern "C" int fg_spmm_dds_f32(fg_spmm_plan *plan, const int32_t *s1_pos_dev,
                                const int32_t *s1_idx_dev, const float *vals_dev, const float *x_dev,
                                float *out_dev, int F, int num_feat_partitions, void *stream) {
     return spmm_run(plan, s1_pos_dev, s1_idx_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
 }
 
-extern "C" int fg_gspmm_f32(const fg_spmm_plan *plan, const int32_t *pos_dev, const int32_t *idx_dev,
+extern "C" int fg_gspmm_f32(fg_spmm_plan *plan, const int32_t *pos_dev, const int32_t *idx_dev,
                             const float *vals_dev, const float *x_dev, float *out_dev, int F, int heads,
                             int vals_head_major, int reduce, int num_feat_partitions, void *stream) {
     return spmm_run(plan, pos_dev, idx_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream, heads,
                     reduce, /*allow_no_vals=*/true, vals_head_major != 0);
 }
 
-extern "C" int fg_gspmm_arg_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev, const int32_t *indices_dev,
+extern "C" int fg_gspmm_arg_f32(fg_spmm_plan *plan, const int32_t *indptr_dev, const int32_t *indices_dev,
                                 const float *vals_dev, const float *x_dev, float *out_dev, int32_t *arg_dev, int F,
                                 int heads, int vals_head_major, int reduce, int num_feat_partitions, void *stream) {
     if (!arg_dev) return fail(FG_ERR_ARG, "fg_gspmm_arg_f32: arg_dev is null");

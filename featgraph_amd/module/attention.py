@@ -96,6 +96,7 @@ class GraphAttentionhip(object):
         self._t_parts = None if t_parts in (None, 'auto') else int(t_parts)
         self._scale = float(compute_args.get('scale', 1.0 / np.sqrt(head_len)))
         self._active = self._layout(P)
+        common.reserve(self._active['plan'], common.OP_ATTENTION, heads, head_len, 0, self._ctx)
         self._placeholders = [q_ph, k_ph, v_ph]
         self.out_tvm = torch.zeros((self._num_rows, heads, head_len), dtype=torch.float32, device=self._ctx)
         # every row's maximum score and sum of exponentials, per head: what backward() starts from
@@ -133,6 +134,7 @@ class GraphAttentionhip(object):
         t_parts = schedule_args.get('num_dst_partitions')
         self._t_parts = None if t_parts in (None, 'auto') else int(t_parts)
         self._active = self._layout(self._partitions(schedule_args, 4 * head_len))
+        common.reserve(self._active['plan'], common.OP_ATTENTION_ADDITIVE, heads, head_len, 0, self._ctx)
         self._placeholders = [er_ph, el_ph, v_ph]
         self.out_tvm = torch.zeros((self._num_rows, heads, head_len), dtype=torch.float32, device=self._ctx)
         self.state_tvm = torch.zeros((self._num_rows, heads, 2), dtype=torch.float32, device=self._ctx)

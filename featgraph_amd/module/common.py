@@ -72,6 +72,17 @@ def timed_mean_seconds(fn, num_runs):
     return start.elapsed_time(end) * 1e-3 / num_runs
 
 
+# fg_op of include/featgraph_hip.h
+OP_SPMM_SUM, OP_SPMM_EXTREME, OP_SDDMM_DDS, OP_EDGE_SOFTMAX, OP_ATTENTION, OP_ATTENTION_ADDITIVE = range(6)
+
+
+def reserve(plan, op, heads, head_len, num_feat_partitions, dev):
+    """Sizes the plan's device scratch at build() time, so that run() allocates nothing (and can be
+    captured into a HIP graph without a warm-up call)."""
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().fg_spmm_plan_reserve(plan, op, int(heads), int(head_len), int(num_feat_partitions)))
+
+
 def take_args(args, allowed, what):
     """Mirrors the reference's ``**args`` unpacking: an unknown key is a TypeError."""
     for k in args:

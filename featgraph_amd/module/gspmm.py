@@ -70,6 +70,8 @@ class GSpMMhip(VanillaSpMMhip):
         self._reduce, self._msg, self._weights_at_run, self._notes = reduce, msg, weights_at_run, notes
         self._active = self._glayout(P)
         self._func = _lib.lib().fg_gspmm_f32
+        common.reserve(self._active['plan'], common.OP_SPMM_SUM if _REDUCE[reduce] == 0 else common.OP_SPMM_EXTREME,
+                       heads, feat_len // heads, self._num_feat_partitions, self._ctx)
         self._return_arg = return_arg
         self._inv_deg_edge = None
         self._w_head_major = None

@@ -153,9 +153,19 @@ class SDDMMbase(object):
         for t in (T, Ts):
             if t < 1 or (H * D) % t != 0:
                 raise ValueError("feat_len %d is not divisible by num_feat_partitions %d" % (H * D, t))
-        if T != 1 or Ts != 1:
-            notes.append("num_feat_partitions accepted; an edge's dot product is reduced inside one "
-                         "wavefront, so the feature axis is not tiled across workgroups")
+        # The reference's knob (python/featgraph/op/vanilla_sddmm.py:48-60) asks for T feature tiles; it
+        # becomes the tiled traversal's tile count when F / T is a tile width the kernel takes.
+        knob = T if T != 1 else Ts
+        knob_tiles = None
+        if knob != 1:
+            tile_w = (H * D) // knob
+            legal = tile_w % 4 == 0 and 16 <= tile_w <= 256 and (tile_w & (tile_w - 1)) == 0 and \
+                (H == 1 or tile_w % D == 0 or D == tile_w)
+            if legal:
+                knob_tiles = knob
+            else:
+                notes.append("num_feat_partitions=%d gives tiles of %d floats; the kernel takes power-of-two tiles of "
+                             "16..256 floats, so the default tiling is used" % (knob, tile_w))
         blocks = schedule_args.get('num_cuda_blocks')
         if blocks is not None:
             # same bound as schedule_vanilla_sddmm_cuda_tree_reduce (vanilla_sddmm.py:82-83)
@@ -174,6 +184,8 @@ class SDDMMbase(object):
         if order in ('auto', 'tiled') and nnz > 0:
             tiled = tuning.choose_sddmm(self._num_rows, self._num_cols, nnz, H, D)
             p_arg, t_arg = schedule_args.get('num_src_partitions'), schedule_args.get('num_feat_tiles')
+            if t_arg is None and knob_tiles is not None and order != 'coo' and order != 'csr':
+                t_arg = knob_tiles
             if order == 'tiled' or p_arg is not None or t_arg is not None:
                 base = tiled or (1, 1)
                 tiled = (int(p_arg) if p_arg is not None else base[0], int(t_arg) if t_arg is not None else base[1])
@@ -191,7 +203,9 @@ class SDDMMbase(object):
             [SrcFeat (num_cols, feat_len), DstFeat (num_rows, feat_len)]
 
         compute_args : dict
-            {'num_feat_partitions': T} is accepted (see lower_to_ir for what it maps to)
+            {'num_feat_partitions': T}: T feature tiles handled by different workgroups (the tiled
+            traversal), when feat_len / T is a power of two between 16 and 256; otherwise a note is
+            recorded (see lower_to_ir) and the default tiling applies
 
         schedule_args : dict
             'num_feat_partitions', 'num_cuda_blocks' (reference keys); 'order' in
@@ -205,6 +219,7 @@ class SDDMMbase(object):
         self._tiled = None
         if tiled is not None:
             self._tiled = (self._dds_layout(tiled[0]), tiled[1])
+            common.reserve(self._tiled[0]['plan'], common.OP_SDDMM_DDS, H, D, tiled[1], self._ctx)
         self._func = _lib.lib().fg_sddmm_csr_f32 if use_csr else _lib.lib().fg_sddmm_coo_f32
         nnz = self._adj_row_indices.shape[0]
         oshape = (nnz,) if self._out_1d else (nnz, H)

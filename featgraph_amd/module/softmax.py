@@ -62,6 +62,7 @@ class EdgeSoftmaxhip(object):
         self._heads = int(ph.shape[1]) if len(ph.shape) == 2 else 1
         if self._heads < 1:
             raise ValueError("number of heads must be positive")
+        common.reserve(self._plan, common.OP_EDGE_SOFTMAX, self._heads, 1, 0, self._ctx)
         self.out_tvm = torch.zeros(tuple(ph.shape), dtype=torch.float32, device=self._ctx)
         self.grad_tvm = None
 
@@ -150,6 +151,7 @@ class EdgeSoftmaxSpMMhip(object):
         w_shape = (self._nnz,) if heads == 1 else (self._nnz, heads)
         self._agg.build([x_ph, common.placeholder(w_shape)], dict(compute_args or {}), dict(schedule_args or {}))
         self._heads = heads
+        common.reserve(self._agg._layouts[1]['plan'], common.OP_EDGE_SOFTMAX, heads, 1, 0, self._ctx)
         self._placeholders = [s_ph, x_ph]
         self._row_stats = torch.zeros((self._num_rows, heads, 2), dtype=torch.float32, device=self._ctx)
         self._weights = torch.empty((heads, self._nnz), dtype=torch.float32, device=self._ctx)

@@ -29,6 +29,9 @@ class SpMMbase(object):
             adj_scipy_csr = adj_scipy.tocsr()
         else:
             adj_scipy_csr = adj_scipy
+        if adj_scipy_csr.dtype != np.float32:
+            # the kernels compute in fp32 whatever the matrix holds (e.g. scipy.sparse.random's float64)
+            adj_scipy_csr = adj_scipy_csr.astype(np.float32)
         self._num_rows = adj_scipy_csr.shape[0]
         self._num_cols = adj_scipy_csr.shape[1]
         assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
@@ -166,6 +169,7 @@ class SpMMbase(object):
         self._notes = notes
         self._active = self._layout(P)
         self._func = _lib.lib().fg_spmm_dds_f32 if P > 1 else _lib.lib().fg_spmm_csr_f32
+        common.reserve(self._active['plan'], common.OP_SPMM_SUM, 1, feat_len, T, self._ctx)
         self.out_tvm = torch.zeros((self._num_rows, feat_len), dtype=torch.float32, device=self._ctx)
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):

@@ -15,15 +15,19 @@ def util_convert_csr_to_dds(adj_scipy_csr, num_col_partitions):
     -------
     s1_pos : int32 [num_col_partitions * (num_rows + 1)]
     s1_idx : int32 [nnz], partition-local column ids
-    vals   : [nnz], dtype of ``adj_scipy_csr.data`` (which must be 32 bits wide)
+    vals   : [nnz], dtype of ``adj_scipy_csr.data`` (any dtype, as in the reference; values that are
+             not 32 bits wide are permuted on the host through the positions the library returns)
     """
     assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
     num_rows, num_cols = adj_scipy_csr.shape
     indptr = np.ascontiguousarray(adj_scipy_csr.indptr, dtype=np.int32)
     indices = np.ascontiguousarray(adj_scipy_csr.indices, dtype=np.int32)
     data = np.ascontiguousarray(adj_scipy_csr.data)
+    moved = None
     if data.dtype.itemsize != 4:
-        raise ValueError("adjacency values must be 32 bits wide (float32 / int32), got %s" % data.dtype)
+        if indices.shape[0] >= 2 ** 31:
+            raise ValueError("too many stored elements for int32 positions")
+        moved, data = data, np.arange(indices.shape[0], dtype=np.int32)      # the library moves 32-bit words
     s1_pos = np.zeros(num_col_partitions * (num_rows + 1), dtype=np.int32)
     s1_idx = np.zeros(indices.shape, dtype=np.int32)
     vals = np.zeros(data.shape, dtype=data.dtype)
@@ -31,6 +35,8 @@ def util_convert_csr_to_dds(adj_scipy_csr, num_col_partitions):
                                         _lib.host_ptr(data), num_col_partitions, _lib.host_ptr(s1_pos),
                                         _lib.host_ptr(s1_idx), _lib.host_ptr(vals)))
     assert len(s1_idx) == s1_pos[-1] and len(vals) == s1_pos[-1]
+    if moved is not None:
+        vals = moved[vals]
     return s1_pos, s1_idx, vals
 
 

@@ -1,0 +1,108 @@
+"""The benchmark's own configurations at full size: 232,965 nodes / ~114.8M edges.
+
+The CPU oracle would need minutes per product here, so the checks are the size-independent ones:
+closed forms (dst = ones gives the gathered rows' sums), a 200,000-edge sample against float64
+formed on the device, agreement of two different kernels (the tiled traversal over the
+source-column-partitioned edge list against the CSR-order kernel), and head sums against the flat
+single-head product.  Tolerance: rel 1e-4 / abs 1e-5 plus the rounding allowance 8 * eps32 * sum of
+|terms| (the bar of helpers.assert_sum_close, evaluated on the device).
+"""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+from helpers import RTOL, ATOL, MASS_FACTOR
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def graph():
+    import torch
+    from featgraph_amd import synthetic
+    assert torch.cuda.is_available()
+    indptr, indices = synthetic.make_workload("powerlaw-233k")
+    n = indptr.shape[0] - 1
+    adj = sp.csr_matrix((np.ones(indices.shape[0], "float32"), indices, indptr), shape=(n, n))
+    return adj, n, indices.shape[0]
+
+
+def _close(got, ref64, mass):
+    return ((got.double() - ref64).abs() <= ATOL + RTOL * ref64.abs() + MASS_FACTOR * mass).all().item()
+
+
+def test_sddmm_default_at_feat_512(graph):
+    """What bench.py times: the tile-by-tile copy of Src, 8 partitions x 8 tiles, the sum over tiles."""
+    import torch
+    from featgraph_amd.module import VanillaSDDMMhip, placeholder
+    adj, n, nnz = graph
+    F = 512
+    g = torch.Generator(device="cuda"); g.manual_seed(5)
+    src = torch.randn((n, F), generator=g, device="cuda")
+    dst = torch.randn((n, F), generator=g, device="cuda")
+    m = VanillaSDDMMhip(adj)
+    m.build([placeholder((n, F)), placeholder((n, F))], {}, {})
+    text = m.lower_to_ir([placeholder((n, F)), placeholder((n, F))], {}, {})
+    assert m._tiled is not None and m._tiled[1] == 8 and m._tiled[0]['P'] == 8, text
+    col_d, row_d = m._adj_col_indices_dev.long(), m._adj_row_indices_dev.long()
+
+    # dst = ones: every edge's result is the sum of its source row
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([src, torch.ones((n, F), device="cuda")])
+    row_sum = src.double().sum(1)
+    row_mass = src.double().abs().sum(1)
+    assert _close(out, row_sum[col_d], row_mass[col_d])
+
+    # a sample of edges against float64
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([src, dst])
+    assert torch.isfinite(out).all().item()
+    pick = torch.randint(0, nnz, (200000,), generator=g, device="cuda")
+    pick[0], pick[1] = 0, nnz - 1
+    prod = src[col_d[pick]].double() * dst[row_d[pick]].double()
+    assert _close(out[pick], prod.sum(1), prod.abs().sum(1))
+    del prod
+
+    # the CSR-order kernel (one wavefront per row piece, no tiles, no partial sums) on every edge
+    out_tiled = out.clone()
+    m2 = VanillaSDDMMhip(adj)
+    m2.build([placeholder((n, F)), placeholder((n, F))], {}, {'order': 'csr'})
+    assert m2._tiled is None
+    out_csr = m2.run([src, dst])
+    # two fp32 results, each within the allowance of the exact value; sum |terms| <= |a| |b| (Cauchy-Schwarz)
+    bound = src.double().norm(dim=1)[col_d] * dst.double().norm(dim=1)[row_d]
+    assert ((out_tiled.double() - out_csr.double()).abs() <= ATOL + RTOL * out_csr.double().abs()
+            + 2 * MASS_FACTOR * bound).all().item()
+    # repeatable bit for bit
+    assert torch.equal(m.run([src, dst]), out_tiled)
+
+
+@pytest.mark.parametrize("H,D", [(4, 64), (8, 32), (8, 64)])
+def test_multihead_shapes(graph, H, D):
+    import torch
+    from featgraph_amd.module import VanillaSDDMMhip, MultiHeadSDDMMhip, placeholder
+    adj, n, nnz = graph
+    F = H * D
+    g = torch.Generator(device="cuda"); g.manual_seed(H * 100 + D)
+    src = torch.randn((n, H, D), generator=g, device="cuda")
+    dst = torch.randn((n, H, D), generator=g, device="cuda")
+    mh = MultiHeadSDDMMhip(adj)
+    mh.build([placeholder((n, H, D)), placeholder((n, H, D))], {}, {})
+    assert mh._tiled is not None
+    mh.out_tvm.fill_(float("nan"))
+    out = mh.run([src, dst])
+    assert out.shape == (nnz, H) and torch.isfinite(out).all().item()
+    col_d, row_d = mh._adj_col_indices_dev.long(), mh._adj_row_indices_dev.long()
+    pick = torch.randint(0, nnz, (200000,), generator=g, device="cuda")
+    pick[0], pick[1] = 0, nnz - 1
+    prod = src[col_d[pick]].double() * dst[row_d[pick]].double()                        # [S, H, D]
+    assert _close(out[pick], prod.sum(2), prod.abs().sum(2))
+    del prod
+    # the heads' sum is the flat single-head product (another kernel configuration: tile sums)
+    flat = VanillaSDDMMhip(adj)
+    flat.build([placeholder((n, F)), placeholder((n, F))], {}, {})
+    out_flat = flat.run([src.view(n, F), dst.view(n, F)])
+    bound = src.view(n, F).double().norm(dim=1)[col_d] * dst.view(n, F).double().norm(dim=1)[row_d]
+    head_sum = out.double().sum(1)
+    assert ((head_sum - out_flat.double()).abs() <= ATOL + RTOL * out_flat.double().abs()
+            + 2 * MASS_FACTOR * bound).all().item()

@@ -108,3 +108,64 @@ def test_attention_replay(scores):
         for i, (r, e) in enumerate(zip(recorded, eager)):
             assert torch.isfinite(e).all()
             assert torch.equal(r, e), "replay %d: result %d differs from the eager run" % (k, i)
+
+
+def test_scratch_is_reserved_at_build_and_never_grown_under_capture():
+    """build() sizes the plan's scratch (fg_spmm_plan_reserve), so the first run() of a module can be the
+    recorded one; a direct C-ABI call that would have to grow the scratch while its stream is being
+    captured changes nothing and reports FG_ERR_ARG."""
+    import ctypes
+    import torch
+    from featgraph_amd import _lib
+    from featgraph_amd.module import VanillaSpMMhip, placeholder
+    rng = np.random.default_rng(9)
+    n_dst, n_src = 64, 3000
+    adj = sp.random(n_dst, n_src, density=0.01, format="csr", random_state=rng).astype("float32").tolil()
+    adj[5, rng.choice(n_src, size=2600, replace=False)] = 1.0       # split into pieces: needs scratch
+    adj = adj.tocsr().astype("float32"); adj.sort_indices()
+    adj.data = rng.random(adj.nnz).astype("float32")
+    warm = VanillaSpMMhip(adj)
+    warm.build([placeholder((n_src, 8))], {}, {})
+    x8 = torch.randn((n_src, 8), device="cuda")
+    warm.run([x8])                                                  # the library's kernels are loaded
+    torch.cuda.synchronize()
+
+    F = 256
+    m = VanillaSpMMhip(adj)
+    m.build([placeholder((n_src, F))], {}, {})
+    x = torch.randn((n_src, F), device="cuda")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        recorded = m.run([x])                                       # first call of this module
+    graph.replay()
+    torch.cuda.synchronize()
+    ref = adj.astype(np.float64).dot(x.cpu().numpy().astype(np.float64))
+    np.testing.assert_allclose(recorded.cpu().numpy(), ref, rtol=RTOL, atol=1e-4)
+
+    # the C ABI without a reservation
+    L = _lib.lib()
+    plan = ctypes.c_void_p()
+    indptr = np.ascontiguousarray(adj.indptr, dtype=np.int32)
+    assert L.fg_spmm_plan_create(_lib.host_ptr(indptr), n_dst, n_src, 1, None, ctypes.byref(plan)) == 0
+    try:
+        ip, ix, vals = (torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (indptr, adj.indices, adj.data))
+        out = torch.full((n_dst, F), float("nan"), device="cuda")
+        p = _lib.dev_ptr
+        g2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g2):
+            s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            rc = L.fg_spmm_csr_f32(plan, p(ip), p(ix), p(vals), p(x), p(out), F, 0, s)
+        assert rc == -1 and b"fg_spmm_plan_reserve" in L.fg_last_error()
+        assert L.fg_spmm_plan_reserve(plan, 0, 1, F, 0) == 0
+        g3 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g3):
+            s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            rc = L.fg_spmm_csr_f32(plan, p(ip), p(ix), p(vals), p(x), p(out), F, 0, s)
+        assert rc == 0
+        g3.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, recorded)
+        assert L.fg_spmm_plan_reserve(plan, 99, 1, F, 0) == -1
+        assert L.fg_spmm_plan_reserve(plan, 2, 1, 24, 1) == -2          # a tile the tiled SDDMM does not take
+    finally:
+        L.fg_spmm_plan_destroy(plan)

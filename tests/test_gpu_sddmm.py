@@ -49,6 +49,14 @@ def test_reference_x86_cases(torch_cuda, oracle, feat_len, num_feat_partitions, 
     m, out = _run(torch_cuda, VanillaSDDMMx86, coo, src, dst, {'num_feat_partitions': num_feat_partitions},
                   {'num_feat_partitions': num_feat_partitions}, R, C)
     out = out.cpu().numpy()
+    # the reference's knob is honoured: T feature tiles handled by different workgroups
+    from featgraph_amd.module import placeholder
+    text = m.lower_to_ir([placeholder(src.shape), placeholder(dst.shape)], {'num_feat_partitions': num_feat_partitions},
+                         {'num_feat_partitions': num_feat_partitions})
+    if num_feat_partitions > 1:
+        assert "x %d feature tile(s) of %d floats" % (num_feat_partitions, feat_len // num_feat_partitions) in text, text
+    else:
+        assert "feature tile(s)" not in text, text
     if R != 1 or C != 1:
         # stored edge order and the mapping are bit-exact with the reference's partitioner
         eid, prow, pcol = oracle.partition_coo_2d(coo, R, C)

@@ -352,3 +352,19 @@ def test_low_degree_large_graph_properties(torch_cuda):
     for e in (0, nnz - 1):
         rr, cc = int(s._adj_row_indices[e]), int(s._adj_col_indices[e])
         assert abs(e_out[e].item() - float((x[cc].double() * y[rr].double()).sum())) <= 1e-3
+
+
+def test_float64_adjacency_with_partitions(torch_cuda, oracle):
+    """scipy.sparse.random's default dtype: the values are cast to fp32 once, whatever the partition count."""
+    from featgraph_amd.module import VanillaSpMMhip, VanillaSpMMx86
+    rng = np.random.default_rng(21)
+    adj64 = sp.random(90, 140, density=0.1, format="csr", random_state=rng)
+    assert adj64.dtype == np.float64
+    adj64.sort_indices()
+    x = rng.standard_normal((140, 32)).astype("float32")
+    a32 = adj64.astype("float32")
+    ref = oracle.spmm_csr_x86(a32.indptr, a32.indices, a32.data, x)
+    for cls, ctor, sched in ((VanillaSpMMhip, (), {}), (VanillaSpMMhip, (3,), {}), (VanillaSpMMx86, (4,), {}),
+                             (VanillaSpMMhip, (), {'num_src_partitions': 5})):
+        _, out = _run(torch_cuda, cls, adj64, x, {}, sched, *ctor)
+        np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)

@@ -80,8 +80,8 @@ def test_partitioner_edge_cases(fg):
     with pytest.raises(ValueError):
         util_partition_adj_coo_2d(dup, 2, 2)
     f64 = sp.identity(3, dtype="float64", format="csr")
-    with pytest.raises(ValueError):
-        util_convert_csr_to_dds(f64, 2)
+    _, _, v64 = util_convert_csr_to_dds(f64, 2)            # any dtype, as in the reference
+    assert v64.dtype == np.float64 and v64.tolist() == [1.0, 1.0, 1.0]
     # unsorted column ids inside a row keep their stored order within each partition
     uns = sp.csr_matrix((np.array([1, 2, 3, 4], "float32"), np.array([3, 0, 2, 1], "int32"), np.array([0, 4], "int32")),
                         shape=(1, 4))
@@ -222,3 +222,42 @@ def test_partitioners_property_based(fg, oracle):
         assert np.array_equal(eid[mapping], np.arange(1, coo.nnz + 1))
 
     check()
+
+
+@pytest.mark.parametrize("dtype", ["float64", "int64", "int16", "complex64"])
+def test_dds_values_of_any_width(fg, oracle, dtype):
+    """The reference's util keeps the dtype of adj.data (adj_partitioning.py:37-39), e.g. the float64
+    of scipy.sparse.random; values that are not 32 bits wide take the host-side permutation."""
+    from featgraph_amd.util import util_convert_csr_to_dds
+    rng = np.random.default_rng(5)
+    a = sp.random(60, 90, density=0.2, format="csr", random_state=rng)
+    a.data = (a.data * 1000).astype(dtype)
+    a.sort_indices()
+    for P in (1, 3, 8):
+        s1_pos, s1_idx, vals = util_convert_csr_to_dds(a, P)
+        ref_pos, ref_idx, ref_perm = oracle.csr_to_dds(sp.csr_matrix((np.arange(a.nnz, dtype=np.int32), a.indices, a.indptr), shape=a.shape), P)
+        assert vals.dtype == a.data.dtype
+        assert np.array_equal(s1_pos, ref_pos) and np.array_equal(s1_idx, ref_idx)
+        assert np.array_equal(vals, a.data[ref_perm])
+
+
+@pytest.mark.parametrize("R,C", [(4, 1), (1, 3), (2, 5)])
+def test_edge_mapping_restores_stored_order_for_unequal_partition_counts(fg, oracle, R, C):
+    """R != C: the reference's SDDMMbase overwrites num_col_partitions with num_row_partitions
+    (python/featgraph/module/sddmm.py:37) while this build honours both, so the traversal order
+    differs from the reference's there -- but out[edge_mapping] is the unpartitioned result either way."""
+    from featgraph_amd.util import util_partition_adj_coo_2d
+    rng = np.random.default_rng(R * 10 + C)
+    coo = sp.random(50, 70, density=0.15, format="coo", random_state=rng).astype("float32")
+    src = rng.standard_normal((70, 24)).astype("float32")
+    dst = rng.standard_normal((50, 24)).astype("float32")
+    eid, row, col = util_partition_adj_coo_2d(coo, R, C)
+    mapping = np.argsort(eid)
+    assert sorted(eid.tolist()) == list(range(1, coo.nnz + 1))
+    out_part = oracle.sddmm_x86(row, col, src, dst)
+    out_plain = oracle.sddmm_x86(coo.row, coo.col, src, dst)
+    assert np.array_equal(out_part[mapping], out_plain)
+    # blocks in row-major block order: block ids never decrease along the traversal
+    rb = row // -(-50 // R)
+    cb = col // -(-70 // C)
+    assert (np.diff(rb * C + cb) >= 0).all()
