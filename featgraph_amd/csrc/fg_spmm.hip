@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 
 #include <climits>
+#include <mutex>
 #include <string>
 
 #include "fg_common.h"
@@ -965,7 +966,7 @@ fg::ScratchNeed scratch_need(const fg_spmm_plan *pl, const SpmmConfig &c, int F)
 int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
              const float *x, float *out, int F, int T, void *stream, int heads = 1,
              int reduce = FG_REDUCE_SUM, bool allow_no_vals = false, bool head_major = false,
-             int32_t *arg_out = nullptr) {
+             int32_t *arg_out = nullptr, float *fixed_partial = nullptr, size_t fixed_partial_floats = 0) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (arg_out && reduce == FG_REDUCE_SUM) return fail(FG_ERR_ARG, "positions of the selected elements exist for max / min only");
     if (int drc = fg::check_device(pl)) return drc;
@@ -976,7 +977,18 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
     SpmmConfig c;
     int rc = resolve_config(pl, F, T, heads, reduce, aligned16, &c);
     if (rc != FG_OK) return rc;
-    if ((rc = fg::ensure_scratch(pl, scratch_need(pl, c, F), stream)) != FG_OK) return rc;
+    // fixed_partial: the split rows' partial sums go to this buffer of fixed size instead of the plan's,
+    // X is gathered from the caller's matrix (no tile-by-tile copy), and nothing is allocated.
+    fg::ScratchNeed need = scratch_need(pl, c, F);
+    if (fixed_partial) {
+        if (need.partial > fixed_partial_floats)
+            return fail(FG_ERR_SHAPE, "the split rows of this plan need %zu floats of scratch at feature length %d; "
+                        "the fixed buffer of this entry point holds %zu", need.partial, F, fixed_partial_floats);
+        need.tiled = 0;
+    } else if ((rc = fg::ensure_scratch(pl, need, stream)) != FG_OK) {
+        return rc;
+    }
+    float *const partial = fixed_partial ? fixed_partial : pl->partial_dev;
     hipStream_t st = (hipStream_t)stream;
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
@@ -986,7 +998,7 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
     // at F=512, 6.8 -> 6.1 ms at F=256, before the 0.25 / 0.13 ms that the copy takes); the sums
     // are the same, in the same order.
     const int ft = c.V * c.L * c.K;
-    const bool tiled = gathers_tile_major(pl, c, F);
+    const bool tiled = need.tiled > 0;
     if (tiled && (rc = fg::make_tile_major(pl, x, pl->n_src, F, ft, stream)) != FG_OK) return rc;
     for (int p = 0; p < P; ++p) {
         const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
@@ -998,7 +1010,7 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
             a.x = tiled ? pl->tiled_dev + (int64_t)p * width * ft : x + (int64_t)p * width * F;
             a.x_row_bytes = (uint32_t)(tiled ? ft : F) * 4u;
             a.x_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * ft * 4u) : 0u;
-            a.out = out; a.partial = pl->partial_dev;
+            a.out = out; a.partial = partial;
             a.F = F; a.tile_w = c.tile_w; a.sub_per_tile = c.sub_per_tile;
             a.heads = heads; a.head_len = F / heads;
             a.vstride = head_major ? 1 : heads; a.head_stride = head_major ? pl->nnz : 1;
@@ -1025,14 +1037,14 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
             const unsigned blocks = (unsigned)((threads + 255) / 256);
             const Fixup *fx = pl->fixups_dev + x0;
             if (reduce == FG_REDUCE_SUM) {
-                if (fv == 4) hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F, (int)(p > 0));
-                else hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F, (int)(p > 0));
+                if (fv == 4) hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F, (int)(p > 0));
+                else hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F, (int)(p > 0));
             } else if (reduce == FG_REDUCE_MAX) {
-                if (fv == 4) hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<4, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F);
-                else hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<1, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F);
+                if (fv == 4) hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<4, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F);
+                else hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<1, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F);
             } else {
-                if (fv == 4) hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<4, false>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F);
-                else hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<1, false>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pl->partial_dev, out, F);
+                if (fv == 4) hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<4, false>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F);
+                else hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<1, false>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F);
             }
         }
     }

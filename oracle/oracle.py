@@ -57,6 +57,8 @@ def lib():
         L.orc_edge_softmax_backward.argtypes = [_i64, _int, _i32p, _f32p, _f32p, _f32p, _int]
         L.orc_sddmm_x86.argtypes = [_i64, _i64, _i64, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int, _int, _int]
         L.orc_sddmm_multihead.argtypes = [_i64, _int, _int, _i32p, _i32p, _f32p, _f32p, _f32p, _int]
+        for name in ("orc_spmm_csr_x86", "orc_spmm_dds_x86", "orc_sddmm_x86"):       # timing-only copies
+            getattr(L, name.replace("orc_", "orcf_")).argtypes = getattr(L, name).argtypes
         L.orc_csr_to_dds.argtypes = [_i64, _i64, _i32p, _i32p, _u32p, _int, _i32p, _i32p, _u32p]
         L.orc_partition_coo_2d.argtypes = [_i64, _i64, _i64, _i32p, _i32p, _int, _int, _i32p, _i32p, _i32p]
         _lib = L
@@ -81,14 +83,15 @@ def _check(rc, what):
         raise RuntimeError("oracle %s failed with code %d" % (what, rc))
 
 
-def spmm_csr_x86(indptr, indices, vals, x, num_feat_partitions=1, nthreads=1):
-    """python/featgraph/op/vanilla_spmm.py:6-62 + schedule :65-80."""
+def spmm_csr_x86(indptr, indices, vals, x, num_feat_partitions=1, nthreads=1, fast=False):
+    """python/featgraph/op/vanilla_spmm.py:6-62 + schedule :65-80.
+    fast: the timing-only copy (fused multiply-add, AVX-512 where the CPU has it); not a parity reference."""
     indptr = _c(indptr, np.int32); indices = _c(indices, np.int32)
     vals = _c(vals, np.float32); x = _c(x, np.float32)
     n_dst = indptr.shape[0] - 1
     n_src, F = x.shape
     out = np.empty((n_dst, F), dtype=np.float32)
-    _check(lib().orc_spmm_csr_x86(n_dst, n_src, F, _p(indptr, _i32p), _p(indices, _i32p),
+    _check((lib().orcf_spmm_csr_x86 if fast else lib().orc_spmm_csr_x86)(n_dst, n_src, F, _p(indptr, _i32p), _p(indices, _i32p),
                                   _p(vals, _f32p), _p(x, _f32p), _p(out, _f32p),
                                   num_feat_partitions, nthreads), "spmm_csr_x86")
     return out
@@ -108,14 +111,14 @@ def spmm_csr_rowwise(indptr, indices, vals, x, nthreads=1):
 
 
 def spmm_dds_x86(s1_pos, s1_idx, vals, x, n_dst, num_col_partitions,
-                 num_feat_partitions=1, nthreads=1):
-    """python/featgraph/op/vanilla_spmm.py:149-224 + schedule :227-246."""
+                 num_feat_partitions=1, nthreads=1, fast=False):
+    """python/featgraph/op/vanilla_spmm.py:149-224 + schedule :227-246.  fast: as for spmm_csr_x86."""
     s1_pos = _c(s1_pos, np.int32); s1_idx = _c(s1_idx, np.int32)
     vals = _c(vals, np.float32); x = _c(x, np.float32)
     n_src, F = x.shape
     assert s1_pos.shape[0] == num_col_partitions * (n_dst + 1)
     out = np.empty((n_dst, F), dtype=np.float32)
-    _check(lib().orc_spmm_dds_x86(n_dst, n_src, F, num_col_partitions, _p(s1_pos, _i32p),
+    _check((lib().orcf_spmm_dds_x86 if fast else lib().orc_spmm_dds_x86)(n_dst, n_src, F, num_col_partitions, _p(s1_pos, _i32p),
                                   _p(s1_idx, _i32p), _p(vals, _f32p), _p(x, _f32p),
                                   _p(out, _f32p), num_feat_partitions, nthreads), "spmm_dds_x86")
     return out
@@ -188,8 +191,8 @@ def edge_softmax_backward(indptr, a, g, nthreads=1):
     return out
 
 
-def sddmm_x86(row, col, src, dst, num_feat_partitions=1, parallel_edges=False, nthreads=1):
-    """python/featgraph/op/vanilla_sddmm.py:6-63 + schedule :66-74.
+def sddmm_x86(row, col, src, dst, num_feat_partitions=1, parallel_edges=False, nthreads=1, fast=False):
+    """python/featgraph/op/vanilla_sddmm.py:6-63 + schedule :66-74.  fast: as for spmm_csr_x86.
 
     ``src`` is gathered with ``col`` and ``dst`` with ``row`` (:47)."""
     row = _c(row, np.int32); col = _c(col, np.int32)
@@ -198,7 +201,7 @@ def sddmm_x86(row, col, src, dst, num_feat_partitions=1, parallel_edges=False, n
     F = src.shape[1]
     assert dst.shape[1] == F and col.shape[0] == E
     out = np.empty((E,), dtype=np.float32)
-    _check(lib().orc_sddmm_x86(E, src.shape[0], dst.shape[0], F, _p(row, _i32p), _p(col, _i32p),
+    _check((lib().orcf_sddmm_x86 if fast else lib().orc_sddmm_x86)(E, src.shape[0], dst.shape[0], F, _p(row, _i32p), _p(col, _i32p),
                                _p(src, _f32p), _p(dst, _f32p), _p(out, _f32p),
                                num_feat_partitions, int(bool(parallel_edges)), nthreads), "sddmm_x86")
     return out

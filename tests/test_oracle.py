@@ -431,3 +431,30 @@ def test_graph_attention_additive_dense_form(oracle):
     lin = oracle.graph_attention_additive_f64(adj.indptr, adj.indices, er, el, v, 1.0)
     lin0 = oracle.graph_attention_additive_f64(adj.indptr, adj.indices, np.zeros_like(er), el, v, 1.0)
     np.testing.assert_allclose(lin, lin0, rtol=1e-9, atol=1e-12)
+
+
+def test_timing_copies_stay_within_tolerance_of_the_pinned_loops(oracle):
+    """orcf_* (fused multiply-add, AVX-512 clones) are what bench.py times beside the pinned loops; they
+    pin nothing themselves and only have to agree with the pinned functions within the fp32 bar."""
+    rng = np.random.default_rng(77)
+    a = sp.random(300, 500, density=0.08, format="csr", random_state=rng).astype("float32")
+    a.sort_indices()
+    for F, T in ((64, 1), (64, 4), (96, 3), (7, 1)):
+        x = rng.standard_normal((500, F)).astype("float32")
+        y = rng.standard_normal((300, F)).astype("float32")
+        ref = oracle.spmm_csr_x86(a.indptr, a.indices, a.data, x, T, 2)
+        np.testing.assert_allclose(oracle.spmm_csr_x86(a.indptr, a.indices, a.data, x, T, 2, fast=True), ref,
+                                   rtol=1e-4, atol=1e-5)
+        for P in (1, 3):
+            s1_pos, s1_idx, vals = oracle.csr_to_dds(a, P)
+            ref = oracle.spmm_dds_x86(s1_pos, s1_idx, vals, x, 300, P, T, 2)
+            np.testing.assert_allclose(oracle.spmm_dds_x86(s1_pos, s1_idx, vals, x, 300, P, T, 2, fast=True), ref,
+                                       rtol=1e-4, atol=1e-5)
+        coo = a.tocoo()
+        ref = oracle.sddmm_x86(coo.row, coo.col, x, y, T)
+        for par in (False, True):
+            np.testing.assert_allclose(oracle.sddmm_x86(coo.row, coo.col, x, y, T, par, 3, fast=True), ref,
+                                       rtol=1e-4, atol=1e-5)
+    empty = sp.csr_matrix((5, 9), dtype="float32")
+    x = rng.standard_normal((9, 8)).astype("float32")
+    assert (oracle.spmm_csr_x86(empty.indptr, empty.indices, empty.data, x, 2, 2, fast=True) == 0).all()
