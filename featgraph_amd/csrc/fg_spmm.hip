@@ -1112,6 +1112,50 @@ extern "C" int fg_spmm_csr_f32(fg_spmm_plan *plan, const int32_t *indptr_dev,
     return spmm_run(plan, indptr_dev, indices_dev, vals_dev, x_dev, out_dev, F, num_feat_partitions, stream);
 }
 
+// ---- an SpMM entry point that allocates nothing ------------------------------------------------
+//
+// The split rows' partial sums (one row of F floats per piece) live in a file-scope device array
+// instead of plan-owned memory.  Every device the library runs on holds its own copy of the array
+// until the process ends; its address on a device is looked up once, with that device current.
+namespace {
+constexpr size_t kFixedScratchFloats = (size_t)4 << 20;          // 16 MiB
+static __device__ __align__(256) float scratch[kFixedScratchFloats];
+
+constexpr int kMaxDevices = 64;
+float *g_scratch_ptr[kMaxDevices];                                // address of `scratch` per device, once known
+std::mutex g_scratch_mutex;
+
+// The device address of `scratch` on the current device `dev` (the array's name is a host-side
+// handle, never an address a kernel could use).
+int fixed_scratch(int dev, float **ptr) {
+    if (dev < 0 || dev >= kMaxDevices) return fail(FG_ERR_ARG, "device %d: at most %d devices are supported", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(FG_ERR_HIP, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = static_cast<float *>(p);
+    }
+    *ptr = g_scratch_ptr[dev];
+    return FG_OK;
+}
+}  // namespace
+
+extern "C" int fg_spmm_csr_noalloc_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev,
+                                       const int32_t *indices_dev, const float *vals_dev, const float *x_dev,
+                                       float *out_dev, int F, int num_feat_partitions, void *stream) {
+    if (!plan) return fail(FG_ERR_ARG, "plan is null");
+    if (plan->num_col_partitions != 1)
+        return fail(FG_ERR_ARG, "fg_spmm_csr_noalloc_f32 needs a plan with one column partition");
+    if (int drc = fg::check_device(plan)) return drc;        // the plan's device is the current one
+    float *ptr = nullptr;
+    if (int rc = fixed_scratch(plan->device, &ptr)) return rc;
+    // The plan is only read here: every buffer the kernels write is the caller's or the fixed array.
+    return spmm_run(const_cast<fg_spmm_plan *>(plan), indptr_dev, indices_dev, vals_dev, x_dev, out_dev, F,
+                    num_feat_partitions, stream, 1, FG_REDUCE_SUM, false, false, nullptr, ptr, kFixedScratchFloats);
+}
+
 extern "C" int fg_spmm_dds_f32(fg_spmm_plan *plan, const int32_t *s1_pos_dev,
                                const int32_t *s1_idx_dev, const float *vals_dev, const float *x_dev,
                                float *out_dev, int F, int num_feat_partitions, void *stream) {
