@@ -182,7 +182,7 @@ class SDDMMbase(object):
         tiled = None
         nnz = self._adj_row_indices.shape[0]
         if order in ('auto', 'tiled') and nnz > 0:
-            tiled = tuning.choose_sddmm(self._num_rows, self._num_cols, nnz, H, D)
+            tiled = tuning.choose_sddmm(self._num_rows, self._num_cols, nnz, H, D, self._graph_stats() if H == 1 else None)
             p_arg, t_arg = schedule_args.get('num_src_partitions'), schedule_args.get('num_feat_tiles')
             if t_arg is None and knob_tiles is not None and order != 'coo' and order != 'csr':
                 t_arg = knob_tiles
@@ -193,6 +193,43 @@ class SDDMMbase(object):
                 notes.append("tiled traversal: %d source-column partitions x %d feature tiles; results are "
                              "written back in the stored edge order" % tiled)
         return [src_ph, dst_ph], H, D, use_csr, tiled, notes
+
+    def _graph_stats(self):
+        """Column reference counts and row degrees of the adjacency, as the tuning model reads them (once per object)."""
+        if getattr(self, '_stats', None) is None:
+            counts = np.bincount(self._adj_col_indices, minlength=self._num_cols) if len(self._adj_col_indices) else np.zeros(self._num_cols, np.int64)
+            degs = np.bincount(self._adj_row_indices, minlength=self._num_rows) if len(self._adj_row_indices) else np.zeros(self._num_rows, np.int64)
+            cv, cm = np.unique(counts, return_counts=True)
+            dv, dm = np.unique(degs, return_counts=True)
+            self._stats = tuning.GraphStats(self._num_rows, self._num_cols, len(self._adj_col_indices), cv, cm, dv, dm)
+        return self._stats
+
+    def _tune(self, phs, compute_args, schedule_args, how_many):
+        """Times the stored-order kernel(s) and the cost model's `how_many` most promising tiled traversals on
+        this graph (zero features: the kernels' time does not depend on the values); returns the fastest's schedule arguments."""
+        H, D = self._feature_shape(*phs)
+        cands = [{'order': 'coo'}] + ([{'order': 'csr'}] if self._row_sorted else [])
+        if H == 1:
+            for p, t in tuning.rank_sddmm(self._graph_stats(), D)[:max(1, how_many)]:
+                tile = D // t
+                if (p, t) != (1, 1) and tile <= 256 and tile >= 16 and (tile & (tile - 1)) == 0:
+                    cands.append({'order': 'tiled', 'num_src_partitions': p, 'num_feat_tiles': t})
+        else:
+            cands.append({})
+        src = torch.zeros(phs[0].shape, dtype=torch.float32, device=self._ctx)
+        dst = torch.zeros(phs[1].shape, dtype=torch.float32, device=self._ctx)
+        timed = []
+        for extra in cands:
+            sa = {k: v for k, v in schedule_args.items() if k != 'tune'}
+            sa.update(extra)
+            try:
+                self.build(phs, compute_args, sa)
+            except ValueError:
+                continue
+            timed.append((self.measure_average_time([src, dst], 3), sa))
+        timed.sort(key=lambda e: e[0])
+        self._tuned = [(round(s * 1e3, 4), sa) for s, sa in timed]
+        return timed[0][1]
 
     def build(self, input_placeholders, compute_args, schedule_args):
         """Fix the feature shape and kernel variant, allocate the output once.
@@ -211,8 +248,16 @@ class SDDMMbase(object):
             'num_feat_partitions', 'num_cuda_blocks' (reference keys); 'order' in
             {'auto', 'csr', 'coo', 'tiled'}: which kernel walks the edges ('auto' picks the tiled
             traversal when the feature matrices exceed the L2); 'num_src_partitions' /
-            'num_feat_tiles': override the tiled traversal's shape
+            'num_feat_tiles': override the tiled traversal's shape; 'tune': k -- time the stored-order
+            kernels and the cost model's k most promising tiled traversals on this graph and keep the
+            fastest (True: 6), in the manner of the reference's own sweeps
+            (benchmark/bench_vanilla_sddmm.py:41-46); only when no order / shape was given
         """
+        tune = schedule_args.get('tune')
+        if tune and len(input_placeholders) == 2 and not any(k in schedule_args for k in ('order', 'num_src_partitions', 'num_feat_tiles')) \
+                and (compute_args.get('num_feat_partitions', 1) or 1) == 1 and self._adj_row_indices.shape[0] > 0:
+            schedule_args = self._tune(list(input_placeholders), dict(compute_args), dict(schedule_args), 6 if tune is True else int(tune))
+        schedule_args = {k: v for k, v in schedule_args.items() if k != 'tune'}
         phs, H, D, use_csr, tiled, notes = self._resolve(input_placeholders, compute_args, schedule_args)
         self._placeholders = phs
         self._heads, self._head_len, self._use_csr, self._notes = H, D, use_csr, notes
@@ -299,7 +344,7 @@ class SDDMMbase(object):
 class VanillaSDDMMhip(SDDMMbase):
     """Edge-wise dot product on gfx950, optionally over a 2-D partitioned edge order."""
     _compute_keys = ('num_feat_partitions',)
-    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles')
+    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles', 'tune')
     _out_1d = True
 
     def __init__(self, adj_scipy, num_row_partitions=1, num_col_partitions=1):
@@ -313,13 +358,13 @@ class VanillaSDDMMhip(SDDMMbase):
 class VanillaSDDMMx86(VanillaSDDMMhip):
     """Constructor and knobs of the reference's VanillaSDDMMx86
     (python/featgraph/module/sddmm.py:168-176); the partitioned traversal runs on the GPU."""
-    _schedule_keys = ('num_feat_partitions', 'order', 'num_src_partitions', 'num_feat_tiles')
+    _schedule_keys = ('num_feat_partitions', 'order', 'num_src_partitions', 'num_feat_tiles', 'tune')
 
 
 class VanillaSDDMMcuda(VanillaSDDMMhip):
     """Constructor and knobs of the reference's VanillaSDDMMcuda
     (python/featgraph/module/sddmm.py:179-187): no partitioning, hence no edge_mapping."""
-    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles')
+    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles', 'tune')
 
     def __init__(self, adj_scipy):
         super(VanillaSDDMMcuda, self).__init__(adj_scipy, num_row_partitions=1, num_col_partitions=1)

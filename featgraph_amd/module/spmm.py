@@ -132,7 +132,8 @@ class SpMMbase(object):
         P = self._num_col_partitions
         src_parts = schedule_args.get('num_src_partitions', 'auto')
         if P == 1 and src_parts is not None:
-            auto_p, auto_t = tuning.choose_spmm(self._num_rows, self._num_cols, self._adj_indices.shape[0], feat_len)
+            auto_p, auto_t = tuning.choose_spmm(self._num_rows, self._num_cols, self._adj_indices.shape[0], feat_len,
+                                                self._graph_stats())
             P = auto_p if src_parts == 'auto' else int(src_parts)
             if P < 1:
                 raise ValueError("num_src_partitions must be >= 1")
@@ -145,6 +146,29 @@ class SpMMbase(object):
             # (tiling changes which workgroup computes a column, not the sums)
             T = tuning.feature_tiles(feat_len)
         return ph, feat_len, int(T), P, notes
+
+    def _graph_stats(self):
+        """Column reference counts and row degrees of the adjacency, as the tuning model reads them (once per object)."""
+        if getattr(self, '_stats', None) is None:
+            self._stats = tuning.GraphStats.from_csr(self._adj_indptr, self._adj_indices, self._num_cols)
+        return self._stats
+
+    def _tune(self, ph, compute_args, schedule_args, how_many):
+        """Times the model's `how_many` most promising (partitions, tiles) on this graph (zero features:
+        the kernels' time does not depend on the values) and returns the fastest as schedule / compute arguments."""
+        feat_len = ph.shape[1]
+        cands = tuning.rank_spmm(self._graph_stats(), feat_len)[:max(1, how_many)]
+        x = torch.zeros(ph.shape, dtype=torch.float32, device=self._ctx)
+        timed = []
+        for p, t in cands:
+            ca = dict(compute_args, num_feat_partitions=t)
+            sa = dict(schedule_args, num_src_partitions=(p if p > 1 else None))
+            sa.pop('tune', None)
+            self.build([ph], ca, sa)
+            timed.append((self.measure_average_time([x], 3), p, t, ca, sa))
+        timed.sort(key=lambda e: e[0])
+        self._tuned = [(round(s * 1e3, 4), p, t) for s, p, t, _, _ in timed]
+        return timed[0][3], timed[0][4]
 
     def build(self, input_placeholders, compute_args, schedule_args):
         """Fix the feature length and kernel variant, allocate the output once.
@@ -161,7 +185,16 @@ class SpMMbase(object):
             The reference's CUDA keys 'num_cuda_blocks' / 'num_threads_per_cuda_block' are accepted.
             'num_src_partitions': 'auto' (default) | int | None -- source-column partitions used
             when the constructor was left at one partition (None: plain CSR).
+            'tune': k -- time the cost model's k most promising (partitions, tiles) on this graph
+            and keep the fastest (True: 6), in the manner of the reference's own sweeps
+            (benchmark/bench_vanilla_spmm.py:36-41); only when neither knob was given.
         """
+        tune = schedule_args.get('tune') if isinstance(schedule_args, dict) else None
+        if tune and self._num_col_partitions == 1 and not compute_args.get('num_feat_partitions') \
+                and schedule_args.get('num_src_partitions', 'auto') == 'auto' and len(input_placeholders) == 1:
+            compute_args, schedule_args = self._tune(input_placeholders[0], dict(compute_args), dict(schedule_args),
+                                                     6 if tune is True else int(tune))
+        schedule_args = {k: v for k, v in schedule_args.items() if k != 'tune'}
         ph, feat_len, T, P, notes = self._resolve(input_placeholders, compute_args, schedule_args)
         self._placeholders = [ph]
         self._feat_len = feat_len
@@ -228,7 +261,7 @@ class SpMMbase(object):
 class VanillaSpMMhip(SpMMbase):
     """CSR (or, with num_col_partitions > 1, DDS) SpMM on gfx950."""
     _compute_keys = ('num_feat_partitions',)
-    _schedule_keys = ('num_cuda_blocks', 'num_threads_per_cuda_block', 'num_src_partitions')
+    _schedule_keys = ('num_cuda_blocks', 'num_threads_per_cuda_block', 'num_src_partitions', 'tune')
 
     def __init__(self, adj_scipy, num_col_partitions=1):
         super(VanillaSpMMhip, self).__init__(adj_scipy, num_col_partitions)
@@ -242,7 +275,7 @@ class VanillaSpMMx86(VanillaSpMMhip):
     """Constructor and knobs of the reference's VanillaSpMMx86
     (python/featgraph/module/spmm.py:197-209): source-column partitions at init,
     'num_feat_partitions' at build.  Both partitionings are carried out on the GPU."""
-    _schedule_keys = ('num_src_partitions',)
+    _schedule_keys = ('num_src_partitions', 'tune')
 
 
 class VanillaSpMMcuda(VanillaSpMMhip):

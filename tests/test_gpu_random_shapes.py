@@ -149,3 +149,34 @@ def test_random_attention(oracle, monkeypatch, seed):
         ref = oracle.graph_attention_f64(adj.indptr, adj.indices, q, k, v, 1.0 / np.sqrt(D))
         assert np.isfinite(out).all(), what
         np.testing.assert_allclose(out, ref, rtol=1e-4, atol=2e-5, err_msg=what)
+
+
+def test_tuned_choice_is_one_of_the_candidates_and_right():
+    """schedule_args {'tune': k}: the module times the cost model's candidates on its own graph, keeps the
+    fastest, and the result is the same product."""
+    import torch
+    from featgraph_amd import tuning
+    from featgraph_amd.module import VanillaSpMMhip, VanillaSDDMMhip, placeholder
+    rng = np.random.default_rng(5)
+    adj = sp.random(3000, 4000, density=0.01, format="csr", random_state=rng).astype("float32")
+    adj.sort_indices()
+    F = 128
+    x = rng.standard_normal((4000, F)).astype("float32")
+    y = rng.standard_normal((3000, F)).astype("float32")
+    m = VanillaSpMMhip(adj)
+    m.build([placeholder((4000, F))], {}, {'tune': 3})
+    assert len(m._tuned) == 3 and m._tuned[0][0] <= m._tuned[-1][0]
+    ranked = tuning.rank_spmm(m._graph_stats(), F)[:3]
+    assert (m._tuned[0][1], m._tuned[0][2]) in ranked
+    out = m.run([torch.from_numpy(x).cuda()]).cpu().numpy()
+    np.testing.assert_allclose(out, adj.astype(np.float64).dot(x.astype(np.float64)), rtol=1e-4, atol=1e-4)
+    s = VanillaSDDMMhip(adj)
+    s.build([placeholder((4000, F)), placeholder((3000, F))], {}, {'tune': True})
+    assert len(s._tuned) >= 2
+    coo = adj.tocoo()
+    got = s.run([torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda()]).cpu().numpy()
+    ref = (x[coo.col].astype(np.float64) * y[coo.row].astype(np.float64)).sum(1)
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-4)
+    # explicit knobs win over 'tune'
+    m.build([placeholder((4000, F))], {'num_feat_partitions': 2}, {'tune': True, 'num_src_partitions': 2})
+    assert m._active['P'] == 2 and m._num_feat_partitions == 2

@@ -164,23 +164,48 @@ def test_bench_refuses_more_than_one_gpu():
 
 
 def test_default_tilings():
-    """The defaults the modules pick for the benchmark shapes (pure arithmetic, no GPU)."""
+    """The defaults the cost model picks for the benchmark shapes (pure arithmetic, no GPU), with and without
+    the graph's own statistics, and the model's building blocks."""
     from featgraph_amd import tuning
     n, nnz = 232965, 114766039
     assert tuning.choose_spmm(n, n, nnz, 512) == (8, 8)
     assert tuning.choose_spmm(n, n, nnz, 128) == (8, 2)
+    assert tuning.choose_spmm(n, n, nnz, 32) == (4, 0)
     assert tuning.choose_spmm(2450000, 2450000, 61903880, 128) == (1, 1)     # rows too short to partition
+    assert tuning.choose_spmm(1000000, 1000000, 64998031, 128) == (1, 1)     # no slice an L2 could hold: plain CSR
     assert tuning.choose_sddmm(n, n, nnz, 1, 512) == (8, 8)
     assert tuning.choose_sddmm(n, n, nnz, 1, 256) == (8, 4)
     assert tuning.choose_sddmm(n, n, nnz, 1, 1024) == (8, 16)
+    assert tuning.choose_sddmm(2450000, 2450000, 61903880, 1, 128) is None    # stored-order kernels
     assert tuning.choose_sddmm(n, n, nnz, 8, 64) == (16, 4)
     assert tuning.choose_sddmm(n, n, nnz, 4, 64) == (8, 4)
     assert tuning.choose_sddmm(n, n, nnz, 8, 32) == (16, 2)
     assert tuning.choose_sddmm(n, n, nnz, 4, 32) == (8, 2)
     assert tuning.choose_sddmm(10000, 10000, 170000, 1, 32) is None           # fits the caches: plain kernels
-    for F in (32, 64, 128, 256, 512):
+    for F in (32, 64, 96, 128, 256, 512, 2048):
         p, t = tuning.choose_sddmm(n, n, nnz, 1, F)
-        assert F % t == 0 and p >= 1
+        assert F % t == 0 and p >= 1 and F // t >= 32
+        p, t = tuning.choose_spmm(n, n, nnz, F)
+        assert p >= 1 and (t == 0 or F % t == 0)
+    # hit-rate estimate: monotone in the capacity, 0 for an empty cache, compulsory misses only when all fits
+    skew = tuning.GraphStats(1000, 1000, 100000, count_vals=[10, 1000], count_mult=[900, 91], deg_vals=[100], deg_mult=[1000])
+    rates = [skew.hit_rate(k) for k in (1, 10, 91, 300, 991, 5000)]
+    assert all(a <= b + 1e-12 for a, b in zip(rates, rates[1:])) and rates[0] < 0.05
+    assert abs(rates[-1] - (1 - 991 / 100000)) < 1e-9
+    assert rates[2] > 0.5                     # the 91 hot columns carry 91 % of the references
+    flat = tuning.GraphStats(1000, 1000, 100000)
+    assert abs(flat.hit_rate(500) - 0.5) < 0.1
+    # row segments: a row of degree d over P partitions
+    assert flat.segments(1) == 1000 and abs(flat.segments(4) - 4000) < 1
+    short = tuning.GraphStats(1000, 1000, 2000, deg_vals=[2], deg_mult=[1000])
+    assert abs(short.segments(8) - 1000 * 8 * (1 - (7 / 8) ** 2)) < 1e-6
+    # statistics from a CSR
+    ip = np.array([0, 2, 2, 5], np.int32); ix = np.array([0, 3, 3, 1, 0], np.int32)
+    st = tuning.GraphStats.from_csr(ip, ix, 4)
+    assert (st.n_dst, st.n_src, st.nnz) == (3, 4, 5)
+    assert dict(zip(st.count_vals.tolist(), st.count_mult.tolist())) == {1.0: 1.0, 2.0: 2.0}
+    # ranked candidates start with the choice
+    assert tuning.rank_spmm(tuning.GraphStats(n, n, nnz), 512)[0] == (8, 8)
 
 
 def test_partitioners_property_based(fg, oracle):
