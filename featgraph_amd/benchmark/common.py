@@ -24,13 +24,14 @@ def load_adjacency(args, fmt):
         return adj.astype(np.float32)
     indptr, indices = synthetic.make_workload(args.workload)
     n = indptr.shape[0] - 1
+    n_src = synthetic.WORKLOADS[args.workload]["n"]
     vals = synthetic.edge_weights(indices.shape[0], 1) if indices.shape[0] < 5_000_000 else None
     if vals is None:
         import torch
         g = torch.Generator(device="cuda")
         g.manual_seed(1)
         vals = torch.rand(indices.shape[0], generator=g, device="cuda").cpu().numpy()
-    adj = scipy.sparse.csr_matrix((vals, indices, indptr), shape=(n, n))
+    adj = scipy.sparse.csr_matrix((vals, indices, indptr), shape=(n, n_src))
     return adj if fmt == 'csr' else adj.tocoo()
 
 

@@ -103,11 +103,25 @@ WORKLOADS = {
     "powerlaw-233k": dict(kind="powerlaw", n=232965, total_edges=120_600_000, exponent=2.1, max_degree=26500),
     "powerlaw-2.45M": dict(kind="powerlaw", n=2_450_000, total_edges=61_970_000, exponent=2.5, max_degree=17600),
     "powerlaw-23k": dict(kind="powerlaw", n=23296, total_edges=1_146_000, exponent=2.1, max_degree=2000),
+    # graphs of other shapes, for checking that the tiling defaults carry over (seeds of their own)
+    "uniform-1M-deg64": dict(kind="uniform", n=1_000_000, avg_degree=64, seed=11),
+    "powerlaw-1M-deg100-g2.5": dict(kind="powerlaw", n=1_000_000, total_edges=100_000_000, exponent=2.5, max_degree=30000, seed=12),
+    # non-square: the first 100,000 destination rows of a 1M-node graph, all 1M sources
+    "nonsquare-100k-x-1M": dict(kind="powerlaw", n=1_000_000, total_edges=80_000_000, exponent=2.2, max_degree=20000, seed=13,
+                                rows=100_000),
 }
 
 
-def make_workload(name, seed=0xFEA7, num_threads=0):
+def make_workload(name, seed=None, num_threads=0):
+    """(indptr, indices) of a named workload; the number of source vertices is WORKLOADS[name]['n']."""
     spec = WORKLOADS[name]
+    if seed is None:
+        seed = spec.get("seed", 0xFEA7)
     if spec["kind"] == "uniform":
-        return uniform_csr(spec["n"], spec["avg_degree"], seed, num_threads)
-    return powerlaw_csr(spec["n"], spec["total_edges"], spec["exponent"], spec["max_degree"], seed, num_threads)
+        indptr, indices = uniform_csr(spec["n"], spec["avg_degree"], seed, num_threads)
+    else:
+        indptr, indices = powerlaw_csr(spec["n"], spec["total_edges"], spec["exponent"], spec["max_degree"], seed, num_threads)
+    if "rows" in spec:
+        indptr = indptr[:spec["rows"] + 1].copy()
+        indices = indices[:indptr[-1]].copy()
+    return indptr, indices
