@@ -33,13 +33,20 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # Fabric-side bytes (rocprofv3 FETCH_SIZE x2 + WRITE_SIZE, scaled by the X copy of the same run) moved
-# by all launches of the named kernel in one operator call, at the default tiling (the JSON reports
-# them per launch as `traffic` and per operator as `op_traffic`); from
-# profiles/bench_powerlaw233k_f512_rocprofv3.txt.  Other configurations have no measurement: null.
-_PROFILE_F512 = "profiles/bench_powerlaw233k_f512_rocprofv3.txt"
+# by all launches of the gather kernel in one operator call, at the default tiling (the JSON reports
+# them per launch as `traffic` and per operator as `op_traffic`, and names the summary they come from as
+# `traffic_source`).  Configurations without a committed summary: null.
+_PROFILES = "profiles/bench_%s_rocprofv3.txt"
 MEASURED_TRAFFIC = {
-    ("spmm", "powerlaw-233k", 512, 8, 8): (72.4e9, _PROFILE_F512),     # 8 x spmm_items_kernel + fix-ups (copy: +0.95e9)
-    ("sddmm", "powerlaw-233k", 512, 8, 8): (70.9e9, _PROFILE_F512),    # 8 x sddmm_tiled_kernel (copy: +0.95e9, tile sum: +4.7e9)
+    # (operator, workload, F, partitions, tiles): (bytes, summary); tiles 0 = the kernel's own single tile
+    ("spmm", "powerlaw-233k", 512, 8, 8): (72.3e9, _PROFILES % "powerlaw233k_f512"),     # 8 x spmm_items_kernel (copy: +0.95e9)
+    ("sddmm", "powerlaw-233k", 512, 8, 8): (70.9e9, _PROFILES % "powerlaw233k_f512"),    # 8 x sddmm_tiled_kernel (copy: +0.95e9, tile sum: +4.7e9)
+    ("spmm", "powerlaw-233k", 64, 8, 0): (9.05e9, _PROFILES % "powerlaw233k_f64"),
+    ("sddmm", "powerlaw-233k", 64, 8, 1): (9.71e9, _PROFILES % "powerlaw233k_f64"),
+    ("spmm", "powerlaw-233k", 32, 4, 0): (4.80e9, _PROFILES % "powerlaw233k_f32"),
+    ("sddmm", "powerlaw-233k", 32, 4, 1): (5.56e9, _PROFILES % "powerlaw233k_f32"),
+    ("spmm", "powerlaw-2.45M", 128, 1, 1): (33.15e9, _PROFILES % "powerlaw2450k_f128"),
+    ("sddmm", "powerlaw-2.45M", 128, 1, 1): (32.86e9, _PROFILES % "powerlaw2450k_f128"),
 }
 METRIC = "SpMM/SDDMM GFLOP/s + achieved HBM GB/s (% roofline), 233k-node graph, feat 512"
 
