@@ -296,6 +296,12 @@ def main():
         default rule: 4 or more feature tiles, 64 MB or more, 32-bit offsets)."""
         return 1 if (n_tiles >= 4 and (64 << 20) <= 4 * n * F < (1 << 32)) else 0
 
+    def pass_sums(n_parts):
+        """Launches of the kernel that adds the SpMM passes' own buffers into out (the library's default rule:
+        4 or more source partitions, an output of 256 MB or more, buffers of 8 GiB or less)."""
+        out_bytes = 4 * n * F
+        return 1 if (n_parts >= 4 and out_bytes >= (256 << 20) and out_bytes * n_parts <= (8 << 30)) else 0
+
     flops_op = 2.0 * nnz * F
     b_spmm = spmm_bytes(n, n, nnz, F)
     b_sddmm = sddmm_bytes(n, nnz, F, 1, csr=True)
@@ -304,7 +310,8 @@ def main():
                  "hbm_gbs": b_spmm / t_spmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_spmm / 1e6,
                  "kernel": "spmm_items_kernel", "launches": spmm._active['P'],
                  "kernels": {"tile_major_kernel": copies(spmm._num_feat_partitions or 1),
-                             "spmm_items_kernel": spmm._active['P'], "spmm_fixup_kernel": spmm._active['P']},
+                             "spmm_items_kernel": spmm._active['P'], "spmm_fixup_kernel": spmm._active['P'],
+                             "spmm_pass_sum_kernel": pass_sums(spmm._active['P'])},
                  "num_col_partitions": spmm._active['P'], "num_feat_partitions": spmm._num_feat_partitions},
         "sddmm": {"ms": t_sddmm, "gflops": flops_op / t_sddmm / 1e6, "compulsory_gb": b_sddmm / 1e9,
                   "hbm_gbs": b_sddmm / t_sddmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_sddmm / 1e6,

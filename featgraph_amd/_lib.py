@@ -23,7 +23,7 @@ _int = ctypes.c_int
 class FgPlanOpts(ctypes.Structure):
     _fields_ = [("split_threshold", ctypes.c_int32), ("item_edges", ctypes.c_int32),
                 ("wide_offsets", ctypes.c_int32), ("tile_major", ctypes.c_int32),
-                ("reserved", ctypes.c_int32 * 4)]
+                ("pass_buffers", ctypes.c_int32), ("reserved", ctypes.c_int32 * 3)]
 
 
 # Options every module passes to fg_spmm_plan_create (None: the library's defaults).

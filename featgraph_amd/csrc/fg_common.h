@@ -53,6 +53,7 @@ struct fg_spmm_plan {
     int item_edges = 0;              // element budget of a multi-row item
     bool wide_offsets = false;       // never use 32-bit byte offsets into the feature matrices
     int tile_major = 0;              // fg_plan_opts.tile_major
+    int pass_buffers = 0;            // fg_plan_opts.pass_buffers
     int device = 0;
     // per partition: [item_begin, item_end) and [fixup_begin, fixup_end)
     std::vector<int64_t> item_off, fixup_off;

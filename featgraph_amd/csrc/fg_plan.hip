@@ -46,6 +46,7 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
     pl->num_col_partitions = P; pl->split_threshold = split; pl->item_edges = item_edges;
     pl->wide_offsets = opts && opts->wide_offsets != 0;
     pl->tile_major = opts ? opts->tile_major : 0;
+    pl->pass_buffers = opts ? opts->pass_buffers : 0;
     std::vector<Item> items;
     std::vector<Fixup> fixups;
     items.reserve((size_t)(n_dst + n_dst / 8 + 16));
@@ -93,7 +94,8 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
                 ++r;
                 continue;
             }
-            if (total == 0 && p > 0) continue;  // later partitions only add: nothing to do
+            // (runs of empty segments keep their item in later partitions too: a pass that writes a buffer
+            // of its own must write every row of it, and a pass that adds in place skips them in the kernel)
             items.push_back({start, total, (int32_t)r0, -(int32_t)(r - r0)});
             if (r - r0 > 1) pl->n_multi_items++;
         }
