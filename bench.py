@@ -298,9 +298,9 @@ def main():
 
     def pass_sums(n_parts):
         """Launches of the kernel that adds the SpMM passes' own buffers into out (the library's default rule:
-        4 or more source partitions, an output of 256 MB or more, buffers of 8 GiB or less)."""
+        4 or more source partitions, an output of 192 MB or more, buffers of 8 GiB or less)."""
         out_bytes = 4 * n * F
-        return 1 if (n_parts >= 4 and out_bytes >= (256 << 20) and out_bytes * n_parts <= (8 << 30)) else 0
+        return 1 if (n_parts >= 4 and out_bytes >= (192 << 20) and out_bytes * n_parts <= (8 << 30)) else 0
 
     flops_op = 2.0 * nnz * F
     b_spmm = spmm_bytes(n, n, nnz, F)

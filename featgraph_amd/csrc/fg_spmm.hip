@@ -975,13 +975,14 @@ size_t piece_floats(const fg_spmm_plan *pl, int F) {
 // instead of every later pass reading and rewriting `out`.  A wavefront's loads return in order, so a row of
 // `out` that has to come from memory holds up the gathers issued behind it; without those reads a pass over
 // the 232,965-node graph takes 1.37 instead of 1.52 ms at F = 512 and the sum of the 8 buffers 0.85 ms:
-// 12.08 -> 11.68 ms (F = 128: 3.19 -> 3.17 ms).  Same sums in the same order: bit-identical results.
+// 12.11 -> 11.68 ms (F = 256, 238 MB of output: 6.30 -> 6.16 ms; F = 128, 119 MB: 3.27 -> 3.29 ms, hence the size
+// rule below).  Same sums in the same order: bit-identical results.
 bool uses_pass_buffers(const fg_spmm_plan *pl, const SpmmConfig &c, int F, int reduce) {
     const int P = pl->num_col_partitions;
     if (P < 2 || reduce != FG_REDUCE_SUM || c.V != 4 || pl->pass_buffers == 2) return false;
     if (pl->pass_buffers == 1) return true;
     const uint64_t out_bytes = (uint64_t)pl->n_dst * (uint64_t)F * 4u;
-    return P >= 4 && out_bytes >= (256ull << 20) && out_bytes * (uint64_t)P <= (8ull << 30);
+    return P >= 4 && out_bytes >= (192ull << 20) && out_bytes * (uint64_t)P <= (8ull << 30);
 }
 
 fg::ScratchNeed scratch_need(const fg_spmm_plan *pl, const SpmmConfig &c, int F, int reduce) {
