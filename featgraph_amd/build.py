@@ -15,12 +15,15 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libfeatgraph_hip.so")
 
-SOURCES = ["fg_host.cpp", "fg_plan.hip", "fg_spmm.hip", "fg_sddmm.hip", "fg_softmax.hip", "fg_attention.hip", "fg_attention_bwd.hip"]
+SOURCES = ["fg_host.cpp", "fg_plan.hip", "fg_spmm.hip", "fg_sddmm.hip", "fg_softmax.hip", "fg_attention.hip", "fg_attention_bwd.hip", "fg_general.hip"]
 
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 instructions.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=fast",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wall", "-Wno-unused-function"]
+# The broadcasting operators promise separately rounded messages and sums (exact max / min and selected
+# positions, sums in stored order): no fused multiply-add in that file.
+EXTRA_FLAGS = {"fg_general.hip": ["-ffp-contract=off"]}
 
 
 def _hipcc():
@@ -32,7 +35,7 @@ def _hipcc():
 
 def _compile(src):
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc()] + HIP_FLAGS + ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc()] + HIP_FLAGS + EXTRA_FLAGS.get(src, []) + ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     return src, obj, res.returncode, res.stdout
 

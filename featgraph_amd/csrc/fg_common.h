@@ -101,6 +101,7 @@ int check_device(const fg_spmm_plan *plan);
 int spmm_scratch_need(const fg_spmm_plan *plan, int F, int heads, int reduce, int num_feat_partitions, ScratchNeed *need);
 int sddmm_dds_scratch_need(const fg_spmm_plan *plan, int H, int D, int num_feat_partitions, ScratchNeed *need);
 int softmax_scratch_need(const fg_spmm_plan *plan, int heads, ScratchNeed *need);
+int gspmm_bcast_scratch_need(const fg_spmm_plan *plan, int out_len, bool with_arg, ScratchNeed *need);
 int attention_scratch_need(const fg_spmm_plan *plan, int heads, int head_len, bool additive, bool own_row_state,
                            ScratchNeed *need);
 }  // namespace fg

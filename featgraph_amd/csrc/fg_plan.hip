@@ -220,6 +220,8 @@ extern "C" int fg_spmm_plan_reserve(fg_spmm_plan *pl, int op, int heads, int hea
         case FG_OP_EDGE_SOFTMAX: rc = fg::softmax_scratch_need(pl, heads, &need); break;
         case FG_OP_ATTENTION: rc = fg::attention_scratch_need(pl, heads, head_len, false, true, &need); break;
         case FG_OP_ATTENTION_ADDITIVE: rc = fg::attention_scratch_need(pl, heads, head_len, true, true, &need); break;
+        case FG_OP_GSPMM_BCAST: rc = fg::gspmm_bcast_scratch_need(pl, heads * head_len, false, &need); break;
+        case FG_OP_GSPMM_BCAST_ARG: rc = fg::gspmm_bcast_scratch_need(pl, heads * head_len, true, &need); break;
         default: return fail(FG_ERR_ARG, "fg_spmm_plan_reserve: unknown operator %d", op);
     }
     if (rc != FG_OK) return rc;

@@ -908,63 +908,14 @@ extern "C" int fg_sddmm_dds_f32(fg_spmm_plan *pl, const int32_t *s1_pos_dev, con
 
 // ---- element-wise edge operators ---------------------------------------------------------------
 //
-// out[e, f] = src[col[e], f] (+ | - | *) dst[row[e], f]: no reduction, F results per edge, so the
-// kernel is bound by writing out.  One edge per lane group of L lanes, V floats per lane per step.
-
-namespace {
-
-template <int OP> __device__ __forceinline__ float ew(float a, float b) { return OP == 0 ? a + b : OP == 1 ? a - b : a * b; }
-template <int OP> __device__ __forceinline__ float4 ew(const float4 &a, const float4 &b) {
-    return make_float4(ew<OP>(a.x, b.x), ew<OP>(a.y, b.y), ew<OP>(a.z, b.z), ew<OP>(a.w, b.w));
-}
-
-template <int V, int OP>
-__global__ __launch_bounds__(kBlock) void gsddmm_elementwise_kernel(const int32_t *row, const int32_t *col,
-                                                                   int64_t n_edges, const float *src,
-                                                                   const float *dst, float *out, int F, int L) {
-    using vec = typename Vec<V>::type;
-    const int lane = threadIdx.x & 63;
-    const int64_t wave_id = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const int G = 64 / L, g = lane / L, li = lane % L;
-    const int64_t e0 = wave_id * 64;                      // 64 edges per wavefront
-    const int per_row = F / V;
-    for (int64_t e = e0 + g; e < min(e0 + 64, n_edges); e += G) {
-        const float *s = src + (int64_t)col[e] * F;
-        const float *d = dst + (int64_t)row[e] * F;
-        float *o = out + e * F;
-        for (int f = li; f < per_row; f += L)
-            *reinterpret_cast<vec *>(o + f * V) = ew<OP>(*reinterpret_cast<const vec *>(s + f * V),
-                                                         *reinterpret_cast<const vec *>(d + f * V));
-    }
-}
-
-template <int V>
-void launch_elementwise(int op, dim3 grid, hipStream_t st, const int32_t *row, const int32_t *col, int64_t n_edges,
-                        const float *src, const float *dst, float *out, int F, int L) {
-    if (op == FG_EDGE_ADD) hipLaunchKernelGGL((gsddmm_elementwise_kernel<V, 0>), grid, dim3(kBlock), 0, st, row, col, n_edges, src, dst, out, F, L);
-    else if (op == FG_EDGE_SUB) hipLaunchKernelGGL((gsddmm_elementwise_kernel<V, 1>), grid, dim3(kBlock), 0, st, row, col, n_edges, src, dst, out, F, L);
-    else hipLaunchKernelGGL((gsddmm_elementwise_kernel<V, 2>), grid, dim3(kBlock), 0, st, row, col, n_edges, src, dst, out, F, L);
-}
-
-}  // namespace
+// out[e, f] = src[col[e], f] (+ | - | *) dst[row[e], f]: the broadcasting kernel of fg_general.hip with both
+// operands in the output's layout (no reduction, F results per edge: bound by writing out).
 
 extern "C" int fg_gsddmm_elementwise_f32(const int32_t *row_dev, const int32_t *col_dev, int64_t n_edges,
                                          const float *src_dev, const float *dst_dev, float *out_dev, int F,
                                          int op, void *stream) {
-    if (F < 1) return fail(FG_ERR_SHAPE, "feature length must be positive, got %d", F);
     if (op != FG_EDGE_ADD && op != FG_EDGE_SUB && op != FG_EDGE_MUL) return fail(FG_ERR_ARG, "unknown edge operator %d", op);
-    if (n_edges < 0) return fail(FG_ERR_ARG, "negative edge count");
-    if (n_edges == 0) return FG_OK;
-    if (!row_dev || !col_dev || !src_dev || !dst_dev || !out_dev) return fail(FG_ERR_ARG, "null device pointer");
-    const bool v4 = F % 4 == 0 && ((((uintptr_t)src_dev | (uintptr_t)dst_dev | (uintptr_t)out_dev) & 15) == 0);
-    const int lanes = v4 ? F / 4 : F;
-    int L = 1;
-    while (L < lanes && L < 64) L <<= 1;
-    const int64_t blocks = ((n_edges + 63) / 64 + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
-    hipStream_t st = (hipStream_t)stream;
-    if (v4) launch_elementwise<4>(op, dim3((unsigned)blocks), st, row_dev, col_dev, n_edges, src_dev, dst_dev, out_dev, F, L);
-    else launch_elementwise<1>(op, dim3((unsigned)blocks), st, row_dev, col_dev, n_edges, src_dev, dst_dev, out_dev, F, L);
-    FG_HIP_TRY(hipGetLastError());
-    return FG_OK;
+    const int bin = op == FG_EDGE_ADD ? FG_BIN_ADD : op == FG_EDGE_SUB ? FG_BIN_SUB : FG_BIN_MUL;
+    return fg_gsddmm_bcast_f32(row_dev, col_dev, n_edges, bin, src_dev, FG_TARGET_U, F, nullptr, dst_dev, FG_TARGET_V, F,
+                               nullptr, 0, out_dev, F, 1, stream);
 }

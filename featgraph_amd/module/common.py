@@ -73,7 +73,8 @@ def timed_mean_seconds(fn, num_runs):
 
 
 # fg_op of include/featgraph_hip.h
-OP_SPMM_SUM, OP_SPMM_EXTREME, OP_SDDMM_DDS, OP_EDGE_SOFTMAX, OP_ATTENTION, OP_ATTENTION_ADDITIVE = range(6)
+(OP_SPMM_SUM, OP_SPMM_EXTREME, OP_SDDMM_DDS, OP_EDGE_SOFTMAX, OP_ATTENTION, OP_ATTENTION_ADDITIVE,
+ OP_GSPMM_BCAST, OP_GSPMM_BCAST_ARG) = range(8)
 
 
 def reserve(plan, op, heads, head_len, num_feat_partitions, dev):

@@ -12,6 +12,7 @@ from .. import _lib
 from .. import tuning
 from ..util import util_convert_csr_to_dds
 from . import common
+from . import general
 from .spmm import VanillaSpMMhip
 
 _REDUCE = {'sum': 0, 'mean': 0, 'max': 1, 'min': 2}
@@ -28,6 +29,14 @@ class GSpMMhip(VanillaSpMMhip):
     Rows without edges give 0 for every reduce.
     'return_arg': True (max / min only) also fills self.arg_tvm, int32 of out's shape: the position, in
     the adjacency's CSR edge order, of the edge whose message was selected (-1 for rows without edges).
+
+    Any other message goes to the library's broadcasting kernel: 'msg' = '<lhs>_<op>_<rhs>' with
+    lhs, rhs in {'u', 'e'} and op in {'add', 'sub', 'mul', 'div'}, or 'copy_e'; the inputs are the two
+    operands in that order ('u': (num_cols, ...), 'e': (nnz, ...) in CSR edge order), whose feature shapes
+    broadcast against each other the numpy way, e.g. 'u_mul_e' with (num_cols, H, D) and (nnz, H, 1), or
+    'u_add_e' with (num_cols, F) and (nnz, F).  out[v] = reduce over row v's edges of the message; out
+    has the broadcast feature shape.  (With 'u_mul_e', a second input of shape (nnz,) or (nnz, H) keeps
+    its meaning of one weight per edge, or per edge and head.)
     """
     _compute_keys = ('num_feat_partitions', 'reduce', 'msg', 'return_arg')
 
@@ -40,8 +49,9 @@ class GSpMMhip(VanillaSpMMhip):
             raise ValueError("return_arg is defined for reduce='max' / 'min' only")
         if reduce not in _REDUCE:
             raise ValueError("reduce must be one of %s" % sorted(_REDUCE))
-        if msg not in ('u_mul_e', 'copy_u'):
-            raise ValueError("msg must be 'u_mul_e' or 'copy_u'")
+        self._bop = None
+        if self._is_broadcast_message(msg, input_placeholders):
+            return self._build_broadcast(input_placeholders, compute_args, schedule_args, msg, reduce, return_arg)
         if len(input_placeholders) not in (1, 2):
             raise ValueError("GSpMM takes SrcFeat and optionally the edge weights")
         src_ph = input_placeholders[0]
@@ -82,6 +92,69 @@ class GSpMMhip(VanillaSpMMhip):
             self._inv_deg_edge = common.to_device_f32(np.repeat(inv, np.diff(self._adj_indptr)), self._ctx)
         self.out_tvm = torch.zeros((self._num_rows,) + tuple(src_ph.shape[1:]), dtype=torch.float32, device=self._ctx)
         self.arg_tvm = torch.full(self.out_tvm.shape, -1, dtype=torch.int32, device=self._ctx) if return_arg else None
+
+    def _is_broadcast_message(self, msg, input_placeholders):
+        if msg not in ('u_mul_e', 'copy_u'):
+            return True
+        if msg == 'u_mul_e' and len(input_placeholders) == 2 and len(input_placeholders[0].shape) in (2, 3):
+            src_ph, e_ph = input_placeholders
+            heads = src_ph.shape[1] if len(src_ph.shape) == 3 else 1
+            nnz = self._adj_indices.shape[0]
+            return tuple(e_ph.shape) not in ((nnz,), (nnz, heads))
+        return False
+
+    def _build_broadcast(self, input_placeholders, compute_args, schedule_args, msg, reduce, return_arg):
+        """Messages with vector edge features or broadcasting between the operands."""
+        common.take_args(compute_args, self._compute_keys, "compute_func")
+        common.take_args(schedule_args, self._schedule_keys, "schedule_func")
+        op, lt, rt = general.parse_message(msg)
+        if len(input_placeholders) != (1 if rt is None else 2):
+            raise ValueError("message %r takes %d input(s), got %d" % (msg, 1 if rt is None else 2, len(input_placeholders)))
+        if self._num_col_partitions != 1:
+            raise ValueError("message %r needs num_col_partitions == 1" % (msg,))
+        nnz = self._adj_indices.shape[0]
+        lhs_ph = input_placeholders[0]
+        rhs_ph = input_placeholders[1] if rt is not None else None
+        self._bop = general.BroadcastOp(op, lt, rt, lhs_ph, rhs_ph, self._num_rows, self._num_cols, nnz, self._ctx, allow_v=False)
+        self._placeholders = list(input_placeholders)
+        self._feat_len, self._heads, self._num_feat_partitions = self._bop.out_len, 1, 0
+        self._reduce, self._msg, self._return_arg = reduce, msg, return_arg
+        self._notes = [self._bop.describe()]
+        if compute_args.get('num_feat_partitions') or schedule_args:
+            self._notes.append("tiling and partitioning knobs do not apply to this message; ignored")
+        self._active = self._layout(1)
+        self._func = _lib.lib().fg_gspmm_bcast_f32
+        common.reserve(self._active['plan'], common.OP_GSPMM_BCAST_ARG if return_arg else common.OP_GSPMM_BCAST,
+                       1, self._bop.out_len, 0, self._ctx)
+        self._row_scale = None
+        if reduce == 'mean':
+            deg = np.diff(self._adj_indptr).astype(np.float32)
+            self._row_scale = common.to_device_f32(np.where(deg > 0, 1.0 / np.maximum(deg, 1), 0), self._ctx)
+        self.out_tvm = torch.zeros((self._num_rows,) + self._bop.out_shape, dtype=torch.float32, device=self._ctx)
+        self.arg_tvm = torch.full(self.out_tvm.shape, -1, dtype=torch.int32, device=self._ctx) if return_arg else None
+
+    def _launch_broadcast(self, inputs):
+        lay = self._active
+        lhs = inputs[0]
+        rhs = inputs[1] if len(inputs) > 1 else None
+        self._bop.run_spmm(lay['plan'], lay['pos'], lay['idx'], _REDUCE[self._reduce], lhs, rhs, self._row_scale,
+                           self.out_tvm, self.arg_tvm)
+
+    def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
+        compute_args = dict(compute_args)
+        msg = compute_args.get('msg', 'u_mul_e')
+        if self._is_broadcast_message(msg, input_placeholders):
+            op, lt, rt = general.parse_message(msg)
+            nnz = self._adj_indices.shape[0]
+            bop = general.BroadcastOp(op, lt, rt, input_placeholders[0], input_placeholders[1] if rt is not None else None,
+                                      self._num_rows, self._num_cols, nnz, self._ctx, allow_v=False)
+            buf = ctypes.create_string_buffer(4096)
+            _lib.check(_lib.lib().fg_spmm_plan_describe(self._layout(1)['plan'], 0, 0, buf, len(buf)))
+            return buf.value.decode() + "  kernel           : gspmm_bcast_kernel, one wavefront per work item\n  note             : %s\n" % bop.describe()
+        for k in ('reduce', 'msg', 'return_arg'):
+            compute_args.pop(k, None)
+        flat = common.placeholder((self._num_cols, int(np.prod(input_placeholders[0].shape[1:]))))
+        return super(GSpMMhip, self).lower_to_ir([flat], compute_args, schedule_args)
 
     def _glayout(self, P):
         """Layout for P source partitions plus, for P > 1, each DDS element's CSR position (so that
@@ -181,13 +254,18 @@ class GSpMMhip(VanillaSpMMhip):
         if self._func is None:
             raise RuntimeError("call build() before run()")
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
-        self._launch(input_tvm_ndarrays[0], input_tvm_ndarrays[1] if self._weights_at_run else None)
+        if self._bop is not None:
+            self._launch_broadcast(input_tvm_ndarrays)
+        else:
+            self._launch(input_tvm_ndarrays[0], input_tvm_ndarrays[1] if self._weights_at_run else None)
         return self.out_tvm
 
     def measure_average_time(self, input_tvm_ndarrays, num_runs):
         if self._func is None:
             raise RuntimeError("call build() before measure_average_time()")
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        if self._bop is not None:
+            return common.timed_mean_seconds(lambda: self._launch_broadcast(input_tvm_ndarrays), num_runs)
         x = input_tvm_ndarrays[0]
         w = input_tvm_ndarrays[1] if self._weights_at_run else None
         return common.timed_mean_seconds(lambda: self._launch(x, w), num_runs)

@@ -9,6 +9,7 @@ from .. import _lib
 from .. import tuning
 from ..util import util_convert_csr_to_dds, util_partition_adj_coo_2d
 from . import common
+from . import general
 
 
 class SDDMMbase(object):
@@ -387,29 +388,99 @@ class MultiHeadSDDMMhip(VanillaSDDMMhip):
 
 
 class GSDDMMhip(VanillaSDDMMhip):
-    """Generalised SDDMM: compute_args {'op': 'dot' | 'add' | 'sub' | 'mul'}.  'dot' is
-    VanillaSDDMMhip; the others give out[e, :] = SrcFeat[col[e], :] op DstFeat[row[e], :] with
-    shape (num_edges, feat_len), in the stored edge order.  Not present in the reference."""
-    _compute_keys = ('num_feat_partitions', 'op')
+    """Generalised SDDMM.  compute_args:
+      'op'         : 'dot' | 'add' | 'sub' | 'mul' | 'div' | 'copy_lhs' | 'copy_rhs'   (default 'dot')
+      'lhs_target' : 'u' | 'v' | 'e'   (default 'u': the first input is indexed by the edge's column)
+      'rhs_target' : 'u' | 'v' | 'e'   (default 'v': the second input is indexed by the edge's row)
+    'dot' with the default targets and equal shapes is VanillaSDDMMhip (2-D inputs) or MultiHeadSDDMMhip (3-D
+    inputs, one result per head) and the element-wise
+    'add' / 'sub' / 'mul' with the default targets and equal 2-D shapes give out[e, :] = SrcFeat[col[e], :]
+    op DstFeat[row[e], :].  Everything else goes to the library's broadcasting kernel: an operand on 'u' has
+    num_cols rows, on 'v' num_rows rows, on 'e' one row per stored edge, in the stored edge order (what
+    edge_mapping refers to); the feature shapes broadcast against each other the numpy way; 'dot' contracts
+    the last axis.  out is (num_edges,) + the broadcast
+    shape, in the stored edge order.
+    Not present in the reference (README.md:9-11 names it)."""
+    _compute_keys = ('num_feat_partitions', 'op', 'lhs_target', 'rhs_target')
     _EDGE_OPS = {'add': 0, 'sub': 1, 'mul': 2}
+
+    def _feature_shape(self, src_ph, dst_ph):
+        if len(src_ph.shape) == 3 and len(dst_ph.shape) == 3:
+            return src_ph.shape[1], src_ph.shape[2]
+        return super(GSDDMMhip, self)._feature_shape(src_ph, dst_ph)
 
     def build(self, input_placeholders, compute_args, schedule_args):
         compute_args = dict(compute_args)
         self._op = compute_args.pop('op', 'dot')
-        if self._op == 'dot':
+        lt = compute_args.pop('lhs_target', 'u')
+        rt = compute_args.pop('rhs_target', 'v')
+        self._bop = None
+        if self._op not in general.BINARY:
+            raise ValueError("op must be one of %s" % sorted(general.BINARY))
+        same = (lt, rt) == ('u', 'v') and len(input_placeholders) == 2 and \
+            input_placeholders[0].shape[1:] == input_placeholders[1].shape[1:]
+        plain = same and len(input_placeholders[0].shape) == 2
+        self._out_1d = True
+        if self._op == 'dot' and same and len(input_placeholders[0].shape) in (2, 3):
+            # the dot-product kernels proper: single head (2-D inputs) or one result per head (3-D inputs)
+            self._out_1d = len(input_placeholders[0].shape) == 2
             return super(GSDDMMhip, self).build(input_placeholders, compute_args, schedule_args)
-        if self._op not in self._EDGE_OPS:
-            raise ValueError("op must be 'dot', 'add', 'sub' or 'mul'")
-        phs, H, D, _, _, notes = self._resolve(input_placeholders, compute_args, dict(schedule_args, order='coo'))
-        self._placeholders, self._heads, self._head_len, self._notes = phs, H, D, notes
+        if plain and self._op in self._EDGE_OPS:
+            phs, H, D, _, _, notes = self._resolve(input_placeholders, compute_args, dict(schedule_args, order='coo'))
+            self._placeholders, self._heads, self._head_len, self._notes = phs, H, D, notes
+            self._tiled, self._use_csr = None, False
+            self._func = _lib.lib().fg_gsddmm_elementwise_f32
+            self.out_tvm = torch.zeros((self._adj_row_indices.shape[0], H * D), dtype=torch.float32, device=self._ctx)
+            return
+        common.take_args(compute_args, self._compute_keys, "compute_func")
+        common.take_args(schedule_args, self._schedule_keys, "schedule_func")
+        single = self._op in ('copy_lhs', 'copy_rhs')
+        if len(input_placeholders) != (1 if single else 2):
+            raise ValueError("op %r takes %d input(s), got %d" % (self._op, 1 if single else 2, len(input_placeholders)))
+        nnz = self._adj_row_indices.shape[0]
+        if single:
+            # one operand: it is the left one of the library call
+            target = lt if self._op == 'copy_lhs' else rt
+            bop = general.BroadcastOp('copy_lhs', target, None, input_placeholders[0], None,
+                                      self._num_rows, self._num_cols, nnz, self._ctx, allow_v=True)
+        else:
+            bop = general.BroadcastOp(self._op, lt, rt, input_placeholders[0], input_placeholders[1],
+                                      self._num_rows, self._num_cols, nnz, self._ctx, allow_v=True)
+        self._bop = bop
+        self._placeholders = list(input_placeholders)
+        self._heads, self._head_len = 1, bop.out_len
+        self._notes = [bop.describe()]
         self._tiled, self._use_csr = None, False
-        self._func = _lib.lib().fg_gsddmm_elementwise_f32
-        self.out_tvm = torch.zeros((self._adj_row_indices.shape[0], H * D), dtype=torch.float32, device=self._ctx)
+        self._func = _lib.lib().fg_gsddmm_bcast_f32
+        self.out_tvm = torch.zeros((nnz,) + tuple(bop.out_shape), dtype=torch.float32, device=self._ctx)
 
     def _launch(self, src_feat, dst_feat):
-        if getattr(self, '_op', 'dot') == 'dot':
+        if getattr(self, '_op', 'dot') == 'dot' and self._bop is None:
             return super(GSDDMMhip, self)._launch(src_feat, dst_feat)
+        if self._bop is not None:
+            self._bop.run_sddmm(self._adj_row_indices_dev, self._adj_col_indices_dev, self._adj_row_indices.shape[0],
+                                src_feat, dst_feat, self.out_tvm)
+            return
         _lib.check(self._func(_lib.dev_ptr(self._adj_row_indices_dev), _lib.dev_ptr(self._adj_col_indices_dev),
                               self._adj_row_indices.shape[0], _lib.dev_ptr(src_feat), _lib.dev_ptr(dst_feat),
                               _lib.dev_ptr(self.out_tvm), self._heads * self._head_len,
                               self._EDGE_OPS[self._op], common.stream_ptr()))
+
+    def run(self, input_tvm_ndarrays):
+        if self._func is None:
+            raise RuntimeError("call build() before run()")
+        if self._bop is None:
+            return super(GSDDMMhip, self).run(input_tvm_ndarrays)
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        self._launch(input_tvm_ndarrays[0], input_tvm_ndarrays[1] if len(input_tvm_ndarrays) > 1 else None)
+        return self.out_tvm
+
+    def measure_average_time(self, input_tvm_ndarrays, num_runs):
+        if self._func is None:
+            raise RuntimeError("call build() before measure_average_time()")
+        if self._bop is None:
+            return super(GSDDMMhip, self).measure_average_time(input_tvm_ndarrays, num_runs)
+        common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
+        a = input_tvm_ndarrays[0]
+        b = input_tvm_ndarrays[1] if len(input_tvm_ndarrays) > 1 else None
+        return common.timed_mean_seconds(lambda: self._launch(a, b), num_runs)

@@ -14,7 +14,10 @@ Two kinds of checker live here:
   restatement and the HIP kernels are compared with.
 
 ``sddmm_multihead`` is PARITY UNPINNED by the reference (it has no multi-head
-op); see the header of ``fg_oracle.c``.
+op); see the header of ``fg_oracle.c``.  So are ``gspmm_bcast`` / ``gsddmm_bcast``
+(numpy restatements of generalised SpMM / SDDMM with broadcasting, which the
+reference only names): the tests pin them by special cases that reduce to the
+pinned operators and to scipy products.
 """
 import ctypes
 import os
@@ -166,6 +169,66 @@ def gspmm_arg(indptr, indices, vals, x, reduce="max", nthreads=1):
     _check(lib().orc_gspmm_arg(n_dst, F, H, _p(indptr, _i32p), _p(indices, _i32p), vp, _p(x2, _f32p),
                                _p(out, _f32p), _p(arg, _i32p), REDUCE[reduce], nthreads), "gspmm_arg")
     return out.reshape((n_dst,) + shape[1:]), arg.reshape((n_dst,) + shape[1:])
+
+
+_BINARY = {
+    "add": lambda l, r: l + r, "sub": lambda l, r: l - r, "mul": lambda l, r: l * r, "div": lambda l, r: l / r,
+    "copy_lhs": lambda l, r: l, "copy_rhs": lambda l, r: r,
+}
+
+
+def _edge_messages(row, col, op, lhs, rhs, lhs_target, rhs_target):
+    """Per stored element e: lhs[i_l(e)] op rhs[i_r(e)] with numpy broadcasting over the feature axes, in
+    float32 (one correctly rounded operation per result, so the values are exact); targets 'u' (column),
+    'v' (row), 'e' (the element).  'dot' contracts the last axis in float64."""
+    e = np.arange(len(row))
+    pick = {"u": col, "v": row, "e": e}
+    l = None if lhs is None else np.asarray(lhs, np.float32)[pick[lhs_target]]
+    r = None if rhs is None else np.asarray(rhs, np.float32)[pick[rhs_target]]
+    if l is not None and r is not None:
+        nd = max(l.ndim, r.ndim)      # align the feature axes to the right, the element axis stays first
+        l = l.reshape((l.shape[0],) + (1,) * (nd - l.ndim) + l.shape[1:])
+        r = r.reshape((r.shape[0],) + (1,) * (nd - r.ndim) + r.shape[1:])
+    if op == "dot":
+        return (l.astype(np.float64) * r.astype(np.float64)).sum(-1)
+    with np.errstate(all="ignore"):
+        m = _BINARY[op](l, r)
+    return np.asarray(m, np.float32)
+
+
+def gsddmm_bcast(row, col, op, lhs, rhs, lhs_target="u", rhs_target="v"):
+    """Generalised SDDMM with broadcasting: out[e] = lhs[..] op rhs[..] per stored edge (op in add / sub / mul /
+    div / copy_lhs / copy_rhs: float32, exact; 'dot': float64).  Not in the reference (README.md:9-11 names it);
+    semantics: numpy broadcasting of the operands' feature shapes."""
+    return _edge_messages(np.asarray(row), np.asarray(col), op, lhs, rhs, lhs_target, rhs_target)
+
+
+def gspmm_bcast(indptr, indices, op, reduce, lhs, rhs, lhs_target="u", rhs_target="e"):
+    """Generalised SpMM with broadcasting: out[v] = reduce over row v's elements of the message
+    lhs[..] op rhs[..] (targets 'u' / 'e').  Returns (out, arg): sum / mean in float64 (out is float64),
+    max / min exact with arg = the first element whose message equals the result (-1 for an empty row; arg
+    is None for sum / mean).  Rows without elements give 0.  Not in the reference."""
+    indptr = np.asarray(indptr, np.int64); indices = np.asarray(indices)
+    n = len(indptr) - 1
+    row = np.repeat(np.arange(n), np.diff(indptr))
+    m = _edge_messages(row, indices, op, lhs, rhs, lhs_target, rhs_target)
+    feat = m.shape[1:]
+    m2 = m.reshape(len(indices), -1)
+    if reduce in ("sum", "mean"):
+        out = np.zeros((n, m2.shape[1]), np.float64)
+        np.add.at(out, row, m2.astype(np.float64))
+        if reduce == "mean":
+            out /= np.maximum(np.diff(indptr), 1)[:, None]
+        return out.reshape((n,) + feat), None
+    out = np.zeros((n, m2.shape[1]), np.float32)
+    arg = np.full((n, m2.shape[1]), -1, np.int32)
+    for v in range(n):
+        a, b = indptr[v], indptr[v + 1]
+        if b > a:
+            seg = m2[a:b]
+            out[v] = seg.max(0) if reduce == "max" else seg.min(0)
+            arg[v] = a + (seg == out[v]).argmax(0)
+    return out.reshape((n,) + feat), arg.reshape((n,) + feat)
 
 
 def edge_softmax(indptr, x, nthreads=1):
