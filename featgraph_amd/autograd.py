@@ -13,8 +13,9 @@ import numpy as np
 import scipy.sparse
 import torch
 
-from .module import (EdgeSoftmaxhip, GraphAttentionhip, GSpMMhip, MultiHeadSDDMMhip, VanillaSDDMMhip,
+from .module import (EdgeSoftmaxhip, GraphAttentionhip, GSDDMMhip, GSpMMhip, MultiHeadSDDMMhip, VanillaSDDMMhip,
                      placeholder)
+from .module.general import parse_message
 
 
 class Graph(object):
@@ -154,6 +155,85 @@ class Graph(object):
             self._mods[key] = m
         return self._mods[key]
 
+    # ---- generalised operators with broadcasting -------------------------------------------------------
+
+    def gspmm(self, msg, lhs, rhs=None, reduce="sum"):
+        """out[v] = sum (or mean) over the edges e into v of the message msg = '<u|e>_<add|sub|mul>_<u|e>' or 'copy_e'
+        (DGL's names): operands on 'u' are (num_cols, ...), on 'e' (nnz, ...) in CSR edge order, and their feature
+        shapes broadcast the numpy way.  Differentiable in both operands.  ('u_mul_e' with one weight per edge or
+        per edge and head is spmm(); 'copy_u' is aggregate().)"""
+        op, lt, rt = parse_message(msg)
+        if reduce not in ("sum", "mean") or op not in ("add", "sub", "mul", "copy_lhs") or "v" in (lt, rt) or lt == rt:
+            raise ValueError("differentiable here: sum / mean of add, sub, mul between an operand on 'u' and one on 'e', or copy_e")
+        if rt is None:
+            return _GSpMM.apply(self, msg, reduce, lhs)
+        return _GSpMM.apply(self, msg, reduce, lhs, rhs)
+
+    def gsddmm(self, op, lhs, rhs, lhs_target="u", rhs_target="v"):
+        """out[e] = lhs[..] op rhs[..] per edge, op in {'add', 'sub', 'mul'}, operands on 'u' (num_cols, ...), 'v'
+        (num_rows, ...) or 'e' (nnz, ...), feature shapes broadcasting the numpy way; out is (nnz, ...) in CSR edge
+        order.  Differentiable in both operands.  (The dot product is sddmm().)"""
+        if op not in ("add", "sub", "mul") or lhs_target == rhs_target or not {lhs_target, rhs_target} <= {"u", "v", "e"}:
+            raise ValueError("differentiable here: add, sub, mul between operands on two different targets of u / v / e")
+        return _GSDDMM.apply(self, op, lhs_target, rhs_target, lhs, rhs)
+
+    def _tr_pos(self, device):
+        if getattr(self, "_tr_pos_dev", None) is None or self._tr_pos_dev.device != device:
+            self._tr_pos_dev = torch.from_numpy(self._tr_pos_host).to(device)
+        return self._tr_pos_dev
+
+    def _bcast_spmm_raw(self, msg, arrays, reduce="sum", transposed=False):
+        """Generalised SpMM over the adjacency or its transpose (edge operands then in the transpose's edge order)."""
+        arrays = [a.contiguous() for a in arrays]
+        key = ('gspmm', msg, reduce, transposed) + tuple(tuple(a.shape) for a in arrays)
+        if key not in self._mods:
+            m = GSpMMhip(self._tr if transposed else self._csr)
+            m.build([placeholder(tuple(a.shape)) for a in arrays], {'msg': msg, 'reduce': reduce}, {})
+            self._mods[key] = m
+        return _fresh_run(self._mods[key], arrays)
+
+    def _bcast_sddmm_raw(self, op, lt, rt, arrays):
+        arrays = [a.contiguous() for a in arrays]
+        key = ('gsddmm', op, lt, rt) + tuple(tuple(a.shape) for a in arrays)
+        if key not in self._mods:
+            m = GSDDMMhip(self._csr)
+            args = {'op': op}
+            if lt is not None:
+                args['lhs_target'] = lt
+            if rt is not None:
+                args['rhs_target'] = rt
+            m.build([placeholder(tuple(a.shape)) for a in arrays], args, {})
+            self._mods[key] = m
+        return _fresh_run(self._mods[key], arrays)
+
+    def _to_edges(self, x, target):
+        """x on 'v' or 'u' copied to the edges (CSR order); x on 'e' as it is."""
+        if target == "e":
+            return x
+        return self._bcast_sddmm_raw('copy_lhs', target, None, [x])
+
+    def _from_edges(self, m, target):
+        """Sum of the per-edge array m (CSR order) over the edges of each node of `target`; 'e': m itself."""
+        if target == "e":
+            return m
+        if target == "v":
+            return self._bcast_spmm_raw('copy_e', [m])
+        return self._bcast_spmm_raw('copy_e', [m.index_select(0, self._tr_pos(m.device))], transposed=True)
+
+    def _edge_product_sum(self, m, q, tq, target):
+        """For every node of `target` ('v' or 'u'): the sum over its edges of m[e] * q(e), m per edge (CSR order),
+        q on `tq`; the products are formed inside the aggregation, no per-edge array is written."""
+        if target == "v":               # rows of the adjacency: q on 'u' or 'e'
+            if tq == "v":
+                raise ValueError("both operands on the same target")
+            return self._bcast_spmm_raw('e_mul_' + tq, [m, q])
+        tp = self._tr_pos(m.device)     # rows of the transpose: its 'u' are this graph's 'v'
+        if tq == "u":
+            raise ValueError("both operands on the same target")
+        if tq == "v":
+            return self._bcast_spmm_raw('e_mul_u', [m.index_select(0, tp), q], transposed=True)
+        return self._bcast_spmm_raw('e_mul_e', [m.index_select(0, tp), q.index_select(0, tp)], transposed=True)
+
     def edge_softmax(self, scores):
         """Softmax of scores, (nnz,) or (nnz, H), over the edges of each destination row, per head."""
         return _EdgeSoftmax.apply(self, scores)
@@ -248,6 +328,91 @@ class _EdgeSoftmax(torch.autograd.Function):
         mod = ctx.g._softmax_mod(tuple(a.shape))
         mod.grad_tvm = torch.empty_like(a)          # handed to the caller; the module takes a new one next time
         return None, mod.backward(a, da.contiguous())
+
+
+def _reduce_to(full, shape):
+    """Sums `full` (rows, *broadcast feature shape) over the axes along which an operand of `shape` was broadcast."""
+    shape = tuple(shape)
+    lead = full.dim() - len(shape)
+    if lead > 0:
+        full = full.sum(dim=tuple(range(1, 1 + lead)))
+    return full.sum_to_size(shape) if tuple(full.shape) != shape else full
+
+
+class _GSpMM(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, g, msg, reduce, lhs, rhs=None):
+        ctx.g, ctx.msg, ctx.reduce = g, msg, reduce
+        arrays = [lhs] if rhs is None else [lhs, rhs]
+        ctx.save_for_backward(*arrays)
+        return g._bcast_spmm_raw(msg, arrays, reduce)
+
+    @staticmethod
+    def backward(ctx, dout):
+        g = ctx.g
+        op, lt, rt = parse_message(ctx.msg)
+        arrays = ctx.saved_tensors
+        dout = dout.contiguous()
+        if ctx.reduce == "mean":
+            deg = torch.from_numpy(np.maximum(np.diff(g._csr.indptr), 1).astype(np.float32)).to(dout.device)
+            dout = dout / deg.reshape((-1,) + (1,) * (dout.dim() - 1))
+        grads = []
+        targets = [lt] if rt is None else [lt, rt]
+        for i, (p, tp) in enumerate(zip(arrays, targets)):
+            if not ctx.needs_input_grad[3 + i]:
+                grads.append(None)
+                continue
+            if op in ("add", "sub", "copy_lhs"):
+                # the message is linear in p with coefficient +-1: reduce dout to p's feature shape first
+                d = _reduce_to(dout, (dout.shape[0],) + tuple(p.shape[1:]))
+                full = g._to_edges(d, "v") if tp == "e" else _sum_over_out_edges(g, d)
+                if op == "sub" and i == 1:
+                    full = -full
+                grads.append(full.reshape(p.shape))
+            else:   # mul: d message / d p = the other operand
+                q, tq = arrays[1 - i], targets[1 - i]
+                if tp == "u":       # sum over the edges that leave u of dout[row e] * q[e]
+                    full = g._bcast_spmm_raw('u_mul_e', [dout, q.index_select(0, g._tr_pos(q.device))], transposed=True)
+                else:               # per edge: dout[row e] * q[col e]
+                    full = g._bcast_sddmm_raw('mul', 'v', tq, [dout, q])
+                grads.append(_reduce_to(full, p.shape))
+        return (None, None, None) + tuple(grads)
+
+
+def _sum_over_out_edges(g, d):
+    """For every source node: the sum of d[row e] over the edges that leave it (d on the destination nodes)."""
+    return g._bcast_spmm_raw('copy_u', [d.reshape(d.shape[0], -1)], transposed=True).reshape((g.shape[1],) + tuple(d.shape[1:]))
+
+
+class _GSDDMM(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, g, op, lt, rt, lhs, rhs):
+        ctx.g, ctx.op, ctx.targets = g, op, (lt, rt)
+        ctx.save_for_backward(lhs, rhs)
+        return g._bcast_sddmm_raw(op, lt, rt, [lhs, rhs])
+
+    @staticmethod
+    def backward(ctx, dout):
+        g, op = ctx.g, ctx.op
+        arrays, targets = ctx.saved_tensors, ctx.targets
+        dout = dout.contiguous()
+        grads = []
+        for i, (p, tp) in enumerate(zip(arrays, targets)):
+            if not ctx.needs_input_grad[4 + i]:
+                grads.append(None)
+                continue
+            if op in ("add", "sub"):
+                d = _reduce_to(dout, (dout.shape[0],) + tuple(p.shape[1:]))
+                full = g._from_edges(d.reshape(d.shape[0], -1), tp).reshape(p.shape)
+                grads.append(-full if (op == "sub" and i == 1) else full)
+            else:
+                q, tq = arrays[1 - i], targets[1 - i]
+                if tp == "e":
+                    full = g._bcast_sddmm_raw('mul', 'e', tq, [dout, q])
+                else:
+                    full = g._edge_product_sum(dout, q, tq, tp)
+                grads.append(_reduce_to(full, p.shape))
+        return (None, None, None, None) + tuple(grads)
 
 
 class _Aggregate(torch.autograd.Function):

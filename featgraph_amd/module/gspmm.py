@@ -96,7 +96,9 @@ class GSpMMhip(VanillaSpMMhip):
     def _is_broadcast_message(self, msg, input_placeholders):
         if msg not in ('u_mul_e', 'copy_u'):
             return True
-        if msg == 'u_mul_e' and len(input_placeholders) == 2 and len(input_placeholders[0].shape) in (2, 3):
+        if len(input_placeholders) >= 1 and len(input_placeholders[0].shape) not in (2, 3):
+            return True                   # the weighted-sum kernels take (num_cols, F) or (num_cols, H, D)
+        if msg == 'u_mul_e' and len(input_placeholders) == 2:
             src_ph, e_ph = input_placeholders
             heads = src_ph.shape[1] if len(src_ph.shape) == 3 else 1
             nnz = self._adj_indices.shape[0]

@@ -138,3 +138,99 @@ def test_gat_attention_gradients():
     np.testing.assert_allclose(out.detach().cpu().numpy(), ref.detach().numpy(), rtol=1e-4, atol=2e-5)
     for got, want in ((er.grad, er64.grad), (el.grad, el64.grad), (v.grad, v64.grad)):
         np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=1e-3, atol=1e-4)
+
+
+def _dense_pick(t, target, rows, cols):
+    import torch
+    if target == 'u':
+        return t[cols]
+    if target == 'v':
+        return t[rows]
+    return t
+
+
+def _align(a, b):
+    nd = max(a.dim(), b.dim())
+    a = a.reshape((a.shape[0],) + (1,) * (nd - a.dim()) + tuple(a.shape[1:]))
+    b = b.reshape((b.shape[0],) + (1,) * (nd - b.dim()) + tuple(b.shape[1:]))
+    return a, b
+
+
+_TORCH_OP = {'add': lambda a, b: a + b, 'sub': lambda a, b: a - b, 'mul': lambda a, b: a * b}
+
+
+@pytest.mark.parametrize("msg,l_shape,r_shape", [
+    ("u_mul_e", (24,), (24,)), ("u_mul_e", (4, 8), (4, 1)), ("e_mul_u", (1,), (16,)), ("u_add_e", (8,), (8,)),
+    ("u_sub_e", (3, 1), (1, 5)), ("e_sub_u", (6,), (1,)), ("copy_e", (12,), None), ("u_add_e", (), (4,)),
+])
+@pytest.mark.parametrize("reduce", ["sum", "mean"])
+def test_generalised_spmm_gradients(msg, l_shape, r_shape, reduce):
+    """Graph.gspmm against torch autograd on the same formula in float64 (gather / index_add)."""
+    import torch
+    from featgraph_amd.autograd import Graph
+    from featgraph_amd.module.general import parse_message
+    rng = np.random.default_rng(len(msg) + len(l_shape))
+    adj = sp.random(90, 140, density=0.08, format="csr", random_state=rng).astype("float32")
+    adj.sort_indices()
+    g = Graph(adj)
+    coo = adj.tocoo()
+    rows = torch.from_numpy(coo.row.astype(np.int64)).cuda()
+    cols = torch.from_numpy(coo.col.astype(np.int64)).cuda()
+    op, lt, rt = parse_message(msg)
+    n_of = {'u': adj.shape[1], 'e': adj.nnz}
+    gen = torch.Generator(device="cuda"); gen.manual_seed(1)
+    lhs = torch.randn((n_of[lt],) + l_shape, generator=gen, device="cuda", requires_grad=True)
+    rhs = torch.randn((n_of[rt],) + r_shape, generator=gen, device="cuda", requires_grad=True) if rt else None
+    out = g.gspmm(msg, lhs, rhs, reduce) if rt else g.gspmm(msg, lhs, reduce=reduce)
+    up = torch.randn(out.shape, generator=gen, device="cuda")
+    (out * up).sum().backward()
+
+    l64 = lhs.detach().double().requires_grad_()
+    r64 = rhs.detach().double().requires_grad_() if rt else None
+    if rt:
+        a, b = _align(_dense_pick(l64, lt, rows, cols), _dense_pick(r64, rt, rows, cols))
+        m = _TORCH_OP[op](a, b)
+    else:
+        m = l64 if len(l_shape) else l64[:, None]
+    ref = torch.zeros((adj.shape[0],) + tuple(m.shape[1:]), dtype=torch.float64, device="cuda").index_add(0, rows, m)
+    if reduce == "mean":
+        deg = torch.from_numpy(np.maximum(np.diff(adj.indptr), 1)).cuda().double()
+        ref = ref / deg.reshape((-1,) + (1,) * (ref.dim() - 1))
+    assert out.shape == ref.shape
+    (ref * up.double()).sum().backward()
+    assert torch.allclose(out.double(), ref, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(lhs.grad.double(), l64.grad, rtol=1e-4, atol=1e-4)
+    if rt:
+        assert torch.allclose(rhs.grad.double(), r64.grad, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("op,lt,l_shape,rt,r_shape", [
+    ("add", 'u', (16,), 'v', (16,)), ("sub", 'u', (4, 1), 'v', (1, 6)), ("mul", 'u', (12,), 'v', (12,)),
+    ("mul", 'v', (4, 8), 'u', (4, 1)), ("mul", 'e', (8,), 'u', (8,)), ("mul", 'e', (1,), 'v', (20,)),
+    ("sub", 'e', (5,), 'v', (5,)), ("mul", 'u', (3,), 'e', (3,)), ("add", 'v', (2, 3), 'e', (3,)),
+])
+def test_generalised_sddmm_gradients(op, lt, l_shape, rt, r_shape):
+    import torch
+    from featgraph_amd.autograd import Graph
+    rng = np.random.default_rng(len(op) + sum(l_shape))
+    adj = sp.random(90, 140, density=0.08, format="csr", random_state=rng).astype("float32")
+    adj.sort_indices()
+    g = Graph(adj)
+    coo = adj.tocoo()
+    rows = torch.from_numpy(coo.row.astype(np.int64)).cuda()
+    cols = torch.from_numpy(coo.col.astype(np.int64)).cuda()
+    n_of = {'u': adj.shape[1], 'v': adj.shape[0], 'e': adj.nnz}
+    gen = torch.Generator(device="cuda"); gen.manual_seed(2)
+    lhs = torch.randn((n_of[lt],) + l_shape, generator=gen, device="cuda", requires_grad=True)
+    rhs = torch.randn((n_of[rt],) + r_shape, generator=gen, device="cuda", requires_grad=True)
+    out = g.gsddmm(op, lhs, rhs, lt, rt)
+    up = torch.randn(out.shape, generator=gen, device="cuda")
+    (out * up).sum().backward()
+    l64, r64 = lhs.detach().double().requires_grad_(), rhs.detach().double().requires_grad_()
+    a, b = _align(_dense_pick(l64, lt, rows, cols), _dense_pick(r64, rt, rows, cols))
+    ref = _TORCH_OP[op](a, b)
+    assert out.shape == ref.shape
+    (ref * up.double()).sum().backward()
+    assert torch.allclose(out.double(), ref, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(lhs.grad.double(), l64.grad, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(rhs.grad.double(), r64.grad, rtol=1e-4, atol=1e-4)
