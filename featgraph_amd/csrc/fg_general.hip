@@ -263,9 +263,10 @@ int lanes_for(int F) {
     return L;
 }
 
-int check_operand(const char *name, bool used, const float *p, int len, int target, bool allow_v) {
+// rows: how many rows the operand has in this call (an operand without rows may be a null pointer)
+int check_operand(const char *name, bool used, const float *p, int64_t rows, int len, int target, bool allow_v) {
     if (!used) return FG_OK;
-    if (!p) return fail(FG_ERR_ARG, "%s is null", name);
+    if (!p && rows > 0) return fail(FG_ERR_ARG, "%s is null", name);
     if (len < 1) return fail(FG_ERR_SHAPE, "%s feature length must be positive, got %d", name, len);
     if (!(target == FG_TARGET_U || target == FG_TARGET_E || (allow_v && target == FG_TARGET_V)))
         return fail(FG_ERR_ARG, "%s target %d is not valid here", name, target);
@@ -375,8 +376,8 @@ extern "C" int fg_gspmm_bcast_f32(fg_spmm_plan *pl, const int32_t *indptr_dev, c
     fg::ScratchNeed need;
     if (int rc = fg::gspmm_bcast_scratch_need(pl, out_len, arg_dev != nullptr, &need)) return rc;
     const bool uses_l = op != FG_BIN_COPY_RHS, uses_r = op != FG_BIN_COPY_LHS;
-    if (int rc = check_operand("lhs", uses_l, lhs_dev, lhs_len, lhs_target, false)) return rc;
-    if (int rc = check_operand("rhs", uses_r, rhs_dev, rhs_len, rhs_target, false)) return rc;
+    if (int rc = check_operand("lhs", uses_l, lhs_dev, lhs_target == FG_TARGET_E ? pl->nnz : pl->n_src, lhs_len, lhs_target, false)) return rc;
+    if (int rc = check_operand("rhs", uses_r, rhs_dev, rhs_target == FG_TARGET_E ? pl->nnz : pl->n_src, rhs_len, rhs_target, false)) return rc;
     if ((uses_l && !lhs_off_dev && lhs_len != out_len) || (uses_r && !rhs_off_dev && rhs_len != out_len))
         return fail(FG_ERR_SHAPE, "an operand without an offset array must have the output's feature length %d", out_len);
     if (pl->n_dst == 0) return FG_OK;
@@ -431,8 +432,9 @@ extern "C" int fg_gsddmm_bcast_f32(const int32_t *row_dev, const int32_t *col_de
     if (n_edges < 0) return fail(FG_ERR_ARG, "negative edge count");
     if (out_len < 1) return fail(FG_ERR_SHAPE, "feature length must be positive, got %d", out_len);
     const bool uses_l = op != FG_BIN_COPY_RHS, uses_r = op != FG_BIN_COPY_LHS;
-    if (int rc = check_operand("lhs", uses_l, lhs_dev, lhs_len, lhs_target, true)) return rc;
-    if (int rc = check_operand("rhs", uses_r, rhs_dev, rhs_len, rhs_target, true)) return rc;
+    // with edges every operand has rows to read; without, nothing is read
+    if (int rc = check_operand("lhs", uses_l, lhs_dev, n_edges, lhs_len, lhs_target, true)) return rc;
+    if (int rc = check_operand("rhs", uses_r, rhs_dev, n_edges, rhs_len, rhs_target, true)) return rc;
     const int R = op == FG_BIN_DOT ? reduce_len : 1;
     if (R < 1) return fail(FG_ERR_SHAPE, "the contracted length must be positive, got %d", reduce_len);
     if (op == FG_BIN_DOT && (lhs_len % R != 0 || rhs_len % R != 0))

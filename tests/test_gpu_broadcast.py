@@ -280,3 +280,29 @@ def test_gsddmm_broadcast_errors():
         m.build([placeholder((nc, 4)), placeholder((nr, 4))], {'op': 'pow'}, {})
     with pytest.raises(ValueError):
         m.build([placeholder((nc, 4)), placeholder((nr, 4))], {'op': 'copy_lhs'}, {})
+
+
+def test_graphs_without_edges_or_rows(oracle):
+    """No edges: every output row is 0 (also for max / min) and the per-edge result is empty."""
+    import torch
+    from featgraph_amd.module import GSpMMhip, GSDDMMhip, placeholder
+    adj = sp.csr_matrix((7, 9), dtype="float32")
+    x = np.ones((9, 5), "float32")
+    ef = np.zeros((0, 5), "float32")
+    for reduce in ("sum", "max", "mean"):
+        m = GSpMMhip(adj)
+        m.build([placeholder(x.shape), placeholder(ef.shape)], {'msg': 'u_add_e', 'reduce': reduce}, {})
+        m.out_tvm.fill_(float("nan"))
+        out = m.run([torch.from_numpy(x).cuda(), torch.from_numpy(ef).cuda()]).cpu().numpy()
+        assert out.shape == (7, 5) and (out == 0).all()
+    g = GSDDMMhip(adj.tocoo())
+    g.build([placeholder((9, 5)), placeholder((7, 1))], {'op': 'mul'}, {})
+    out = g.run([torch.from_numpy(x).cuda(), torch.ones((7, 1), device="cuda")])
+    assert tuple(out.shape) == (0, 5)
+    # one row, one element
+    one = sp.csr_matrix((np.ones(1, "float32"), np.array([3], np.int32), np.array([0, 1], np.int32)), shape=(1, 9))
+    m = GSpMMhip(one)
+    m.build([placeholder((9, 5)), placeholder((1, 5))], {'msg': 'u_sub_e', 'reduce': 'min', 'return_arg': True}, {})
+    xs = np.arange(45, dtype="float32").reshape(9, 5)
+    out = m.run([torch.from_numpy(xs).cuda(), torch.ones((1, 5), device="cuda")]).cpu().numpy()
+    assert np.array_equal(out, xs[3:4] - 1) and (m.arg_tvm.cpu().numpy() == 0).all()
