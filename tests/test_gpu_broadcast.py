@@ -306,3 +306,31 @@ def test_graphs_without_edges_or_rows(oracle):
     xs = np.arange(45, dtype="float32").reshape(9, 5)
     out = m.run([torch.from_numpy(xs).cuda(), torch.ones((1, 5), device="cuda")]).cpu().numpy()
     assert np.array_equal(out, xs[3:4] - 1) and (m.arg_tvm.cpu().numpy() == 0).all()
+
+
+def test_operands_that_are_not_16_byte_aligned(oracle):
+    """Contiguous views that start 4 bytes into an allocation: the 128-bit paths must not be taken for them."""
+    import torch
+    from featgraph_amd.module import GSpMMhip, GSDDMMhip, placeholder
+    rng = np.random.default_rng(21)
+    adj = _hub_graph(rng)
+    n, nnz, F = adj.shape[1], adj.nnz, 32
+    x = _operand(rng, n, (F,)); ef = _operand(rng, nnz, (F,)); y = _operand(rng, adj.shape[0], (F,))
+
+    def shifted(a):
+        flat = torch.empty(a.size + 1, dtype=torch.float32, device="cuda")
+        view = flat[1:].view(a.shape)
+        view.copy_(torch.from_numpy(a))
+        assert view.data_ptr() % 16 == 4 and view.is_contiguous()
+        return view
+
+    m = GSpMMhip(adj)
+    m.build([placeholder(x.shape), placeholder(ef.shape)], {'msg': 'u_mul_e', 'reduce': 'max'}, {})
+    ref, _ = oracle.gspmm_bcast(adj.indptr, adj.indices, 'mul', 'max', x, ef, 'u', 'e')
+    for xs, es in ((shifted(x), torch.from_numpy(ef).cuda()), (torch.from_numpy(x).cuda(), shifted(ef)), (shifted(x), shifted(ef))):
+        assert np.array_equal(m.run([xs, es]).cpu().numpy(), ref)
+    coo = adj.tocoo()
+    g = GSDDMMhip(coo)
+    g.build([placeholder(ef.shape), placeholder(y.shape)], {'op': 'sub', 'lhs_target': 'e'}, {})
+    ref = oracle.gsddmm_bcast(coo.row, coo.col, 'sub', ef, y, 'e', 'v')
+    assert np.array_equal(g.run([shifted(ef), shifted(y)]).cpu().numpy(), ref)
