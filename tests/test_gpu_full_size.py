@@ -106,3 +106,55 @@ def test_multihead_shapes(graph, H, D):
     head_sum = out.double().sum(1)
     assert ((head_sum - out_flat.double()).abs() <= ATOL + RTOL * out_flat.double().abs()
             + 2 * MASS_FACTOR * bound).all().item()
+
+
+def test_broadcasting_operators_at_full_size(graph):
+    """Closed forms that need no CPU pass over 114.8M edges: the sum of all-ones edge features is the row's degree;
+    edge features that repeat one weight per edge give the weighted SpMM; an all-ones edge operand leaves the
+    destination rows' features on the edges."""
+    import torch
+    from featgraph_amd.module import GSpMMhip, GSDDMMhip, VanillaSpMMhip, placeholder
+    adj, n, nnz = graph
+    F = 16
+    g = torch.Generator(device="cuda"); g.manual_seed(7)
+    deg = torch.from_numpy(np.diff(adj.indptr).astype(np.float32)).cuda()
+    ones = torch.ones((nnz, F), device="cuda")
+    m = GSpMMhip(adj)
+    m.build([placeholder((nnz, F))], {'msg': 'copy_e', 'reduce': 'sum'}, {})
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([ones])
+    assert torch.equal(out, deg[:, None].expand(n, F))               # integers below 2^24: exact in any order
+    m.build([placeholder((nnz, F))], {'msg': 'copy_e', 'reduce': 'max', 'return_arg': True}, {})
+    out = m.run([ones])
+    assert torch.equal(out, (deg > 0).float()[:, None].expand(n, F))
+    first = torch.from_numpy(adj.indptr[:-1].astype(np.int32)).cuda()
+    want_arg = torch.where(deg > 0, first, torch.full_like(first, -1))
+    assert torch.equal(m.arg_tvm, want_arg[:, None].expand(n, F))     # ties: the row's first edge
+    del ones
+
+    w = torch.rand(nnz, generator=g, device="cuda")
+    x = torch.randn((n, F), generator=g, device="cuda")
+    ef = w[:, None].expand(nnz, F).contiguous()
+    m.build([placeholder((n, F)), placeholder((nnz, F))], {'msg': 'u_mul_e', 'reduce': 'sum'}, {})
+    out = m.run([x, ef]).clone()
+    wadj = sp.csr_matrix((w.cpu().numpy(), adj.indices, adj.indptr), shape=adj.shape)
+    plain = VanillaSpMMhip(wadj)
+    plain.build([placeholder((n, F))], {}, {})
+    ref = plain.run([x])
+    mass = VanillaSpMMhip(wadj)
+    mass.build([placeholder((n, F))], {}, {})
+    row_mass = mass.run([x.abs()]).double()
+    assert ((out.double() - ref.double()).abs() <= ATOL + RTOL * ref.double().abs() + 2 * MASS_FACTOR * row_mass).all().item()
+    del ef
+
+    y = torch.randn((n, F), generator=g, device="cuda")
+    e1 = torch.ones((nnz, 1), device="cuda")
+    gs = GSDDMMhip(adj.tocoo())
+    gs.build([placeholder((nnz, 1)), placeholder((n, F))], {'op': 'mul', 'lhs_target': 'e', 'rhs_target': 'v'}, {})
+    gs.out_tvm.fill_(float("nan"))
+    out = gs.run([e1, y])
+    rows = gs._adj_row_indices_dev.long()
+    pick = torch.randint(0, nnz, (500000,), generator=g, device="cuda")
+    pick[0], pick[1] = 0, nnz - 1
+    assert torch.equal(out[pick], y[rows[pick]])
+    assert torch.isfinite(out).all().item()
