@@ -213,7 +213,7 @@ def gspmm_bcast(indptr, indices, op, reduce, lhs, rhs, lhs_target="u", rhs_targe
     row = np.repeat(np.arange(n), np.diff(indptr))
     m = _edge_messages(row, indices, op, lhs, rhs, lhs_target, rhs_target)
     feat = m.shape[1:]
-    m2 = m.reshape(len(indices), -1)
+    m2 = m.reshape(len(indices), int(np.prod(feat)))
     if reduce in ("sum", "mean"):
         out = np.zeros((n, m2.shape[1]), np.float64)
         np.add.at(out, row, m2.astype(np.float64))

@@ -151,6 +151,81 @@ def test_random_attention(oracle, monkeypatch, seed):
         np.testing.assert_allclose(out, ref, rtol=1e-4, atol=2e-5, err_msg=what)
 
 
+def _random_feature_shapes(rng):
+    """Two feature shapes that broadcast against each other (possibly of different rank)."""
+    nd = int(rng.integers(1, 4))
+    dims = [int(rng.choice([1, 2, 3, 4, 5, 8, 16, 33])) for _ in range(nd)]
+    l, r = [], []
+    for d in dims:
+        which = rng.integers(0, 4)
+        l.append(1 if which == 1 else d)
+        r.append(1 if which == 2 else d)
+    cut = int(rng.integers(0, nd))          # drop leading axes of one operand
+    if rng.random() < 0.5:
+        l = l[cut:]
+    else:
+        r = r[cut:]
+    return tuple(l), tuple(r)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_broadcast_operators(oracle, monkeypatch, seed):
+    """Generalised SpMM / SDDMM with broadcasting: random graphs, operators, targets and feature shapes (odd
+    seeds: rows split into pieces of 64 elements, so that split rows occur on these small graphs)."""
+    import torch
+    from featgraph_amd import _lib
+    from featgraph_amd.module import GSpMMhip, GSDDMMhip, placeholder
+    if seed % 2:
+        monkeypatch.setattr(_lib, "plan_opts", _lib.FgPlanOpts(split_threshold=64))
+    rng = np.random.default_rng(SEED_BASE + 5000 + seed)
+    for case in range(16):
+        adj = _random_graph(rng)
+        nnz = adj.nnz
+        l_shape, r_shape = _random_feature_shapes(rng)
+        op = str(rng.choice(["add", "sub", "mul", "div"]))
+        what = "seed %d case %d: %s nnz %d %s %s %s" % (seed, case, adj.shape, nnz, op, l_shape, r_shape)
+
+        def operand(rows, shape):
+            x = rng.standard_normal((rows,) + shape).astype("float32")
+            return (np.abs(x) + 0.5).astype("float32") if op == "div" else x
+
+        # SpMM: operands on (u, e) or (e, u)
+        lt, rt = ("u", "e") if rng.random() < 0.5 else ("e", "u")
+        rows = {"u": adj.shape[1], "e": nnz}
+        lhs, rhs = operand(rows[lt], l_shape), operand(rows[rt], r_shape)
+        reduce = str(rng.choice(["sum", "mean", "max", "min"]))
+        m = GSpMMhip(adj)
+        args = {'msg': "%s_%s_%s" % (lt, op, rt), 'reduce': reduce}
+        if reduce in ("max", "min"):
+            args['return_arg'] = True
+        m.build([placeholder(lhs.shape), placeholder(rhs.shape)], args, {})
+        m.out_tvm.fill_(float("nan"))
+        out = m.run([torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda()]).cpu().numpy()
+        ref, ref_arg = oracle.gspmm_bcast(adj.indptr, adj.indices, op, reduce, lhs, rhs, lt, rt)
+        assert out.shape == ref.shape, what
+        if reduce in ("max", "min"):
+            assert np.array_equal(out, ref), what + " " + reduce
+            assert np.array_equal(m.arg_tvm.cpu().numpy(), ref_arg), what + " arg " + reduce
+        else:
+            mass_op = "add" if op == "sub" else op
+            mass, _ = oracle.gspmm_bcast(adj.indptr, adj.indices, mass_op, reduce, np.abs(lhs), np.abs(rhs), lt, rt)
+            assert_sum_close(out, ref, mass, what + " " + reduce)
+
+        # SDDMM: any two different targets
+        targets = ["u", "v", "e"]
+        lt = str(rng.choice(targets))
+        rt = str(rng.choice([t for t in targets if t != lt]))
+        coo = adj.tocoo()
+        rows = {"u": adj.shape[1], "v": adj.shape[0], "e": nnz}
+        lhs, rhs = operand(rows[lt], l_shape), operand(rows[rt], r_shape)
+        g = GSDDMMhip(coo)
+        g.build([placeholder(lhs.shape), placeholder(rhs.shape)], {'op': op, 'lhs_target': lt, 'rhs_target': rt}, {})
+        g.out_tvm.fill_(float("nan"))
+        out = g.run([torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda()]).cpu().numpy()
+        ref = oracle.gsddmm_bcast(coo.row, coo.col, op, lhs, rhs, lt, rt)
+        assert out.shape == ref.shape and np.array_equal(out, ref), what + " sddmm %s %s" % (lt, rt)
+
+
 def test_tuned_choice_is_one_of_the_candidates_and_right():
     """schedule_args {'tune': k}: the module times the cost model's candidates on its own graph, keeps the
     fastest, and the result is the same product."""
