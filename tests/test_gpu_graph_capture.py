@@ -169,3 +169,44 @@ def test_scratch_is_reserved_at_build_and_never_grown_under_capture():
         assert L.fg_spmm_plan_reserve(plan, 2, 1, 24, 1) == -2          # a tile the tiled SDDMM does not take
     finally:
         L.fg_spmm_plan_destroy(plan)
+
+
+def test_broadcasting_operators_replay_without_a_warm_up_call():
+    """build() reserves the split rows' scratch, so the first run() may already be the recorded one."""
+    import torch
+    from featgraph_amd.module import GSpMMhip, GSDDMMhip, placeholder
+    rng = np.random.default_rng(8)
+    n_dst, n_src, F = 300, 2500, 24
+    adj = sp.random(n_dst, n_src, density=0.02, format="csr", random_state=rng).astype("float32").tolil()
+    adj[7, rng.choice(n_src, size=2200, replace=False)] = 1.0       # a row that is split into pieces
+    adj = adj.tocsr().astype("float32"); adj.sort_indices()
+    nnz = adj.nnz
+    agg = GSpMMhip(adj)
+    agg.build([placeholder((n_src, F)), placeholder((nnz, F))], {'msg': 'u_mul_e', 'reduce': 'max', 'return_arg': True}, {})
+    edge = GSDDMMhip(adj.tocoo())
+    edge.build([placeholder((nnz, F)), placeholder((n_dst, 1))], {'op': 'add', 'lhs_target': 'e', 'rhs_target': 'v'}, {})
+    x = torch.zeros((n_src, F), device="cuda")
+    ef = torch.zeros((nnz, F), device="cuda")
+    b = torch.zeros((n_dst, 1), device="cuda")
+
+    def chain():
+        return agg.run([x, ef]), edge.run([ef, b])
+
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_out, g_edge = chain()
+    gen = torch.Generator(device="cuda")
+    for k in range(3):
+        gen.manual_seed(20 + k)
+        x.copy_(torch.randn((n_src, F), generator=gen, device="cuda"))
+        ef.copy_(torch.randn((nnz, F), generator=gen, device="cuda"))
+        b.copy_(torch.randn((n_dst, 1), generator=gen, device="cuda"))
+        e_out, e_edge = (t.clone() for t in chain())
+        e_arg = agg.arg_tvm.clone()
+        torch.cuda.synchronize()
+        agg.out_tvm.fill_(float("nan")); agg.arg_tvm.fill_(-7); edge.out_tvm.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_out, e_out) and torch.equal(agg.arg_tvm, e_arg), "aggregation replay %d" % k
+        assert torch.equal(g_edge, e_edge), "edge operator replay %d" % k
