@@ -256,6 +256,7 @@ struct SddmmTiledArgs {
     uint32_t src_row_bytes;
     uint32_t src_tile_bytes;
     int first_part, conc, n_parts;   // this launch works on partitions [first_part, first_part + conc)
+    int all_parts;                   // 1: the launch walks the items of all partitions, partition by partition (conc == 1)
     int tile_base;                   // ... and on tiles [tile_base, tile_base + n_tiles)
     const float *dst;
     float *out;               // out (direct mode) or partial (tile-sum mode)
@@ -376,11 +377,21 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     const unsigned per = (unsigned)(a.n_tiles * a.conc);
     const int slot = (int)(blockIdx.x % per);
     const int tile = a.tile_base + slot % a.n_tiles;
-    const int part = a.first_part + slot / a.n_tiles;
-    if (part >= a.n_parts) return;
-    const int64_t i0 = a.item_off[part];
-    const int64_t item_id = (int64_t)(blockIdx.x / per) * kWavesPerBlock + wave;
-    if (item_id >= a.item_off[part + 1] - i0) return;
+    int part = a.first_part + slot / a.n_tiles;
+    int64_t item_id = (int64_t)(blockIdx.x / per) * kWavesPerBlock + wave;
+    int64_t i0 = 0;
+    if (a.all_parts) {
+        // item_id counts through all partitions' items; its partition is uniform over the wavefront
+        const int64_t id = ((int64_t)__builtin_amdgcn_readfirstlane((int)(item_id >> 32)) << 32) |
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)item_id);
+        if (id >= a.item_off[a.n_parts]) return;
+        part = 0;
+        while (part + 1 < a.n_parts && id >= a.item_off[part + 1]) ++part;
+    } else {
+        if (part >= a.n_parts) return;
+        i0 = a.item_off[part];
+        if (item_id >= a.item_off[part + 1] - i0) return;
+    }
     const Item it = a.items[i0 + item_id];
     const int32_t *pos = a.pos + part * a.pos_stride;
     const float *src = a.src + part * a.src_stride;
@@ -879,7 +890,22 @@ extern "C" int fg_sddmm_dds_f32(fg_spmm_plan *pl, const int32_t *s1_pos_dev, con
     // More than 8 tiles: 8 per launch (one per XCD), as for SpMM.
     const int per_launch = (T > 8 && T % 8 == 0) ? 8 : T;
     a.n_tiles = per_launch;
-    for (int p0 = 0; p0 < P; p0 += conc) {
+    a.all_parts = 0;
+    // One partition at a time and several of them: a single launch walks all partitions' items in partition order
+    // (edges of different partitions write different results, so nothing orders the passes); the next partition's
+    // first workgroups fill the compute units that the previous one's last workgroups leave idle.
+    if (conc == 1 && P > 1) {
+        a.all_parts = 1; a.first_part = 0;
+        const int64_t blocks = ((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
+        if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
+        for (int tb = 0; tb < T && blocks > 0; tb += per_launch) {
+            a.tile_base = tb;
+            const bool ok = (tile_sum || staged) ? launch_tiled_l<false>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a)
+                                                 : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
+            if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);
+        }
+    }
+    for (int p0 = 0; p0 < P && !a.all_parts; p0 += conc) {
         int64_t most = 0;
         for (int p = p0; p < std::min(P, p0 + conc); ++p) most = std::max(most, pl->item_off[p + 1] - pl->item_off[p]);
         if (most == 0) continue;

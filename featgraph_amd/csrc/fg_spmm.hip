@@ -76,6 +76,12 @@ struct SpmmArgs {
     int32_t *arg;          // arg kernel: stored position of the element that gave out[v, f]
     int vstride;           // weight of element t, head h: vals[t * vstride + h * head_stride]
     int64_t head_stride;
+    // One launch over the items of all source partitions (sum kernel, every pass into a buffer of its own): the
+    // plan's item_off on the device (n_parts + 1 entries; null: the launch holds one partition's items and the
+    // strides are unused) and the distance from one partition's pos / x / out / partial to the next, in elements.
+    const int64_t *item_off = nullptr;
+    int n_parts = 1;
+    int64_t pos_stride = 0, x_stride = 0, out_stride = 0, partial_stride = 0;
 };
 
 
@@ -258,6 +264,18 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
     const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_ftiles) * kWavesPerBlock + wave;
     if (item_id >= a.n_items) return;      // uniform per wavefront; no workgroup barriers below
     const Item it = a.items[item_id];
+    // the partition this item belongs to (uniform per wavefront): selects its position array, its slice of x,
+    // its output buffer and its share of the split rows' scratch
+    int part = 0;
+    if (a.item_off) {
+        const int64_t id = ((int64_t)__builtin_amdgcn_readfirstlane((int)(item_id >> 32)) << 32) |
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)item_id);
+        while (part + 1 < a.n_parts && id >= a.item_off[part + 1]) ++part;
+    }
+    const int32_t *const pos_p = a.pos + part * a.pos_stride;
+    const float *const x_p = a.x + part * a.x_stride;
+    float *const out_p = a.out + part * a.out_stride;
+    float *const partial_p = a.partial + part * a.partial_stride;
     const int g = lane / L, li = lane % L;
 
     const int rt = tile / a.sub_per_tile, st = tile % a.sub_per_tile;
@@ -296,7 +314,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
                 const int t = lane + 64 * i;
                 const int r = min(t / kLines, nrows - 1);
                 const int f = min(f_tile + (t % kLines) * 32, f_last);
-                touched[i] = a.out[(int64_t)(it.row + r) * F + f];
+                touched[i] = out_p[(int64_t)(it.row + r) * F + f];
             }
         }
         if (it.len > 0) {
@@ -305,7 +323,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
             stage_store(edge, lane, regs);
             if (HPT > 1) stage_store_w<HPT>(s_w[wave], lane, wregs);
         }
-        s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        s_end[wave][lane] = pos_p[it.row + min(lane, nrows - 1) + 1] - it.start;
         if (lane == 0) s_next[wave] = 0;
         wave_lds_sync();
         if (ACC) {
@@ -318,7 +336,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
             for (int q = 0; q < nrows; ++q) {
                 const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
                 if (e > b || !ACC) {
-                    float *dst = a.out + (int64_t)(it.row + q) * F + f_lo;
+                    float *dst = out_p + (int64_t)(it.row + q) * F + f_lo;
                     if (ACC) {
 #pragma unroll
                         for (int k = 0; k < K; ++k)
@@ -326,7 +344,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
                     }
 #pragma unroll
                     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
-                    gather_rows<V, L, K, FULL, U, OFF32, HPT>(edge, wrow, b, e, g, a.x, lane_bytes, F, on, acc);
+                    gather_rows<V, L, K, FULL, U, OFF32, HPT>(edge, wrow, b, e, g, x_p, lane_bytes, F, on, acc);
                     finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
                 }
                 b = e;
@@ -341,7 +359,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
         for (;;) {
             if (!done && j >= e) {
                 if (q >= 0 && (!ACC || nonempty)) {       // the row this group just finished
-                    float *dst = a.out + (int64_t)(it.row + q) * F + f_lo;
+                    float *dst = out_p + (int64_t)(it.row + q) * F + f_lo;
 #pragma unroll
                     for (int k = 0; k < K; ++k)
                         if (FULL || on[k]) {
@@ -362,7 +380,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
 #pragma unroll
                     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
                     if (ACC && nonempty) {
-                        const float *src = a.out + (int64_t)(it.row + q) * F + f_lo;
+                        const float *src = out_p + (int64_t)(it.row + q) * F + f_lo;
 #pragma unroll
                         for (int k = 0; k < K; ++k)
                             if (FULL || on[k]) old[k] = *reinterpret_cast<const vec *>(src + k * L * V);
@@ -386,7 +404,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
 #pragma unroll
                     for (int k = 0; k < K; ++k)
                         if (FULL || on[k])
-                            xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<OFF32>(a.x, lane_bytes, F, cw[u].x) + k * L * V);
+                            xv[u][k] = *reinterpret_cast<const vec *>(row_ptr<OFF32>(x_p, lane_bytes, F, cw[u].x) + k * L * V);
 #pragma unroll
                 for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -404,7 +422,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
 
     // one row, or one piece of a long row: 256 elements at a time, the next 256 on their way
     // while the current ones are used
-    float *dst = (it.info < 0 ? a.out + (int64_t)it.row * F : a.partial + (int64_t)it.info * F) + f_lo;
+    float *dst = (it.info < 0 ? out_p + (int64_t)it.row * F : partial_p + (int64_t)it.info * F) + f_lo;
     const bool add = ACC && it.info < 0;
 #pragma unroll
     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
@@ -430,7 +448,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
                 stage_load_w<HPT>(a.vals, (int64_t)it.start + base + fg::kItemEdges, it.len - base - fg::kItemEdges,
                                   lane, a.vstride, voff, a.head_stride, wregs);
         }
-        gather_rows<V, L, K, FULL, U, OFF32, HPT>(edge, wrow, 0, n, g, a.x, lane_bytes, F, on, acc);
+        gather_rows<V, L, K, FULL, U, OFF32, HPT>(edge, wrow, 0, n, g, x_p, lane_bytes, F, on, acc);
     }
     finish_row<V, L, K, FULL, ACC>(acc, old, g, on, dst);
 }
@@ -974,21 +992,24 @@ size_t piece_floats(const fg_spmm_plan *pl, int F) {
 // Whether the passes over the source partitions write buffers of their own that one last kernel adds up,
 // instead of every later pass reading and rewriting `out`.  A wavefront's loads return in order, so a row of
 // `out` that has to come from memory holds up the gathers issued behind it; without those reads a pass over
-// the 232,965-node graph takes 1.37 instead of 1.52 ms at F = 512 and the sum of the 8 buffers 0.85 ms:
-// 12.11 -> 11.68 ms (F = 256, 238 MB of output: 6.30 -> 6.16 ms; F = 128, 119 MB: 3.27 -> 3.29 ms, hence the size
-// rule below).  Same sums in the same order: bit-identical results.
+// the 232,965-node graph takes 1.37 instead of 1.52 ms at F = 512 and the sum of the 8 buffers 0.77 ms.  Passes
+// that do not read each other's results need no ordering either, so one launch walks all partitions' items.
+// Together (232,965-node graph): 12.11 -> 11.53 ms at F = 512, 6.19 -> 5.90 ms at F = 256, 3.13 -> 3.03 ms at F = 128,
+// 1.76 -> 1.66 ms at F = 64, 0.93 -> 0.90 ms at F = 32.  Same sums in the same order: bit-identical results.
+// The buffers take P times the output's size; beyond 8 GiB the passes add to `out` in place.
 bool uses_pass_buffers(const fg_spmm_plan *pl, const SpmmConfig &c, int F, int reduce) {
     const int P = pl->num_col_partitions;
     if (P < 2 || reduce != FG_REDUCE_SUM || c.V != 4 || pl->pass_buffers == 2) return false;
     if (pl->pass_buffers == 1) return true;
     const uint64_t out_bytes = (uint64_t)pl->n_dst * (uint64_t)F * 4u;
-    return P >= 4 && out_bytes >= (192ull << 20) && out_bytes * (uint64_t)P <= (8ull << 30);
+    return out_bytes * (uint64_t)P <= (8ull << 30);
 }
 
 fg::ScratchNeed scratch_need(const fg_spmm_plan *pl, const SpmmConfig &c, int F, int reduce) {
     fg::ScratchNeed need;
     need.partial = piece_floats(pl, F);                                  // one row of F floats per piece of a split row
-    if (uses_pass_buffers(pl, c, F, reduce)) need.partial += (size_t)pl->num_col_partitions * (size_t)pl->n_dst * (size_t)F;
+    if (uses_pass_buffers(pl, c, F, reduce))                             // every pass: pieces and a buffer of its own
+        need.partial = (size_t)pl->num_col_partitions * (need.partial + (size_t)pl->n_dst * (size_t)F);
     if (gathers_tile_major(pl, c, F)) need.tiled = (size_t)pl->n_src * (size_t)F;
     return need;
 }
@@ -1024,10 +1045,11 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
     float *const partial = fixed_partial ? fixed_partial : pl->partial_dev;
     // per-pass buffers [P][n_dst][F] behind the pieces (every row of every buffer is written by its pass:
     // the plan holds an item or a fix-up for every row of every partition)
-    float *const pass_buf = (!fixed_partial && uses_pass_buffers(pl, c, F, reduce)) ? pl->partial_dev + piece_floats(pl, F) : nullptr;
+    const int P = pl->num_col_partitions;
+    const size_t piece = piece_floats(pl, F);
+    float *const pass_buf = (!fixed_partial && uses_pass_buffers(pl, c, F, reduce)) ? pl->partial_dev + (size_t)P * piece : nullptr;
     const size_t pass_stride = (size_t)pl->n_dst * (size_t)F;
     hipStream_t st = (hipStream_t)stream;
-    const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
     // With several feature tiles an XCD gathers one tile's 256 bytes (or less) out of every source
     // row, F * 4 bytes apart.  Gathered from a copy that stores each tile's slices back to back, the
@@ -1037,9 +1059,36 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
     const int ft = c.V * c.L * c.K;
     const bool tiled = need.tiled > 0;
     if (tiled && (rc = fg::make_tile_major(pl, x, pl->n_src, F, ft, stream)) != FG_OK) return rc;
+    if (pass_buf && pl->n_items > 0) {
+        // The passes are independent (each writes a buffer and pieces of its own), so one launch walks the items of all
+        // partitions, partition by partition in workgroup order: the next partition's first workgroups fill the
+        // compute units that the previous one's last workgroups leave idle, and seven launch gaps go away.
+        SpmmArgs a;
+        a.items = pl->items_dev; a.n_items = pl->n_items;
+        a.item_off = pl->item_off_dev; a.n_parts = P;
+        a.pos = pos; a.pos_stride = pl->n_dst + 1;
+        a.indices = idx; a.vals = vals;
+        a.x = tiled ? pl->tiled_dev : x; a.x_stride = width * (tiled ? ft : F);
+        a.x_row_bytes = (uint32_t)(tiled ? ft : F) * 4u;
+        a.x_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * ft * 4u) : 0u;
+        a.out = pass_buf; a.out_stride = (int64_t)pass_stride;
+        a.partial = partial; a.partial_stride = (int64_t)piece;
+        a.F = F; a.tile_w = c.tile_w; a.sub_per_tile = c.sub_per_tile;
+        a.heads = heads; a.head_len = F / heads;
+        a.vstride = head_major ? 1 : heads; a.head_stride = head_major ? pl->nnz : 1;
+        a.accumulate = 0;
+        const int per_launch = (c.n_ftiles > 8 && c.n_ftiles % 8 == 0) ? 8 : c.n_ftiles;
+        for (int tb = 0; tb < c.n_ftiles; tb += per_launch) {
+            a.n_ftiles = per_launch; a.tile_base = tb;
+            const int64_t blocks = ((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
+            if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
+            rc = (c.V == 4) ? launch_v<4>(c, dim3((unsigned)blocks), st, a) : launch_v<1>(c, dim3((unsigned)blocks), st, a);
+            if (rc != FG_OK) return rc;
+        }
+    }
     for (int p = 0; p < P; ++p) {
         const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
-        if (i1 > i0) {
+        if (i1 > i0 && !pass_buf) {
             SpmmArgs a;
             a.items = pl->items_dev + i0; a.n_items = i1 - i0;
             a.pos = pos + (int64_t)p * (pl->n_dst + 1);
@@ -1052,7 +1101,6 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
             a.heads = heads; a.head_len = F / heads;
             a.vstride = head_major ? 1 : heads; a.head_stride = head_major ? pl->nnz : 1;
             a.accumulate = p > 0;
-            if (pass_buf) { a.out = pass_buf + (size_t)p * pass_stride; a.accumulate = 0; }
             // More than 8 tiles: 8 at a time (one per XCD), so that an XCD's L2 serves one tile's
             // slice of this partition per launch; the partition's index arrays stay in the
             // memory-side cache between the launches.
@@ -1076,9 +1124,10 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
             const Fixup *fx = pl->fixups_dev + x0;
             if (reduce == FG_REDUCE_SUM) {
                 float *dst = pass_buf ? pass_buf + (size_t)p * pass_stride : out;
+                const float *pieces = pass_buf ? partial + (size_t)p * piece : partial;
                 const int add = (p > 0 && !pass_buf) ? 1 : 0;
-                if (fv == 4) hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, dst, F, add);
-                else hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, dst, F, add);
+                if (fv == 4) hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pieces, dst, F, add);
+                else hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pieces, dst, F, add);
             } else if (reduce == FG_REDUCE_MAX) {
                 if (fv == 4) hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<4, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F);
                 else hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<1, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F);

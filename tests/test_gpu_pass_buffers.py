@@ -1,5 +1,6 @@
 """SpMM over several source partitions: every pass either adds to `out` in place or writes a buffer of its
-own that a last kernel adds up (plan option `pass_buffers`: 1 = always, 2 = never; default: by size).  The
+own that a last kernel adds up, all passes in one launch (plan option `pass_buffers`: 1 = always, 2 = never;
+default: buffers unless they would take more than 8 GiB).  The
 sums and their order are the same, so the two must agree bit for bit -- on graphs with empty rows, rows
 whose elements all lie in one partition, partitions without any element, and rows split over wavefronts."""
 import numpy as np
