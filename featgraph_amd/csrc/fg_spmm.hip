@@ -1195,7 +1195,7 @@ std::string spmm_launch_text(const fg_spmm_plan *pl, int F, int T) {
     text += gathers_tile_major(pl, c, F) ? "  source features  : gathered from a tile-by-tile copy made at the start of every call\n"
                                          : "  source features  : gathered from the caller's row-major matrix\n";
     if (pl->num_col_partitions > 1)
-        text += uses_pass_buffers(pl, c, F, FG_REDUCE_SUM) ? "  passes           : each writes a buffer of its own; one last kernel adds the buffers into out\n"
+        text += uses_pass_buffers(pl, c, F, FG_REDUCE_SUM) ? "  passes           : one launch walks all partitions, each into a buffer of its own; one last kernel adds the buffers into out\n"
                                                            : "  passes           : later passes add to out in place\n";
     return text;
 }
