@@ -10,12 +10,13 @@ python/featgraph/module/spmm.py:179-186).  Prints ONE JSON line; `value` is
 2 * (2 * nnz * F) flops per step over the measured step time.
 
 `roofline` prices the slower of the two operators against the 8 TB/s HBM peak with the
-compulsory-traffic byte model (an operator is one C-ABI call; on this graph it is several
-launches of one kernel, one per source-column partition, plus a short closing kernel -- the
-fix-ups of split rows for SpMM, the sum over feature tiles for SDDMM -- so `achieved` = the
+compulsory-traffic byte model (an operator is one C-ABI call; on this graph it is one launch of
+the gather kernel that walks all source-column partitions, preceded by the tile-by-tile copy of the
+gathered operand and followed by short closing kernels -- the fix-ups of split rows and the sum of
+the passes' buffers for SpMM, the sum over feature tiles for SDDMM -- so `achieved` = the
 operator's algorithmic bytes / the HIP-event time of all its launches; `kernels` lists them and
 `avg_launch_ms` is that time divided by the number of launches of the gather kernel, i.e. it
-carries the closing kernel's share as well):
+carries the other kernels' share as well):
     SpMM  : 4(N+1) + 8 nnz + 4 N F (X once) + 4 N F (out once)
     SDDMM : 4(N+1) + 4 nnz (CSR order; 8 nnz in COO order) + 8 N F + 4 nnz H
 `cpu_baseline` times the CPU oracle (a C restatement of the reference's x86 schedules: SpMM
@@ -39,11 +40,11 @@ HBM_PEAK_GBS = 8000.0
 _PROFILES = "profiles/bench_%s_rocprofv3.txt"
 MEASURED_TRAFFIC = {
     # (operator, workload, F, partitions, tiles): (bytes, summary); tiles 0 = the kernel's own single tile
-    ("spmm", "powerlaw-233k", 512, 8, 8): (63.2e9, _PROFILES % "powerlaw233k_f512"),     # 8 x spmm_items_kernel (copy: +0.95e9, sum of the passes: +4.3e9)
-    ("sddmm", "powerlaw-233k", 512, 8, 8): (70.9e9, _PROFILES % "powerlaw233k_f512"),    # 8 x sddmm_tiled_kernel (copy: +0.95e9, tile sum: +4.7e9)
-    ("spmm", "powerlaw-233k", 64, 8, 0): (9.05e9, _PROFILES % "powerlaw233k_f64"),
+    ("spmm", "powerlaw-233k", 512, 8, 8): (63.7e9, _PROFILES % "powerlaw233k_f512"),     # spmm_items_kernel (copy: +0.95e9, sum of the passes: +4.3e9)
+    ("sddmm", "powerlaw-233k", 512, 8, 8): (71.2e9, _PROFILES % "powerlaw233k_f512"),    # sddmm_tiled_kernel (copy: +0.95e9, tile sum: +4.7e9)
+    ("spmm", "powerlaw-233k", 64, 8, 0): (8.50e9, _PROFILES % "powerlaw233k_f64"),
     ("sddmm", "powerlaw-233k", 64, 8, 1): (9.71e9, _PROFILES % "powerlaw233k_f64"),
-    ("spmm", "powerlaw-233k", 32, 4, 0): (4.80e9, _PROFILES % "powerlaw233k_f32"),
+    ("spmm", "powerlaw-233k", 32, 4, 0): (4.72e9, _PROFILES % "powerlaw233k_f32"),
     ("sddmm", "powerlaw-233k", 32, 4, 1): (5.56e9, _PROFILES % "powerlaw233k_f32"),
     ("spmm", "powerlaw-2.45M", 128, 1, 1): (33.15e9, _PROFILES % "powerlaw2450k_f128"),
     ("sddmm", "powerlaw-2.45M", 128, 1, 1): (32.86e9, _PROFILES % "powerlaw2450k_f128"),
@@ -283,13 +284,19 @@ def main():
     t_spmm = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps      # ms, HIP events on the launch stream
     t_sddmm = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
 
+    def tile_groups(n_tiles):
+        """More than 8 feature tiles are launched 8 at a time (one per XCD)."""
+        return n_tiles // 8 if (n_tiles > 8 and n_tiles % 8 == 0) else 1
+
     def sddmm_launches():
-        """Launches of the tiled kernel: with T < 8 tiles, 8 / T partitions share a launch."""
+        """Launches of the tiled kernel: one launch walks all partitions (8 / T of them at a time when there are
+        fewer than 8 tiles); only beyond 32 such groups does every group get a launch of its own."""
         if not sddmm._tiled:
             return 1
         P, T = sddmm._tiled[0]['P'], sddmm._tiled[1]
         conc = min(8 // T, P) if (T < 8 and 8 % T == 0) else 1
-        return (P + conc - 1) // conc
+        groups = (P + conc - 1) // conc
+        return tile_groups(T) * (1 if groups <= 32 else groups)
 
     def copies(n_tiles):
         """Launches of the kernel that makes the tile-by-tile copy of the gathered operand (the library's
@@ -298,9 +305,13 @@ def main():
 
     def pass_sums(n_parts):
         """Launches of the kernel that adds the SpMM passes' own buffers into out (the library's default rule:
-        4 or more source partitions, an output of 192 MB or more, buffers of 8 GiB or less)."""
-        out_bytes = 4 * n * F
-        return 1 if (n_parts >= 4 and out_bytes >= (192 << 20) and out_bytes * n_parts <= (8 << 30)) else 0
+        several source partitions and buffers of 8 GiB or less)."""
+        return 1 if (n_parts >= 2 and 4 * n * F * n_parts <= (8 << 30)) else 0
+
+    def spmm_launches():
+        """Launches of the gather kernel: with buffers per pass one launch walks all partitions, else one per partition."""
+        P = spmm._active['P']
+        return tile_groups(spmm._num_feat_partitions or 1) * (1 if (P == 1 or pass_sums(P)) else P)
 
     flops_op = 2.0 * nnz * F
     b_spmm = spmm_bytes(n, n, nnz, F)
@@ -308,9 +319,9 @@ def main():
     ops = {
         "spmm": {"ms": t_spmm, "gflops": flops_op / t_spmm / 1e6, "compulsory_gb": b_spmm / 1e9,
                  "hbm_gbs": b_spmm / t_spmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_spmm / 1e6,
-                 "kernel": "spmm_items_kernel", "launches": spmm._active['P'],
+                 "kernel": "spmm_items_kernel", "launches": spmm_launches(),
                  "kernels": {"tile_major_kernel": copies(spmm._num_feat_partitions or 1),
-                             "spmm_items_kernel": spmm._active['P'], "spmm_fixup_kernel": spmm._active['P'],
+                             "spmm_items_kernel": spmm_launches(), "spmm_fixup_kernel": spmm._active['P'],
                              "spmm_pass_sum_kernel": pass_sums(spmm._active['P'])},
                  "num_col_partitions": spmm._active['P'], "num_feat_partitions": spmm._num_feat_partitions},
         "sddmm": {"ms": t_sddmm, "gflops": flops_op / t_sddmm / 1e6, "compulsory_gb": b_sddmm / 1e9,
