@@ -321,7 +321,8 @@ def main():
                  "hbm_gbs": b_spmm / t_spmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_spmm / 1e6,
                  "kernel": "spmm_items_kernel", "launches": spmm_launches(),
                  "kernels": {"tile_major_kernel": copies(spmm._num_feat_partitions or 1),
-                             "spmm_items_kernel": spmm_launches(), "spmm_fixup_kernel": spmm._active['P'],
+                             "spmm_items_kernel": spmm_launches(),
+                             "spmm_fixup_kernel": 1 if pass_sums(spmm._active['P']) else spmm._active['P'],
                              "spmm_pass_sum_kernel": pass_sums(spmm._active['P'])},
                  "num_col_partitions": spmm._active['P'], "num_feat_partitions": spmm._num_feat_partitions},
         "sddmm": {"ms": t_sddmm, "gflops": flops_op / t_sddmm / 1e6, "compulsory_gb": b_sddmm / 1e9,

@@ -41,7 +41,7 @@ struct Fixup {
     int32_t row;
     int32_t slot0;
     int32_t n_pieces;
-    int32_t pad;
+    int32_t part;     // the source partition the segment belongs to
 };
 
 }  // namespace fg

@@ -67,7 +67,7 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
                 int32_t made = 0;
                 for (int32_t s = 0; s < len; s += piece_len, ++made)
                     items.push_back({start + s, std::min(piece_len, len - s), (int32_t)r, slot + made});
-                fixups.push_back({(int32_t)r, slot, made, 0});
+                fixups.push_back({(int32_t)r, slot, made, (int32_t)p});
                 slot += made;
                 pl->n_split_rows++;
                 ++r;

@@ -791,16 +791,20 @@ int launch_arg_v(int L, int K, bool full, dim3 grid, hipStream_t st, const SpmmA
 }
 
 // out[row, :] (+)= sum of the row's pieces, in piece order.  One lane per V columns.
+// part_stride / out_stride (floats; 0 for a launch over one partition's fix-ups): with every pass in a buffer of
+// its own, partition p's pieces start at partial + p * part_stride and its rows at out + p * out_stride.
 template <int V>
 __global__ __launch_bounds__(256) void spmm_fixup_kernel(const Fixup *fixups, int64_t n_fixups,
                                                          const float *partial, float *out, int F,
-                                                         int accumulate) {
+                                                         int accumulate, int64_t part_stride, int64_t out_stride) {
     using vec = typename Vec<V>::type;
     const int per_row = F / V;
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n_fixups * per_row) return;
     const Fixup fx = fixups[t / per_row];
     const int f = (int)(t % per_row) * V;
+    partial += fx.part * part_stride;
+    out += fx.part * out_stride;
     vec sum = *reinterpret_cast<const vec *>(partial + (int64_t)fx.slot0 * F + f);
     for (int p = 1; p < fx.n_pieces; ++p)
         vadd(sum, *reinterpret_cast<const vec *>(partial + (int64_t)(fx.slot0 + p) * F + f));
@@ -1086,9 +1090,17 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
             if (rc != FG_OK) return rc;
         }
     }
-    for (int p = 0; p < P; ++p) {
+    if (pass_buf && pl->n_fixups > 0) {
+        // the split rows of all partitions in one launch, each into its partition's buffer
+        const int fv = (aligned16 && F % 4 == 0) ? 4 : 1;
+        const int64_t threads = pl->n_fixups * (F / fv);
+        const unsigned blocks = (unsigned)((threads + 255) / 256);
+        if (fv == 4) hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, pl->fixups_dev, pl->n_fixups, partial, pass_buf, F, 0, (int64_t)piece, (int64_t)pass_stride);
+        else hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, pl->fixups_dev, pl->n_fixups, partial, pass_buf, F, 0, (int64_t)piece, (int64_t)pass_stride);
+    }
+    for (int p = 0; p < P && !pass_buf; ++p) {
         const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
-        if (i1 > i0 && !pass_buf) {
+        if (i1 > i0) {
             SpmmArgs a;
             a.items = pl->items_dev + i0; a.n_items = i1 - i0;
             a.pos = pos + (int64_t)p * (pl->n_dst + 1);
@@ -1123,11 +1135,9 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
             const unsigned blocks = (unsigned)((threads + 255) / 256);
             const Fixup *fx = pl->fixups_dev + x0;
             if (reduce == FG_REDUCE_SUM) {
-                float *dst = pass_buf ? pass_buf + (size_t)p * pass_stride : out;
-                const float *pieces = pass_buf ? partial + (size_t)p * piece : partial;
-                const int add = (p > 0 && !pass_buf) ? 1 : 0;
-                if (fv == 4) hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pieces, dst, F, add);
-                else hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, pieces, dst, F, add);
+                const int add = p > 0 ? 1 : 0;
+                if (fv == 4) hipLaunchKernelGGL(spmm_fixup_kernel<4>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F, add, (int64_t)0, (int64_t)0);
+                else hipLaunchKernelGGL(spmm_fixup_kernel<1>, dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F, add, (int64_t)0, (int64_t)0);
             } else if (reduce == FG_REDUCE_MAX) {
                 if (fv == 4) hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<4, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F);
                 else hipLaunchKernelGGL((gspmm_extreme_fixup_kernel<1, true>), dim3(blocks), dim3(256), 0, st, fx, x1 - x0, partial, out, F);
