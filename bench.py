@@ -47,7 +47,7 @@ MEASURED_TRAFFIC = {
     ("spmm", "powerlaw-233k", 32, 4, 0): (4.72e9, _PROFILES % "powerlaw233k_f32"),
     ("sddmm", "powerlaw-233k", 32, 4, 1): (5.56e9, _PROFILES % "powerlaw233k_f32"),
     ("spmm", "powerlaw-2.45M", 128, 1, 1): (33.15e9, _PROFILES % "powerlaw2450k_f128"),
-    ("sddmm", "powerlaw-2.45M", 128, 1, 1): (32.86e9, _PROFILES % "powerlaw2450k_f128"),
+    ("sddmm", "powerlaw-2.45M", 128, 1, 1): (33.41e9, _PROFILES % "powerlaw2450k_f128"),
 }
 METRIC = "SpMM/SDDMM GFLOP/s + achieved HBM GB/s (% roofline), 233k-node graph, feat 512"
 
@@ -313,6 +313,7 @@ def main():
         P = spmm._active['P']
         return tile_groups(spmm._num_feat_partitions or 1) * (1 if (P == 1 or pass_sums(P)) else P)
 
+    plain_sddmm = "sddmm_csr_kernel" if sddmm._use_csr else "sddmm_coo_kernel"     # the stored-order kernels
     flops_op = 2.0 * nnz * F
     b_spmm = spmm_bytes(n, n, nnz, F)
     b_sddmm = sddmm_bytes(n, nnz, F, 1, csr=True)
@@ -327,11 +328,11 @@ def main():
                  "num_col_partitions": spmm._active['P'], "num_feat_partitions": spmm._num_feat_partitions},
         "sddmm": {"ms": t_sddmm, "gflops": flops_op / t_sddmm / 1e6, "compulsory_gb": b_sddmm / 1e9,
                   "hbm_gbs": b_sddmm / t_sddmm / 1e6, "gathered_gbs": 4.0 * nnz * F / t_sddmm / 1e6,
-                  "kernel": "sddmm_tiled_kernel" if sddmm._tiled else "sddmm_csr_kernel",
+                  "kernel": "sddmm_tiled_kernel" if sddmm._tiled else plain_sddmm,
                   "launches": sddmm_launches(),
                   "kernels": ({"tile_major_kernel": copies(sddmm._tiled[1]), "sddmm_tiled_kernel": sddmm_launches(),
                                "sddmm_tile_sum_kernel": 1}
-                              if sddmm._tiled else {"sddmm_csr_kernel": 1}),
+                              if sddmm._tiled else {plain_sddmm: 1}),
                   "num_src_partitions": sddmm._tiled[0]['P'] if sddmm._tiled else 1,
                   "num_feat_tiles": sddmm._tiled[1] if sddmm._tiled else 1},
     }

@@ -237,8 +237,11 @@ def choose_sddmm(n_rows, n_cols, nnz, heads, head_len, stats=None):
             return None                                # the whole operand sits in every L2: nothing to tile
         ranked = [(p, t) for p, t in rank_sddmm(stats, feat_len)
                   if feat_len // t <= 256 and _is_pow2(feat_len // t) and feat_len // t >= 16]
-        if not ranked or ranked[0] == (1, 1):
-            return None                                # the stored-order kernels (measured 2-8 % ahead of a 1 x 1 traversal)
+        if not ranked or ranked[0][0] == 1:
+            # No source partitions: the stored-order kernels.  Without partitions the traversal has no slice to keep in
+            # the L2s and still pays for its partial sums and the scatter to the stored order (measured: 2-8 % behind at
+            # 1 x 1; 2.45M-node graph at F = 512: 1 x 2 tiles 22.5 ms, stored order 20.1 ms; uniform 1M-node graph: 23.3 / 22.7 ms).
+            return None
         return ranked[0]
     return _choose_sddmm_heads(n_rows, n_cols, nnz, heads, head_len)
 
