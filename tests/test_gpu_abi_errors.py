@@ -79,3 +79,58 @@ def test_plan_rejects_bad_positions(env):
     assert not bad.value
     assert L.fg_spmm_plan_create(lib.host_ptr(dec), 3, 4, 0, None, ctypes.byref(bad)) == FG_ERR_ARG
     assert L.fg_spmm_plan_create(None, 3, 4, 1, None, ctypes.byref(bad)) == FG_ERR_ARG
+
+
+def test_broadcasting_entry_points(env):
+    """fg_gspmm_bcast_f32 / fg_gsddmm_bcast_f32 called directly: a correct call, then every refusal."""
+    import torch
+    L, lib, plan, plan2, t = env
+    p = lib.dev_ptr
+    U, E, V = 0, 1, 2
+    ADD, MUL, COPY_LHS, DOT = 0, 2, 4, 6
+    SUM, MAX = 0, 1
+    ef = torch.full((6, 8), 2.0, device="cuda")
+    out = torch.zeros((4, 8), device="cuda")
+    arg = torch.zeros((4, 8), dtype=torch.int32, device="cuda")
+
+    def spmm(pl=plan, op=MUL, red=SUM, lhs=t['x'], lt=U, ll=8, loff=None, rhs=ef, rt=E, rl=8, roff=None, flags=0, o=out, a=None, n=8):
+        return L.fg_gspmm_bcast_f32(pl, p(t['indptr']), p(t['indices']), op, red, p(lhs), lt, ll, p(loff), p(rhs), rt, rl, p(roff),
+                                    flags, None, p(o), p(a), n, None)
+
+    assert spmm() == FG_OK
+    torch.cuda.synchronize()
+    deg = torch.tensor([2., 0., 3., 1.], device="cuda")
+    assert torch.equal(out, (2 * deg)[:, None].expand(4, 8))          # x = 1, edge features = 2
+    assert spmm(red=MAX, a=arg) == FG_OK
+    torch.cuda.synchronize()
+    assert arg[:, 0].tolist() == [0, -1, 2, 5]                        # first element of every row, -1 for the empty one
+    assert spmm(pl=None) == FG_ERR_ARG
+    assert spmm(pl=plan2) == FG_ERR_ARG and b"one column partition" in L.fg_last_error()
+    assert spmm(op=DOT) == FG_ERR_ARG
+    assert spmm(red=5) == FG_ERR_ARG
+    assert spmm(a=arg) == FG_ERR_ARG                                  # positions exist for max / min only
+    assert spmm(lhs=None) == FG_ERR_ARG and b"lhs" in L.fg_last_error()
+    assert spmm(lt=V) == FG_ERR_ARG                                   # destination-node operands: SDDMM only
+    assert spmm(ll=4) == FG_ERR_SHAPE                                 # no offset array: the length must be the output's
+    assert spmm(n=0) == FG_ERR_SHAPE
+    assert spmm(o=None) == FG_ERR_ARG
+    assert spmm(op=COPY_LHS, rhs=None, rl=0) == FG_OK                 # the unused operand may be absent
+
+    row = torch.tensor([0, 0, 2, 2, 2, 3], dtype=torch.int32, device="cuda")
+    eo = torch.zeros((6, 8), device="cuda")
+
+    def sddmm(r=row, c=t['indices'], n_edges=6, op=ADD, lhs=t['x'], lt=U, ll=8, rhs=t['y'], rt=V, rl=8, o=eo, n=8, red_len=1):
+        return L.fg_gsddmm_bcast_f32(p(r), p(c), n_edges, op, p(lhs), lt, ll, None, p(rhs), rt, rl, None, 0, p(o), n, red_len, None)
+
+    assert sddmm() == FG_OK
+    torch.cuda.synchronize()
+    assert torch.equal(eo, torch.full((6, 8), 2.0, device="cuda"))
+    assert sddmm(op=9) == FG_ERR_ARG
+    assert sddmm(n_edges=-1) == FG_ERR_ARG
+    assert sddmm(lhs=None) == FG_ERR_ARG
+    assert sddmm(c=None) == FG_ERR_ARG                                # an operand on u needs the column ids
+    assert sddmm(r=None) == FG_ERR_ARG
+    assert sddmm(ll=4) == FG_ERR_SHAPE
+    assert sddmm(op=DOT, n=2, red_len=3) == FG_ERR_SHAPE              # 8 is not a multiple of the contracted length
+    assert sddmm(op=DOT, n=2, red_len=4, o=eo) == FG_OK
+    assert sddmm(n_edges=0, lhs=None, rhs=None) == FG_OK              # nothing to read, nothing refused
