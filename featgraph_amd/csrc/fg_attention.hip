@@ -50,6 +50,12 @@ struct AttnArgs {
     // scalar per vertex and head; floats from one head's block to the next; negative slope of the leaky ReLU
     int64_t q_head_floats, k_head_floats;
     float slope;
+    // One launch over the items of all source partitions, every partition into buffers of its own (FIRST in every
+    // pass): the plan's item_off on the device (n_parts + 1 entries; null: one partition's items, strides unused) and
+    // the distance from one partition's pos / k / v / out / state to the next, in elements.
+    const int64_t *item_off = nullptr;
+    int n_parts = 1;
+    int64_t pos_stride = 0, k_stride = 0, v_stride = 0, out_stride = 0, state_stride = 0;
 };
 
 // Running softmax-weighted sum of one lane group: maximum, sum of exponentials, weighted sum.
@@ -222,13 +228,25 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
     const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_heads) * kWavesPerBlock + wave;
     if (item_id >= a.n_items) return;
     const Item it = a.items[item_id];
+    // the partition this item belongs to (uniform per wavefront)
+    int part = 0;
+    if (a.item_off) {
+        const int64_t id = ((int64_t)__builtin_amdgcn_readfirstlane((int)(item_id >> 32)) << 32) |
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)item_id);
+        while (part + 1 < a.n_parts && id >= a.item_off[part + 1]) ++part;
+    }
+    const int32_t *const pos_p = a.pos + part * a.pos_stride;
+    const float *const k_p = a.k + part * a.k_stride;
+    const float *const v_p = a.v + part * a.v_stride;
+    float *const out_p = a.out + part * a.out_stride;
+    float *const state_p = a.state + part * a.state_stride;
     const int g = lane / L, li = lane % L;
     const int f_lo = head * D + li * 4;
     const uint32_t lane_bytes = a.kv_tile_bytes ? (uint32_t)head * a.kv_tile_bytes + (uint32_t)li * 16u : (uint32_t)f_lo * 4u;
     const int64_t F = a.F;
     S *cols = s_col[wave];
     // ADD: this head's scalars; the score's second parameter is the negative slope
-    const float *kptr = ADD ? a.k + (int64_t)head * a.k_head_floats : a.k;
+    const float *kptr = ADD ? k_p + (int64_t)head * a.k_head_floats : k_p;
     const float *q_head = a.q + (int64_t)head * a.q_head_floats;
     const float sparam = ADD ? a.slope : a.scale;
 
@@ -256,8 +274,8 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
         if constexpr (ADD) return make_float4(q_head[row], 0.f, 0.f, 0.f);
         else return *reinterpret_cast<const float4 *>(a.q + row * F + f_lo);
     };
-    auto out_row = [&](int64_t row) { return a.out + row * F + f_lo; };
-    auto state_row = [&](int64_t row) { return a.state + (row * a.H + head) * 2; };
+    auto out_row = [&](int64_t row) { return out_p + row * F + f_lo; };
+    auto state_row = [&](int64_t row) { return state_p + (row * a.H + head) * 2; };
 
     if (it.info < -1) {
         // several whole rows, at most 256 elements: staged once
@@ -273,10 +291,10 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
             const int t = lane + 64 * i;
             const int64_t at = (int64_t)(it.row + min(t / kLines, nrows - 1)) * F + head * D + min((t % kLines) * 32, D - 1);
             if (!ADD) touched += a.q[at];
-            if (!FIRST) touched += a.out[at];
+            if (!FIRST) touched += out_p[at];
         }
         if (it.len > 0) stage(it.start, it.len);
-        s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+        s_end[wave][lane] = pos_p[it.row + min(lane, nrows - 1) + 1] - it.start;
         if (lane == 0) s_next[wave] = 0;
         wave_lds_sync();
         asm volatile("" ::"v"(touched));      // keeps the loads
@@ -314,7 +332,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
                 }
                 if (__all(done)) break;
                 if (!done && j < e) {
-                    own_batch<L, ADD>(cols, j, e, kptr, a.v, lane_bytes, q, sparam, run);
+                    own_batch<L, ADD>(cols, j, e, kptr, v_p, lane_bytes, q, sparam, run);
                     j += kU;
                 }
             }
@@ -327,7 +345,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
                 const float4 q = own_q(it.row + r);
                 const Running old = load_state<FIRST>(out_row(it.row + r), state_row(it.row + r));
                 Running run = running_empty();
-                walk<L, ADD>(cols, b, e, g, kptr, a.v, lane_bytes, q, sparam, run);
+                walk<L, ADD>(cols, b, e, g, kptr, v_p, lane_bytes, q, sparam, run);
                 finish_row<L, FIRST>(run, old, g, li, out_row(it.row + r), state_row(it.row + r));
             }
             b = e;
@@ -343,7 +361,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
         wave_lds_sync();
         stage((int64_t)it.start + base, n);
         wave_lds_sync();
-        walk<L, ADD>(cols, 0, n, g, kptr, a.v, lane_bytes, q, sparam, run);
+        walk<L, ADD>(cols, 0, n, g, kptr, v_p, lane_bytes, q, sparam, run);
     }
     if (it.len > 0 || FIRST) finish_row<L, FIRST>(run, old, g, li, out_row(it.row), state_row(it.row));
 }
@@ -359,6 +377,36 @@ __global__ __launch_bounds__(256) void attention_finish_kernel(float4 *out, cons
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     o.x *= inv; o.y *= inv; o.z *= inv; o.w *= inv;
     out[i] = l > 0.f ? o : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// The partitions' buffers merged, partition after partition, and the row divided by its sum of exponentials:
+// out[r, h, :] and state[r, h] = (maximum, sum) from buf_out [P][n_dst][F] and buf_state [P][n_dst][H][2].
+__global__ __launch_bounds__(256) void attention_merge_kernel(float4 *out, float *state, const float4 *buf_out,
+                                                              const float *buf_state, uint32_t n_words, uint32_t row_words,
+                                                              uint32_t head_words, int H, int P) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= n_words) return;
+    const uint32_t r = i / row_words, w = i - r * row_words, h = w / head_words;
+    const uint64_t srow = ((uint64_t)r * H + h) * 2, sstride = (uint64_t)(n_words / row_words) * H * 2;
+    // the row's maximum over the partitions first, so that every buffer enters with one factor and the loads of the
+    // running sums do not wait for each other
+    float m = -INFINITY;
+    for (int p = 0; p < P; ++p) m = fmaxf(m, buf_state[p * sstride + srow]);
+    Running run = running_empty();
+    if (m != -INFINITY) {
+        run.m = m;
+#pragma unroll 4
+        for (int p = 0; p < P; ++p) {
+            const float f = __expf(buf_state[p * sstride + srow] - m);      // exp(-inf) = 0 for a partition without elements
+            const float4 a = buf_out[(uint64_t)p * n_words + i];
+            run.acc.x += a.x * f; run.acc.y += a.y * f; run.acc.z += a.z * f; run.acc.w += a.w * f;
+            run.l += buf_state[p * sstride + srow + 1] * f;
+        }
+    }
+    const float inv = run.l > 0.f ? 1.0f / run.l : 0.f;
+    out[i] = run.l > 0.f ? make_float4(run.acc.x * inv, run.acc.y * inv, run.acc.z * inv, run.acc.w * inv)
+                         : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (w == h * head_words) { state[srow] = run.m; state[srow + 1] = run.l; }
 }
 
 template <int L, bool ADD>
@@ -408,6 +456,42 @@ int run_forward(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev
         }
     }
     const int row_floats = tiled ? head_len : F;
+    const size_t own_state = row_state_dev == pl->partial_dev ? (size_t)pl->n_dst * heads * 2 : 0;
+    const size_t buf_out_floats = (size_t)pl->n_dst * F, buf_state_floats = (size_t)pl->n_dst * heads * 2;
+    if (fg::attention_pass_buffers(pl, heads, head_len) && pl->n_items > 0) {
+        // Every partition into buffers of its own (no reads of the rows' earlier state inside the gather kernel, no
+        // order between the passes): one launch walks all partitions' items, one kernel merges the buffers.
+        float *buf_out = pl->partial_dev + ((own_state + 3) & ~(size_t)3);
+        float *buf_state = buf_out + (size_t)P * buf_out_floats;
+        AttnArgs a;
+        a.items = pl->items_dev; a.n_items = pl->n_items; a.item_off = pl->item_off_dev; a.n_parts = P;
+        a.pos = pos_dev; a.pos_stride = pl->n_dst + 1;
+        a.indices = idx_dev; a.q = q_dev;
+        a.k = k; a.k_stride = ADD ? width : width * row_floats;
+        a.v = v; a.v_stride = width * row_floats;
+        a.kv_row_bytes = (uint32_t)row_floats * 4u;
+        a.kv_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * head_len * 4u) : 0u;
+        a.out = buf_out; a.out_stride = (int64_t)buf_out_floats;
+        a.state = buf_state; a.state_stride = (int64_t)buf_state_floats;
+        a.F = F; a.H = heads; a.scale = param; a.slope = param;
+        a.q_head_floats = ADD ? pl->n_dst : 0; a.k_head_floats = ADD ? pl->n_src : 0;
+        const int per_launch = (heads > 8 && heads % 8 == 0) ? 8 : heads;
+        for (int hb = 0; hb < heads; hb += per_launch) {
+            a.n_heads = per_launch; a.head_base = hb;
+            const int64_t blocks = ((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
+            if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
+            const dim3 grid((unsigned)blocks);
+            if (head_len == 64) launch<16, ADD>(true, grid, st, a);
+            else if (head_len == 32) launch<8, ADD>(true, grid, st, a);
+            else launch<4, ADD>(true, grid, st, a);
+        }
+        const uint32_t n_words = (uint32_t)((uint64_t)pl->n_dst * F / 4);
+        hipLaunchKernelGGL(attention_merge_kernel, dim3((n_words + 255u) / 256u), dim3(256), 0, st,
+                           reinterpret_cast<float4 *>(out_dev), row_state_dev, reinterpret_cast<const float4 *>(buf_out), buf_state,
+                           n_words, (uint32_t)(F / 4), (uint32_t)(head_len / 4), heads, P);
+        FG_HIP_TRY(hipGetLastError());
+        return FG_OK;
+    }
     for (int p = 0; p < P; ++p) {
         const int64_t i0 = pl->item_off[p], i1 = pl->item_off[p + 1];
         if (i1 == i0) continue;
@@ -443,14 +527,26 @@ int run_forward(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev
 }  // namespace
 
 namespace fg {
+// Whether the forward passes over the source partitions write buffers of their own ([P][n_dst][F] running sums and
+// [P][n_dst][H][2] maxima / sums of exponentials) that one kernel merges: several partitions, unless the plan's
+// pass_buffers option says never or the buffers would take more than 8 GiB.
+bool attention_pass_buffers(const fg_spmm_plan *pl, int heads, int head_len) {
+    const int P = pl->num_col_partitions;
+    if (P < 2 || pl->pass_buffers == 2) return false;
+    const uint64_t floats = (uint64_t)pl->n_dst * heads * (head_len + 2);
+    return floats * 4u * (uint64_t)P <= (8ull << 30);
+}
 // The rows' (max, sum) state when the caller passes none, and the head-by-head copies of the gathered
 // operands (V, and K for dot-product scores); the gradient kernels need the same copies and no state.
 int attention_scratch_need(const fg_spmm_plan *pl, int heads, int head_len, bool additive, bool own_row_state,
-                           ScratchNeed *need) {
+                           ScratchNeed *need, bool forward) {
     if (heads < 1 || !(head_len == 16 || head_len == 32 || head_len == 64))
         return fail(FG_ERR_SHAPE, "attention takes heads of 16, 32 or 64 floats, got %d heads of %d", heads, head_len);
     const uint64_t F = (uint64_t)heads * head_len;
     need->partial = own_row_state ? (size_t)pl->n_dst * heads * 2 : 0;
+    if (forward && attention_pass_buffers(pl, heads, head_len))
+        need->partial = ((need->partial + 3) & ~(size_t)3) +
+                        (size_t)pl->num_col_partitions * ((size_t)pl->n_dst * F + (size_t)pl->n_dst * heads * 2);
     need->tiled = 0;
     if (pl->nnz > 0 && wants_tile_major(pl, heads, (uint64_t)pl->n_src * F * 4u))
         need->tiled = (size_t)pl->n_src * F * (additive ? 1 : 2);

@@ -347,7 +347,7 @@ int run_backward(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_de
     const int P = pl->num_col_partitions;
     const int64_t width = (pl->n_src + P - 1) / P;
     fg::ScratchNeed need;
-    int rc = fg::attention_scratch_need(pl, heads, head_len, ADD, false, &need);
+    int rc = fg::attention_scratch_need(pl, heads, head_len, ADD, false, &need, false);
     if (rc == FG_OK) rc = fg::ensure_scratch(pl, need, stream);
     if (rc != FG_OK) return rc;
     const bool tiled = need.tiled > 0;

@@ -102,6 +102,9 @@ int spmm_scratch_need(const fg_spmm_plan *plan, int F, int heads, int reduce, in
 int sddmm_dds_scratch_need(const fg_spmm_plan *plan, int H, int D, int num_feat_partitions, ScratchNeed *need);
 int softmax_scratch_need(const fg_spmm_plan *plan, int heads, ScratchNeed *need);
 int gspmm_bcast_scratch_need(const fg_spmm_plan *plan, int out_len, bool with_arg, ScratchNeed *need);
+bool attention_pass_buffers(const fg_spmm_plan *plan, int heads, int head_len);
+// forward: the call is the forward pass (whose partitions may write buffers of their own); the gradient sweeps need
+// only the head-by-head copies of the gathered operands.
 int attention_scratch_need(const fg_spmm_plan *plan, int heads, int head_len, bool additive, bool own_row_state,
-                           ScratchNeed *need);
+                           ScratchNeed *need, bool forward = true);
 }  // namespace fg
