@@ -211,8 +211,9 @@ __device__ __forceinline__ void finish_row(Running r, const Running &old, int g,
     if (li == 0) { state_row[0] = r.m; state_row[1] = r.l; }
 }
 
-// L lanes x 128 bits cover one head.  FIRST: the first partition's pass writes every row's state; later
-// passes merge into it and skip rows without elements in their partition.
+// L lanes x 128 bits cover one head.  FIRST: the pass writes every row's state -- the first partition's pass, or
+// every partition's when each has buffers of its own (one launch over all partitions, merged afterwards);
+// otherwise later passes merge into the stored state and skip rows without elements in their partition.
 // ADD: scores are leaky_relu(el[col e, h] + er[row e, h]) (a.k = el and a.q = er, one scalar per vertex and head,
 // head by head) instead of scaled dot products of K and Q slices.
 template <int L, bool FIRST, bool ADD>

@@ -128,7 +128,7 @@ class SpMMbase(object):
         if T < 0 or (T > 0 and feat_len % T != 0):
             raise ValueError("feat_len %d is not divisible by num_feat_partitions %d" % (feat_len, T))
         # Source-column partitions: the constructor's count when it was given, else chosen for
-        # the L2 size (the product is the same; later partitions add to the output in place).
+        # the L2 size (the product is the same; the partitions' results are summed in partition order).
         P = self._num_col_partitions
         src_parts = schedule_args.get('num_src_partitions', 'auto')
         if P == 1 and src_parts is not None:
