@@ -158,23 +158,27 @@ class Graph(object):
     # ---- generalised operators with broadcasting -------------------------------------------------------
 
     def gspmm(self, msg, lhs, rhs=None, reduce="sum"):
-        """out[v] = sum (or mean) over the edges e into v of the message msg = '<u|e>_<add|sub|mul>_<u|e>' or 'copy_e'
-        (DGL's names): operands on 'u' are (num_cols, ...), on 'e' (nnz, ...) in CSR edge order, and their feature
-        shapes broadcast the numpy way.  Differentiable in both operands.  ('u_mul_e' with one weight per edge or
-        per edge and head is spmm(); 'copy_u' is aggregate().)"""
+        """out[v] = reduce over the edges e into v of the message msg = '<u|e>_<add|sub|mul|div>_<u|e>' or 'copy_e'
+        (DGL's names), reduce in {'sum', 'mean', 'max', 'min'}: operands on 'u' are (num_cols, ...), on 'e' (nnz, ...) in
+        CSR edge order, and their feature shapes broadcast the numpy way.  Differentiable in both operands (max / min:
+        the gradient goes to the selected edge's operands).  ('u_mul_e' with one weight per edge or per edge and head
+        is spmm(); 'copy_u' is aggregate().)"""
         op, lt, rt = parse_message(msg)
-        if reduce not in ("sum", "mean") or op not in ("add", "sub", "mul", "copy_lhs") or "v" in (lt, rt) or lt == rt:
-            raise ValueError("differentiable here: sum / mean of add, sub, mul between an operand on 'u' and one on 'e', or copy_e")
+        if reduce not in ("sum", "mean", "max", "min") or op not in ("add", "sub", "mul", "div", "copy_lhs") \
+                or "v" in (lt, rt) or lt == rt:
+            raise ValueError("differentiable here: sum / mean / max / min of add, sub, mul, div between an operand on 'u' "
+                             "and one on 'e', or copy_e")
+        fn = _GSpMM if reduce in ("sum", "mean") else _GSpMMExtreme
         if rt is None:
-            return _GSpMM.apply(self, msg, reduce, lhs)
-        return _GSpMM.apply(self, msg, reduce, lhs, rhs)
+            return fn.apply(self, msg, reduce, lhs)
+        return fn.apply(self, msg, reduce, lhs, rhs)
 
     def gsddmm(self, op, lhs, rhs, lhs_target="u", rhs_target="v"):
-        """out[e] = lhs[..] op rhs[..] per edge, op in {'add', 'sub', 'mul'}, operands on 'u' (num_cols, ...), 'v'
+        """out[e] = lhs[..] op rhs[..] per edge, op in {'add', 'sub', 'mul', 'div'}, operands on 'u' (num_cols, ...), 'v'
         (num_rows, ...) or 'e' (nnz, ...), feature shapes broadcasting the numpy way; out is (nnz, ...) in CSR edge
         order.  Differentiable in both operands.  (The dot product is sddmm().)"""
-        if op not in ("add", "sub", "mul") or lhs_target == rhs_target or not {lhs_target, rhs_target} <= {"u", "v", "e"}:
-            raise ValueError("differentiable here: add, sub, mul between operands on two different targets of u / v / e")
+        if op not in ("add", "sub", "mul", "div") or lhs_target == rhs_target or not {lhs_target, rhs_target} <= {"u", "v", "e"}:
+            raise ValueError("differentiable here: add, sub, mul, div between operands on two different targets of u / v / e")
         return _GSDDMM.apply(self, op, lhs_target, rhs_target, lhs, rhs)
 
     def _tr_pos(self, device):
@@ -182,15 +186,23 @@ class Graph(object):
             self._tr_pos_dev = torch.from_numpy(self._tr_pos_host).to(device)
         return self._tr_pos_dev
 
-    def _bcast_spmm_raw(self, msg, arrays, reduce="sum", transposed=False):
-        """Generalised SpMM over the adjacency or its transpose (edge operands then in the transpose's edge order)."""
+    def _bcast_spmm_raw(self, msg, arrays, reduce="sum", transposed=False, return_arg=False):
+        """Generalised SpMM over the adjacency or its transpose (edge operands then in the transpose's edge order);
+        return_arg (max / min): also the CSR position of the selected edge per output, as a tensor of the caller's own."""
         arrays = [a.contiguous() for a in arrays]
-        key = ('gspmm', msg, reduce, transposed) + tuple(tuple(a.shape) for a in arrays)
+        key = ('gspmm', msg, reduce, transposed, return_arg) + tuple(tuple(a.shape) for a in arrays)
         if key not in self._mods:
             m = GSpMMhip(self._tr if transposed else self._csr)
-            m.build([placeholder(tuple(a.shape)) for a in arrays], {'msg': msg, 'reduce': reduce}, {})
+            args = {'msg': msg, 'reduce': reduce}
+            if return_arg:
+                args['return_arg'] = True
+            m.build([placeholder(tuple(a.shape)) for a in arrays], args, {})
             self._mods[key] = m
-        return _fresh_run(self._mods[key], arrays)
+        mod = self._mods[key]
+        if return_arg:
+            mod.arg_tvm = torch.empty_like(mod.arg_tvm)
+            return _fresh_run(mod, arrays), mod.arg_tvm
+        return _fresh_run(mod, arrays)
 
     def _bcast_sddmm_raw(self, op, lt, rt, arrays):
         arrays = [a.contiguous() for a in arrays]
@@ -220,19 +232,19 @@ class Graph(object):
             return self._bcast_spmm_raw('copy_e', [m])
         return self._bcast_spmm_raw('copy_e', [m.index_select(0, self._tr_pos(m.device))], transposed=True)
 
-    def _edge_product_sum(self, m, q, tq, target):
-        """For every node of `target` ('v' or 'u'): the sum over its edges of m[e] * q(e), m per edge (CSR order),
-        q on `tq`; the products are formed inside the aggregation, no per-edge array is written."""
+    def _edge_product_sum(self, m, q, tq, target, op="mul"):
+        """For every node of `target` ('v' or 'u'): the sum over its edges of m[e] * q(e) (op='div': m[e] / q(e)), m per
+        edge (CSR order), q on `tq`; the messages are formed inside the aggregation, no per-edge array is written."""
         if target == "v":               # rows of the adjacency: q on 'u' or 'e'
             if tq == "v":
                 raise ValueError("both operands on the same target")
-            return self._bcast_spmm_raw('e_mul_' + tq, [m, q])
+            return self._bcast_spmm_raw('e_%s_%s' % (op, tq), [m, q])
         tp = self._tr_pos(m.device)     # rows of the transpose: its 'u' are this graph's 'v'
         if tq == "u":
             raise ValueError("both operands on the same target")
         if tq == "v":
-            return self._bcast_spmm_raw('e_mul_u', [m.index_select(0, tp), q], transposed=True)
-        return self._bcast_spmm_raw('e_mul_e', [m.index_select(0, tp), q.index_select(0, tp)], transposed=True)
+            return self._bcast_spmm_raw('e_%s_u' % op, [m.index_select(0, tp), q], transposed=True)
+        return self._bcast_spmm_raw('e_%s_e' % op, [m.index_select(0, tp), q.index_select(0, tp)], transposed=True)
 
     def edge_softmax(self, scores):
         """Softmax of scores, (nnz,) or (nnz, H), over the edges of each destination row, per head."""
@@ -369,13 +381,75 @@ class _GSpMM(torch.autograd.Function):
                 if op == "sub" and i == 1:
                     full = -full
                 grads.append(full.reshape(p.shape))
-            else:   # mul: d message / d p = the other operand
+            else:
+                # mul: d message / d p = the other operand q;  div: 1 / q for the numerator, -l / p^2 for the denominator
                 q, tq = arrays[1 - i], targets[1 - i]
-                if tp == "u":       # sum over the edges that leave u of dout[row e] * q[e]
-                    full = g._bcast_spmm_raw('u_mul_e', [dout, q.index_select(0, g._tr_pos(q.device))], transposed=True)
-                else:               # per edge: dout[row e] * q[col e]
-                    full = g._bcast_sddmm_raw('mul', 'v', tq, [dout, q])
+                inner = "div" if (op == "div" and i == 0) else "mul"
+                if tp == "u":       # sum over the edges that leave u of dout[row e] (* or /) q[e]
+                    full = g._bcast_spmm_raw('u_%s_e' % inner, [dout, q.index_select(0, g._tr_pos(q.device))], transposed=True)
+                else:               # per edge: dout[row e] (* or /) q[col e]
+                    full = g._bcast_sddmm_raw(inner, 'v', tq, [dout, q])
+                if op == "div" and i == 1:
+                    full = -full / _align_features(p, full) ** 2
                 grads.append(_reduce_to(full, p.shape))
+        return (None, None, None) + tuple(grads)
+
+
+def _align_features(x, like):
+    """View of x (rows, *feat) with its feature axes right-aligned to those of `like` (rows, *broadcast feat)."""
+    return x.reshape((x.shape[0],) + (1,) * (like.dim() - x.dim()) + tuple(x.shape[1:]))
+
+
+class _GSpMMExtreme(torch.autograd.Function):
+    """max / min aggregation of a generalised message: the gradient of out[v, f] goes to the operands of the edge
+    that was selected (the first one on ties, as the kernel reports it)."""
+
+    @staticmethod
+    def forward(ctx, g, msg, reduce, lhs, rhs=None):
+        arrays = [lhs] if rhs is None else [lhs, rhs]
+        out, arg = g._bcast_spmm_raw(msg, arrays, reduce, return_arg=True)
+        ctx.g, ctx.msg = g, msg
+        ctx.save_for_backward(arg, *arrays)
+        ctx.mark_non_differentiable(arg)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        g = ctx.g
+        op, lt, rt = parse_message(ctx.msg)
+        arg, *arrays = ctx.saved_tensors
+        targets = [lt] if rt is None else [lt, rt]
+        n_dst, out_shape = dout.shape[0], tuple(dout.shape[1:])
+        n_out = int(np.prod(out_shape)) if out_shape else 1
+        g._mean_weights(dout.device)                                   # makes g._cols
+        e = arg.reshape(n_dst, n_out).long()
+        valid = e >= 0
+        e = e.clamp(min=0)
+        rows_of = {"u": g._cols[e], "e": e}                            # operand row per output element
+
+        def spread(x):      # (rows, *feat) -> (rows, n_out): the operand feature every output feature reads
+            return _align_features(x, dout).expand((x.shape[0],) + out_shape).reshape(x.shape[0], n_out)
+
+        picked = [spread(x).gather(0, rows_of[t]) for x, t in zip(arrays, targets)]
+        d = dout.reshape(n_dst, n_out) * valid
+        grads = []
+        for i, (p, tp) in enumerate(zip(arrays, targets)):
+            if not ctx.needs_input_grad[3 + i]:
+                grads.append(None)
+                continue
+            if op in ("add", "copy_lhs") or (op == "sub" and i == 0):
+                c = d
+            elif op == "sub":
+                c = -d
+            elif op == "mul":
+                c = d * picked[1 - i]
+            elif i == 0:                                               # div, numerator
+                c = d / picked[1]
+            else:                                                      # div, denominator
+                c = -d * picked[0] / picked[1] ** 2
+            c = torch.where(valid, c, torch.zeros_like(c))
+            full = torch.zeros((p.shape[0], n_out), dtype=dout.dtype, device=dout.device).scatter_add_(0, rows_of[tp], c)
+            grads.append(_reduce_to(full.reshape((p.shape[0],) + out_shape), p.shape))
         return (None, None, None) + tuple(grads)
 
 
@@ -406,11 +480,15 @@ class _GSDDMM(torch.autograd.Function):
                 full = g._from_edges(d.reshape(d.shape[0], -1), tp).reshape(p.shape)
                 grads.append(-full if (op == "sub" and i == 1) else full)
             else:
+                # mul: d out / d p = q;  div: 1 / q for the numerator, -l / p^2 for the denominator
                 q, tq = arrays[1 - i], targets[1 - i]
+                inner = "div" if (op == "div" and i == 0) else "mul"
                 if tp == "e":
-                    full = g._bcast_sddmm_raw('mul', 'e', tq, [dout, q])
+                    full = g._bcast_sddmm_raw(inner, 'e', tq, [dout, q])
                 else:
-                    full = g._edge_product_sum(dout, q, tq, tp)
+                    full = g._edge_product_sum(dout, q, tq, tp, inner)
+                if op == "div" and i == 1:
+                    full = -full / _align_features(p, full) ** 2
                 grads.append(_reduce_to(full, p.shape))
         return (None, None, None, None) + tuple(grads)
 

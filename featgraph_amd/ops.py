@@ -6,9 +6,10 @@ neither.  Operand conventions are DGL's: node features of the source nodes are `
 destination nodes `(num_dst, ...)`, edge features `(nnz, ...)` in the graph's CSR edge order, and the feature
 shapes of two operands broadcast against each other the numpy way.
 
-Gradients: every call routes to a differentiable operator where one exists (weighted sums, sum / mean of
-add / sub / mul messages, copies, per-edge add / sub / mul / dot, max / min of copied source features); the
-rest (division, max / min of two-operand messages) runs forward only and refuses inputs that require grad.
+Gradients: every call routes to a differentiable operator (weighted sums; sum / mean / max / min of add / sub /
+mul / div messages and copies; per-edge add / sub / mul / div and dot products of node features); what is left --
+operators between two operands on the same target, dot products that involve edge features or broadcasting --
+runs forward only and refuses inputs that require grad.
 """
 import torch
 
@@ -34,10 +35,7 @@ def gspmm(g, op, reduce_op, lhs_data, rhs_data):
             return g.aggregate(x[:, None], reduce_op)[:, 0]
         return g.aggregate(x.reshape(x.shape[0], -1), reduce_op).reshape((g.shape[0],) + tuple(x.shape[1:]))
     if op == "copy_rhs":
-        if reduce_op in ("sum", "mean"):
-            return g.gspmm("copy_e", rhs_data, reduce=reduce_op)
-        _no_grad_inputs("max / min of edge features", rhs_data)
-        return g._bcast_spmm_raw("copy_e", [rhs_data], reduce_op)
+        return g.gspmm("copy_e", rhs_data, reduce=reduce_op)
     if op not in _BINARY:
         raise ValueError("op must be one of %s, 'copy_lhs', 'copy_rhs'" % (_BINARY,))
     if op == "mul" and reduce_op == "sum" and lhs_data.dim() in (2, 3):
@@ -49,11 +47,7 @@ def gspmm(g, op, reduce_op, lhs_data, rhs_data):
             return g.spmm(lhs_data, rhs_data[:, :, 0])
         if lhs_data.dim() == 2 and tuple(rhs_data.shape[1:]) == (1,):
             return g.spmm(lhs_data, rhs_data[:, 0])
-    msg = "u_%s_e" % op
-    if op != "div" and reduce_op in ("sum", "mean"):
-        return g.gspmm(msg, lhs_data, rhs_data, reduce_op)
-    _no_grad_inputs("gspmm(%s, %s)" % (op, reduce_op), lhs_data, rhs_data)
-    return g._bcast_spmm_raw(msg, [lhs_data, rhs_data], reduce_op)
+    return g.gspmm("u_%s_e" % op, lhs_data, rhs_data, reduce_op)
 
 
 def gsddmm(g, op, lhs_data, rhs_data, lhs_target="u", rhs_target="v"):
@@ -76,7 +70,7 @@ def gsddmm(g, op, lhs_data, rhs_data, lhs_target="u", rhs_target="v"):
         return g._bcast_sddmm_raw("dot", lhs_target, rhs_target, [lhs_data, rhs_data]).unsqueeze(-1)
     if op not in _BINARY:
         raise ValueError("op must be one of %s, 'dot', 'copy_lhs', 'copy_rhs'" % (_BINARY,))
-    if op != "div" and lhs_target != rhs_target:
+    if lhs_target != rhs_target:
         return g.gsddmm(op, lhs_data, rhs_data, lhs_target, rhs_target)
     _no_grad_inputs("gsddmm(%s) between '%s' and '%s'" % (op, lhs_target, rhs_target), lhs_data, rhs_data)
     return g._bcast_sddmm_raw(op, lhs_target, rhs_target, [lhs_data, rhs_data])

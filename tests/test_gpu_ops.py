@@ -44,6 +44,7 @@ def _reduce64(torch, m, rows, n_dst, reduce_op, deg):
 @pytest.mark.parametrize("op,reduce_op,l_shape,r_shape", [
     ("mul", "sum", (32,), ()), ("mul", "sum", (4, 8), (4, 1)), ("mul", "sum", (16,), (16,)), ("add", "mean", (8,), (1,)),
     ("sub", "sum", (2, 3), (3,)), ("div", "sum", (8,), (8,)), ("mul", "max", (8,), (8,)), ("add", "min", (5,), (1,)),
+    ("div", "mean", (4, 1), (1, 6)), ("div", "max", (6,), (1,)), ("sub", "min", (1,), (7,)), ("mul", "min", (2, 4), (2, 1)),
     ("copy_lhs", "sum", (12,), None), ("copy_lhs", "max", (3, 4), None), ("copy_rhs", "sum", None, (6,)),
     ("copy_rhs", "min", None, (2, 2)), ("copy_lhs", "mean", (), None),
 ])
@@ -53,7 +54,7 @@ def test_gspmm(op, reduce_op, l_shape, r_shape):
     gen = torch.Generator(device="cuda"); gen.manual_seed(3)
     n_dst, n_src, nnz = adj.shape[0], adj.shape[1], adj.nnz
     deg = torch.from_numpy(np.diff(adj.indptr)).cuda().double()
-    differentiable = op != "div" and (reduce_op in ("sum", "mean") or op == "copy_lhs")
+    differentiable = True
 
     def make(n, shape):
         if shape is None:
@@ -96,7 +97,8 @@ def test_gspmm(op, reduce_op, l_shape, r_shape):
 @pytest.mark.parametrize("op,lt,l_shape,rt,r_shape", [
     ("dot", 'u', (24,), 'v', (24,)), ("dot", 'u', (4, 8), 'v', (4, 8)), ("dot", 'v', (16,), 'u', (16,)),
     ("dot", 'e', (2, 4), 'u', (1, 4)), ("add", 'u', (8,), 'v', (8,)), ("mul", 'e', (4, 1), 'v', (4, 8)),
-    ("sub", 'v', (3,), 'u', (1,)), ("div", 'u', (6,), 'e', (6,)), ("copy_lhs", 'u', (5,), 'v', (1,)),
+    ("sub", 'v', (3,), 'u', (1,)), ("div", 'u', (6,), 'e', (6,)), ("div", 'e', (2, 3), 'v', (3,)), ("div", 'v', (1,), 'u', (5,)),
+    ("copy_lhs", 'u', (5,), 'v', (1,)),
     ("copy_rhs", 'u', (1,), 'v', (2, 3)), ("copy_lhs", 'e', (4,), 'v', (1,)),
 ])
 def test_gsddmm(op, lt, l_shape, rt, r_shape):
@@ -104,7 +106,7 @@ def test_gsddmm(op, lt, l_shape, rt, r_shape):
     torch, g, adj, rows, cols = _setup(len(op) + sum(l_shape))
     gen = torch.Generator(device="cuda"); gen.manual_seed(4)
     n_of = {'u': adj.shape[1], 'v': adj.shape[0], 'e': adj.nnz}
-    differentiable = op in ("add", "sub", "mul", "copy_lhs", "copy_rhs") or (op == "dot" and {lt, rt} == {'u', 'v'})
+    differentiable = op in ("add", "sub", "mul", "div", "copy_lhs", "copy_rhs") or (op == "dot" and {lt, rt} == {'u', 'v'})
 
     def make(n, shape):
         t = torch.randn((n,) + shape, generator=gen, device="cuda")
