@@ -10,7 +10,6 @@ Prints one JSON line per point: mean of 5 runs, GFLOP/s, compulsory-model GB/s a
 """
 import argparse
 
-import numpy as np
 import torch
 
 from ..module import VanillaSpMMhip, placeholder

@@ -9,7 +9,6 @@ import scipy.sparse
 import torch
 
 from .. import _lib
-from .. import tuning
 from ..util import util_convert_csr_to_dds
 from . import common
 from . import general

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import scipy.sparse as sp
 
-from helpers import RTOL, ATOL
+from helpers import RTOL
 
 pytestmark = pytest.mark.gpu
 

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import scipy.sparse as sp
 
-from helpers import RTOL, ATOL, assert_sum_close, spmm_mass
+from helpers import assert_sum_close, spmm_mass
 
 pytestmark = pytest.mark.gpu
 

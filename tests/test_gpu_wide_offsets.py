@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import scipy.sparse as sp
 
-from helpers import RTOL, ATOL, assert_sum_close, spmm_mass, sddmm_mass
+from helpers import assert_sum_close, spmm_mass, sddmm_mass
 
 pytestmark = pytest.mark.gpu
 
