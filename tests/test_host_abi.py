@@ -177,6 +177,8 @@ def test_default_tilings():
     assert tuning.choose_sddmm(n, n, nnz, 1, 256) == (8, 4)
     assert tuning.choose_sddmm(n, n, nnz, 1, 1024) == (8, 16)
     assert tuning.choose_sddmm(2450000, 2450000, 61903880, 1, 128) is None    # stored-order kernels
+    assert tuning.choose_sddmm(2450000, 2450000, 61903880, 1, 512) is None    # no source partitions: stored order, not 1 x 2 tiles
+    assert tuning.choose_sddmm(1000000, 1000000, 64998031, 1, 512) is None
     assert tuning.choose_sddmm(n, n, nnz, 8, 64) == (16, 4)
     assert tuning.choose_sddmm(n, n, nnz, 4, 64) == (8, 4)
     assert tuning.choose_sddmm(n, n, nnz, 8, 32) == (16, 2)
