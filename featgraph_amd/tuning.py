@@ -153,7 +153,8 @@ def _gather_seconds(stats, feat_len, P, T, c):
 def predict_spmm(stats, feat_len, P, T, coef=SPMM_COEF):
     """Modelled seconds of one SpMM with P source-column partitions and T feature tiles."""
     t = _gather_seconds(stats, feat_len, P, T, coef)
-    return t + 4.0 * stats.n_dst * feat_len * (2 * P - 1) / coef['stream']      # out: written per pass, re-read by later ones
+    # out: one buffer written per pass and read back once by the sum (fitted as (2P - 1) when later passes re-read `out`)
+    return t + 4.0 * stats.n_dst * feat_len * (2 * P - 1) / coef['stream']
 
 
 def predict_sddmm(stats, feat_len, P, T, coef=SDDMM_COEF):
