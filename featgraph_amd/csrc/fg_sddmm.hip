@@ -373,6 +373,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     __shared__ __align__(16) int2 s_edge[kWavesPerBlock][fg::kItemEdges + kTilePad];     // x = column word, y = edge_pos
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
     __shared__ int32_t s_next[kWavesPerBlock];
+    __shared__ __align__(16) float4 s_dst[kWavesPerBlock][128 * K];      // destination slices of an item with few rows
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane / L, li = lane % L;
@@ -428,10 +429,45 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
 
     if (it.info < -1) {
         const int nrows = -it.info;
-        // The destination rows of this item are read once here, one word per 128 bytes, while the
-        // edges are on their way.  Loads return in order, so a row fetched from memory at the moment
-        // it is needed would hold up every gather issued after it; fetched here, all rows' misses
-        // overlap each other and the staging loads, and the later reads hit the cache.
+        if (nrows < 2 * G) {
+            // Few, longer rows: all lane groups share each row in turn.  The rows' destination slices (fewer than
+            // 128 * K 128-bit words) are read once here, together with the staging loads, and kept in LDS: a slice
+            // fetched at the moment its row starts would sit in front of that row's gathers (loads return in order),
+            // and one that was only touched here has left the L2 again by the time a later row of the item needs it.
+            constexpr int RV = L * K;                    // 128-bit words per row slice
+            float4 held[2 * K];
+#pragma unroll
+            for (int i = 0; i < 2 * K; ++i) {
+                const int t = lane + 64 * i;
+                const int r = min(t / RV, nrows - 1);
+                held[i] = *reinterpret_cast<const float4 *>(a.dst + (int64_t)(it.row + r) * F + tile * (RV * 4) + (t % RV) * 4);
+            }
+            stage(it.start, it.len);
+            s_end[wave][lane] = pos[it.row + min(lane, nrows - 1) + 1] - it.start;
+#pragma unroll
+            for (int i = 0; i < 2 * K; ++i) s_dst[wave][lane + 64 * i] = held[i];
+            wave_lds_sync();
+            int b = 0;
+            for (int q = 0; q < nrows; ++q) {
+                const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
+                if (e > b) {
+#pragma unroll
+                    for (int k = 0; k < K; ++k) dv[k] = s_dst[wave][q * RV + k * L + li];
+                    int s0 = b;
+                    for (; s0 + G * U <= e; s0 += G * U)
+                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, e, src, lane_bytes, F, dv,
+                                                                                 out, a.out_edge_stride, it.start, seg_pos);
+                    if (s0 < e)
+                        sddmm_tile_tail<L, K, RW, KH, U, SCATTER, OFF32>((e - s0 + G - 1) / G, edge, s0 + g, G, e, src, lane_bytes,
+                                                                         F, dv, out, a.out_edge_stride, it.start, seg_pos);
+                }
+                b = e;
+            }
+            return;
+        }
+        // Many short rows.  Their destination slices are touched once here, one word per 128 bytes, while the
+        // edges are on their way, so that all rows' misses overlap each other and the staging loads and the
+        // reads at the rows' starts hit the cache.
         constexpr int kLines = (L * K * 16 + 127) / 128;
         constexpr int kTouch = (fg::kItemRows * kLines + 63) / 64;
         float touched[kTouch];
@@ -448,25 +484,6 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         wave_lds_sync();
 #pragma unroll
         for (int i = 0; i < kTouch; ++i) asm volatile("" ::"v"(touched[i]));    // keeps the loads
-        if (nrows < 2 * G) {
-            // few, longer rows: all lane groups share each row in turn
-            int b = 0;
-            for (int q = 0; q < nrows; ++q) {
-                const int e = __builtin_amdgcn_readfirstlane(s_end[wave][q]);
-                if (e > b) {
-                    load_dst(it.row + q);
-                    int s0 = b;
-                    for (; s0 + G * U <= e; s0 += G * U)
-                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, e, src, lane_bytes, F, dv,
-                                                                                 out, a.out_edge_stride, it.start, seg_pos);
-                    if (s0 < e)
-                        sddmm_tile_tail<L, K, RW, KH, U, SCATTER, OFF32>((e - s0 + G - 1) / G, edge, s0 + g, G, e, src, lane_bytes,
-                                                                         F, dv, out, a.out_edge_stride, it.start, seg_pos);
-                }
-                b = e;
-            }
-            return;
-        }
         // many short rows: every lane group walks rows of its own
         int q = -1, j = 0, e = 0;
         bool done = false;
