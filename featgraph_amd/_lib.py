@@ -56,6 +56,7 @@ SIGNATURES = {
     "fg_sddmm_dds_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp]),
     "fg_gsddmm_elementwise_f32": (_int, [_vp, _vp, _i64, _vp, _vp, _vp, _int, _int, _vp]),
     "fg_gspmm_bcast_f32": (_int, [_vp, _vp, _vp, _int, _int, _vp, _int, _int, _vp, _vp, _int, _int, _vp, _int, _vp, _vp, _vp, _int, _vp]),
+    "fg_gspmm_bcast_dds_f32": (_int, [_vp, _vp, _vp, _vp, _int, _int, _vp, _int, _int, _vp, _vp, _int, _int, _vp, _int, _vp, _vp, _vp, _int, _vp]),
     "fg_gsddmm_bcast_f32": (_int, [_vp, _vp, _i64, _int, _vp, _int, _int, _vp, _vp, _int, _int, _vp, _int, _vp, _int, _int, _vp]),
     "fg_edge_softmax_f32": (_int, [_vp, _vp, _vp, _vp, _int, _vp]),
     "fg_edge_softmax_backward_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp]),

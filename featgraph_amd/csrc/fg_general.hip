@@ -19,6 +19,12 @@
 // 64 vectors at a time.  With one group (64 vectors or more) a row's sum is formed in the stored element
 // order.  The edge operand, when there is one, is the dominant stream ([nnz, len] floats read once,
 // coalesced); the node operand is gathered.
+//
+// Over a plan with several source-column partitions (fg_gspmm_bcast_dds_f32) one launch walks all partitions'
+// items in partition order, so that the gathered operand's rows of the current partition stay in the L2s: a
+// partition's row segments are reduced into a buffer of its own and a closing kernel combines the buffers in
+// partition order.  The elements then come in the partitioned layout's order and reach the operands on the edges
+// (and the reported positions) through the layout's element -> stored position array.
 #include <hip/hip_runtime.h>
 
 #include <climits>
@@ -50,18 +56,32 @@ struct GenArgs {
     const int32_t *lhs_off, *rhs_off;
     int lhs_len, rhs_len;
     int lhs_target, rhs_target;
+    float sign;                  // -1: the launch computes a minimum as the negated maximum of the negated messages; else 1
     const float *row_scale;      // out[v, :] *= row_scale[v] (null: 1), applied where a row is completed
     float *out;
     int32_t *arg;                // optional: stored position of the selected element (max / min)
     float *partial;              // pieces of split rows: [slot][F] values
     int32_t *partial_arg;        //                       [slot][F] positions
     int F, L;
+    // Several source-column partitions (PART): indptr / indices are the partitioned layout's position and local
+    // column arrays, item_off the plan's item ranges per partition, edge_pos the stored position of every element;
+    // out / arg are the partitions' buffers.  Strides in elements, per partition.
+    const int64_t *item_off;
+    const int32_t *edge_pos;
+    int n_parts;
+    int64_t pos_stride, col_width, out_stride, partial_stride;
 };
 
 // The operand features of a lane's V outputs: V consecutive ones (CONTIG: one 128-bit load) or one value V times.
-template <int V, bool CONTIG>
+// NT: a non-temporal load, for an operand on the stored elements, which is read once from end to end and should not
+// displace the gathered operand's rows from the L2.
+typedef float nt_f4 __attribute__((ext_vector_type(4)));
+template <int V, bool CONTIG, bool NT = false>
 __device__ __forceinline__ void load_operand(const float *p, float (&o)[V]) {
-    if (V == 4 && CONTIG) {
+    if (V == 4 && CONTIG && NT) {
+        const nt_f4 t = __builtin_nontemporal_load(reinterpret_cast<const nt_f4 *>(p));
+        o[0] = t.x; o[1 % V] = t.y; o[2 % V] = t.z; o[3 % V] = t.w;
+    } else if (V == 4 && CONTIG) {
         const float4 t = *reinterpret_cast<const float4 *>(p);
         o[0] = t.x; o[1 % V] = t.y; o[2 % V] = t.z; o[3 % V] = t.w;
     } else {
@@ -91,8 +111,15 @@ template <int RED> __device__ __forceinline__ bool replaces(float m, int em, flo
 // LC / RC (V == 4 only): the operand's 4 features are consecutive (one 128-bit load), else one value 4 times.
 // No branch stands between the loads of a step: one around a load would make the wavefront wait for everything
 // issued before it.
-template <int OP, int RED, bool ARG, int V, bool LC, bool RC>
+// PART: the items of several source-column partitions (see GenArgs); a row segment without elements then keeps the
+// reduction's identity and no row is scaled, both being the combining kernel's business.
+// LNT / RNT: see load_operand.  RED: FG_REDUCE_SUM or FG_REDUCE_MAX; a minimum runs as the maximum of the negated
+// messages (a.sign = -1; negation is exact, so values, ties and selected positions are those of the minimum).
+template <int OP, int RED, bool ARG, int V, bool LC, bool RC, bool LNT, bool RNT, bool PART>
 __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
+    static_assert(RED == FG_REDUCE_SUM || RED == FG_REDUCE_MAX, "a minimum is a maximum with a.sign = -1");
+    constexpr bool kLhs = kUsesLhs<OP>, kRhs = kUsesRhs<OP>;
+    const float sign = RED == FG_REDUCE_SUM ? 1.f : a.sign;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int64_t item_id = (int64_t)blockIdx.x * kWavesPerBlock + wave;
@@ -100,6 +127,18 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
     const Item it = a.items[item_id];
     const int L = a.L, G = 64 / L, g = lane / L, li = lane % L;
     const int F = a.F, FV = F / V;
+    int part = 0;
+    if (PART) {
+        const int64_t id = ((int64_t)__builtin_amdgcn_readfirstlane((int)(item_id >> 32)) << 32) |
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)item_id);
+        while (part + 1 < a.n_parts && id >= a.item_off[part + 1]) ++part;
+    }
+    const int32_t *const pos_p = a.indptr + (PART ? part * a.pos_stride : 0);
+    const int64_t ubase = PART ? part * a.col_width : 0;       // the partition's first column
+    float *const out_p = a.out + (PART ? part * a.out_stride : 0);
+    int32_t *const arg_p = ARG ? a.arg + (PART ? part * a.out_stride : 0) : nullptr;
+    float *const partial_p = a.partial + (PART ? part * a.partial_stride : 0);
+    int32_t *const partial_arg_p = ARG ? a.partial_arg + (PART ? part * a.partial_stride : 0) : nullptr;
     const bool l_on_e = a.lhs_target == FG_TARGET_E, r_on_e = a.rhs_target == FG_TARGET_E;
     constexpr int U = V == 4 ? 4 : 8;     // elements in flight per lane group: the loads of a step are issued before its sums
 
@@ -108,8 +147,8 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
         for (int f0 = 0; f0 < FV; f0 += L) {
             const bool active = f0 + li < FV;
             const int fc = (active ? f0 + li : FV - 1) * V;       // the lane's first output feature
-            const int fl = kUsesLhs<OP> ? (a.lhs_off ? a.lhs_off[fc] : fc) : 0;
-            const int fr = kUsesRhs<OP> ? (a.rhs_off ? a.rhs_off[fc] : fc) : 0;
+            const int fl = kLhs ? (a.lhs_off ? a.lhs_off[fc] : fc) : 0;
+            const int fr = kRhs ? (a.rhs_off ? a.rhs_off[fc] : fc) : 0;
             float acc[V];
             int at[V];
 #pragma unroll
@@ -117,21 +156,27 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
             for (int64_t eb = e0 + g; eb < e1; eb += (int64_t)G * U) {
                 float m[U][V];
                 bool ok[U];
+                int stored[U];          // the element's position in the caller's edge order
 #pragma unroll
                 for (int k = 0; k < U; ++k) {
                     const int64_t e = eb + (int64_t)k * G;
                     ok[k] = e < e1;
                     const int64_t ec = ok[k] ? e : eb;
-                    const int64_t u = a.indices[ec];          // read also when no operand lives on u: no branch
+                    const int64_t u = a.indices[ec] + ubase;  // read also when no operand lives on u: no branch
+                    stored[k] = PART ? a.edge_pos[ec] : (int)e;
+                    const int64_t ee = PART ? (int64_t)stored[k] : ec;
                     float l[V], r[V];
-                    if (kUsesLhs<OP>) load_operand<V, LC>(a.lhs + (l_on_e ? ec : u) * a.lhs_len + fl, l);
-                    if (kUsesRhs<OP>) load_operand<V, RC>(a.rhs + (r_on_e ? ec : u) * a.rhs_len + fr, r);
+                    if (kLhs) load_operand<V, LC, LNT>(a.lhs + (l_on_e ? ee : u) * a.lhs_len + fl, l);
+                    if (kRhs) load_operand<V, RC, RNT>(a.rhs + (r_on_e ? ee : u) * a.rhs_len + fr, r);
 #pragma unroll
-                    for (int i = 0; i < V; ++i) m[k][i] = binary<OP>(kUsesLhs<OP> ? l[i] : 0.f, kUsesRhs<OP> ? r[i] : 0.f);
+                    for (int i = 0; i < V; ++i) {
+                        m[k][i] = binary<OP>(kLhs ? l[i] : 0.f, kRhs ? r[i] : 0.f);
+                        if (RED != FG_REDUCE_SUM) m[k][i] *= sign;
+                    }
                 }
 #pragma unroll
                 for (int k = 0; k < U; ++k) {
-                    const int e = (int)(eb + (int64_t)k * G);
+                    const int e = stored[k];
 #pragma unroll
                     for (int i = 0; i < V; ++i) {
                         if (RED == FG_REDUCE_SUM) {
@@ -160,7 +205,8 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
                 const float scale = (done && a.row_scale) ? a.row_scale[v] : 1.f;
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
-                    acc[i] = (RED != FG_REDUCE_SUM && empty) ? 0.f : acc[i];
+                    if (RED != FG_REDUCE_SUM) acc[i] *= sign;
+                    acc[i] = (RED != FG_REDUCE_SUM && empty && !PART) ? 0.f : acc[i];
                     if (done && a.row_scale) acc[i] *= scale;
                     if (ARG) at[i] = (at[i] == INT_MAX) ? -1 : at[i];
                 }
@@ -179,64 +225,125 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
         const int nrows = -it.info;
         for (int q = 0; q < nrows; ++q) {
             const int v = it.row + q;
-            const int64_t e0 = a.indptr[v], e1 = a.indptr[v + 1];
-            reduce_range(e0, e1, v, a.out + (int64_t)v * F, ARG ? a.arg + (int64_t)v * F : nullptr, true);
+            const int64_t e0 = pos_p[v], e1 = pos_p[v + 1];
+            reduce_range(e0, e1, v, out_p + (int64_t)v * F, ARG ? arg_p + (int64_t)v * F : nullptr, !PART);
         }
         return;
     }
-    reduce_range(it.start, (int64_t)it.start + it.len, it.row, a.partial + (int64_t)it.info * F,
-                 ARG ? a.partial_arg + (int64_t)it.info * F : nullptr, false);
+    reduce_range(it.start, (int64_t)it.start + it.len, it.row, partial_p + (int64_t)it.info * F,
+                 ARG ? partial_arg_p + (int64_t)it.info * F : nullptr, false);
 }
 
 // The pieces of a split row, combined in stored order.
+// partial_stride / out_stride: per source partition (0 with one partition); the split segment's partition is fx.part.
 template <int RED, bool ARG>
 __global__ __launch_bounds__(256) void gspmm_bcast_fixup_kernel(const Fixup *fixups, int64_t n_fixups, const float *partial,
                                                                 const int32_t *partial_arg, const float *row_scale,
-                                                                float *out, int32_t *arg, int F) {
+                                                                float *out, int32_t *arg, int F, int64_t partial_stride,
+                                                                int64_t out_stride) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n_fixups * F) return;
     const Fixup fx = fixups[t / F];
     const int f = (int)(t % F);
+    const int64_t from = fx.part * partial_stride, to = fx.part * out_stride;
     float acc = identity<RED>();
     int at = INT_MAX;
     for (int p = 0; p < fx.n_pieces; ++p) {
-        const float m = partial[(int64_t)(fx.slot0 + p) * F + f];
+        const float m = partial[from + (int64_t)(fx.slot0 + p) * F + f];
         if (RED == FG_REDUCE_SUM) acc = p == 0 ? m : acc + m;
         else if (ARG) {
-            const int am = partial_arg[(int64_t)(fx.slot0 + p) * F + f];
+            const int am = partial_arg[from + (int64_t)(fx.slot0 + p) * F + f];
             if (am >= 0 && replaces<RED>(m, am, acc, at)) { acc = m; at = am; }
         } else acc = RED == FG_REDUCE_MAX ? fmaxf(acc, m) : fminf(acc, m);
     }
     if (row_scale) acc *= row_scale[fx.row];
-    out[(int64_t)fx.row * F + f] = acc;
-    if (ARG) arg[(int64_t)fx.row * F + f] = (at == INT_MAX) ? -1 : at;
+    out[to + (int64_t)fx.row * F + f] = acc;
+    if (ARG) arg[to + (int64_t)fx.row * F + f] = (at == INT_MAX) ? -1 : at;
+}
+
+// out[v, f] = the partitions' results for row v combined in partition order (buf[p * buf_stride + v * F + f], positions abuf likewise, with -1
+// for "none"); a row without elements in any partition gives 0 for max / min; rows are scaled here.
+template <int RED, bool ARG>
+__global__ __launch_bounds__(256) void gspmm_bcast_combine_kernel(const float *buf, const int32_t *abuf, const int32_t *pos,
+                                                                  int n_parts, int64_t pos_stride, int64_t buf_stride,
+                                                                  int64_t n_rows, int F, const float *row_scale, float *out,
+                                                                  int32_t *arg) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_rows * F) return;
+    const int64_t v = t / F;
+    float acc = identity<RED>();
+    int at = INT_MAX;
+    bool any = false;
+    for (int p = 0; p < n_parts; ++p) {
+        const float m = buf[p * buf_stride + t];
+        if (RED == FG_REDUCE_SUM) acc = p == 0 ? m : acc + m;
+        else {
+            any = any || pos[p * pos_stride + v + 1] > pos[p * pos_stride + v];
+            if (ARG) {
+                const int am = abuf[p * buf_stride + t];
+                if (am >= 0 && replaces<RED>(m, am, acc, at)) { acc = m; at = am; }
+            } else acc = RED == FG_REDUCE_MAX ? fmaxf(acc, m) : fminf(acc, m);
+        }
+    }
+    if (RED != FG_REDUCE_SUM && !any) acc = 0.f;
+    if (row_scale) acc *= row_scale[v];
+    out[t] = acc;
+    if (ARG) arg[t] = (at == INT_MAX) ? -1 : at;
 }
 
 // vec: 0 = one feature per lane; else 4 per lane with (lhs, rhs) read as 1 = (consecutive, consecutive),
-// 2 = (consecutive, one value), 3 = (one value, consecutive)
+// 2 = (consecutive, one value), 3 = (one value, consecutive); lnt / rnt: that operand streams from the stored elements
+template <int OP, int RED, bool ARG, bool PART>
+void launch_spmm_variant(int vec, bool lnt, bool rnt, dim3 grid, hipStream_t st, const GenArgs &a) {
+    constexpr int USES = (kUsesLhs<OP> ? 1 : 0) | (kUsesRhs<OP> ? 2 : 0);
+#define FG_GO(V, LC, RC, LNT, RNT) \
+    hipLaunchKernelGGL((gspmm_bcast_kernel<OP, RED, ARG, V, LC, RC, LNT, RNT, PART>), grid, dim3(kBlock), 0, st, a)
+    if (vec == 0) { FG_GO(1, true, true, false, false); return; }
+    const bool lc = vec != 3, rc = vec != 2;
+    lnt = lnt && lc; rnt = rnt && rc;
+    if constexpr (USES == 1) {             // the right operand is not read: one instantiation stands for all its modes
+        if (!lc) FG_GO(4, false, true, false, false);
+        else if (lnt) FG_GO(4, true, true, true, false);
+        else FG_GO(4, true, true, false, false);
+    } else if constexpr (USES == 2) {
+        if (!rc) FG_GO(4, true, false, false, false);
+        else if (rnt) FG_GO(4, true, true, false, true);
+        else FG_GO(4, true, true, false, false);
+    } else {
+        if (lc && rc) {
+            if (lnt && rnt) FG_GO(4, true, true, true, true);
+            else if (lnt) FG_GO(4, true, true, true, false);
+            else if (rnt) FG_GO(4, true, true, false, true);
+            else FG_GO(4, true, true, false, false);
+        } else if (lc) {
+            if (lnt) FG_GO(4, true, false, true, false);
+            else FG_GO(4, true, false, false, false);
+        } else {
+            if (rnt) FG_GO(4, false, true, false, true);
+            else FG_GO(4, false, true, false, false);
+        }
+    }
+#undef FG_GO
+}
 template <int OP, int RED, bool ARG>
-void launch_spmm_ora(int vec, dim3 grid, hipStream_t st, const GenArgs &a) {
-    if (vec == 1) hipLaunchKernelGGL((gspmm_bcast_kernel<OP, RED, ARG, 4, true, true>), grid, dim3(kBlock), 0, st, a);
-    else if (vec == 2) hipLaunchKernelGGL((gspmm_bcast_kernel<OP, RED, ARG, 4, true, false>), grid, dim3(kBlock), 0, st, a);
-    else if (vec == 3) hipLaunchKernelGGL((gspmm_bcast_kernel<OP, RED, ARG, 4, false, true>), grid, dim3(kBlock), 0, st, a);
-    else hipLaunchKernelGGL((gspmm_bcast_kernel<OP, RED, ARG, 1, true, true>), grid, dim3(kBlock), 0, st, a);
+void launch_spmm_ora(int vec, bool lnt, bool rnt, dim3 grid, hipStream_t st, const GenArgs &a) {
+    if (a.n_parts > 1) launch_spmm_variant<OP, RED, ARG, true>(vec, lnt, rnt, grid, st, a);
+    else launch_spmm_variant<OP, RED, ARG, false>(vec, lnt, rnt, grid, st, a);
 }
 template <int OP>
-void launch_spmm_o(int reduce, bool with_arg, int vec, dim3 grid, hipStream_t st, const GenArgs &a) {
-    if (reduce == FG_REDUCE_SUM) launch_spmm_ora<OP, FG_REDUCE_SUM, false>(vec, grid, st, a);
-    else if (reduce == FG_REDUCE_MAX && with_arg) launch_spmm_ora<OP, FG_REDUCE_MAX, true>(vec, grid, st, a);
-    else if (reduce == FG_REDUCE_MAX) launch_spmm_ora<OP, FG_REDUCE_MAX, false>(vec, grid, st, a);
-    else if (with_arg) launch_spmm_ora<OP, FG_REDUCE_MIN, true>(vec, grid, st, a);
-    else launch_spmm_ora<OP, FG_REDUCE_MIN, false>(vec, grid, st, a);
+void launch_spmm_o(int reduce, bool with_arg, int vec, bool lnt, bool rnt, dim3 grid, hipStream_t st, const GenArgs &a) {
+    if (reduce == FG_REDUCE_SUM) launch_spmm_ora<OP, FG_REDUCE_SUM, false>(vec, lnt, rnt, grid, st, a);
+    else if (with_arg) launch_spmm_ora<OP, FG_REDUCE_MAX, true>(vec, lnt, rnt, grid, st, a);       // max, or min by a.sign
+    else launch_spmm_ora<OP, FG_REDUCE_MAX, false>(vec, lnt, rnt, grid, st, a);
 }
-void launch_spmm(int op, int reduce, bool with_arg, int vec, dim3 grid, hipStream_t st, const GenArgs &a) {
+void launch_spmm(int op, int reduce, bool with_arg, int vec, bool lnt, bool rnt, dim3 grid, hipStream_t st, const GenArgs &a) {
     switch (op) {
-        case FG_BIN_ADD: launch_spmm_o<FG_BIN_ADD>(reduce, with_arg, vec, grid, st, a); break;
-        case FG_BIN_SUB: launch_spmm_o<FG_BIN_SUB>(reduce, with_arg, vec, grid, st, a); break;
-        case FG_BIN_MUL: launch_spmm_o<FG_BIN_MUL>(reduce, with_arg, vec, grid, st, a); break;
-        case FG_BIN_DIV: launch_spmm_o<FG_BIN_DIV>(reduce, with_arg, vec, grid, st, a); break;
-        case FG_BIN_COPY_LHS: launch_spmm_o<FG_BIN_COPY_LHS>(reduce, with_arg, vec, grid, st, a); break;
-        default: launch_spmm_o<FG_BIN_COPY_RHS>(reduce, with_arg, vec, grid, st, a); break;
+        case FG_BIN_ADD: launch_spmm_o<FG_BIN_ADD>(reduce, with_arg, vec, lnt, rnt, grid, st, a); break;
+        case FG_BIN_SUB: launch_spmm_o<FG_BIN_SUB>(reduce, with_arg, vec, lnt, rnt, grid, st, a); break;
+        case FG_BIN_MUL: launch_spmm_o<FG_BIN_MUL>(reduce, with_arg, vec, lnt, rnt, grid, st, a); break;
+        case FG_BIN_DIV: launch_spmm_o<FG_BIN_DIV>(reduce, with_arg, vec, lnt, rnt, grid, st, a); break;
+        case FG_BIN_COPY_LHS: launch_spmm_o<FG_BIN_COPY_LHS>(reduce, with_arg, vec, lnt, rnt, grid, st, a); break;
+        default: launch_spmm_o<FG_BIN_COPY_RHS>(reduce, with_arg, vec, lnt, rnt, grid, st, a); break;
     }
 }
 
@@ -273,10 +380,24 @@ int check_operand(const char *name, bool used, const float *p, int64_t rows, int
     return FG_OK;
 }
 
-size_t gspmm_piece_floats(const fg_spmm_plan *pl, int F, bool with_arg) {
-    const size_t per = (((size_t)pl->max_slots_in_partition * (size_t)F) + 3) & ~(size_t)3;
-    return with_arg ? 2 * per : per;
+// Scratch of one call, in floats: per partition the pieces of its split rows ([slot][F], rounded up to 16 bytes) and,
+// with several partitions, a buffer of [n_dst][F] results; the selected positions, when wanted, take as much again.
+struct BcastScratch {
+    size_t pieces = 0;      // per partition
+    size_t buffers = 0;     // per partition (0 with one partition)
+    size_t half = 0;        // all partitions' values; the positions follow
+    size_t total = 0;
+};
+BcastScratch bcast_scratch(const fg_spmm_plan *pl, int F, bool with_arg) {
+    BcastScratch b;
+    const size_t P = (size_t)pl->num_col_partitions;
+    b.pieces = (((size_t)pl->max_slots_in_partition * (size_t)F) + 3) & ~(size_t)3;
+    b.buffers = P > 1 ? (((size_t)pl->n_dst * (size_t)F) + 3) & ~(size_t)3 : 0;
+    b.half = P * (b.pieces + b.buffers);
+    b.total = with_arg ? 2 * b.half : b.half;
+    return b;
 }
+constexpr size_t kMaxBufferBytes = (size_t)8 << 30;     // all partitions' result buffers together
 
 // ---- SDDMM ------------------------------------------------------------------------------------------
 
@@ -335,7 +456,7 @@ __global__ __launch_bounds__(kBlock) void gsddmm_bcast_kernel(const EdgeArgs a) 
             for (int k = 0; k < U; ++k) {
                 if (!ok[k]) continue;
                 float *o = a.out + (eb + (int64_t)k * G) * a.F + fc;
-                if (V == 4) *reinterpret_cast<float4 *>(o) = make_float4(m[k][0], m[k][1 % V], m[k][2 % V], m[k][3 % V]);
+                if (V == 4) { nt_f4 t4; t4.x = m[k][0]; t4.y = m[k][1 % V]; t4.z = m[k][2 % V]; t4.w = m[k][3 % V]; __builtin_nontemporal_store(t4, reinterpret_cast<nt_f4 *>(o)); }
                 else *o = m[k][0];
             }
         }
@@ -354,13 +475,104 @@ void launch_sddmm(int vec, dim3 grid, hipStream_t st, const EdgeArgs &a) {
 
 namespace fg {
 int gspmm_bcast_scratch_need(const fg_spmm_plan *pl, int F, bool with_arg, ScratchNeed *need) {
-    if (pl->num_col_partitions != 1) return fail(FG_ERR_ARG, "the broadcasting SpMM needs a plan with one column partition");
     if (F < 1) return fail(FG_ERR_SHAPE, "feature length must be positive, got %d", F);
-    need->partial = gspmm_piece_floats(pl, F, with_arg);
+    const BcastScratch b = bcast_scratch(pl, F, with_arg);
+    if ((size_t)pl->num_col_partitions * b.buffers * 4 * (with_arg ? 2 : 1) > kMaxBufferBytes)
+        return fail(FG_ERR_SHAPE, "%d source partitions of [%lld, %d] results need more than 8 GiB of buffers; use fewer partitions",
+                    pl->num_col_partitions, (long long)pl->n_dst, F);
+    need->partial = b.total;
     need->tiled = 0;
     return FG_OK;
 }
 }  // namespace fg
+
+namespace {
+
+// pos / idx: indptr / indices of the CSR arrays with one partition, else the partitioned layout's position and local
+// column arrays, with edge_pos the stored position of each of its elements.
+int gspmm_bcast_run(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev, const int32_t *edge_pos_dev, int op,
+                    int reduce, const float *lhs_dev, int lhs_target, int lhs_len, const int32_t *lhs_off_dev,
+                    const float *rhs_dev, int rhs_target, int rhs_len, const int32_t *rhs_off_dev, int flags,
+                    const float *row_scale_dev, float *out_dev, int32_t *arg_dev, int out_len, void *stream) {
+    if (op < FG_BIN_ADD || op > FG_BIN_COPY_RHS) return fail(FG_ERR_ARG, "unknown message operator %d", op);
+    if (reduce != FG_REDUCE_SUM && reduce != FG_REDUCE_MAX && reduce != FG_REDUCE_MIN)
+        return fail(FG_ERR_ARG, "unknown reduce op %d", reduce);
+    if (arg_dev && reduce == FG_REDUCE_SUM) return fail(FG_ERR_ARG, "positions of the selected elements exist for max / min only");
+    fg::ScratchNeed need;
+    if (int rc = fg::gspmm_bcast_scratch_need(pl, out_len, arg_dev != nullptr, &need)) return rc;
+    const int P = pl->num_col_partitions;
+    const bool uses_l = op != FG_BIN_COPY_RHS, uses_r = op != FG_BIN_COPY_LHS;
+    if (int rc = check_operand("lhs", uses_l, lhs_dev, lhs_target == FG_TARGET_E ? pl->nnz : pl->n_src, lhs_len, lhs_target, false)) return rc;
+    if (int rc = check_operand("rhs", uses_r, rhs_dev, rhs_target == FG_TARGET_E ? pl->nnz : pl->n_src, rhs_len, rhs_target, false)) return rc;
+    if ((uses_l && !lhs_off_dev && lhs_len != out_len) || (uses_r && !rhs_off_dev && rhs_len != out_len))
+        return fail(FG_ERR_SHAPE, "an operand without an offset array must have the output's feature length %d", out_len);
+    if (pl->n_dst == 0) return FG_OK;
+    if (!out_dev || !pos_dev || (pl->nnz > 0 && (!idx_dev || (P > 1 && !edge_pos_dev)))) return fail(FG_ERR_ARG, "null device pointer");
+    if (int rc = fg::ensure_scratch(pl, need, stream)) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const BcastScratch b = bcast_scratch(pl, out_len, arg_dev != nullptr);
+    const int lmode = vector_mode(uses_l, lhs_dev, lhs_len, lhs_off_dev, flags, FG_BCAST_LHS_VEC4, FG_BCAST_LHS_SPLAT4);
+    const int rmode = vector_mode(uses_r, rhs_dev, rhs_len, rhs_off_dev, flags, FG_BCAST_RHS_VEC4, FG_BCAST_RHS_SPLAT4);
+    const int vec = vector_variant(out_len % 4 == 0 && (((uintptr_t)out_dev | (uintptr_t)arg_dev) & 15) == 0, lmode, rmode);
+    const int V = vec ? 4 : 1;
+    float *const values = pl->partial_dev;                                          // [P][pieces] then [P][buffers]
+    int32_t *const positions = reinterpret_cast<int32_t *>(pl->partial_dev + b.half);
+    float *const buf = values + (size_t)P * b.pieces;
+    int32_t *const abuf = positions + (size_t)P * b.pieces;
+    GenArgs a;
+    a.items = pl->items_dev; a.n_items = pl->n_items;
+    a.indptr = pos_dev; a.indices = idx_dev;
+    a.lhs = lhs_dev; a.rhs = rhs_dev; a.lhs_off = lhs_off_dev; a.rhs_off = rhs_off_dev;
+    a.lhs_len = lhs_len; a.rhs_len = rhs_len; a.lhs_target = lhs_target; a.rhs_target = rhs_target;
+    a.sign = reduce == FG_REDUCE_MIN ? -1.f : 1.f;
+    a.row_scale = P > 1 ? nullptr : row_scale_dev;
+    a.out = P > 1 ? buf : out_dev;
+    a.arg = P > 1 ? (arg_dev ? abuf : nullptr) : arg_dev;
+    a.partial = values; a.partial_arg = positions;
+    a.F = out_len; a.L = lanes_for(out_len / V);
+    a.item_off = pl->item_off_dev; a.edge_pos = edge_pos_dev; a.n_parts = P;
+    a.pos_stride = pl->n_dst + 1; a.col_width = (pl->n_src + P - 1) / P;
+    a.out_stride = (int64_t)b.buffers; a.partial_stride = (int64_t)b.pieces;
+    const int64_t blocks = (pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
+    // an operand on the stored elements that is read with 128-bit loads streams past the caches
+    const bool lnt = uses_l && lhs_target == FG_TARGET_E && lmode == 1, rnt = uses_r && rhs_target == FG_TARGET_E && rmode == 1;
+    if (blocks > 0) launch_spmm(op, reduce, arg_dev != nullptr, vec, lnt, rnt, dim3((unsigned)blocks), st, a);
+    const int which = reduce == FG_REDUCE_SUM ? 0 : (reduce == FG_REDUCE_MAX ? 1 : 3) + (arg_dev ? 1 : 0);
+    if (pl->n_fixups > 0) {
+        const int64_t threads = pl->n_fixups * (int64_t)out_len;
+        const dim3 grid((unsigned)((threads + 255) / 256));
+#define FG_FIXUP(RED, ARG) hipLaunchKernelGGL((gspmm_bcast_fixup_kernel<RED, ARG>), grid, dim3(256), 0, st, pl->fixups_dev, pl->n_fixups, \
+                                              a.partial, a.partial_arg, a.row_scale, a.out, a.arg, out_len, a.partial_stride, a.out_stride)
+        switch (which) {
+            case 0: FG_FIXUP(FG_REDUCE_SUM, false); break;
+            case 1: FG_FIXUP(FG_REDUCE_MAX, false); break;
+            case 2: FG_FIXUP(FG_REDUCE_MAX, true); break;
+            case 3: FG_FIXUP(FG_REDUCE_MIN, false); break;
+            default: FG_FIXUP(FG_REDUCE_MIN, true); break;
+        }
+#undef FG_FIXUP
+    }
+    if (P > 1) {
+        const int64_t threads = pl->n_dst * (int64_t)out_len;
+        if ((threads + 255) / 256 > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "output of %lld values is too large", (long long)threads);
+        const dim3 grid((unsigned)((threads + 255) / 256));
+#define FG_COMBINE(RED, ARG) hipLaunchKernelGGL((gspmm_bcast_combine_kernel<RED, ARG>), grid, dim3(256), 0, st, buf, abuf, pos_dev, P, \
+                                                a.pos_stride, a.out_stride, pl->n_dst, out_len, row_scale_dev, out_dev, arg_dev)
+        switch (which) {
+            case 0: FG_COMBINE(FG_REDUCE_SUM, false); break;
+            case 1: FG_COMBINE(FG_REDUCE_MAX, false); break;
+            case 2: FG_COMBINE(FG_REDUCE_MAX, true); break;
+            case 3: FG_COMBINE(FG_REDUCE_MIN, false); break;
+            default: FG_COMBINE(FG_REDUCE_MIN, true); break;
+        }
+#undef FG_COMBINE
+    }
+    FG_HIP_TRY(hipGetLastError());
+    return FG_OK;
+}
+
+}  // namespace
 
 extern "C" int fg_gspmm_bcast_f32(fg_spmm_plan *pl, const int32_t *indptr_dev, const int32_t *indices_dev, int op,
                                   int reduce, const float *lhs_dev, int lhs_target, int lhs_len,
@@ -369,59 +581,21 @@ extern "C" int fg_gspmm_bcast_f32(fg_spmm_plan *pl, const int32_t *indptr_dev, c
                                   int32_t *arg_dev, int out_len, void *stream) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (int drc = fg::check_device(pl)) return drc;
-    if (op < FG_BIN_ADD || op > FG_BIN_COPY_RHS) return fail(FG_ERR_ARG, "unknown message operator %d", op);
-    if (reduce != FG_REDUCE_SUM && reduce != FG_REDUCE_MAX && reduce != FG_REDUCE_MIN)
-        return fail(FG_ERR_ARG, "unknown reduce op %d", reduce);
-    if (arg_dev && reduce == FG_REDUCE_SUM) return fail(FG_ERR_ARG, "positions of the selected elements exist for max / min only");
-    fg::ScratchNeed need;
-    if (int rc = fg::gspmm_bcast_scratch_need(pl, out_len, arg_dev != nullptr, &need)) return rc;
-    const bool uses_l = op != FG_BIN_COPY_RHS, uses_r = op != FG_BIN_COPY_LHS;
-    if (int rc = check_operand("lhs", uses_l, lhs_dev, lhs_target == FG_TARGET_E ? pl->nnz : pl->n_src, lhs_len, lhs_target, false)) return rc;
-    if (int rc = check_operand("rhs", uses_r, rhs_dev, rhs_target == FG_TARGET_E ? pl->nnz : pl->n_src, rhs_len, rhs_target, false)) return rc;
-    if ((uses_l && !lhs_off_dev && lhs_len != out_len) || (uses_r && !rhs_off_dev && rhs_len != out_len))
-        return fail(FG_ERR_SHAPE, "an operand without an offset array must have the output's feature length %d", out_len);
-    if (pl->n_dst == 0) return FG_OK;
-    if (!out_dev || !indptr_dev || (pl->nnz > 0 && !indices_dev)) return fail(FG_ERR_ARG, "null device pointer");
-    if (int rc = fg::ensure_scratch(pl, need, stream)) return rc;
-    hipStream_t st = (hipStream_t)stream;
-    const int lmode = vector_mode(uses_l, lhs_dev, lhs_len, lhs_off_dev, flags, FG_BCAST_LHS_VEC4, FG_BCAST_LHS_SPLAT4);
-    const int rmode = vector_mode(uses_r, rhs_dev, rhs_len, rhs_off_dev, flags, FG_BCAST_RHS_VEC4, FG_BCAST_RHS_SPLAT4);
-    const int vec = vector_variant(out_len % 4 == 0 && (((uintptr_t)out_dev | (uintptr_t)arg_dev) & 15) == 0, lmode, rmode);
-    const int V = vec ? 4 : 1;
-    GenArgs a;
-    a.items = pl->items_dev; a.n_items = pl->n_items;
-    a.indptr = indptr_dev; a.indices = indices_dev;
-    a.lhs = lhs_dev; a.rhs = rhs_dev; a.lhs_off = lhs_off_dev; a.rhs_off = rhs_off_dev;
-    a.lhs_len = lhs_len; a.rhs_len = rhs_len; a.lhs_target = lhs_target; a.rhs_target = rhs_target;
-    a.row_scale = row_scale_dev;
-    a.out = out_dev; a.arg = arg_dev;
-    a.partial = pl->partial_dev;
-    a.partial_arg = reinterpret_cast<int32_t *>(pl->partial_dev + need.partial / 2);
-    a.F = out_len; a.L = lanes_for(out_len / V);
-    const int64_t blocks = (pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
-    if (blocks > 0) launch_spmm(op, reduce, arg_dev != nullptr, vec, dim3((unsigned)blocks), st, a);
-    if (pl->n_fixups > 0) {
-        const int64_t threads = pl->n_fixups * (int64_t)out_len;
-        const dim3 grid((unsigned)((threads + 255) / 256));
-        if (reduce == FG_REDUCE_SUM)
-            hipLaunchKernelGGL((gspmm_bcast_fixup_kernel<FG_REDUCE_SUM, false>), grid, dim3(256), 0, st, pl->fixups_dev, pl->n_fixups,
-                               a.partial, a.partial_arg, row_scale_dev, out_dev, arg_dev, out_len);
-        else if (reduce == FG_REDUCE_MAX && arg_dev)
-            hipLaunchKernelGGL((gspmm_bcast_fixup_kernel<FG_REDUCE_MAX, true>), grid, dim3(256), 0, st, pl->fixups_dev, pl->n_fixups,
-                               a.partial, a.partial_arg, row_scale_dev, out_dev, arg_dev, out_len);
-        else if (reduce == FG_REDUCE_MAX)
-            hipLaunchKernelGGL((gspmm_bcast_fixup_kernel<FG_REDUCE_MAX, false>), grid, dim3(256), 0, st, pl->fixups_dev, pl->n_fixups,
-                               a.partial, a.partial_arg, row_scale_dev, out_dev, arg_dev, out_len);
-        else if (arg_dev)
-            hipLaunchKernelGGL((gspmm_bcast_fixup_kernel<FG_REDUCE_MIN, true>), grid, dim3(256), 0, st, pl->fixups_dev, pl->n_fixups,
-                               a.partial, a.partial_arg, row_scale_dev, out_dev, arg_dev, out_len);
-        else
-            hipLaunchKernelGGL((gspmm_bcast_fixup_kernel<FG_REDUCE_MIN, false>), grid, dim3(256), 0, st, pl->fixups_dev, pl->n_fixups,
-                               a.partial, a.partial_arg, row_scale_dev, out_dev, arg_dev, out_len);
-    }
-    FG_HIP_TRY(hipGetLastError());
-    return FG_OK;
+    if (pl->num_col_partitions != 1)
+        return fail(FG_ERR_ARG, "fg_gspmm_bcast_f32 takes a plan with one column partition (fg_gspmm_bcast_dds_f32: several)");
+    return gspmm_bcast_run(pl, indptr_dev, indices_dev, nullptr, op, reduce, lhs_dev, lhs_target, lhs_len, lhs_off_dev, rhs_dev,
+                           rhs_target, rhs_len, rhs_off_dev, flags, row_scale_dev, out_dev, arg_dev, out_len, stream);
+}
+
+extern "C" int fg_gspmm_bcast_dds_f32(fg_spmm_plan *pl, const int32_t *s1_pos_dev, const int32_t *s1_idx_dev,
+                                      const int32_t *edge_pos_dev, int op, int reduce, const float *lhs_dev, int lhs_target,
+                                      int lhs_len, const int32_t *lhs_off_dev, const float *rhs_dev, int rhs_target,
+                                      int rhs_len, const int32_t *rhs_off_dev, int flags, const float *row_scale_dev,
+                                      float *out_dev, int32_t *arg_dev, int out_len, void *stream) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
+    return gspmm_bcast_run(pl, s1_pos_dev, s1_idx_dev, edge_pos_dev, op, reduce, lhs_dev, lhs_target, lhs_len, lhs_off_dev, rhs_dev,
+                           rhs_target, rhs_len, rhs_off_dev, flags, row_scale_dev, out_dev, arg_dev, out_len, stream);
 }
 
 extern "C" int fg_gsddmm_bcast_f32(const int32_t *row_dev, const int32_t *col_dev, int64_t n_edges, int op,

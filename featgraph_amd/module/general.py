@@ -107,12 +107,21 @@ class BroadcastOp(object):
                    "" if self.reduce_len == 1 else ", %d contracted" % self.reduce_len,
                    "" if self.lhs_off is None and self.rhs_off is None else ", broadcast through offset arrays"))
 
-    def run_spmm(self, plan, indptr_dev, indices_dev, reduce, lhs, rhs, row_scale, out, arg):
-        _lib.check(_lib.lib().fg_gspmm_bcast_f32(
-            plan, _lib.dev_ptr(indptr_dev), _lib.dev_ptr(indices_dev), BINARY[self.op], reduce,
-            _lib.dev_ptr(lhs), TARGET[self.lhs_target or 'u'], self.lhs_len, _lib.dev_ptr(self.lhs_off),
-            _lib.dev_ptr(rhs), TARGET[self.rhs_target or 'e'], self.rhs_len, _lib.dev_ptr(self.rhs_off), self.flags,
-            _lib.dev_ptr(row_scale), _lib.dev_ptr(out), _lib.dev_ptr(arg), self.out_len, common.stream_ptr()))
+    def gathered_len(self):
+        """Feature length of the operand that is gathered from the source nodes (0: none is)."""
+        return max(self.lhs_len if self.lhs_target == 'u' else 0, self.rhs_len if self.rhs_target == 'u' else 0)
+
+    def run_spmm(self, plan, pos_dev, idx_dev, reduce, lhs, rhs, row_scale, out, arg, edge_pos_dev=None):
+        """pos_dev / idx_dev: indptr / indices, or (edge_pos_dev given) the arrays of a source-partitioned layout."""
+        operands = (BINARY[self.op], reduce,
+                    _lib.dev_ptr(lhs), TARGET[self.lhs_target or 'u'], self.lhs_len, _lib.dev_ptr(self.lhs_off),
+                    _lib.dev_ptr(rhs), TARGET[self.rhs_target or 'e'], self.rhs_len, _lib.dev_ptr(self.rhs_off), self.flags,
+                    _lib.dev_ptr(row_scale), _lib.dev_ptr(out), _lib.dev_ptr(arg), self.out_len, common.stream_ptr())
+        if edge_pos_dev is None:
+            _lib.check(_lib.lib().fg_gspmm_bcast_f32(plan, _lib.dev_ptr(pos_dev), _lib.dev_ptr(idx_dev), *operands))
+        else:
+            _lib.check(_lib.lib().fg_gspmm_bcast_dds_f32(plan, _lib.dev_ptr(pos_dev), _lib.dev_ptr(idx_dev),
+                                                         _lib.dev_ptr(edge_pos_dev), *operands))
 
     def run_sddmm(self, row_dev, col_dev, n_edges, lhs, rhs, out):
         _lib.check(_lib.lib().fg_gsddmm_bcast_f32(

@@ -10,6 +10,7 @@ import torch
 
 from .. import _lib
 from ..util import util_convert_csr_to_dds
+from .. import tuning
 from . import common
 from . import general
 from .spmm import VanillaSpMMhip
@@ -35,7 +36,9 @@ class GSpMMhip(VanillaSpMMhip):
     broadcast against each other the numpy way, e.g. 'u_mul_e' with (num_cols, H, D) and (nnz, H, 1), or
     'u_add_e' with (num_cols, F) and (nnz, F).  out[v] = reduce over row v's edges of the message; out
     has the broadcast feature shape.  (With 'u_mul_e', a second input of shape (nnz,) or (nnz, H) keeps
-    its meaning of one weight per edge, or per edge and head.)
+    its meaning of one weight per edge, or per edge and head.)  schedule_args {'num_src_partitions': 'auto' | int |
+    None} cuts the source columns into partitions as for the weighted sum (default 'auto': chosen from the size of the
+    operand that is gathered from the source nodes); operands on the edges and the reported positions stay in CSR order.
     """
     _compute_keys = ('num_feat_partitions', 'reduce', 'msg', 'return_arg')
 
@@ -111,8 +114,6 @@ class GSpMMhip(VanillaSpMMhip):
         op, lt, rt = general.parse_message(msg)
         if len(input_placeholders) != (1 if rt is None else 2):
             raise ValueError("message %r takes %d input(s), got %d" % (msg, 1 if rt is None else 2, len(input_placeholders)))
-        if self._num_col_partitions != 1:
-            raise ValueError("message %r needs num_col_partitions == 1" % (msg,))
         nnz = self._adj_indices.shape[0]
         lhs_ph = input_placeholders[0]
         rhs_ph = input_placeholders[1] if rt is not None else None
@@ -121,10 +122,13 @@ class GSpMMhip(VanillaSpMMhip):
         self._feat_len, self._heads, self._num_feat_partitions = self._bop.out_len, 1, 0
         self._reduce, self._msg, self._return_arg = reduce, msg, return_arg
         self._notes = [self._bop.describe()]
-        if compute_args.get('num_feat_partitions') or schedule_args:
-            self._notes.append("tiling and partitioning knobs do not apply to this message; ignored")
-        self._active = self._layout(1)
-        self._func = _lib.lib().fg_gspmm_bcast_f32
+        P = self._broadcast_partitions(schedule_args, return_arg)
+        if P > 1:
+            self._notes.append("%d source-column partitions, one buffer of results each, combined in partition order" % P)
+        if compute_args.get('num_feat_partitions') or any(k != 'num_src_partitions' for k in schedule_args):
+            self._notes.append("the feature axis of this message is not tiled; tiling knobs ignored")
+        self._active = self._glayout(P)
+        self._func = _lib.lib().fg_gspmm_bcast_dds_f32 if P > 1 else _lib.lib().fg_gspmm_bcast_f32
         common.reserve(self._active['plan'], common.OP_GSPMM_BCAST_ARG if return_arg else common.OP_GSPMM_BCAST,
                        1, self._bop.out_len, 0, self._ctx)
         self._row_scale = None
@@ -134,12 +138,31 @@ class GSpMMhip(VanillaSpMMhip):
         self.out_tvm = torch.zeros((self._num_rows,) + self._bop.out_shape, dtype=torch.float32, device=self._ctx)
         self.arg_tvm = torch.full(self.out_tvm.shape, -1, dtype=torch.int32, device=self._ctx) if return_arg else None
 
+    def _broadcast_partitions(self, schedule_args, return_arg):
+        """Source-column partitions of a broadcasting message: the constructor's count when it was given, else
+        schedule_args['num_src_partitions'] ('auto', the default: chosen for the operand gathered from the source
+        nodes, if there is one; None: the CSR arrays as they are)."""
+        if self._num_col_partitions != 1:
+            return self._num_col_partitions
+        want = schedule_args.get('num_src_partitions', 'auto')
+        if want is None:
+            return 1
+        if want != 'auto':
+            if int(want) < 1:
+                raise ValueError("num_src_partitions must be >= 1")
+            return int(want)
+        bop = self._bop
+        if bop.gathered_len() == 0:
+            return 1
+        return tuning.choose_gather_partitions(self._num_rows, self._num_cols, self._adj_indices.shape[0], bop.gathered_len(),
+                                               bop.out_len * (2 if return_arg else 1), self._graph_stats())
+
     def _launch_broadcast(self, inputs):
         lay = self._active
         lhs = inputs[0]
         rhs = inputs[1] if len(inputs) > 1 else None
         self._bop.run_spmm(lay['plan'], lay['pos'], lay['idx'], _REDUCE[self._reduce], lhs, rhs, self._row_scale,
-                           self.out_tvm, self.arg_tvm)
+                           self.out_tvm, self.arg_tvm, edge_pos_dev=(lay['edge_pos32'] if lay['P'] > 1 else None))
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         compute_args = dict(compute_args)
@@ -149,8 +172,14 @@ class GSpMMhip(VanillaSpMMhip):
             nnz = self._adj_indices.shape[0]
             bop = general.BroadcastOp(op, lt, rt, input_placeholders[0], input_placeholders[1] if rt is not None else None,
                                       self._num_rows, self._num_cols, nnz, self._ctx, allow_v=False)
+            self._bop, keep = bop, self._bop
+            try:
+                P = self._broadcast_partitions(common.take_args(schedule_args, self._schedule_keys, "schedule_func"),
+                                               bool(compute_args.get('return_arg', False)))
+            finally:
+                self._bop = keep
             buf = ctypes.create_string_buffer(4096)
-            _lib.check(_lib.lib().fg_spmm_plan_describe(self._layout(1)['plan'], 0, 0, buf, len(buf)))
+            _lib.check(_lib.lib().fg_spmm_plan_describe(self._layout(P)['plan'], 0, 0, buf, len(buf)))
             return buf.value.decode() + "  kernel           : gspmm_bcast_kernel, one wavefront per work item\n  note             : %s\n" % bop.describe()
         for k in ('reduce', 'msg', 'return_arg'):
             compute_args.pop(k, None)

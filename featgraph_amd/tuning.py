@@ -225,6 +225,28 @@ def choose_spmm(n_dst, n_src, nnz, feat_len, stats=None):
     return p, (t if t > 1 else 0)
 
 
+# The broadcasting kernel reads a row segment's index words and then gathers, segment after segment, where the
+# weighted-sum kernel stages a whole work item's indices first: a segment costs it ~0.45 ns of machine time more
+# (233k-node graph, u_add_e with one weight per edge: F=64 3.07 / 2.49 / 2.60 / 2.99 ms at 1 / 4 / 8 / 16 partitions
+# against 2.94 / 1.93 / 1.60 / 1.86 ms modelled for the weighted sum; F=128 6.80 / 5.21 / 4.76 / 5.16 against
+# 6.63 / 4.90 / 3.97 / 3.53).
+BCAST_COEF = dict(SPMM_COEF, seg=4.5e-10)
+
+
+def choose_gather_partitions(n_dst, n_src, nnz, gathered_len, out_len, stats=None):
+    """Source-column partitions for a generalised SpMM whose gathered operand has `gathered_len` floats per source
+    node and whose result has `out_len` per destination: the kernel does not tile the feature axis, so the model is
+    asked for the untiled traversal; every partition's results take a buffer of their own (8 GiB at most)."""
+    if nnz == 0 or n_dst == 0 or gathered_len < 1:
+        return 1
+    if stats is None:
+        stats = GraphStats(n_dst, n_src, nnz)
+    cands = [(p, 1) for p in (1, 2, 4, 8, 16, 32)
+             if p <= min(MAX_PARTITIONS, max(1, n_src)) and (p == 1 or 4.0 * p * n_dst * out_len <= float(8 << 30))]
+    predict = lambda st, f, p, t: predict_spmm(st, f, p, t, BCAST_COEF)
+    return _rank(stats, gathered_len, predict, cands, _spmm_tie)[0][0]
+
+
 def choose_sddmm(n_rows, n_cols, nnz, heads, head_len, stats=None):
     """(num_src_partitions, num_feat_tiles) for the tiled traversal, or None when the plain
     kernels should be used (small feature matrices, or a shape the tiled kernel does not take)."""

@@ -116,6 +116,32 @@ def test_broadcasting_entry_points(env):
     assert spmm(o=None) == FG_ERR_ARG
     assert spmm(op=COPY_LHS, rhs=None, rl=0) == FG_OK                 # the unused operand may be absent
 
+    # the same matrix in two source-column partitions (columns 0-2 and 3-4): fg_gspmm_bcast_dds_f32
+    s1_pos = np.array([0, 1, 1, 3, 4, 4, 5, 5, 6, 6], dtype=np.int32)
+    s1_idx = torch.tensor([0, 1, 2, 0, 0, 1], dtype=torch.int32, device="cuda")
+    edge_pos = torch.tensor([0, 2, 3, 5, 1, 4], dtype=torch.int32, device="cuda")
+    plan_dds = ctypes.c_void_p()
+    assert L.fg_spmm_plan_create(lib.host_ptr(s1_pos), 4, 5, 2, None, ctypes.byref(plan_dds)) == FG_OK
+    pos_dev = torch.from_numpy(s1_pos).cuda()
+    ramp = torch.arange(6, dtype=torch.float32, device="cuda")[:, None].expand(6, 8).contiguous()      # edge e holds e
+
+    def dds(pl=plan_dds, red=SUM, ep=edge_pos, a=None, op=COPY_LHS, pos=pos_dev, idx=s1_idx):
+        return L.fg_gspmm_bcast_dds_f32(pl, p(pos), p(idx), p(ep), op, red, p(ramp), E, 8, None, None, E, 0, None,
+                                        0, None, p(out), p(a), 8, None)
+
+    assert dds() == FG_OK
+    torch.cuda.synchronize()
+    assert out[:, 0].tolist() == [1.0, 0.0, 9.0, 5.0]                 # sums of the rows' CSR positions: 0+1, -, 2+3+4, 5
+    assert dds(red=MAX, a=arg) == FG_OK
+    torch.cuda.synchronize()
+    assert out[:, 3].tolist() == [1.0, 0.0, 4.0, 5.0] and arg[:, 3].tolist() == [1, -1, 4, 5]     # positions in CSR order
+    assert dds(ep=None) == FG_ERR_ARG                                 # several partitions need the stored positions
+    assert dds(pl=None) == FG_ERR_ARG
+    assert dds(pl=plan, ep=None, pos=t['indptr'], idx=t['indices']) == FG_OK      # one partition: the CSR arrays themselves
+    torch.cuda.synchronize()
+    assert out[:, 0].tolist() == [1.0, 0.0, 9.0, 5.0]
+    L.fg_spmm_plan_destroy(plan_dds)
+
     row = torch.tensor([0, 0, 2, 2, 2, 3], dtype=torch.int32, device="cuda")
     eo = torch.zeros((6, 8), device="cuda")
 

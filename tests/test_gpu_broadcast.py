@@ -35,14 +35,17 @@ def _operand(rng, rows, shape, positive=False):
     return (np.abs(x) + 0.5).astype("float32") if positive else x
 
 
-def _run_spmm(adj, msg, reduce, arrays, return_arg=False):
+def _run_spmm(adj, msg, reduce, arrays, return_arg=False, partitions=None):
+    """partitions: None = the CSR arrays as they are (these graphs are too small for the default to partition them);
+    an int = that many source-column partitions."""
     import torch
     from featgraph_amd.module import GSpMMhip, placeholder
     m = GSpMMhip(adj)
     args = {'reduce': reduce, 'msg': msg}
     if return_arg:
         args['return_arg'] = True
-    m.build([placeholder(a.shape) for a in arrays], args, {})
+    m.build([placeholder(a.shape) for a in arrays], args, {'num_src_partitions': partitions})
+    assert m._active['P'] == (partitions or 1)
     m.out_tvm.fill_(float("nan"))
     out = m.run([torch.from_numpy(a).cuda() for a in arrays]).cpu().numpy()
     return (out, m.arg_tvm.cpu().numpy()) if return_arg else out
@@ -109,6 +112,66 @@ def test_gspmm_broadcast_extreme_is_exact(oracle, msg, l_shape, r_shape, reduce)
     out2, arg = _run_spmm(adj, msg, reduce, arrays, return_arg=True)
     assert np.array_equal(out2, ref)
     assert np.array_equal(arg, ref_arg)
+
+
+@pytest.mark.parametrize("reduce", ["sum", "mean"])
+@pytest.mark.parametrize("msg,l_shape,r_shape", CASES)
+@pytest.mark.parametrize("partitions", [2, 5])
+def test_gspmm_broadcast_sum_over_source_partitions(oracle, msg, l_shape, r_shape, reduce, partitions):
+    """The same messages with the source columns cut into partitions (2: the hub row's segments are still split into
+    pieces; 5: most segments are empty): operands on the edges stay in CSR order."""
+    rng = np.random.default_rng(len(msg) + sum(l_shape) + partitions)
+    adj = _hub_graph(rng)
+    op, lt, rt, lhs, rhs = _arrays(rng, adj, msg, l_shape, r_shape)
+    arrays = [lhs] + ([rhs] if rhs is not None else [])
+    out = _run_spmm(adj, msg, reduce, arrays, partitions=partitions)
+    ref, _ = oracle.gspmm_bcast(adj.indptr, adj.indices, op, reduce, lhs, rhs, lt, rt or 'e')
+    mass, _ = oracle.gspmm_bcast(adj.indptr, adj.indices, 'add' if op == 'sub' else op, reduce,
+                                 np.abs(lhs), None if rhs is None else np.abs(rhs), lt, rt or 'e')
+    assert out.shape == ref.shape
+    assert_sum_close(out, ref, mass, "%s %s P=%d" % (msg, reduce, partitions))
+    assert (out[np.diff(adj.indptr) == 0] == 0).all()
+
+
+@pytest.mark.parametrize("reduce", ["max", "min"])
+@pytest.mark.parametrize("msg,l_shape,r_shape", CASES)
+@pytest.mark.parametrize("partitions", [2, 5])
+def test_gspmm_broadcast_extreme_over_source_partitions_is_exact(oracle, msg, l_shape, r_shape, reduce, partitions):
+    rng = np.random.default_rng(len(msg) * 3 + sum(l_shape) + partitions)
+    adj = _hub_graph(rng)
+    op, lt, rt, lhs, rhs = _arrays(rng, adj, msg, l_shape, r_shape)
+    arrays = [lhs] + ([rhs] if rhs is not None else [])
+    ref, ref_arg = oracle.gspmm_bcast(adj.indptr, adj.indices, op, reduce, lhs, rhs, lt, rt or 'e')
+    out = _run_spmm(adj, msg, reduce, arrays, partitions=partitions)
+    assert np.array_equal(out, ref), (msg, reduce)
+    out2, arg = _run_spmm(adj, msg, reduce, arrays, return_arg=True, partitions=partitions)
+    assert np.array_equal(out2, ref)
+    assert np.array_equal(arg, ref_arg)          # positions in the caller's CSR order
+    assert (out[np.diff(adj.indptr) == 0] == 0).all() and (arg[np.diff(adj.indptr) == 0] == -1).all()
+
+
+def test_source_partitions_with_unsorted_columns_and_ties(oracle):
+    """Rows whose columns are not stored in ascending order: a partition's elements are then not consecutive in the
+    CSR arrays, and the first stored one among equal candidates may lie in a later partition."""
+    rng = np.random.default_rng(21)
+    adj = _hub_graph(rng)
+    indices = adj.indices.copy()
+    perm = np.arange(adj.nnz)
+    for r in range(adj.shape[0]):
+        lo, hi = adj.indptr[r], adj.indptr[r + 1]
+        perm[lo:hi] = lo + rng.permutation(hi - lo)
+    shuffled = sp.csr_matrix((adj.data[perm], indices[perm], adj.indptr), shape=adj.shape)
+    assert not shuffled.has_sorted_indices
+    lhs = rng.integers(0, 3, size=(adj.shape[1], 8)).astype("float32")
+    rhs = rng.integers(0, 3, size=(adj.nnz, 1)).astype("float32")
+    for reduce in ("max", "min"):
+        out, arg = _run_spmm(shuffled, "u_add_e", reduce, [lhs, rhs], return_arg=True, partitions=4)
+        ref, ref_arg = oracle.gspmm_bcast(shuffled.indptr, shuffled.indices, "add", reduce, lhs, rhs, 'u', 'e')
+        assert np.array_equal(out, ref)
+        assert np.array_equal(arg, ref_arg)
+    out = _run_spmm(shuffled, "u_mul_e", "sum", [lhs, rhs], partitions=4)
+    ref, _ = oracle.gspmm_bcast(shuffled.indptr, shuffled.indices, "mul", "sum", lhs, rhs, 'u', 'e')
+    assert np.array_equal(out, ref)              # small integers: every sum is exact in any order
 
 
 def test_selected_position_with_ties(oracle):
@@ -182,9 +245,11 @@ def test_gspmm_broadcast_errors():
         m.build([placeholder((nnz, 4)), placeholder((nnz, 4))], {'msg': 'copy_e'}, {})
     with pytest.raises(ValueError):
         m.build([placeholder((n, 4)), placeholder((nnz, 4))], {'msg': 'u_add_e', 'reduce': 'sum', 'return_arg': True}, {})
-    m2 = GSpMMhip(adj, 2)
     with pytest.raises(ValueError):
-        m2.build([placeholder((n, 4)), placeholder((nnz, 4))], {'msg': 'u_add_e'}, {})
+        m.build([placeholder((n, 4)), placeholder((nnz, 4))], {'msg': 'u_add_e'}, {'num_src_partitions': 0})
+    m2 = GSpMMhip(adj, 2)               # the constructor's partitions are honoured
+    m2.build([placeholder((n, 4)), placeholder((nnz, 4))], {'msg': 'u_add_e'}, {})
+    assert m2._active['P'] == 2
     m.build([placeholder((n, 4)), placeholder((nnz, 4))], {'msg': 'u_add_e'}, {})
     assert "gspmm_bcast_kernel" in m.lower_to_ir([placeholder((n, 4)), placeholder((nnz, 4))], {'msg': 'u_add_e'}, {})
 

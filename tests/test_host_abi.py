@@ -208,6 +208,14 @@ def test_default_tilings():
     assert dict(zip(st.count_vals.tolist(), st.count_mult.tolist())) == {1.0: 1.0, 2.0: 2.0}
     # ranked candidates start with the choice
     assert tuning.rank_spmm(tuning.GraphStats(n, n, nnz), 512)[0] == (8, 8)
+    # source partitions of a broadcasting message: none without a gathered operand, for an operand that fits the caches
+    # or when every partition's buffer of results would not fit 8 GiB together; fewer than for the weighted sum
+    assert tuning.choose_gather_partitions(n, n, nnz, 0, 64) == 1
+    assert tuning.choose_gather_partitions(10000, 10000, 170000, 32, 32) == 1
+    assert tuning.choose_gather_partitions(n, n, nnz, 64, 64) in (2, 4, 8)
+    assert tuning.choose_gather_partitions(n, n, nnz, 64, 64) <= tuning.choose_spmm(n, n, nnz, 64)[0]
+    assert tuning.choose_gather_partitions(n, n, nnz, 64, 1 << 14) == 1
+    assert tuning.choose_gather_partitions(0, n, 0, 64, 64) == 1
 
 
 def test_partitioners_property_based(fg, oracle):
