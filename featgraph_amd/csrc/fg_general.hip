@@ -35,6 +35,7 @@
 using fg::fail;
 using fg::Fixup;
 using fg::Item;
+using fg::wave_lds_sync;
 
 // Every message is one correctly rounded float32 operation and every sum adds the rounded messages one by
 // one, so that max / min, the selected positions and (with one lane group per row) the sums in stored
@@ -46,6 +47,7 @@ namespace {
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = 64 * kWavesPerBlock;
+constexpr int kStage = 256;             // elements whose index words a wavefront keeps in LDS at a time
 
 struct GenArgs {
     const Item *items;
@@ -142,8 +144,20 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
     const bool l_on_e = a.lhs_target == FG_TARGET_E, r_on_e = a.rhs_target == FG_TARGET_E;
     constexpr int U = V == 4 ? 4 : 8;     // elements in flight per lane group: the loads of a step are issued before its sums
 
-    // the elements [e0, e1) of output row v: reduce and store to (dst_v, dst_a); `done`: the row is complete
-    auto reduce_range = [&](int64_t e0, int64_t e1, int v, float *dst_v, int32_t *dst_a, bool done) {
+    // The column and the stored position of up to kStage consecutive elements, read once with coalesced loads: the
+    // gathers of a step then wait for LDS, not for a load of their own index words.
+    __shared__ int2 s_el[kWavesPerBlock][kStage];
+    int2 *const el = s_el[wave];
+    auto stage = [&](int64_t c0, int n) {
+        for (int t = lane; t < n; t += 64)
+            el[t] = make_int2((int)(a.indices[c0 + t] + ubase), PART ? a.edge_pos[c0 + t] : (int)(c0 + t));
+        wave_lds_sync();
+    };
+
+    // the elements [e0, e1) of output row v: reduce and store to (dst_v, dst_a); `done`: the row is complete.
+    // staged_at >= 0: the range lies inside the elements staged from that position on; else it is staged here, kStage
+    // elements at a time (a lane group keeps its elements and their order: kStage is a multiple of the groups).
+    auto reduce_range = [&](int64_t e0, int64_t e1, int64_t staged_at, int v, float *dst_v, int32_t *dst_a, bool done) {
         for (int f0 = 0; f0 < FV; f0 += L) {
             const bool active = f0 + li < FV;
             const int fc = (active ? f0 + li : FV - 1) * V;       // the lane's first output feature
@@ -153,18 +167,26 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
             int at[V];
 #pragma unroll
             for (int i = 0; i < V; ++i) { acc[i] = identity<RED>(); at[i] = INT_MAX; }
-            for (int64_t eb = e0 + g; eb < e1; eb += (int64_t)G * U) {
+            for (int64_t c0 = e0; c0 < e1; c0 += kStage) {
+            const int64_t c1 = min(c0 + kStage, e1);
+            int64_t base = staged_at;
+            if (staged_at < 0) {
+                wave_lds_sync();          // the reads of what was staged before
+                stage(c0, (int)(c1 - c0));
+                base = c0;
+            }
+            const int t1 = (int)(c1 - base);       // positions in the staged window
+            for (int tb = (int)(c0 - base) + g; tb < t1; tb += G * U) {
                 float m[U][V];
                 bool ok[U];
                 int stored[U];          // the element's position in the caller's edge order
 #pragma unroll
                 for (int k = 0; k < U; ++k) {
-                    const int64_t e = eb + (int64_t)k * G;
-                    ok[k] = e < e1;
-                    const int64_t ec = ok[k] ? e : eb;
-                    const int64_t u = a.indices[ec] + ubase;  // read also when no operand lives on u: no branch
-                    stored[k] = PART ? a.edge_pos[ec] : (int)e;
-                    const int64_t ee = PART ? (int64_t)stored[k] : ec;
+                    const int t = tb + k * G;
+                    ok[k] = t < t1;
+                    const int2 w = el[ok[k] ? t : tb];
+                    const int64_t u = w.x, ee = w.y;
+                    stored[k] = w.y;
                     float l[V], r[V];
                     if (kLhs) load_operand<V, LC, LNT>(a.lhs + (l_on_e ? ee : u) * a.lhs_len + fl, l);
                     if (kRhs) load_operand<V, RC, RNT>(a.rhs + (r_on_e ? ee : u) * a.rhs_len + fr, r);
@@ -188,6 +210,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
                         }
                     }
                 }
+            }
             }
             for (int off = L; off < 64; off <<= 1) {
 #pragma unroll
@@ -223,14 +246,16 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
 
     if (it.info < 0) {
         const int nrows = -it.info;
+        const bool fits = it.len <= kStage;       // always, for an item of several rows
+        if (fits) stage(it.start, it.len);
         for (int q = 0; q < nrows; ++q) {
             const int v = it.row + q;
             const int64_t e0 = pos_p[v], e1 = pos_p[v + 1];
-            reduce_range(e0, e1, v, out_p + (int64_t)v * F, ARG ? arg_p + (int64_t)v * F : nullptr, !PART);
+            reduce_range(e0, e1, fits ? (int64_t)it.start : -1, v, out_p + (int64_t)v * F, ARG ? arg_p + (int64_t)v * F : nullptr, !PART);
         }
         return;
     }
-    reduce_range(it.start, (int64_t)it.start + it.len, it.row, partial_p + (int64_t)it.info * F,
+    reduce_range(it.start, (int64_t)it.start + it.len, -1, it.row, partial_p + (int64_t)it.info * F,
                  ARG ? partial_arg_p + (int64_t)it.info * F : nullptr, false);
 }
 

@@ -225,11 +225,12 @@ def choose_spmm(n_dst, n_src, nnz, feat_len, stats=None):
     return p, (t if t > 1 else 0)
 
 
-# The broadcasting kernel reads a row segment's index words and then gathers, segment after segment, where the
-# weighted-sum kernel stages a whole work item's indices first: a segment costs it ~0.45 ns of machine time more
-# (233k-node graph, u_add_e with one weight per edge: F=64 3.07 / 2.49 / 2.60 / 2.99 ms at 1 / 4 / 8 / 16 partitions
-# against 2.94 / 1.93 / 1.60 / 1.86 ms modelled for the weighted sum; F=128 6.80 / 5.21 / 4.76 / 5.16 against
-# 6.63 / 4.90 / 3.97 / 3.53).
+# The broadcasting kernel reduces one row segment after the other, all lane groups on the same segment, where the
+# weighted-sum kernel gives short segments a lane group each: a segment costs it a few tenths of a nanosecond of
+# machine time more.  With this coefficient the choice was the fastest or within 3 % of it on the 233k-node graph
+# (u_add_e with one weight per edge, ms at 1 / 2 / 4 / 8 / 16 partitions: F=32 1.30 / 1.20 / 1.22 / 1.38 / 1.98,
+# F=64 3.02 / - / 2.14 / 2.20 / 2.56, F=128 6.58 / 5.95 / 4.99 / 4.14 / 4.38, F=256 15.7 / 14.1 / 12.3 / 10.2 / 8.87;
+# u_mul_e with [nnz, F] edge features: F=64 6.87 / - / 6.19 / 6.66 / 7.23, F=128 14.4 / 13.7 / 12.7 / 13.1 / 14.1).
 BCAST_COEF = dict(SPMM_COEF, seg=4.5e-10)
 
 
