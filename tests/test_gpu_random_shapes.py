@@ -171,7 +171,8 @@ def _random_feature_shapes(rng):
 @pytest.mark.parametrize("seed", range(6))
 def test_random_broadcast_operators(oracle, monkeypatch, seed):
     """Generalised SpMM / SDDMM with broadcasting: random graphs, operators, targets and feature shapes (odd
-    seeds: rows split into pieces of 64 elements, so that split rows occur on these small graphs)."""
+    seeds: rows split into pieces of 64 elements, so that split rows occur on these small graphs; the SpMM over the
+    CSR arrays or over 2, 3 or 7 source-column partitions)."""
     import torch
     from featgraph_amd import _lib
     from featgraph_amd.module import GSpMMhip, GSDDMMhip, placeholder
@@ -198,7 +199,9 @@ def test_random_broadcast_operators(oracle, monkeypatch, seed):
         args = {'msg': "%s_%s_%s" % (lt, op, rt), 'reduce': reduce}
         if reduce in ("max", "min"):
             args['return_arg'] = True
-        m.build([placeholder(lhs.shape), placeholder(rhs.shape)], args, {})
+        parts = [None, 2, 3, 7][int(rng.integers(0, 4))]         # source-column partitions (None: the CSR arrays as they are)
+        what += " parts %s" % parts
+        m.build([placeholder(lhs.shape), placeholder(rhs.shape)], args, {'num_src_partitions': parts})
         m.out_tvm.fill_(float("nan"))
         out = m.run([torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda()]).cpu().numpy()
         ref, ref_arg = oracle.gspmm_bcast(adj.indptr, adj.indices, op, reduce, lhs, rhs, lt, rt)
