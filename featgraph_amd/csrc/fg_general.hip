@@ -28,6 +28,7 @@
 #include <hip/hip_runtime.h>
 
 #include <climits>
+#include <type_traits>
 
 #include "fg_common.h"
 #include "fg_device.h"
@@ -157,7 +158,14 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
     // the elements [e0, e1) of output row v: reduce and store to (dst_v, dst_a); `done`: the row is complete.
     // staged_at >= 0: the range lies inside the elements staged from that position on; else it is staged here, kStage
     // elements at a time (a lane group keeps its elements and their order: kStage is a multiple of the groups).
-    auto reduce_range = [&](int64_t e0, int64_t e1, int64_t staged_at, int v, float *dst_v, int32_t *dst_a, bool done) {
+    // own (a std::bool_constant): false = the wavefront's lane groups share the row, taking every G-th element each, and
+    // their results are combined; true = every lane group has a row of its own (e0, e1, v and the destinations differ
+    // from group to group, `mine` says whether the group has a row at all), walks it element by element in stored
+    // order and stores it itself -- for items of many short rows, whose elements are all staged.
+    auto reduce_range = [&](auto own, bool mine, int64_t e0, int64_t e1, int64_t staged_at, int v, float *dst_v, int32_t *dst_a,
+                            bool done) {
+        constexpr bool OWN = decltype(own)::value;
+        const int first = OWN ? 0 : g, step = OWN ? 1 : G;
         for (int f0 = 0; f0 < FV; f0 += L) {
             const bool active = f0 + li < FV;
             const int fc = (active ? f0 + li : FV - 1) * V;       // the lane's first output feature
@@ -170,19 +178,19 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
             for (int64_t c0 = e0; c0 < e1; c0 += kStage) {
             const int64_t c1 = min(c0 + kStage, e1);
             int64_t base = staged_at;
-            if (staged_at < 0) {
+            if (!OWN && staged_at < 0) {
                 wave_lds_sync();          // the reads of what was staged before
                 stage(c0, (int)(c1 - c0));
                 base = c0;
             }
             const int t1 = (int)(c1 - base);       // positions in the staged window
-            for (int tb = (int)(c0 - base) + g; tb < t1; tb += G * U) {
+            for (int tb = (int)(c0 - base) + first; tb < t1; tb += step * U) {
                 float m[U][V];
                 bool ok[U];
                 int stored[U];          // the element's position in the caller's edge order
 #pragma unroll
                 for (int k = 0; k < U; ++k) {
-                    const int t = tb + k * G;
+                    const int t = tb + k * step;
                     ok[k] = t < t1;
                     const int2 w = el[ok[k] ? t : tb];
                     const int64_t u = w.x, ee = w.y;
@@ -212,7 +220,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
                 }
             }
             }
-            for (int off = L; off < 64; off <<= 1) {
+            for (int off = L; !OWN && off < 64; off <<= 1) {
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
                     const float o = __shfl_xor(acc[i], off);
@@ -223,7 +231,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
                     } else acc[i] = RED == FG_REDUCE_MAX ? fmaxf(acc[i], o) : fminf(acc[i], o);
                 }
             }
-            if (g == 0 && active) {
+            if ((OWN ? mine : g == 0) && active) {
                 const bool empty = e1 <= e0;
                 const float scale = (done && a.row_scale) ? a.row_scale[v] : 1.f;
 #pragma unroll
@@ -248,14 +256,26 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
         const int nrows = -it.info;
         const bool fits = it.len <= kStage;       // always, for an item of several rows
         if (fits) stage(it.start, it.len);
+        if (fits && nrows >= 2 * G) {
+            // many short rows: a lane group per row, G rows at a time
+            for (int q0 = 0; q0 < nrows; q0 += G) {
+                const bool mine = q0 + g < nrows;
+                const int v = it.row + min(q0 + g, nrows - 1);
+                const int64_t e0 = pos_p[v], e1 = mine ? pos_p[v + 1] : e0;
+                reduce_range(std::true_type{}, mine, e0, e1, it.start, v, out_p + (int64_t)v * F,
+                             ARG ? arg_p + (int64_t)v * F : nullptr, !PART);
+            }
+            return;
+        }
         for (int q = 0; q < nrows; ++q) {
             const int v = it.row + q;
             const int64_t e0 = pos_p[v], e1 = pos_p[v + 1];
-            reduce_range(e0, e1, fits ? (int64_t)it.start : -1, v, out_p + (int64_t)v * F, ARG ? arg_p + (int64_t)v * F : nullptr, !PART);
+            reduce_range(std::false_type{}, true, e0, e1, fits ? (int64_t)it.start : -1, v, out_p + (int64_t)v * F,
+                         ARG ? arg_p + (int64_t)v * F : nullptr, !PART);
         }
         return;
     }
-    reduce_range(it.start, (int64_t)it.start + it.len, -1, it.row, partial_p + (int64_t)it.info * F,
+    reduce_range(std::false_type{}, true, it.start, (int64_t)it.start + it.len, -1, it.row, partial_p + (int64_t)it.info * F,
                  ARG ? partial_arg_p + (int64_t)it.info * F : nullptr, false);
 }
 
