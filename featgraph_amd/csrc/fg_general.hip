@@ -15,10 +15,12 @@
 // The SpMM kernel walks the plan's work items, one wavefront each, like the weighted-sum kernel.  A lane holds
 // V output features (V = 4 with 128-bit accesses when the shapes allow it, else 1); a group of L lanes
 // (L = the power of two that covers the F / V vectors, at most 64) takes one element at a time and the
-// 64 / L groups take different elements of the row, several steps in flight; longer feature axes are walked
-// 64 vectors at a time.  With one group (64 vectors or more) a row's sum is formed in the stored element
-// order.  The edge operand, when there is one, is the dominant stream ([nnz, len] floats read once,
-// coalesced); the node operand is gathered.
+// 64 / L groups take different elements of the row, several steps in flight (in an item of many short rows
+// every group takes a row of its own instead); longer feature axes are walked 64 vectors at a time.  With one
+// group (64 vectors or more), and for rows that a group has to itself, a row's sum is formed in the stored
+// element order.  The edge operand, when there is one, is the dominant stream ([nnz, len] floats read once,
+// coalesced, past the caches); the node operand is gathered, through column words that the wavefront has staged
+// in LDS for the whole item.
 //
 // Over a plan with several source-column partitions (fg_gspmm_bcast_dds_f32) one launch walks all partitions'
 // items in partition order, so that the gathered operand's rows of the current partition stay in the L2s: a
