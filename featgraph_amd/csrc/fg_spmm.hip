@@ -1294,6 +1294,37 @@ __global__ __launch_bounds__(256) void edge_values_head_major_kernel(const float
     const float *s = src + (pos ? (int64_t)pos[e] : e) * H;
     for (int h = 0; h < H; ++h) dst[(int64_t)h * n + e] = s[h];
 }
+// The same for H = 4 * Q heads and a 16-byte aligned src: an element's heads by Q 128-bit loads, two elements per lane
+// (a block apart, so that every store of a wavefront still covers 64 consecutive elements of one head).
+template <int Q>
+__global__ __launch_bounds__(256) void edge_values_head_major_vec_kernel(const float *src, const int32_t *pos,
+                                                                         int64_t n, float *dst) {
+    constexpr int H = 4 * Q;
+    const int64_t e0 = (int64_t)blockIdx.x * 512 + threadIdx.x;
+    float4 v[2][Q];
+    bool ok[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int64_t e = e0 + 256 * j;
+        ok[j] = e < n;
+        const int64_t ec = ok[j] ? e : n - 1;                  // clamped: no branch around the loads
+        const float4 *s = reinterpret_cast<const float4 *>(src + (pos ? (int64_t)pos[ec] : ec) * H);
+#pragma unroll
+        for (int q = 0; q < Q; ++q) v[j][q] = s[q];
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        if (!ok[j]) continue;
+        float *d = dst + e0 + 256 * j;
+#pragma unroll
+        for (int q = 0; q < Q; ++q) {
+            d[(int64_t)(4 * q + 0) * n] = v[j][q].x;
+            d[(int64_t)(4 * q + 1) * n] = v[j][q].y;
+            d[(int64_t)(4 * q + 2) * n] = v[j][q].z;
+            d[(int64_t)(4 * q + 3) * n] = v[j][q].w;
+        }
+    }
+}
 }  // namespace
 
 extern "C" int fg_edge_values_head_major_f32(const float *src_dev, const int32_t *edge_pos_dev, int64_t n_edges,
@@ -1303,8 +1334,18 @@ extern "C" int fg_edge_values_head_major_f32(const float *src_dev, const int32_t
     if (!src_dev || !dst_dev) return fail(FG_ERR_ARG, "null device pointer");
     const int64_t blocks = (n_edges + 255) / 256;
     if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "too many edges for one grid");
-    hipLaunchKernelGGL(edge_values_head_major_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       src_dev, edge_pos_dev, n_edges, heads, dst_dev);
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 wide((unsigned)((n_edges + 511) / 512));
+    const bool aligned = ((uintptr_t)src_dev & 15) == 0;
+    if (aligned && heads == 4)
+        hipLaunchKernelGGL(edge_values_head_major_vec_kernel<1>, wide, dim3(256), 0, st, src_dev, edge_pos_dev, n_edges, dst_dev);
+    else if (aligned && heads == 8)
+        hipLaunchKernelGGL(edge_values_head_major_vec_kernel<2>, wide, dim3(256), 0, st, src_dev, edge_pos_dev, n_edges, dst_dev);
+    else if (aligned && heads == 16)
+        hipLaunchKernelGGL(edge_values_head_major_vec_kernel<4>, wide, dim3(256), 0, st, src_dev, edge_pos_dev, n_edges, dst_dev);
+    else
+        hipLaunchKernelGGL(edge_values_head_major_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
+                           src_dev, edge_pos_dev, n_edges, heads, dst_dev);
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;
 }

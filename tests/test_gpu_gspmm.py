@@ -175,3 +175,20 @@ def test_selected_elements(torch_cuda, oracle, reduce, feat_len):
         assert (arg[np.diff(adj.indptr) == 0] == -1).all()
     with pytest.raises(ValueError):
         GSpMMhip(adj).build([placeholder(x.shape)], {'reduce': 'sum', 'return_arg': True}, {})
+
+
+@pytest.mark.parametrize("heads", [1, 3, 4, 8, 16])
+@pytest.mark.parametrize("n", [1, 511, 513, 70001])
+def test_edge_values_head_major(torch_cuda, heads, n):
+    """dst[h, e] = src[pos[e], h]: the relayout of per-head edge weights, through the C ABI; heads of 4, 8 and 16 take
+    the kernel with 128-bit loads, the others (and a misaligned source) the scalar one."""
+    from featgraph_amd import _lib
+    torch = torch_cuda
+    g = torch.Generator(device="cuda").manual_seed(n * 31 + heads)
+    src = torch.randn((n + 1, heads), device="cuda", generator=g)
+    pos = torch.randperm(n, device="cuda", generator=g).to(torch.int32)
+    for s, p in ((src[:n], None), (src[:n], pos), (src.reshape(-1)[1:1 + n * heads].reshape(n, heads), pos)):
+        dst = torch.full((heads, n), float("nan"), device="cuda")
+        _lib.check(_lib.lib().fg_edge_values_head_major_f32(_lib.dev_ptr(s), _lib.dev_ptr(p), n, heads, _lib.dev_ptr(dst), None))
+        want = (s if p is None else s[p.long()]).t()
+        assert torch.equal(dst, want)
