@@ -403,6 +403,44 @@ __global__ __launch_bounds__(256) void edge_softmax_head_major_kernel(const floa
     for (int h = 0; h < H; ++h) dst[(int64_t)h * n + e] = __expf(xs[h] - st[h].x) / st[h].y;
 }
 
+// The same for H = 4 * Q heads and 16-byte aligned arrays: an element's scores by Q 128-bit loads and its row's
+// statistics by 2 Q, two elements per lane (a block apart: every store of a wavefront covers 64 consecutive elements
+// of one head); exp and division as in the kernel above, so both give the same bits.
+template <int Q>
+__global__ __launch_bounds__(256) void edge_softmax_head_major_vec_kernel(const float *x, const float2 *row_stats,
+                                                                          const int32_t *edge_row, const int32_t *pos,
+                                                                          int64_t n, float *dst) {
+    constexpr int H = 4 * Q;
+    const int64_t e0 = (int64_t)blockIdx.x * 512 + threadIdx.x;
+    float4 xs[2][Q], st[2][2 * Q];
+    bool ok[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int64_t e = e0 + 256 * j;
+        ok[j] = e < n;
+        const int64_t ec = ok[j] ? e : n - 1;                   // clamped: no branch around the loads
+        const int64_t at = pos ? (int64_t)pos[ec] : ec;
+        const float4 *xp = reinterpret_cast<const float4 *>(x + at * H);
+        const float4 *sp = reinterpret_cast<const float4 *>(row_stats + (int64_t)edge_row[at] * H);
+#pragma unroll
+        for (int q = 0; q < Q; ++q) xs[j][q] = xp[q];
+#pragma unroll
+        for (int q = 0; q < 2 * Q; ++q) st[j][q] = sp[q];       // (max, sum) of heads 2q and 2q + 1
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        if (!ok[j]) continue;
+        float *d = dst + e0 + 256 * j;
+#pragma unroll
+        for (int q = 0; q < Q; ++q) {
+            d[(int64_t)(4 * q + 0) * n] = __expf(xs[j][q].x - st[j][2 * q].x) / st[j][2 * q].y;
+            d[(int64_t)(4 * q + 1) * n] = __expf(xs[j][q].y - st[j][2 * q].z) / st[j][2 * q].w;
+            d[(int64_t)(4 * q + 2) * n] = __expf(xs[j][q].z - st[j][2 * q + 1].x) / st[j][2 * q + 1].y;
+            d[(int64_t)(4 * q + 3) * n] = __expf(xs[j][q].w - st[j][2 * q + 1].z) / st[j][2 * q + 1].w;
+        }
+    }
+}
+
 template <bool BWD, bool LANEHEAD>
 void launch_both(const fg_spmm_plan *pl, const SoftmaxArgs &a, hipStream_t st) {
     const dim3 grid((unsigned)((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock));
@@ -497,9 +535,19 @@ extern "C" int fg_edge_softmax_head_major_f32(const float *scores_dev, const flo
     if (!scores_dev || !row_stats_dev || !edge_row_dev || !dst_dev) return fail(FG_ERR_ARG, "null device pointer");
     const int64_t blocks = (n_edges + 255) / 256;
     if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "too many edges for one grid");
-    hipLaunchKernelGGL(edge_softmax_head_major_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       scores_dev, reinterpret_cast<const float2 *>(row_stats_dev), edge_row_dev, edge_pos_dev, n_edges,
-                       heads, dst_dev);
+    hipStream_t st = (hipStream_t)stream;
+    const float2 *stats = reinterpret_cast<const float2 *>(row_stats_dev);
+    const dim3 wide((unsigned)((n_edges + 511) / 512));
+    const bool aligned = (((uintptr_t)scores_dev | (uintptr_t)row_stats_dev) & 15) == 0;
+    if (aligned && heads == 4)
+        hipLaunchKernelGGL(edge_softmax_head_major_vec_kernel<1>, wide, dim3(256), 0, st, scores_dev, stats, edge_row_dev,
+                           edge_pos_dev, n_edges, dst_dev);
+    else if (aligned && heads == 8)
+        hipLaunchKernelGGL(edge_softmax_head_major_vec_kernel<2>, wide, dim3(256), 0, st, scores_dev, stats, edge_row_dev,
+                           edge_pos_dev, n_edges, dst_dev);
+    else
+        hipLaunchKernelGGL(edge_softmax_head_major_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
+                           scores_dev, stats, edge_row_dev, edge_pos_dev, n_edges, heads, dst_dev);
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;
 }
