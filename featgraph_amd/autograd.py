@@ -181,13 +181,9 @@ class Graph(object):
             raise ValueError("differentiable here: add, sub, mul, div between operands on two different targets of u / v / e")
         return _GSDDMM.apply(self, op, lhs_target, rhs_target, lhs, rhs)
 
-    def _tr_pos(self, device):
-        if getattr(self, "_tr_pos_dev", None) is None or self._tr_pos_dev.device != device:
-            self._tr_pos_dev = torch.from_numpy(self._tr_pos_host).to(device)
-        return self._tr_pos_dev
-
     def _bcast_spmm_raw(self, msg, arrays, reduce="sum", transposed=False, return_arg=False):
-        """Generalised SpMM over the adjacency or its transpose (edge operands then in the transpose's edge order);
+        """Generalised SpMM over the adjacency or its transpose; edge operands in this graph's CSR edge order either
+        way (over the transpose the kernel addresses them through the transposed edges' CSR positions);
         return_arg (max / min): also the CSR position of the selected edge per output, as a tensor of the caller's own."""
         arrays = [a.contiguous() for a in arrays]
         key = ('gspmm', msg, reduce, transposed, return_arg) + tuple(tuple(a.shape) for a in arrays)
@@ -197,10 +193,13 @@ class Graph(object):
             if return_arg:
                 args['return_arg'] = True
             m.build([placeholder(tuple(a.shape)) for a in arrays], args, {})
+            if transposed:
+                m.set_weight_order(self._tr_pos_host)
             self._mods[key] = m
         mod = self._mods[key]
         if return_arg:
-            mod.arg_tvm = torch.empty_like(mod.arg_tvm)
+            mod.arg_tvm = torch.empty(mod._fresh_like[0] if getattr(mod, '_fresh_like', None) else mod.out_tvm.shape,
+                                      dtype=torch.int32, device=mod._ctx)
             return _fresh_run(mod, arrays), mod.arg_tvm
         return _fresh_run(mod, arrays)
 
@@ -230,7 +229,7 @@ class Graph(object):
             return m
         if target == "v":
             return self._bcast_spmm_raw('copy_e', [m])
-        return self._bcast_spmm_raw('copy_e', [m.index_select(0, self._tr_pos(m.device))], transposed=True)
+        return self._bcast_spmm_raw('copy_e', [m], transposed=True)
 
     def _edge_product_sum(self, m, q, tq, target, op="mul"):
         """For every node of `target` ('v' or 'u'): the sum over its edges of m[e] * q(e) (op='div': m[e] / q(e)), m per
@@ -239,12 +238,11 @@ class Graph(object):
             if tq == "v":
                 raise ValueError("both operands on the same target")
             return self._bcast_spmm_raw('e_%s_%s' % (op, tq), [m, q])
-        tp = self._tr_pos(m.device)     # rows of the transpose: its 'u' are this graph's 'v'
-        if tq == "u":
+        if tq == "u":                   # rows of the transpose: its 'u' are this graph's 'v'
             raise ValueError("both operands on the same target")
         if tq == "v":
-            return self._bcast_spmm_raw('e_%s_u' % op, [m.index_select(0, tp), q], transposed=True)
-        return self._bcast_spmm_raw('e_%s_e' % op, [m.index_select(0, tp), q.index_select(0, tp)], transposed=True)
+            return self._bcast_spmm_raw('e_%s_u' % op, [m, q], transposed=True)
+        return self._bcast_spmm_raw('e_%s_e' % op, [m, q], transposed=True)
 
     def edge_softmax(self, scores):
         """Softmax of scores, (nnz,) or (nnz, H), over the edges of each destination row, per head."""
@@ -253,9 +251,15 @@ class Graph(object):
 
 def _fresh_run(mod, inputs):
     """run() into a tensor of the caller's own: the module's output buffer (every element of which a run
-    overwrites) is replaced first, so nothing has to be copied out of it."""
-    mod.out_tvm = torch.empty_like(mod.out_tvm)
-    return mod.run(inputs)
+    overwrites) is replaced first, so nothing has to be copied out of it, and the module lets go of it
+    afterwards -- autograd takes a gradient it alone refers to as it is, and clones one that is shared."""
+    like = getattr(mod, '_fresh_like', None)
+    if like is None:
+        like = mod._fresh_like = (tuple(mod.out_tvm.shape), mod.out_tvm.dtype, mod.out_tvm.device)
+    mod.out_tvm = torch.empty(like[0], dtype=like[1], device=like[2])
+    out = mod.run(inputs)
+    mod.out_tvm = None
+    return out
 
 
 class _SpMM(torch.autograd.Function):
@@ -339,7 +343,9 @@ class _EdgeSoftmax(torch.autograd.Function):
         (a,) = ctx.saved_tensors
         mod = ctx.g._softmax_mod(tuple(a.shape))
         mod.grad_tvm = torch.empty_like(a)          # handed to the caller; the module takes a new one next time
-        return None, mod.backward(a, da.contiguous())
+        grad = mod.backward(a, da.contiguous())
+        mod.grad_tvm = None
+        return None, grad
 
 
 def _reduce_to(full, shape):
@@ -386,7 +392,7 @@ class _GSpMM(torch.autograd.Function):
                 q, tq = arrays[1 - i], targets[1 - i]
                 inner = "div" if (op == "div" and i == 0) else "mul"
                 if tp == "u":       # sum over the edges that leave u of dout[row e] (* or /) q[e]
-                    full = g._bcast_spmm_raw('u_%s_e' % inner, [dout, q.index_select(0, g._tr_pos(q.device))], transposed=True)
+                    full = g._bcast_spmm_raw('u_%s_e' % inner, [dout, q], transposed=True)
                 else:               # per edge: dout[row e] (* or /) q[col e]
                     full = g._bcast_sddmm_raw(inner, 'v', tq, [dout, q])
                 if op == "div" and i == 1:

@@ -68,12 +68,15 @@ struct GenArgs {
     float *partial;              // pieces of split rows: [slot][F] values
     int32_t *partial_arg;        //                       [slot][F] positions
     int F, L;
-    // Several source-column partitions (PART): indptr / indices are the partitioned layout's position and local
-    // column arrays, item_off the plan's item ranges per partition, edge_pos the stored position of every element;
-    // out / arg are the partitions' buffers.  Strides in elements, per partition.
+    // PART: the elements are not addressed by their own positions -- several source-column partitions (indptr /
+    // indices are the partitioned layout's position and local column arrays, item_off the plan's item ranges per
+    // partition, out / arg the partitions' buffers; strides in elements, per partition), or edge operands that the
+    // caller keeps in another order: edge_pos gives every element's row in the edge operands (and the position that
+    // is reported for it).
     const int64_t *item_off;
     const int32_t *edge_pos;
     int n_parts;
+    int final;                   // the kernel's rows are results (one partition), not a partition's share of them
     int64_t pos_stride, col_width, out_stride, partial_stride;
 };
 
@@ -116,8 +119,8 @@ template <int RED> __device__ __forceinline__ bool replaces(float m, int em, flo
 // LC / RC (V == 4 only): the operand's 4 features are consecutive (one 128-bit load), else one value 4 times.
 // No branch stands between the loads of a step: one around a load would make the wavefront wait for everything
 // issued before it.
-// PART: the items of several source-column partitions (see GenArgs); a row segment without elements then keeps the
-// reduction's identity and no row is scaled, both being the combining kernel's business.
+// PART: see GenArgs; with several partitions (a.final == 0) a row segment without elements keeps the reduction's
+// identity and no row is scaled, both being the combining kernel's business.
 // LNT / RNT: see load_operand.  RED: FG_REDUCE_SUM or FG_REDUCE_MAX; a minimum runs as the maximum of the negated
 // messages (a.sign = -1; negation is exact, so values, ties and selected positions are those of the minimum).
 template <int OP, int RED, bool ARG, int V, bool LC, bool RC, bool LNT, bool RNT, bool PART>
@@ -125,6 +128,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
     static_assert(RED == FG_REDUCE_SUM || RED == FG_REDUCE_MAX, "a minimum is a maximum with a.sign = -1");
     constexpr bool kLhs = kUsesLhs<OP>, kRhs = kUsesRhs<OP>;
     const float sign = RED == FG_REDUCE_SUM ? 1.f : a.sign;
+    const bool final = !PART || a.final != 0;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int64_t item_id = (int64_t)blockIdx.x * kWavesPerBlock + wave;
@@ -239,7 +243,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
                     if (RED != FG_REDUCE_SUM) acc[i] *= sign;
-                    acc[i] = (RED != FG_REDUCE_SUM && empty && !PART) ? 0.f : acc[i];
+                    acc[i] = (RED != FG_REDUCE_SUM && empty && final) ? 0.f : acc[i];
                     if (done && a.row_scale) acc[i] *= scale;
                     if (ARG) at[i] = (at[i] == INT_MAX) ? -1 : at[i];
                 }
@@ -265,7 +269,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
                 const int v = it.row + min(q0 + g, nrows - 1);
                 const int64_t e0 = pos_p[v], e1 = mine ? pos_p[v + 1] : e0;
                 reduce_range(std::true_type{}, mine, e0, e1, it.start, v, out_p + (int64_t)v * F,
-                             ARG ? arg_p + (int64_t)v * F : nullptr, !PART);
+                             ARG ? arg_p + (int64_t)v * F : nullptr, final);
             }
             return;
         }
@@ -273,7 +277,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
             const int v = it.row + q;
             const int64_t e0 = pos_p[v], e1 = pos_p[v + 1];
             reduce_range(std::false_type{}, true, e0, e1, fits ? (int64_t)it.start : -1, v, out_p + (int64_t)v * F,
-                         ARG ? arg_p + (int64_t)v * F : nullptr, !PART);
+                         ARG ? arg_p + (int64_t)v * F : nullptr, final);
         }
         return;
     }
@@ -374,7 +378,7 @@ void launch_spmm_variant(int vec, bool lnt, bool rnt, dim3 grid, hipStream_t st,
 }
 template <int OP, int RED, bool ARG>
 void launch_spmm_ora(int vec, bool lnt, bool rnt, dim3 grid, hipStream_t st, const GenArgs &a) {
-    if (a.n_parts > 1) launch_spmm_variant<OP, RED, ARG, true>(vec, lnt, rnt, grid, st, a);
+    if (a.n_parts > 1 || a.edge_pos) launch_spmm_variant<OP, RED, ARG, true>(vec, lnt, rnt, grid, st, a);
     else launch_spmm_variant<OP, RED, ARG, false>(vec, lnt, rnt, grid, st, a);
 }
 template <int OP>
@@ -536,7 +540,7 @@ int gspmm_bcast_scratch_need(const fg_spmm_plan *pl, int F, bool with_arg, Scrat
 namespace {
 
 // pos / idx: indptr / indices of the CSR arrays with one partition, else the partitioned layout's position and local
-// column arrays, with edge_pos the stored position of each of its elements.
+// column arrays; edge_pos (required with several partitions): the row of each element in the edge operands.
 int gspmm_bcast_run(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev, const int32_t *edge_pos_dev, int op,
                     int reduce, const float *lhs_dev, int lhs_target, int lhs_len, const int32_t *lhs_off_dev,
                     const float *rhs_dev, int rhs_target, int rhs_len, const int32_t *rhs_off_dev, int flags,
@@ -577,7 +581,7 @@ int gspmm_bcast_run(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx
     a.arg = P > 1 ? (arg_dev ? abuf : nullptr) : arg_dev;
     a.partial = values; a.partial_arg = positions;
     a.F = out_len; a.L = lanes_for(out_len / V);
-    a.item_off = pl->item_off_dev; a.edge_pos = edge_pos_dev; a.n_parts = P;
+    a.item_off = pl->item_off_dev; a.edge_pos = edge_pos_dev; a.n_parts = P; a.final = P == 1;
     a.pos_stride = pl->n_dst + 1; a.col_width = (pl->n_src + P - 1) / P;
     a.out_stride = (int64_t)b.buffers; a.partial_stride = (int64_t)b.pieces;
     const int64_t blocks = (pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock;

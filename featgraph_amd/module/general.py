@@ -112,7 +112,8 @@ class BroadcastOp(object):
         return max(self.lhs_len if self.lhs_target == 'u' else 0, self.rhs_len if self.rhs_target == 'u' else 0)
 
     def run_spmm(self, plan, pos_dev, idx_dev, reduce, lhs, rhs, row_scale, out, arg, edge_pos_dev=None):
-        """pos_dev / idx_dev: indptr / indices, or (edge_pos_dev given) the arrays of a source-partitioned layout."""
+        """pos_dev / idx_dev: indptr / indices, or the arrays of a source-partitioned layout; edge_pos_dev: where each
+        of their elements lies in the edge operands (required with partitions; None: at its own position)."""
         operands = (BINARY[self.op], reduce,
                     _lib.dev_ptr(lhs), TARGET[self.lhs_target or 'u'], self.lhs_len, _lib.dev_ptr(self.lhs_off),
                     _lib.dev_ptr(rhs), TARGET[self.rhs_target or 'e'], self.rhs_len, _lib.dev_ptr(self.rhs_off), self.flags,

@@ -161,8 +161,9 @@ class GSpMMhip(VanillaSpMMhip):
         lay = self._active
         lhs = inputs[0]
         rhs = inputs[1] if len(inputs) > 1 else None
+        # where each element of the layout lies in the edge operands (None: at its own position)
         self._bop.run_spmm(lay['plan'], lay['pos'], lay['idx'], _REDUCE[self._reduce], lhs, rhs, self._row_scale,
-                           self.out_tvm, self.arg_tvm, edge_pos_dev=(lay['edge_pos32'] if lay['P'] > 1 else None))
+                           self.out_tvm, self.arg_tvm, edge_pos_dev=self._given_pos(lay))
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         compute_args = dict(compute_args)
@@ -227,9 +228,11 @@ class GSpMMhip(VanillaSpMMhip):
         return self._weights_in_layout(w, lay, given=True)
 
     def set_weight_order(self, position_of_edge):
-        """Weights given to run() are stored in another edge order: position_of_edge[i] is where the
-        weight of this adjacency's i-th edge (CSR order) lies in the given array (int array of nnz entries,
-        or None for CSR order).  The library's relayout kernel follows it; no separate permutation pass."""
+        """Weights and edge operands given to run() are stored in another edge order: position_of_edge[i] is
+        where the weight (or operand row) of this adjacency's i-th edge (CSR order) lies in the given array (int
+        array of nnz entries, or None for CSR order).  The library's relayout kernel, or the broadcasting kernel's
+        own addressing, follows it: no separate permutation pass.  Positions reported by 'return_arg' then refer
+        to the given order too (broadcasting messages)."""
         if position_of_edge is None:
             self._weight_perm = None
         else:
