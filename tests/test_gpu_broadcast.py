@@ -174,6 +174,45 @@ def test_source_partitions_with_unsorted_columns_and_ties(oracle):
     assert np.array_equal(out, ref)              # small integers: every sum is exact in any order
 
 
+@pytest.mark.parametrize("partitions", [None, 3])
+def test_edge_operands_in_another_order(oracle, partitions):
+    """set_weight_order: the edge operands given to run() lie in another edge order (as those of the transposed graph's
+    calls do); the kernel follows the positions, and the positions it reports refer to the given order."""
+    import torch
+    from featgraph_amd.module import GSpMMhip, placeholder
+    rng = np.random.default_rng(31)
+    adj = _hub_graph(rng)
+    nnz = adj.nnz
+    where = rng.permutation(nnz)                           # edge i of the adjacency lies at where[i] in the given arrays
+    x = _operand(rng, adj.shape[1], (8, 4))
+    ef_csr = _operand(rng, nnz, (8, 1))
+    given = np.empty_like(ef_csr); given[where] = ef_csr
+    for reduce in ("sum", "max"):
+        m = GSpMMhip(adj)
+        args = {'msg': 'u_mul_e', 'reduce': reduce}
+        if reduce == "max":
+            args['return_arg'] = True
+        m.build([placeholder(x.shape), placeholder(given.shape)], args, {'num_src_partitions': partitions})
+        m.set_weight_order(where)
+        out = m.run([torch.from_numpy(x).cuda(), torch.from_numpy(given).cuda()]).cpu().numpy()
+        ref, ref_arg = oracle.gspmm_bcast(adj.indptr, adj.indices, 'mul', reduce, x, ef_csr, 'u', 'e')
+        if reduce == "sum":
+            mass, _ = oracle.gspmm_bcast(adj.indptr, adj.indices, 'mul', reduce, np.abs(x), np.abs(ef_csr), 'u', 'e')
+            assert_sum_close(out, ref, mass, "given order, sum")
+        else:
+            assert np.array_equal(out, ref)
+            arg = m.arg_tvm.cpu().numpy()
+            # the same values are selected; among equal candidates the one that comes first in the given order
+            picked = np.where(arg >= 0, np.argsort(where)[np.maximum(arg, 0)], -1)
+            rows = np.repeat(np.arange(adj.shape[0]), np.diff(adj.indptr))
+            assert ((arg >= 0) == (ref_arg >= 0)).all()
+            ok = arg >= 0
+            assert (rows[picked[ok]] == np.nonzero(ok)[0]).all()          # an edge of the output's own row
+            msgs = x[adj.indices[picked[ok]]] * ef_csr[picked[ok]]
+            f = np.nonzero(ok)[1:]
+            assert np.array_equal(msgs.reshape(msgs.shape[0], -1)[np.arange(msgs.shape[0]), np.ravel_multi_index(f, (8, 4))], out[ok])
+
+
 def test_selected_position_with_ties(oracle):
     """Integer-valued messages: many equal candidates per row, the first stored one is reported (also across
     the lane groups that share a row and across the pieces of the split row)."""
