@@ -1294,6 +1294,18 @@ __global__ __launch_bounds__(256) void edge_values_head_major_kernel(const float
     const float *s = src + (pos ? (int64_t)pos[e] : e) * H;
     for (int h = 0; h < H; ++h) dst[(int64_t)h * n + e] = s[h];
 }
+// One head, weights in another order: dst[e] = src[pos[e]], four consecutive elements per lane (their positions by one
+// 128-bit load, the results by one 128-bit store; pos and dst 16-byte aligned).
+__global__ __launch_bounds__(256) void edge_values_permute_kernel(const float *src, const int32_t *pos, int64_t n, float *dst) {
+    const int64_t e = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (e >= n) return;
+    if (e + 4 <= n) {
+        const int4 p = *reinterpret_cast<const int4 *>(pos + e);
+        *reinterpret_cast<float4 *>(dst + e) = make_float4(src[p.x], src[p.y], src[p.z], src[p.w]);
+    } else {
+        for (int64_t i = e; i < n; ++i) dst[i] = src[pos[i]];
+    }
+}
 // The same for H = 4 * Q heads and a 16-byte aligned src: an element's heads by Q 128-bit loads, two elements per lane
 // (a block apart, so that every store of a wavefront still covers 64 consecutive elements of one head).
 template <int Q>
@@ -1337,7 +1349,10 @@ extern "C" int fg_edge_values_head_major_f32(const float *src_dev, const int32_t
     hipStream_t st = (hipStream_t)stream;
     const dim3 wide((unsigned)((n_edges + 511) / 512));
     const bool aligned = ((uintptr_t)src_dev & 15) == 0;
-    if (aligned && heads == 4)
+    if (heads == 1 && edge_pos_dev && (((uintptr_t)edge_pos_dev | (uintptr_t)dst_dev) & 15) == 0)
+        hipLaunchKernelGGL(edge_values_permute_kernel, dim3((unsigned)((n_edges + 1023) / 1024)), dim3(256), 0, st,
+                           src_dev, edge_pos_dev, n_edges, dst_dev);
+    else if (aligned && heads == 4)
         hipLaunchKernelGGL(edge_values_head_major_vec_kernel<1>, wide, dim3(256), 0, st, src_dev, edge_pos_dev, n_edges, dst_dev);
     else if (aligned && heads == 8)
         hipLaunchKernelGGL(edge_values_head_major_vec_kernel<2>, wide, dim3(256), 0, st, src_dev, edge_pos_dev, n_edges, dst_dev);
