@@ -52,7 +52,7 @@ class GSpMMhip(VanillaSpMMhip):
         if reduce not in _REDUCE:
             raise ValueError("reduce must be one of %s" % sorted(_REDUCE))
         self._bop = None
-        if self._is_broadcast_message(msg, input_placeholders):
+        if self._is_broadcast_message(msg, input_placeholders, reduce):
             return self._build_broadcast(input_placeholders, compute_args, schedule_args, msg, reduce, return_arg)
         if len(input_placeholders) not in (1, 2):
             raise ValueError("GSpMM takes SrcFeat and optionally the edge weights")
@@ -95,8 +95,12 @@ class GSpMMhip(VanillaSpMMhip):
         self.out_tvm = torch.zeros((self._num_rows,) + tuple(src_ph.shape[1:]), dtype=torch.float32, device=self._ctx)
         self.arg_tvm = torch.full(self.out_tvm.shape, -1, dtype=torch.int32, device=self._ctx) if return_arg else None
 
-    def _is_broadcast_message(self, msg, input_placeholders):
+    def _is_broadcast_message(self, msg, input_placeholders, reduce='sum'):
         if msg not in ('u_mul_e', 'copy_u'):
+            return True
+        if msg == 'copy_u' and reduce in ('max', 'min') and len(input_placeholders) == 1 and self._num_col_partitions == 1:
+            # the broadcasting kernel takes source partitions and finds the selected elements in the same sweep
+            # (232,965-node graph, F=64: 2.2 ms against 3.0 ms, 4.3 against 6.0 ms with the positions)
             return True
         if len(input_placeholders) >= 1 and len(input_placeholders[0].shape) not in (2, 3):
             return True                   # the weighted-sum kernels take (num_cols, F) or (num_cols, H, D)
@@ -168,7 +172,7 @@ class GSpMMhip(VanillaSpMMhip):
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         compute_args = dict(compute_args)
         msg = compute_args.get('msg', 'u_mul_e')
-        if self._is_broadcast_message(msg, input_placeholders):
+        if self._is_broadcast_message(msg, input_placeholders, compute_args.get('reduce', 'sum')):
             op, lt, rt = general.parse_message(msg)
             nnz = self._adj_indices.shape[0]
             bop = general.BroadcastOp(op, lt, rt, input_placeholders[0], input_placeholders[1] if rt is not None else None,
