@@ -98,10 +98,14 @@ class GSpMMhip(VanillaSpMMhip):
     def _is_broadcast_message(self, msg, input_placeholders, reduce='sum'):
         if msg not in ('u_mul_e', 'copy_u'):
             return True
-        if msg == 'copy_u' and reduce in ('max', 'min') and len(input_placeholders) == 1 and self._num_col_partitions == 1:
+        if reduce in ('max', 'min') and self._num_col_partitions == 1:
             # the broadcasting kernel takes source partitions and finds the selected elements in the same sweep
-            # (232,965-node graph, F=64: 2.2 ms against 3.0 ms, 4.3 against 6.0 ms with the positions)
-            return True
+            # (232,965-node graph, F=64: 2.0 ms against 3.0 ms, 4.1 against 6.1 ms with the positions)
+            if msg == 'copy_u' and len(input_placeholders) == 1:
+                return True
+            if msg == 'u_mul_e' and len(input_placeholders) == 2 and len(input_placeholders[0].shape) == 2 \
+                    and tuple(input_placeholders[1].shape) == (self._adj_indices.shape[0],):
+                return True                   # one weight per edge, given to run()
         if len(input_placeholders) >= 1 and len(input_placeholders[0].shape) not in (2, 3):
             return True                   # the weighted-sum kernels take (num_cols, F) or (num_cols, H, D)
         if msg == 'u_mul_e' and len(input_placeholders) == 2:

@@ -192,3 +192,24 @@ def test_edge_values_head_major(torch_cuda, heads, n):
         _lib.check(_lib.lib().fg_edge_values_head_major_f32(_lib.dev_ptr(s), _lib.dev_ptr(p), n, heads, _lib.dev_ptr(dst), None))
         want = (s if p is None else s[p.long()]).t()
         assert torch.equal(dst, want)
+
+
+@pytest.mark.parametrize("reduce", ["max", "min"])
+@pytest.mark.parametrize("partitions", ['auto', 3])
+def test_extreme_of_weighted_messages_with_positions(torch_cuda, oracle, reduce, partitions):
+    """max / min of x[col] * w[e] with one weight per edge given to run() (the path over source partitions that finds
+    the selected elements in the same sweep): values exact, positions = the oracle's first occurrence."""
+    from featgraph_amd.module import GSpMMhip, placeholder
+    torch = torch_cuda
+    rng = np.random.default_rng(12)
+    adj = _graph(rng)
+    x = rng.integers(-2, 3, size=(3000, 20)).astype("float32")          # few distinct values: many ties
+    w = rng.integers(-2, 3, size=adj.nnz).astype("float32")
+    m = GSpMMhip(adj)
+    m.build([placeholder(x.shape), placeholder(w.shape)], {'reduce': reduce, 'return_arg': True}, {'num_src_partitions': partitions})
+    assert m._bop is not None
+    out = m.run([torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()]).cpu().numpy()
+    ref = oracle.gspmm(adj.indptr, adj.indices, w, x, reduce)
+    assert np.array_equal(out, ref)
+    ref_b, ref_arg = oracle.gspmm_bcast(adj.indptr, adj.indices, 'mul', reduce, x, w[:, None], 'u', 'e')
+    assert np.array_equal(ref_b, ref) and np.array_equal(m.arg_tvm.cpu().numpy(), ref_arg)
