@@ -171,8 +171,10 @@ def test_scratch_is_reserved_at_build_and_never_grown_under_capture():
         L.fg_spmm_plan_destroy(plan)
 
 
-def test_broadcasting_operators_replay_without_a_warm_up_call():
-    """build() reserves the split rows' scratch, so the first run() may already be the recorded one."""
+@pytest.mark.parametrize("partitions", [None, 2])
+def test_broadcasting_operators_replay_without_a_warm_up_call(partitions):
+    """build() reserves the split rows' scratch (and, over source partitions, the partitions' buffers of results), so the
+    first run() may already be the recorded one."""
     import torch
     from featgraph_amd.module import GSpMMhip, GSDDMMhip, placeholder
     rng = np.random.default_rng(8)
@@ -182,7 +184,9 @@ def test_broadcasting_operators_replay_without_a_warm_up_call():
     adj = adj.tocsr().astype("float32"); adj.sort_indices()
     nnz = adj.nnz
     agg = GSpMMhip(adj)
-    agg.build([placeholder((n_src, F)), placeholder((nnz, F))], {'msg': 'u_mul_e', 'reduce': 'max', 'return_arg': True}, {})
+    agg.build([placeholder((n_src, F)), placeholder((nnz, F))], {'msg': 'u_mul_e', 'reduce': 'max', 'return_arg': True},
+              {'num_src_partitions': partitions})
+    assert agg._active['P'] == (partitions or 1)
     edge = GSDDMMhip(adj.tocoo())
     edge.build([placeholder((nnz, F)), placeholder((n_dst, 1))], {'op': 'add', 'lhs_target': 'e', 'rhs_target': 'v'}, {})
     x = torch.zeros((n_src, F), device="cuda")
