@@ -106,6 +106,8 @@ class GSpMMhip(VanillaSpMMhip):
             if msg == 'u_mul_e' and len(input_placeholders) == 2 and len(input_placeholders[0].shape) == 2 \
                     and tuple(input_placeholders[1].shape) == (self._adj_indices.shape[0],):
                 return True                   # one weight per edge, given to run()
+            if msg == 'u_mul_e' and len(input_placeholders) == 1 and len(input_placeholders[0].shape) == 2:
+                return True                   # ... or the adjacency's own values
         if len(input_placeholders) >= 1 and len(input_placeholders[0].shape) not in (2, 3):
             return True                   # the weighted-sum kernels take (num_cols, F) or (num_cols, H, D)
         if msg == 'u_mul_e' and len(input_placeholders) == 2:
@@ -120,13 +122,18 @@ class GSpMMhip(VanillaSpMMhip):
         common.take_args(compute_args, self._compute_keys, "compute_func")
         common.take_args(schedule_args, self._schedule_keys, "schedule_func")
         op, lt, rt = general.parse_message(msg)
+        nnz = self._adj_indices.shape[0]
+        # 'u_mul_e' with SrcFeat alone: the adjacency's own values are the edge operand (CSR order, already on the device)
+        self._static_rhs = None
+        if msg == 'u_mul_e' and len(input_placeholders) == 1:
+            self._static_rhs = self._layout(1)['vals']
+            input_placeholders = [input_placeholders[0], common.placeholder((nnz,))]
         if len(input_placeholders) != (1 if rt is None else 2):
             raise ValueError("message %r takes %d input(s), got %d" % (msg, 1 if rt is None else 2, len(input_placeholders)))
-        nnz = self._adj_indices.shape[0]
         lhs_ph = input_placeholders[0]
         rhs_ph = input_placeholders[1] if rt is not None else None
         self._bop = general.BroadcastOp(op, lt, rt, lhs_ph, rhs_ph, self._num_rows, self._num_cols, nnz, self._ctx, allow_v=False)
-        self._placeholders = list(input_placeholders)
+        self._placeholders = list(input_placeholders[:1] if self._static_rhs is not None else input_placeholders)
         self._feat_len, self._heads, self._num_feat_partitions = self._bop.out_len, 1, 0
         self._reduce, self._msg, self._return_arg = reduce, msg, return_arg
         self._notes = [self._bop.describe()]
@@ -168,10 +175,13 @@ class GSpMMhip(VanillaSpMMhip):
     def _launch_broadcast(self, inputs):
         lay = self._active
         lhs = inputs[0]
-        rhs = inputs[1] if len(inputs) > 1 else None
-        # where each element of the layout lies in the edge operands (None: at its own position)
+        rhs = inputs[1] if len(inputs) > 1 else self._static_rhs
+        # where each element of the layout lies in the edge operands (None: at its own position); the adjacency's own
+        # values are in CSR order whatever order was announced for operands given to run()
+        own = len(inputs) == 1 and self._static_rhs is not None
+        pos = (lay['edge_pos32'] if lay['P'] > 1 else None) if own else self._given_pos(lay)
         self._bop.run_spmm(lay['plan'], lay['pos'], lay['idx'], _REDUCE[self._reduce], lhs, rhs, self._row_scale,
-                           self.out_tvm, self.arg_tvm, edge_pos_dev=self._given_pos(lay))
+                           self.out_tvm, self.arg_tvm, edge_pos_dev=pos)
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         compute_args = dict(compute_args)
@@ -179,6 +189,8 @@ class GSpMMhip(VanillaSpMMhip):
         if self._is_broadcast_message(msg, input_placeholders, compute_args.get('reduce', 'sum')):
             op, lt, rt = general.parse_message(msg)
             nnz = self._adj_indices.shape[0]
+            if msg == 'u_mul_e' and len(input_placeholders) == 1:
+                input_placeholders = [input_placeholders[0], common.placeholder((nnz,))]       # the adjacency's own values
             bop = general.BroadcastOp(op, lt, rt, input_placeholders[0], input_placeholders[1] if rt is not None else None,
                                       self._num_rows, self._num_cols, nnz, self._ctx, allow_v=False)
             self._bop, keep = bop, self._bop
