@@ -189,7 +189,7 @@ class Graph(object):
         key = ('gspmm', msg, reduce, transposed, return_arg) + tuple(tuple(a.shape) for a in arrays)
         if key not in self._mods:
             m = GSpMMhip(self._tr if transposed else self._csr)
-            args = {'msg': msg, 'reduce': reduce}
+            args = {'msg': msg, 'reduce': reduce, 'broadcast': True}      # numpy broadcasting, whatever the shapes
             if return_arg:
                 args['return_arg'] = True
             m.build([placeholder(tuple(a.shape)) for a in arrays], args, {})

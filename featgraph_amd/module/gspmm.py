@@ -36,23 +36,26 @@ class GSpMMhip(VanillaSpMMhip):
     broadcast against each other the numpy way, e.g. 'u_mul_e' with (num_cols, H, D) and (nnz, H, 1), or
     'u_add_e' with (num_cols, F) and (nnz, F).  out[v] = reduce over row v's edges of the message; out
     has the broadcast feature shape.  (With 'u_mul_e', a second input of shape (nnz,) or (nnz, H) keeps
-    its meaning of one weight per edge, or per edge and head.)  schedule_args {'num_src_partitions': 'auto' | int |
+    its meaning of one weight per edge, or per edge and head; compute_args {'broadcast': True} makes every message
+    follow numpy broadcasting instead, as DGL's gspmm does -- the two readings differ only for SrcFeat (num_cols, H, D)
+    with D == H and a second input (nnz, H).)  schedule_args {'num_src_partitions': 'auto' | int |
     None} cuts the source columns into partitions as for the weighted sum (default 'auto': chosen from the size of the
     operand that is gathered from the source nodes); operands on the edges and the reported positions stay in CSR order.
     """
-    _compute_keys = ('num_feat_partitions', 'reduce', 'msg', 'return_arg')
+    _compute_keys = ('num_feat_partitions', 'reduce', 'msg', 'return_arg', 'broadcast')
 
     def build(self, input_placeholders, compute_args, schedule_args):
         compute_args = dict(compute_args)
         reduce = compute_args.pop('reduce', 'sum')
         msg = compute_args.pop('msg', 'u_mul_e')
         return_arg = bool(compute_args.pop('return_arg', False))
+        force = bool(compute_args.pop('broadcast', False))
         if return_arg and reduce not in ('max', 'min'):
             raise ValueError("return_arg is defined for reduce='max' / 'min' only")
         if reduce not in _REDUCE:
             raise ValueError("reduce must be one of %s" % sorted(_REDUCE))
         self._bop = None
-        if self._is_broadcast_message(msg, input_placeholders, reduce):
+        if self._is_broadcast_message(msg, input_placeholders, reduce, force):
             return self._build_broadcast(input_placeholders, compute_args, schedule_args, msg, reduce, return_arg)
         if len(input_placeholders) not in (1, 2):
             raise ValueError("GSpMM takes SrcFeat and optionally the edge weights")
@@ -95,9 +98,16 @@ class GSpMMhip(VanillaSpMMhip):
         self.out_tvm = torch.zeros((self._num_rows,) + tuple(src_ph.shape[1:]), dtype=torch.float32, device=self._ctx)
         self.arg_tvm = torch.full(self.out_tvm.shape, -1, dtype=torch.int32, device=self._ctx) if return_arg else None
 
-    def _is_broadcast_message(self, msg, input_placeholders, reduce='sum'):
+    def _is_broadcast_message(self, msg, input_placeholders, reduce='sum', force=False):
         if msg not in ('u_mul_e', 'copy_u'):
             return True
+        if force and len(input_placeholders) == 2:
+            # numpy broadcasting throughout; what the weighted-sum kernels also compute stays with them
+            src_ph, e_ph = input_placeholders
+            nnz = self._adj_indices.shape[0]
+            one_weight = tuple(e_ph.shape) == (nnz,) and len(src_ph.shape) == 2
+            if not (msg == 'u_mul_e' and reduce in ('sum', 'mean') and one_weight):
+                return True
         if reduce in ('max', 'min') and self._num_col_partitions == 1:
             # the broadcasting kernel takes source partitions and finds the selected elements in the same sweep
             # (232,965-node graph, F=64: 2.0 ms against 3.0 ms, 4.1 against 6.1 ms with the positions)
@@ -114,7 +124,7 @@ class GSpMMhip(VanillaSpMMhip):
             src_ph, e_ph = input_placeholders
             heads = src_ph.shape[1] if len(src_ph.shape) == 3 else 1
             nnz = self._adj_indices.shape[0]
-            return tuple(e_ph.shape) not in ((nnz,), (nnz, heads))
+            return tuple(e_ph.shape) != ((nnz,) if heads == 1 else (nnz, heads))
         return False
 
     def _build_broadcast(self, input_placeholders, compute_args, schedule_args, msg, reduce, return_arg):
@@ -186,7 +196,7 @@ class GSpMMhip(VanillaSpMMhip):
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         compute_args = dict(compute_args)
         msg = compute_args.get('msg', 'u_mul_e')
-        if self._is_broadcast_message(msg, input_placeholders, compute_args.get('reduce', 'sum')):
+        if self._is_broadcast_message(msg, input_placeholders, compute_args.get('reduce', 'sum'), bool(compute_args.get('broadcast'))):
             op, lt, rt = general.parse_message(msg)
             nnz = self._adj_indices.shape[0]
             if msg == 'u_mul_e' and len(input_placeholders) == 1:
@@ -202,7 +212,7 @@ class GSpMMhip(VanillaSpMMhip):
             buf = ctypes.create_string_buffer(4096)
             _lib.check(_lib.lib().fg_spmm_plan_describe(self._layout(P)['plan'], 0, 0, buf, len(buf)))
             return buf.value.decode() + "  kernel           : gspmm_bcast_kernel, one wavefront per work item\n  note             : %s\n" % bop.describe()
-        for k in ('reduce', 'msg', 'return_arg'):
+        for k in ('reduce', 'msg', 'return_arg', 'broadcast'):
             compute_args.pop(k, None)
         flat = common.placeholder((self._num_cols, int(np.prod(input_placeholders[0].shape[1:]))))
         return super(GSpMMhip, self).lower_to_ir([flat], compute_args, schedule_args)

@@ -438,3 +438,31 @@ def test_operands_that_are_not_16_byte_aligned(oracle):
     g.build([placeholder(ef.shape), placeholder(y.shape)], {'op': 'sub', 'lhs_target': 'e'}, {})
     ref = oracle.gsddmm_bcast(coo.row, coo.col, 'sub', ef, y, 'e', 'v')
     assert np.array_equal(g.run([shifted(ef), shifted(y)]).cpu().numpy(), ref)
+
+
+def test_square_head_shapes_follow_numpy_broadcasting_on_request(oracle):
+    """SrcFeat (num_cols, H, D) with D == H and a second input (nnz, H): the module reads it as one weight per edge and
+    head unless compute_args say 'broadcast', in which case (as for DGL's gspmm, and in featgraph_amd.ops) the second
+    input lines up with the last axis; (num_cols, H, D) with one weight per edge (nnz,) is a broadcast either way."""
+    import torch
+    from featgraph_amd.module import GSpMMhip, placeholder
+    from featgraph_amd import ops
+    from featgraph_amd.autograd import Graph
+    rng = np.random.default_rng(4)
+    adj = _graph(rng)
+    x = _operand(rng, adj.shape[1], (4, 4))
+    w = _operand(rng, adj.nnz, (4,))
+    xd, wd = torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()
+    per_head, _ = oracle.gspmm_bcast(adj.indptr, adj.indices, 'mul', 'sum', x, w[:, :, None], 'u', 'e')
+    last_axis, _ = oracle.gspmm_bcast(adj.indptr, adj.indices, 'mul', 'sum', x, w, 'u', 'e')
+    assert not np.allclose(per_head, last_axis)
+    m = GSpMMhip(adj)
+    m.build([placeholder(x.shape), placeholder(w.shape)], {'msg': 'u_mul_e'}, {})
+    assert np.allclose(m.run([xd, wd]).cpu().numpy(), per_head, rtol=1e-4, atol=1e-4)
+    m.build([placeholder(x.shape), placeholder(w.shape)], {'msg': 'u_mul_e', 'broadcast': True}, {})
+    assert np.allclose(m.run([xd, wd]).cpu().numpy(), last_axis, rtol=1e-4, atol=1e-4)
+    assert np.allclose(ops.gspmm(Graph(adj), "mul", "sum", xd, wd).cpu().numpy(), last_axis, rtol=1e-4, atol=1e-4)
+    one = _operand(rng, adj.nnz, ())
+    m.build([placeholder(x.shape), placeholder(one.shape)], {'msg': 'u_mul_e'}, {})
+    ref, _ = oracle.gspmm_bcast(adj.indptr, adj.indices, 'mul', 'sum', x, one, 'u', 'e')
+    assert np.allclose(m.run([xd, torch.from_numpy(one).cuda()]).cpu().numpy(), ref, rtol=1e-4, atol=1e-4)

@@ -196,7 +196,7 @@ def test_random_broadcast_operators(oracle, monkeypatch, seed):
         lhs, rhs = operand(rows[lt], l_shape), operand(rows[rt], r_shape)
         reduce = str(rng.choice(["sum", "mean", "max", "min"]))
         m = GSpMMhip(adj)
-        args = {'msg': "%s_%s_%s" % (lt, op, rt), 'reduce': reduce}
+        args = {'msg': "%s_%s_%s" % (lt, op, rt), 'reduce': reduce, 'broadcast': True}     # numpy broadcasting throughout
         if reduce in ("max", "min"):
             args['return_arg'] = True
         parts = [None, 2, 3, 7][int(rng.integers(0, 4))]         # source-column partitions (None: the CSR arrays as they are)
