@@ -514,6 +514,51 @@ __global__ __launch_bounds__(kBlock) void gsddmm_bcast_kernel(const EdgeArgs a) 
     }
 }
 
+// Dot products over a contracted axis of R floats (R a multiple of 4, operands 16-byte aligned): a group of L lanes
+// (4 L >= R up to 64 lanes) reads the two operands' R floats of one (edge, output feature) pair with 128-bit loads and
+// adds its products up with shuffles; the 64 / L groups take different pairs of the wavefront's 64 edges, U pairs in
+// flight each.  (gsddmm_bcast_kernel<FG_BIN_DOT> walks the axis lane by lane and serves every other shape.)
+template <int L>
+__global__ __launch_bounds__(kBlock) void gsddmm_dot_kernel(const EdgeArgs a) {
+    constexpr int G = 64 / L, U = 4;
+    const int lane = threadIdx.x & 63, g = lane / L, li = lane % L;
+    const int64_t wave_id = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int64_t e0 = wave_id * 64;
+    if (e0 >= a.n_edges) return;
+    const int n_e = (int)min((int64_t)64, a.n_edges - e0);
+    const int F = a.F, R = a.R;
+    const int n_pairs = n_e * F;
+    const bool l_on_e = a.lhs_target == FG_TARGET_E, r_on_e = a.rhs_target == FG_TARGET_E;
+    for (int pb = g; pb < n_pairs; pb += G * U) {
+        float s[U];
+        bool ok[U];
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            const int p = pb + k * G;
+            ok[k] = p < n_pairs;
+            const int pc = ok[k] ? p : pb;
+            const int64_t e = e0 + pc / F;
+            const int f = pc % F;
+            const int64_t il = a.lhs_index[e], ir = a.rhs_index[e];
+            const int fl = a.lhs_off ? a.lhs_off[f] : f, fr = a.rhs_off ? a.rhs_off[f] : f;
+            const float *lp = a.lhs + (l_on_e ? e : il) * a.lhs_len + (int64_t)fl * R;
+            const float *rp = a.rhs + (r_on_e ? e : ir) * a.rhs_len + (int64_t)fr * R;
+            float acc = 0.f;
+            for (int c = li * 4; c < R; c += L * 4) {
+                const float4 x = *reinterpret_cast<const float4 *>(lp + c), y = *reinterpret_cast<const float4 *>(rp + c);
+                acc += (x.x * y.x + x.y * y.y) + (x.z * y.z + x.w * y.w);
+            }
+            s[k] = acc;
+        }
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            for (int off = 1; off < L; off <<= 1) s[k] += __shfl_xor(s[k], off);
+            const int p = pb + k * G;
+            if (li == 0 && ok[k]) a.out[(e0 + p / F) * F + p % F] = s[k];
+        }
+    }
+}
+
 template <int OP>
 void launch_sddmm(int vec, dim3 grid, hipStream_t st, const EdgeArgs &a) {
     if (vec == 1) hipLaunchKernelGGL((gsddmm_bcast_kernel<OP, 4, true, true>), grid, dim3(kBlock), 0, st, a);
@@ -696,7 +741,16 @@ extern "C" int fg_gsddmm_bcast_f32(const int32_t *row_dev, const int32_t *col_de
         case FG_BIN_DIV: launch_sddmm<FG_BIN_DIV>(vec, grid, st, a); break;
         case FG_BIN_COPY_LHS: launch_sddmm<FG_BIN_COPY_LHS>(vec, grid, st, a); break;
         case FG_BIN_COPY_RHS: launch_sddmm<FG_BIN_COPY_RHS>(vec, grid, st, a); break;
-        default: hipLaunchKernelGGL((gsddmm_bcast_kernel<FG_BIN_DOT, 1, true, true>), grid, dim3(kBlock), 0, st, a); break;
+        default: {
+            const bool wide = R % 4 == 0 && lhs_len % 4 == 0 && rhs_len % 4 == 0 && (((uintptr_t)lhs_dev | (uintptr_t)rhs_dev) & 15) == 0;
+            if (!wide) hipLaunchKernelGGL((gsddmm_bcast_kernel<FG_BIN_DOT, 1, true, true>), grid, dim3(kBlock), 0, st, a);
+            else if (R <= 16) hipLaunchKernelGGL(gsddmm_dot_kernel<4>, grid, dim3(kBlock), 0, st, a);
+            else if (R <= 32) hipLaunchKernelGGL(gsddmm_dot_kernel<8>, grid, dim3(kBlock), 0, st, a);
+            else if (R <= 64) hipLaunchKernelGGL(gsddmm_dot_kernel<16>, grid, dim3(kBlock), 0, st, a);
+            else if (R <= 128) hipLaunchKernelGGL(gsddmm_dot_kernel<32>, grid, dim3(kBlock), 0, st, a);
+            else hipLaunchKernelGGL(gsddmm_dot_kernel<64>, grid, dim3(kBlock), 0, st, a);
+            break;
+        }
     }
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;

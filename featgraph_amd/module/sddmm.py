@@ -419,6 +419,11 @@ class GSDDMMhip(VanillaSDDMMhip):
         self._bop = None
         if self._op not in general.BINARY:
             raise ValueError("op must be one of %s" % sorted(general.BINARY))
+        self._swap_inputs = False
+        if self._op == 'dot' and (lt, rt) == ('v', 'u') and len(input_placeholders) == 2:
+            # a dot product does not care which operand comes first: (DstFeat, SrcFeat) is the dot-product kernels' pair
+            lt, rt, input_placeholders = 'u', 'v', [input_placeholders[1], input_placeholders[0]]
+            self._swap_inputs = True
         same = (lt, rt) == ('u', 'v') and len(input_placeholders) == 2 and \
             input_placeholders[0].shape[1:] == input_placeholders[1].shape[1:]
         plain = same and len(input_placeholders[0].shape) == 2
@@ -471,6 +476,8 @@ class GSDDMMhip(VanillaSDDMMhip):
     def run(self, input_tvm_ndarrays):
         if self._func is None:
             raise RuntimeError("call build() before run()")
+        if getattr(self, '_swap_inputs', False):
+            input_tvm_ndarrays = list(input_tvm_ndarrays)[::-1]
         if self._bop is None:
             return super(GSDDMMhip, self).run(input_tvm_ndarrays)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
@@ -480,6 +487,8 @@ class GSDDMMhip(VanillaSDDMMhip):
     def measure_average_time(self, input_tvm_ndarrays, num_runs):
         if self._func is None:
             raise RuntimeError("call build() before measure_average_time()")
+        if getattr(self, '_swap_inputs', False):
+            input_tvm_ndarrays = list(input_tvm_ndarrays)[::-1]
         if self._bop is None:
             return super(GSDDMMhip, self).measure_average_time(input_tvm_ndarrays, num_runs)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)

@@ -310,6 +310,11 @@ EDGE_CASES = [
     ("dot", 'u', (40,), 'v', (40,)),
     ("dot", 'e', (3, 8), 'u', (1, 8)),
     ("dot", 'v', (2, 1, 4), 'e', (5, 4)),
+    ("dot", 'u', (8, 64), 'v', (1, 64)),          # contracted axes of 16 floats and more: lane groups with 128-bit loads
+    ("dot", 'u', (100,), 'u', (100,)),            # 25 of a group's 32 lanes hold a word
+    ("dot", 'e', (2, 256), 'v', (256,)),
+    ("dot", 'v', (520,), 'u', (3, 520)),          # more than 64 words: a lane walks the axis
+    ("dot", 'u', (3, 6), 'e', (6,)),              # not a multiple of 4: lane by lane
     ("copy_lhs", 'u', (7,), None, None),
     ("copy_lhs", 'v', (70,), None, None),
     ("copy_rhs", None, None, 'e', (3,)),
@@ -438,6 +443,11 @@ def test_operands_that_are_not_16_byte_aligned(oracle):
     g.build([placeholder(ef.shape), placeholder(y.shape)], {'op': 'sub', 'lhs_target': 'e'}, {})
     ref = oracle.gsddmm_bcast(coo.row, coo.col, 'sub', ef, y, 'e', 'v')
     assert np.array_equal(g.run([shifted(ef), shifted(y)]).cpu().numpy(), ref)
+    g.build([placeholder(ef.shape), placeholder(y.shape)], {'op': 'dot', 'lhs_target': 'e'}, {})
+    ref = oracle.gsddmm_bcast(coo.row, coo.col, 'dot', ef, y, 'e', 'v')
+    mass = oracle.gsddmm_bcast(coo.row, coo.col, 'dot', np.abs(ef), np.abs(y), 'e', 'v')
+    for es, ys in ((shifted(ef), torch.from_numpy(y).cuda()), (torch.from_numpy(ef).cuda(), shifted(y))):
+        assert_sum_close(g.run([es, ys]).cpu().numpy(), ref, mass, "dot of a shifted operand")
 
 
 def test_square_head_shapes_follow_numpy_broadcasting_on_request(oracle):
