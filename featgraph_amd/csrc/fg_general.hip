@@ -16,9 +16,10 @@
 // V output features (V = 4 with 128-bit accesses when the shapes allow it, else 1); a group of L lanes
 // (L = the power of two that covers the F / V vectors, at most 64) takes one element at a time and the
 // 64 / L groups take different elements of the row, several steps in flight (in an item of many short rows
-// every group takes a row of its own instead); longer feature axes are walked 64 vectors at a time.  With one
-// group (64 vectors or more), and for rows that a group has to itself, a row's sum is formed in the stored
-// element order.  The edge operand, when there is one, is the dominant stream ([nnz, len] floats read once,
+// every group takes a row of its own instead); feature axes of 128 floats and more, in multiples of 64, are cut
+// into 64-float tiles for different workgroups when an operand is gathered (each L2 then holds one tile's slice of
+// the gathered rows); other long axes are walked 64 vectors at a time.  With one group (64 vectors or more, no
+// tiles), and for rows that a group has to itself, a row's sum is formed in the stored element order.  The edge operand, when there is one, is the dominant stream ([nnz, len] floats read once,
 // coalesced, past the caches); the node operand is gathered, through column words that the wavefront has staged
 // in LDS for the whole item.
 //
@@ -76,6 +77,7 @@ struct GenArgs {
     const int64_t *item_off;
     const int32_t *edge_pos;
     int n_parts;
+    int n_tiles, tile_vecs;      // the feature axis in n_tiles tiles of tile_vecs vectors (V floats each), one per workgroup
     int final;                   // the kernel's rows are results (one partition), not a partition's share of them
     int64_t pos_stride, col_width, out_stride, partial_stride;
 };
@@ -131,11 +133,15 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
     const bool final = !PART || a.final != 0;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int64_t item_id = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+    // workgroup id = item block * n_tiles + tile: the XCDs, dealt workgroups in turn, work on different feature tiles
+    // of the same items, so that each L2 holds one tile's slice of the gathered rows
+    const int tile = (int)(blockIdx.x % (unsigned)a.n_tiles);
+    const int64_t item_id = (int64_t)(blockIdx.x / (unsigned)a.n_tiles) * kWavesPerBlock + wave;
     if (item_id >= a.n_items) return;
     const Item it = a.items[item_id];
     const int L = a.L, G = 64 / L, g = lane / L, li = lane % L;
     const int F = a.F, FV = F / V;
+    const int fv_lo = tile * a.tile_vecs, fv_hi = min(FV, fv_lo + a.tile_vecs);
     int part = 0;
     if (PART) {
         const int64_t id = ((int64_t)__builtin_amdgcn_readfirstlane((int)(item_id >> 32)) << 32) |
@@ -172,9 +178,9 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
                             bool done) {
         constexpr bool OWN = decltype(own)::value;
         const int first = OWN ? 0 : g, step = OWN ? 1 : G;
-        for (int f0 = 0; f0 < FV; f0 += L) {
-            const bool active = f0 + li < FV;
-            const int fc = (active ? f0 + li : FV - 1) * V;       // the lane's first output feature
+        for (int f0 = fv_lo; f0 < fv_hi; f0 += L) {
+            const bool active = f0 + li < fv_hi;
+            const int fc = (active ? f0 + li : fv_hi - 1) * V;       // the lane's first output feature
             const int fl = kLhs ? (a.lhs_off ? a.lhs_off[fc] : fc) : 0;
             const int fr = kRhs ? (a.rhs_off ? a.rhs_off[fc] : fc) : 0;
             float acc[V];
@@ -625,11 +631,19 @@ int gspmm_bcast_run(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx
     a.out = P > 1 ? buf : out_dev;
     a.arg = P > 1 ? (arg_dev ? abuf : nullptr) : arg_dev;
     a.partial = values; a.partial_arg = positions;
-    a.F = out_len; a.L = lanes_for(out_len / V);
+    // Feature tiles of 64 floats over the workgroups (as for the weighted sum) when an operand is gathered from the
+    // source nodes and the 128-bit paths apply: a partition's slice of a tile is what an L2 has to hold.
+    // (Not with the positions of the selected elements, whose kernels hold too many registers to gain from it --
+    // F=256: 17.1 ms tiled against 14.7 ms -- nor with an operand streamed from the edges, which sets the time.)
+    const bool gathers = (uses_l && lhs_target == FG_TARGET_U) || (uses_r && rhs_target == FG_TARGET_U);
+    const bool streams = (uses_l && lhs_target == FG_TARGET_E && lmode == 1) || (uses_r && rhs_target == FG_TARGET_E && rmode == 1);
+    const int T = (V == 4 && gathers && !streams && !arg_dev && out_len >= 128 && out_len % 64 == 0) ? out_len / 64 : 1;
+    a.n_tiles = T; a.tile_vecs = T > 1 ? 16 : (out_len + V - 1) / V;
+    a.F = out_len; a.L = lanes_for(T > 1 ? 16 : out_len / V);
     a.item_off = pl->item_off_dev; a.edge_pos = edge_pos_dev; a.n_parts = P; a.final = P == 1;
     a.pos_stride = pl->n_dst + 1; a.col_width = (pl->n_src + P - 1) / P;
     a.out_stride = (int64_t)b.buffers; a.partial_stride = (int64_t)b.pieces;
-    const int64_t blocks = (pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock;
+    const int64_t blocks = ((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock) * T;
     if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
     // an operand on the stored elements that is read with 128-bit loads streams past the caches
     const bool lnt = uses_l && lhs_target == FG_TARGET_E && lmode == 1, rnt = uses_r && rhs_target == FG_TARGET_E && rmode == 1;

@@ -107,6 +107,24 @@ class BroadcastOp(object):
                    "" if self.reduce_len == 1 else ", %d contracted" % self.reduce_len,
                    "" if self.lhs_off is None and self.rhs_off is None else ", broadcast through offset arrays"))
 
+    def feature_tiles(self, return_arg=False):
+        """The number of 64-float feature tiles the library's SpMM kernel will cut this message into (it does so from
+        128 output features on, when an operand is gathered from the source nodes, none is streamed from the edges
+        with 4 consecutive features per lane, no positions are asked for and 4 features per lane are possible: every
+        operand's groups of 4 consecutive or equal)."""
+        def wide(off, length, vec_flag, splat_flag):
+            if length == 0:
+                return 1                                    # operand not used
+            if off is None or (self.flags & vec_flag):
+                return 1 if length % 4 == 0 else 0
+            return 2 if (self.flags & splat_flag) else 0
+        l, r = wide(self.lhs_off, self.lhs_len, 1, 2), wide(self.rhs_off, self.rhs_len, 4, 8)
+        vec = self.out_len % 4 == 0 and l and r and not (l == 2 and r == 2)
+        streams = (self.lhs_target == 'e' and self.lhs_len > 0 and l == 1) or (self.rhs_target == 'e' and self.rhs_len > 0 and r == 1)
+        if vec and not streams and not return_arg and self.gathered_len() > 0 and self.out_len >= 128 and self.out_len % 64 == 0:
+            return self.out_len // 64
+        return 1
+
     def gathered_len(self):
         """Feature length of the operand that is gathered from the source nodes (0: none is)."""
         return max(self.lhs_len if self.lhs_target == 'u' else 0, self.rhs_len if self.rhs_target == 'u' else 0)

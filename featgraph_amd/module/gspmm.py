@@ -180,7 +180,7 @@ class GSpMMhip(VanillaSpMMhip):
         if bop.gathered_len() == 0:
             return 1
         return tuning.choose_gather_partitions(self._num_rows, self._num_cols, self._adj_indices.shape[0], bop.gathered_len(),
-                                               bop.out_len * (2 if return_arg else 1), self._graph_stats())
+                                               bop.out_len * (2 if return_arg else 1), self._graph_stats(), bop.feature_tiles(return_arg))
 
     def _launch_broadcast(self, inputs):
         lay = self._active

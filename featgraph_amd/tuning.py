@@ -232,19 +232,25 @@ def choose_spmm(n_dst, n_src, nnz, feat_len, stats=None):
 # F=64 3.02 / - / 2.14 / 2.20 / 2.56, F=128 6.58 / 5.95 / 4.99 / 4.14 / 4.38, F=256 15.7 / 14.1 / 12.3 / 10.2 / 8.87;
 # u_mul_e with [nnz, F] edge features: F=64 6.87 / - / 6.19 / 6.66 / 7.23, F=128 14.4 / 13.7 / 12.7 / 13.1 / 14.1).
 BCAST_COEF = dict(SPMM_COEF, seg=4.5e-10)
+# ... and per tile when the feature axis is tiled (u_add_e, F=256 in 4 tiles: 12.8 / 11.2 / 9.21 / 7.83 / 9.54 ms at 1 / 2 / 4 / 8 / 16
+# partitions; F=128 in 2 tiles: 6.03 / 5.16 / 4.04 / 4.08 / 4.93)
+BCAST_TILED_COEF = dict(SPMM_COEF, seg=2.0e-10)
 
 
-def choose_gather_partitions(n_dst, n_src, nnz, gathered_len, out_len, stats=None):
+def choose_gather_partitions(n_dst, n_src, nnz, gathered_len, out_len, stats=None, tiles=1):
     """Source-column partitions for a generalised SpMM whose gathered operand has `gathered_len` floats per source
-    node and whose result has `out_len` per destination: the kernel does not tile the feature axis, so the model is
-    asked for the untiled traversal; every partition's results take a buffer of their own (8 GiB at most)."""
+    node and whose result has `out_len` per destination, with the feature axis in `tiles` tiles (the library's own
+    choice: 64-float tiles from 128 features on, when the 128-bit paths apply); every partition's results take a
+    buffer of their own (8 GiB at most)."""
     if nnz == 0 or n_dst == 0 or gathered_len < 1:
         return 1
     if stats is None:
         stats = GraphStats(n_dst, n_src, nnz)
-    cands = [(p, 1) for p in (1, 2, 4, 8, 16, 32)
+    tiles = max(1, int(tiles))
+    cands = [(p, tiles) for p in (1, 2, 4, 8, 16, 32)
              if p <= min(MAX_PARTITIONS, max(1, n_src)) and (p == 1 or 4.0 * p * n_dst * out_len <= float(8 << 30))]
-    predict = lambda st, f, p, t: predict_spmm(st, f, p, t, BCAST_COEF)
+    coef = BCAST_TILED_COEF if tiles > 1 else BCAST_COEF
+    predict = lambda st, f, p, t: predict_spmm(st, f, p, t, coef)
     return _rank(stats, gathered_len, predict, cands, _spmm_tie)[0][0]
 
 

@@ -64,7 +64,10 @@ CASES = [
     ("e_sub_u", (130,), (130,)),
     ("u_div_e", (32,), (32,)),
     ("e_div_u", (2, 1, 8), (3, 8)),
-    ("e_mul_u", (256,), (256,)),
+    ("e_mul_u", (256,), (256,)),       # 128 features and more, in multiples of 64: feature tiles over the workgroups
+    ("u_mul_e", (2, 64), (2, 64)),
+    ("u_add_e", (192,), (1,)),
+    ("u_mul_e", (8, 64), (8, 1)),
     ("copy_e", (40,), None),
     ("copy_e", (1,), None),
     ("copy_e", (2, 50), None),
@@ -234,8 +237,8 @@ def test_edge_features_that_repeat_a_weight_match_the_weighted_sum(oracle):
     from featgraph_amd.module import VanillaSpMMhip, placeholder
     rng = np.random.default_rng(5)
     adj = _hub_graph(rng)
-    x = _operand(rng, adj.shape[1], (256,))
-    ef = np.repeat(adj.data[:, None], 256, axis=1).astype("float32")
+    x = _operand(rng, adj.shape[1], (260,))
+    ef = np.repeat(adj.data[:, None], 260, axis=1).astype("float32")
     out = _run_spmm(adj, "u_mul_e", "sum", [x, ef])
     m = VanillaSpMMhip(adj)
     m.build([placeholder(x.shape)], {}, {'num_src_partitions': None})
@@ -244,8 +247,8 @@ def test_edge_features_that_repeat_a_weight_match_the_weighted_sum(oracle):
     mass = np.asarray(abs(adj).astype(np.float64).dot(np.abs(x).astype(np.float64)))
     assert_sum_close(out, ref64, mass, "edge features")
     assert_sum_close(plain, ref64, mass, "plain")
-    # 256 features: one lane group per row, so rows that are not split are summed in stored order, with
-    # separately rounded products: the sequential float32 sum, bit for bit
+    # 260 features (65 vectors of 4, not cut into 64-float tiles): one lane group per row, so rows that are not split
+    # are summed in stored order, with separately rounded products: the sequential float32 sum, bit for bit
     seq = oracle.spmm_csr_rowwise(adj.indptr, adj.indices, adj.data, x)
     short = np.diff(adj.indptr) <= 1024
     assert np.array_equal(out[short], seq[short])
