@@ -895,52 +895,52 @@ extern "C" int fg_sddmm_dds_f32(fg_spmm_plan *pl, const int32_t *s1_pos_dev, con
     a.pos = s1_pos_dev; a.pos_stride = pl->n_dst + 1;
     a.src = src_dev; a.src_stride = width * F; a.n_parts = P;
     a.src_row_bytes = (uint32_t)F * 4u; a.src_tile_bytes = 0;
-    // Fewer than 8 tiles: 8 / T partitions per launch, so that every XCD still has one tile of one
-    // partition to itself (no two L2s hold the same slice) and a partition's slice can be smaller
-    // at the same number of launches.  Edges of different partitions write different results.
-    // (232,965-node graph: 3.93 -> 3.71 ms at F=128, 7.89 -> 7.56 ms at F=256, 1.96 -> 1.82 ms at F=64.)
-    const int conc = (T < 8 && 8 % T == 0) ? std::max(1, std::min(8 / T, P)) : 1;
-    a.conc = conc;
     if (ts.tile_major) {
         if ((rc = fg::make_tile_major(pl, src_dev, pl->n_src, F, tile_w, stream)) != FG_OK) return rc;
         a.src = pl->tiled_dev; a.src_stride = width * tile_w;
         a.src_row_bytes = (uint32_t)tile_w * 4u; a.src_tile_bytes = (uint32_t)((uint64_t)pl->n_src * tile_w * 4u);
     }
-    // More than 8 tiles: 8 per launch (one per XCD), as for SpMM.
-    const int per_launch = (T > 8 && T % 8 == 0) ? 8 : T;
-    a.n_tiles = per_launch;
-    // Edges of different partitions write different results, so nothing orders the passes: one launch walks all
-    // groups of `conc` partitions, group after group in workgroup order; the next group's first workgroups fill the
-    // compute units that the previous one's last workgroups leave idle (232,965-node graph, F=512: 13.64 -> 13.51 ms).
-    const int n_groups = (P + conc - 1) / conc;
-    a.n_groups = 0;
-    a.first_part = 0;
-    if (n_groups > 1 && n_groups <= kMaxGroups) {
-        a.n_groups = n_groups;
-        a.group_off[0] = 0;
-        for (int g = 0; g < n_groups; ++g) {
+    // The tiles go out 8, 4, 2 or 1 per launch: counts that divide the 8 XCDs, so that workgroup id % slots always puts
+    // a tile on the same XCDs (10 tiles: 8 + 2; with all 10 in one launch every L2 would see every tile's slice).
+    // Fewer than 8 tiles in a launch: 8 / tiles partitions at a time, so that every XCD still has one tile of one
+    // partition to itself (no two L2s hold the same slice) and a partition's slice can be smaller at the same number
+    // of launches; edges of different partitions write different results.
+    // (232,965-node graph: 3.93 -> 3.71 ms at F=128, 7.89 -> 7.56 ms at F=256, 1.96 -> 1.82 ms at F=64.)
+    for (int tb = 0, per_launch; tb < T; tb += per_launch) {
+        const int left = T - tb;
+        per_launch = left >= 8 ? 8 : left >= 4 ? 4 : left >= 2 ? 2 : 1;
+        const int conc = std::max(1, std::min(8 / per_launch, P));
+        a.conc = conc; a.n_tiles = per_launch; a.tile_base = tb;
+        // Nothing orders the passes over the partitions: one launch walks all groups of `conc` partitions, group after
+        // group in workgroup order; the next group's first workgroups fill the compute units that the previous one's
+        // last workgroups leave idle (232,965-node graph, F=512: 13.64 -> 13.51 ms).
+        const int n_groups = (P + conc - 1) / conc;
+        a.n_groups = 0;
+        a.first_part = 0;
+        if (n_groups > 1 && n_groups <= kMaxGroups) {
+            a.n_groups = n_groups;
+            a.group_off[0] = 0;
+            for (int g = 0; g < n_groups; ++g) {
+                int64_t most = 0;
+                for (int p = g * conc; p < std::min(P, (g + 1) * conc); ++p) most = std::max(most, pl->item_off[p + 1] - pl->item_off[p]);
+                a.group_off[g + 1] = a.group_off[g] + (most + kWavesPerBlock - 1) / kWavesPerBlock;
+            }
+            const int64_t blocks = a.group_off[n_groups] * per_launch * conc;
+            if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
+            if (blocks > 0) {
+                const bool ok = (tile_sum || staged) ? launch_tiled_l<false>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a)
+                                                     : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
+                if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);
+            }
+            continue;
+        }
+        for (int p0 = 0; p0 < P; p0 += conc) {
             int64_t most = 0;
-            for (int p = g * conc; p < std::min(P, (g + 1) * conc); ++p) most = std::max(most, pl->item_off[p + 1] - pl->item_off[p]);
-            a.group_off[g + 1] = a.group_off[g] + (most + kWavesPerBlock - 1) / kWavesPerBlock;
-        }
-        const int64_t blocks = a.group_off[n_groups] * per_launch * conc;
-        if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
-        for (int tb = 0; tb < T && blocks > 0; tb += per_launch) {
-            a.tile_base = tb;
-            const bool ok = (tile_sum || staged) ? launch_tiled_l<false>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a)
-                                                 : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
-            if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);
-        }
-    }
-    for (int p0 = 0; p0 < P && a.n_groups == 0; p0 += conc) {
-        int64_t most = 0;
-        for (int p = p0; p < std::min(P, p0 + conc); ++p) most = std::max(most, pl->item_off[p + 1] - pl->item_off[p]);
-        if (most == 0) continue;
-        a.first_part = p0;
-        const int64_t blocks = ((most + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch * conc;
-        if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
-        for (int tb = 0; tb < T; tb += per_launch) {
-            a.tile_base = tb;
+            for (int p = p0; p < std::min(P, p0 + conc); ++p) most = std::max(most, pl->item_off[p + 1] - pl->item_off[p]);
+            if (most == 0) continue;
+            a.first_part = p0;
+            const int64_t blocks = ((most + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch * conc;
+            if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid too large");
             const bool ok = (tile_sum || staged) ? launch_tiled_l<false>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a)
                                                  : launch_tiled_l<true>(L, K, RW, KH, off32, dim3((unsigned)blocks), st, a);
             if (!ok) return fail(FG_ERR_SHAPE, "no tiled SDDMM kernel for L=%d K=%d RW=%d KH=%d", L, K, RW, KH);

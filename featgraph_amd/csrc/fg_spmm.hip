@@ -1018,6 +1018,13 @@ fg::ScratchNeed scratch_need(const fg_spmm_plan *pl, const SpmmConfig &c, int F,
     return need;
 }
 
+// Kernel tiles per launch: 8, 4, 2 or 1 -- counts that divide the 8 XCDs, so that workgroup id % tiles-per-launch
+// always puts a tile on the same XCDs and an L2 serves one tile's slice at a time (10 tiles: 8 + 2; 5: 4 + 1).  With
+// any other count every XCD would see every tile (232,965-node graph, F=640: 27.4 ms with 10 tiles in one launch).
+int tiles_this_launch(int remaining) {
+    return remaining >= 8 ? 8 : remaining >= 4 ? 4 : remaining >= 2 ? 2 : 1;
+}
+
 // reduce: FG_REDUCE_SUM / MAX / MIN.  heads > 1: vals is [nnz, heads] (or [heads, nnz] when
 // head_major).  vals == nullptr with allow_no_vals: every weight is 1.
 int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const float *vals,
@@ -1081,8 +1088,8 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
         a.heads = heads; a.head_len = F / heads;
         a.vstride = head_major ? 1 : heads; a.head_stride = head_major ? pl->nnz : 1;
         a.accumulate = 0;
-        const int per_launch = (c.n_ftiles > 8 && c.n_ftiles % 8 == 0) ? 8 : c.n_ftiles;
-        for (int tb = 0; tb < c.n_ftiles; tb += per_launch) {
+        for (int tb = 0, per_launch; tb < c.n_ftiles; tb += per_launch) {
+            per_launch = tiles_this_launch(c.n_ftiles - tb);
             a.n_ftiles = per_launch; a.tile_base = tb;
             const int64_t blocks = ((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
             if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
@@ -1116,8 +1123,8 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
             // More than 8 tiles: 8 at a time (one per XCD), so that an XCD's L2 serves one tile's
             // slice of this partition per launch; the partition's index arrays stay in the
             // memory-side cache between the launches.
-            const int per_launch = (c.n_ftiles > 8 && c.n_ftiles % 8 == 0) ? 8 : c.n_ftiles;
-            for (int tb = 0; tb < c.n_ftiles; tb += per_launch) {
+            for (int tb = 0, per_launch; tb < c.n_ftiles; tb += per_launch) {
+                per_launch = tiles_this_launch(c.n_ftiles - tb);
                 a.n_ftiles = per_launch; a.tile_base = tb;
                 const int64_t blocks = ((i1 - i0 + kWavesPerBlock - 1) / kWavesPerBlock) * per_launch;
                 if (blocks > 0x7fffffffLL) return fail(FG_ERR_SHAPE, "grid of %lld workgroups is too large", (long long)blocks);
