@@ -261,7 +261,26 @@ class SDDMMbase(object):
                 and (compute_args.get('num_feat_partitions', 1) or 1) == 1 and self._adj_row_indices.shape[0] > 0:
             schedule_args = self._tune(list(input_placeholders), dict(compute_args), dict(schedule_args), 6 if tune is True else int(tune))
         schedule_args = {k: v for k, v in schedule_args.items() if k != 'tune'}
+        # Single-head rows of an awkward length run at the next friendly one, on zero-padded copies of both operands
+        # (tuning.padded_feature_len): the extra columns add zeros to every dot product.
+        self._pad_from = None
+        given = list(input_placeholders)
+        if len(given) == 2 and len(given[0].shape) == 2 and len(given[1].shape) == 2 and given[0].shape[1] == given[1].shape[1] \
+                and schedule_args.get('pad_features', True) and not compute_args.get('num_feat_partitions') \
+                and not any(schedule_args.get(k) for k in ('num_feat_partitions', 'num_feat_tiles')):
+            D0 = given[0].shape[1]
+            want = tuning.padded_feature_len(D0)
+            if want != D0 and self._adj_row_indices.shape[0] * D0 >= tuning.PAD_MIN_GATHERED:
+                self._pad_from = D0
+                input_placeholders = [common.placeholder((given[0].shape[0], want)), common.placeholder((given[1].shape[0], want))]
+        schedule_args = {k: v for k, v in schedule_args.items() if k != 'pad_features'}
         phs, H, D, use_csr, tiled, notes = self._resolve(input_placeholders, compute_args, schedule_args)
+        self._src_pad = self._dst_pad = None
+        if self._pad_from is not None:
+            notes.append("rows of %d floats run as rows of %d on zero-padded copies" % (self._pad_from, D))
+            phs = given
+            self._src_pad = torch.zeros((self._num_cols, D), dtype=torch.float32, device=self._ctx)
+            self._dst_pad = torch.zeros((self._num_rows, D), dtype=torch.float32, device=self._ctx)
         self._placeholders = phs
         self._heads, self._head_len, self._use_csr, self._notes = H, D, use_csr, notes
         self._tiled = None
@@ -295,6 +314,10 @@ class SDDMMbase(object):
 
     def _launch(self, src_feat, dst_feat):
         s = common.stream_ptr()
+        if getattr(self, '_pad_from', None) is not None:
+            self._src_pad[:, :self._pad_from].copy_(src_feat)       # the padding columns stay zero
+            self._dst_pad[:, :self._pad_from].copy_(dst_feat)
+            src_feat, dst_feat = self._src_pad, self._dst_pad
         if self._tiled is not None:
             d, T = self._tiled
             _lib.check(_lib.lib().fg_sddmm_dds_f32(d['plan'], _lib.dev_ptr(d['pos']), _lib.dev_ptr(d['idx']),
@@ -347,7 +370,7 @@ class SDDMMbase(object):
 class VanillaSDDMMhip(SDDMMbase):
     """Edge-wise dot product on gfx950, optionally over a 2-D partitioned edge order."""
     _compute_keys = ('num_feat_partitions',)
-    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles', 'tune')
+    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles', 'tune', 'pad_features')
     _out_1d = True
 
     def __init__(self, adj_scipy, num_row_partitions=1, num_col_partitions=1):
@@ -361,13 +384,13 @@ class VanillaSDDMMhip(SDDMMbase):
 class VanillaSDDMMx86(VanillaSDDMMhip):
     """Constructor and knobs of the reference's VanillaSDDMMx86
     (python/featgraph/module/sddmm.py:168-176); the partitioned traversal runs on the GPU."""
-    _schedule_keys = ('num_feat_partitions', 'order', 'num_src_partitions', 'num_feat_tiles', 'tune')
+    _schedule_keys = ('num_feat_partitions', 'order', 'num_src_partitions', 'num_feat_tiles', 'tune', 'pad_features')
 
 
 class VanillaSDDMMcuda(VanillaSDDMMhip):
     """Constructor and knobs of the reference's VanillaSDDMMcuda
     (python/featgraph/module/sddmm.py:179-187): no partitioning, hence no edge_mapping."""
-    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles', 'tune')
+    _schedule_keys = ('num_feat_partitions', 'num_cuda_blocks', 'order', 'num_src_partitions', 'num_feat_tiles', 'tune', 'pad_features')
 
     def __init__(self, adj_scipy):
         super(VanillaSDDMMcuda, self).__init__(adj_scipy, num_row_partitions=1, num_col_partitions=1)

@@ -195,7 +195,20 @@ class SpMMbase(object):
             compute_args, schedule_args = self._tune(input_placeholders[0], dict(compute_args), dict(schedule_args),
                                                      6 if tune is True else int(tune))
         schedule_args = {k: v for k, v in schedule_args.items() if k != 'tune'}
+        # Rows of an awkward length run at the next friendly one, on zero-padded copies (tuning.padded_feature_len)
+        self._pad_from = None
+        ph0 = input_placeholders[0] if len(input_placeholders) == 1 else None
+        if ph0 is not None and len(ph0.shape) == 2 and schedule_args.get('pad_features', True) \
+                and not compute_args.get('num_feat_partitions') and not schedule_args.get('num_threads_per_cuda_block'):
+            want = tuning.padded_feature_len(ph0.shape[1])
+            if want != ph0.shape[1] and self._adj_indices.shape[0] * ph0.shape[1] >= tuning.PAD_MIN_GATHERED:
+                self._pad_from = ph0.shape[1]
+                input_placeholders = [common.placeholder((ph0.shape[0], want))]
+        schedule_args = {k: v for k, v in schedule_args.items() if k != 'pad_features'}
         ph, feat_len, T, P, notes = self._resolve(input_placeholders, compute_args, schedule_args)
+        if self._pad_from is not None:
+            notes.append("rows of %d floats run as rows of %d on zero-padded copies" % (self._pad_from, feat_len))
+            ph = ph0
         self._placeholders = [ph]
         self._feat_len = feat_len
         self._num_feat_partitions = T
@@ -203,7 +216,11 @@ class SpMMbase(object):
         self._active = self._layout(P)
         self._func = _lib.lib().fg_spmm_dds_f32 if P > 1 else _lib.lib().fg_spmm_csr_f32
         common.reserve(self._active['plan'], common.OP_SPMM_SUM, 1, feat_len, T, self._ctx)
-        self.out_tvm = torch.zeros((self._num_rows, feat_len), dtype=torch.float32, device=self._ctx)
+        self._x_pad = self._out_pad = None
+        if self._pad_from is not None:
+            self._x_pad = torch.zeros((self._num_cols, feat_len), dtype=torch.float32, device=self._ctx)
+            self._out_pad = torch.zeros((self._num_rows, feat_len), dtype=torch.float32, device=self._ctx)
+        self.out_tvm = torch.zeros((self._num_rows, self._pad_from or feat_len), dtype=torch.float32, device=self._ctx)
 
     def lower_to_ir(self, input_placeholders, compute_args, schedule_args):
         """Return a text description of the plan and launch. This can be useful for debug."""
@@ -217,9 +234,15 @@ class SpMMbase(object):
 
     def _launch(self, src_feat):
         lay = self._active
+        out = self.out_tvm
+        if getattr(self, '_pad_from', None) is not None:
+            self._x_pad[:, :self._pad_from].copy_(src_feat)         # the padding columns stay zero
+            src_feat, out = self._x_pad, self._out_pad
         _lib.check(self._func(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(lay['vals']),
-                              _lib.dev_ptr(src_feat), _lib.dev_ptr(self.out_tvm), self._feat_len,
+                              _lib.dev_ptr(src_feat), _lib.dev_ptr(out), self._feat_len,
                               self._num_feat_partitions, common.stream_ptr()))
+        if out is not self.out_tvm:
+            self.out_tvm.copy_(out[:, :self._pad_from])
 
     def run(self, input_tvm_ndarrays):
         """Run the built func with the given inputs.
@@ -261,7 +284,7 @@ class SpMMbase(object):
 class VanillaSpMMhip(SpMMbase):
     """CSR (or, with num_col_partitions > 1, DDS) SpMM on gfx950."""
     _compute_keys = ('num_feat_partitions',)
-    _schedule_keys = ('num_cuda_blocks', 'num_threads_per_cuda_block', 'num_src_partitions', 'tune')
+    _schedule_keys = ('num_cuda_blocks', 'num_threads_per_cuda_block', 'num_src_partitions', 'tune', 'pad_features')
 
     def __init__(self, adj_scipy, num_col_partitions=1):
         super(VanillaSpMMhip, self).__init__(adj_scipy, num_col_partitions)
@@ -275,7 +298,7 @@ class VanillaSpMMx86(VanillaSpMMhip):
     """Constructor and knobs of the reference's VanillaSpMMx86
     (python/featgraph/module/spmm.py:197-209): source-column partitions at init,
     'num_feat_partitions' at build.  Both partitionings are carried out on the GPU."""
-    _schedule_keys = ('num_src_partitions', 'tune')
+    _schedule_keys = ('num_src_partitions', 'tune', 'pad_features')
 
 
 class VanillaSpMMcuda(VanillaSpMMhip):

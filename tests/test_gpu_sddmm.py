@@ -327,3 +327,27 @@ def test_full_size_properties(torch_cuda):
     out_mh = mh.run([src.view(n, 4, 32), dst.view(n, 4, 32)])
     assert out_mh.shape == (nnz, 4)
     assert ((out_mh.sum(1) - out_csr).abs() <= ATOL + RTOL * out_csr.abs() + 1e-4).all()
+
+
+@pytest.mark.parametrize("feat_len", [30, 100, 200, 300])
+@pytest.mark.parametrize("shuffle", [False, True])
+def test_awkward_feature_lengths_run_on_padded_copies(torch_cuda, oracle, feat_len, shuffle):
+    """Rows whose length is no multiple of 32 run at the next friendly length on zero-padded copies of both operands
+    once the graph is large enough for that to pay: the same dot products, to rounding."""
+    from featgraph_amd import tuning
+    from featgraph_amd.module import VanillaSDDMMhip
+    rng = np.random.default_rng(70 + feat_len)
+    coo = _rand_coo(rng, 2500, 4000, 0.07, shuffle=shuffle)
+    assert coo.nnz * feat_len >= tuning.PAD_MIN_GATHERED
+    src = rng.standard_normal((4000, feat_len)).astype("float32")
+    dst = rng.standard_normal((2500, feat_len)).astype("float32")
+    ref, mass = oracle.sddmm_f64(coo.row, coo.col, src, dst), sddmm_mass(coo.row, coo.col, src, dst)
+    m, out = _run(torch_cuda, VanillaSDDMMhip, coo, src, dst, {}, {})
+    assert m._pad_from == feat_len and m._head_len == tuning.padded_feature_len(feat_len)
+    got = out.cpu().numpy()
+    assert_sum_close(got, ref, mass, "padded F=%d" % feat_len)
+    plain, out2 = _run(torch_cuda, VanillaSDDMMhip, coo, src, dst, {}, {'pad_features': False})
+    assert plain._pad_from is None
+    assert_sum_close(out2.cpu().numpy(), ref, mass, "unpadded F=%d" % feat_len)
+    m.out_tvm.fill_(float("nan"))
+    assert np.array_equal(m.run([torch_cuda.from_numpy(src).cuda(), torch_cuda.from_numpy(dst).cuda()]).cpu().numpy(), got)

@@ -368,3 +368,35 @@ def test_float64_adjacency_with_partitions(torch_cuda, oracle):
                              (VanillaSpMMhip, (), {'num_src_partitions': 5})):
         _, out = _run(torch_cuda, cls, adj64, x, {}, sched, *ctor)
         np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("feat_len", [30, 100, 200, 300])
+def test_awkward_feature_lengths_run_on_padded_copies(torch_cuda, oracle, feat_len):
+    """Rows whose length is no multiple of 32 run at the next friendly length on zero-padded copies once the graph is
+    large enough for that to pay; the result is that of the unpadded kernels (to rounding: the padded shape has other
+    tiles and partitions), every call overwrites all of out, and run() keeps returning the same tensor."""
+    from featgraph_amd import tuning
+    from featgraph_amd.module import VanillaSpMMhip
+    torch = torch_cuda
+    rng = np.random.default_rng(feat_len)
+    adj = _adj_with_long_and_empty_rows(rng, 3000, 3500, 2600)
+    adj = (adj + _rand_csr(rng, 3000, 3500, 0.06)).tocsr().astype("float32"); adj.sort_indices()
+    assert adj.nnz * feat_len >= tuning.PAD_MIN_GATHERED
+    x = rng.standard_normal((3500, feat_len)).astype("float32")
+    m, out = _run(torch, VanillaSpMMhip, adj, x, {}, {})
+    assert m._pad_from == feat_len and m._feat_len == tuning.padded_feature_len(feat_len) and tuple(out.shape) == (3000, feat_len)
+    got = out.cpu().numpy()
+    assert_sum_close(got, oracle.spmm_f64(adj, x), spmm_mass(adj, x), "padded F=%d" % feat_len)
+    plain, out2 = _run(torch, VanillaSpMMhip, adj, x, {}, {'pad_features': False})
+    assert plain._pad_from is None
+    assert_sum_close(out2.cpu().numpy(), oracle.spmm_f64(adj, x), spmm_mass(adj, x), "unpadded F=%d" % feat_len)
+    m.out_tvm.fill_(float("nan"))
+    again = m.run([torch.from_numpy(x).cuda()])
+    assert again is m.out_tvm and np.array_equal(again.cpu().numpy(), got)
+    assert "zero-padded" in "".join(m._notes)
+
+
+def test_padded_feature_lengths():
+    from featgraph_amd import tuning
+    assert [tuning.padded_feature_len(f) for f in (1, 8, 9, 16, 30, 32, 40, 64, 72, 96, 100, 128, 130, 160, 200, 500, 602, 640)] == \
+        [1, 8, 16, 16, 32, 32, 64, 64, 96, 96, 128, 128, 192, 160, 256, 512, 640, 640]
