@@ -78,8 +78,18 @@ class GSpMMhip(VanillaSpMMhip):
             schedule_args = dict(schedule_args, num_src_partitions=None)
             if self._num_col_partitions != 1:
                 raise ValueError("max / min aggregation needs num_col_partitions == 1")
+        # rows of an awkward length run at the next friendly one, on zero-padded copies (tuning.padded_feature_len)
+        self._pad_from = None
+        if heads == 1 and len(src_ph.shape) == 2 and not return_arg and schedule_args.get('pad_features', True) \
+                and not compute_args.get('num_feat_partitions'):
+            want = tuning.padded_feature_len(feat_len)
+            if want != feat_len and nnz * feat_len >= tuning.PAD_MIN_GATHERED:
+                self._pad_from, feat_len = feat_len, want
+        schedule_args = {k: v for k, v in schedule_args.items() if k != 'pad_features'}
         flat = common.placeholder((self._num_cols, feat_len))
         _, _, T, P, notes = self._resolve([flat], compute_args, schedule_args)
+        if self._pad_from is not None:
+            notes.append("rows of %d floats run as rows of %d on zero-padded copies" % (self._pad_from, feat_len))
         self._placeholders = list(input_placeholders)
         self._feat_len, self._heads, self._num_feat_partitions = feat_len, heads, (0 if heads > 1 and 'num_feat_partitions' not in compute_args else T)
         self._reduce, self._msg, self._weights_at_run, self._notes = reduce, msg, weights_at_run, notes
@@ -95,6 +105,10 @@ class GSpMMhip(VanillaSpMMhip):
             deg = np.diff(self._adj_indptr).astype(np.float32)
             inv = np.where(deg > 0, 1.0 / np.maximum(deg, 1), 0).astype(np.float32)
             self._inv_deg_edge = common.to_device_f32(np.repeat(inv, np.diff(self._adj_indptr)), self._ctx)
+        self._x_pad = self._out_pad = None
+        if self._pad_from is not None:
+            self._x_pad = torch.zeros((self._num_cols, feat_len), dtype=torch.float32, device=self._ctx)
+            self._out_pad = torch.zeros((self._num_rows, feat_len), dtype=torch.float32, device=self._ctx)
         self.out_tvm = torch.zeros((self._num_rows,) + tuple(src_ph.shape[1:]), dtype=torch.float32, device=self._ctx)
         self.arg_tvm = torch.full(self.out_tvm.shape, -1, dtype=torch.int32, device=self._ctx) if return_arg else None
 
@@ -133,6 +147,7 @@ class GSpMMhip(VanillaSpMMhip):
         common.take_args(schedule_args, self._schedule_keys, "schedule_func")
         op, lt, rt = general.parse_message(msg)
         nnz = self._adj_indices.shape[0]
+        self._pad_from = None
         # 'u_mul_e' with SrcFeat alone: the adjacency's own values are the edge operand (CSR order, already on the device)
         self._static_rhs = None
         if msg == 'u_mul_e' and len(input_placeholders) == 1:
@@ -308,9 +323,15 @@ class GSpMMhip(VanillaSpMMhip):
                                                    _lib.dev_ptr(self.arg_tvm), self._feat_len, heads, head_major,
                                                    _REDUCE[self._reduce], self._num_feat_partitions, common.stream_ptr()))
             return
+        out = self.out_tvm
+        if getattr(self, '_pad_from', None) is not None:
+            self._x_pad[:, :self._pad_from].copy_(src_feat)         # the padding columns stay zero
+            src_feat, out = self._x_pad, self._out_pad
         _lib.check(self._func(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(w),
-                              _lib.dev_ptr(src_feat), _lib.dev_ptr(self.out_tvm), self._feat_len, heads, head_major,
+                              _lib.dev_ptr(src_feat), _lib.dev_ptr(out), self._feat_len, heads, head_major,
                               _REDUCE[self._reduce], self._num_feat_partitions, common.stream_ptr()))
+        if out is not self.out_tvm:
+            self.out_tvm.copy_(out[:, :self._pad_from])
 
     def run(self, input_tvm_ndarrays):
         """[SrcFeat] or [SrcFeat, edge_weights]; returns self.out_tvm (overwritten in place)."""

@@ -213,3 +213,30 @@ def test_extreme_of_weighted_messages_with_positions(torch_cuda, oracle, reduce,
     assert np.array_equal(out, ref)
     ref_b, ref_arg = oracle.gspmm_bcast(adj.indptr, adj.indices, 'mul', reduce, x, w[:, None], 'u', 'e')
     assert np.array_equal(ref_b, ref) and np.array_equal(m.arg_tvm.cpu().numpy(), ref_arg)
+
+
+@pytest.mark.parametrize("reduce", ["sum", "mean"])
+def test_weights_given_at_run_with_an_awkward_feature_length(torch_cuda, oracle, reduce):
+    """One weight per edge given to run(), rows of 100 floats on a graph large enough for the padded copies."""
+    from featgraph_amd import tuning
+    from featgraph_amd.module import GSpMMhip, placeholder
+    torch = torch_cuda
+    rng = np.random.default_rng(17)
+    adj = sp.random(2500, 3000, density=0.06, format="csr", random_state=rng).astype("float32"); adj.sort_indices()
+    F = 100
+    assert adj.nnz * F >= tuning.PAD_MIN_GATHERED
+    x = rng.standard_normal((3000, F)).astype("float32")
+    w = rng.standard_normal(adj.nnz).astype("float32")
+    m = GSpMMhip(adj)
+    m.build([placeholder(x.shape), placeholder(w.shape)], {'reduce': reduce}, {})
+    assert m._pad_from == F and m._feat_len == 128
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()]).cpu().numpy()
+    aw = sp.csr_matrix((w, adj.indices, adj.indptr), shape=adj.shape)
+    ref = oracle.spmm_f64(aw, x)
+    mass = np.asarray(abs(aw).astype(np.float64).dot(np.abs(x).astype(np.float64)))
+    if reduce == "mean":
+        deg = np.maximum(np.diff(adj.indptr), 1)[:, None]
+        ref, mass = ref / deg, mass / deg
+    assert out.shape == (2500, F)
+    assert_sum_close(out, ref, mass, "padded weighted %s" % reduce)
