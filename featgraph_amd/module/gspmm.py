@@ -85,11 +85,17 @@ class GSpMMhip(VanillaSpMMhip):
             want = tuning.padded_feature_len(feat_len)
             if want != feat_len and nnz * feat_len >= tuning.PAD_MIN_GATHERED:
                 self._pad_from, feat_len = feat_len, want
+        elif heads > 1 and not return_arg and not compute_args.get('num_feat_partitions'):
+            # several heads: a head length the kernels have no tile for is padded to the next one they have
+            D0 = feat_len // heads
+            want = tuning.padded_head_len(D0)
+            if want != D0:
+                self._pad_from, feat_len = D0, heads * want
         schedule_args = {k: v for k, v in schedule_args.items() if k != 'pad_features'}
         flat = common.placeholder((self._num_cols, feat_len))
         _, _, T, P, notes = self._resolve([flat], compute_args, schedule_args)
         if self._pad_from is not None:
-            notes.append("rows of %d floats run as rows of %d on zero-padded copies" % (self._pad_from, feat_len))
+            notes.append("rows (heads) of %d floats run as rows of %d on zero-padded copies" % (self._pad_from, feat_len // heads))
         self._placeholders = list(input_placeholders)
         self._feat_len, self._heads, self._num_feat_partitions = feat_len, heads, (0 if heads > 1 and 'num_feat_partitions' not in compute_args else T)
         self._reduce, self._msg, self._weights_at_run, self._notes = reduce, msg, weights_at_run, notes
@@ -107,8 +113,9 @@ class GSpMMhip(VanillaSpMMhip):
             self._inv_deg_edge = common.to_device_f32(np.repeat(inv, np.diff(self._adj_indptr)), self._ctx)
         self._x_pad = self._out_pad = None
         if self._pad_from is not None:
-            self._x_pad = torch.zeros((self._num_cols, feat_len), dtype=torch.float32, device=self._ctx)
-            self._out_pad = torch.zeros((self._num_rows, feat_len), dtype=torch.float32, device=self._ctx)
+            tail = (feat_len,) if heads == 1 else (heads, feat_len // heads)
+            self._x_pad = torch.zeros((self._num_cols,) + tail, dtype=torch.float32, device=self._ctx)
+            self._out_pad = torch.zeros((self._num_rows,) + tail, dtype=torch.float32, device=self._ctx)
         self.out_tvm = torch.zeros((self._num_rows,) + tuple(src_ph.shape[1:]), dtype=torch.float32, device=self._ctx)
         self.arg_tvm = torch.full(self.out_tvm.shape, -1, dtype=torch.int32, device=self._ctx) if return_arg else None
 
@@ -325,13 +332,13 @@ class GSpMMhip(VanillaSpMMhip):
             return
         out = self.out_tvm
         if getattr(self, '_pad_from', None) is not None:
-            self._x_pad[:, :self._pad_from].copy_(src_feat)         # the padding columns stay zero
+            self._x_pad[..., :self._pad_from].copy_(src_feat)       # the padding columns stay zero
             src_feat, out = self._x_pad, self._out_pad
         _lib.check(self._func(lay['plan'], _lib.dev_ptr(lay['pos']), _lib.dev_ptr(lay['idx']), _lib.dev_ptr(w),
                               _lib.dev_ptr(src_feat), _lib.dev_ptr(out), self._feat_len, heads, head_major,
                               _REDUCE[self._reduce], self._num_feat_partitions, common.stream_ptr()))
         if out is not self.out_tvm:
-            self.out_tvm.copy_(out[:, :self._pad_from])
+            self.out_tvm.copy_(out[..., :self._pad_from])
 
     def run(self, input_tvm_ndarrays):
         """[SrcFeat] or [SrcFeat, edge_weights]; returns self.out_tvm (overwritten in place)."""

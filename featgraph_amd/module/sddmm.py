@@ -273,14 +273,24 @@ class SDDMMbase(object):
             if want != D0 and self._adj_row_indices.shape[0] * D0 >= tuning.PAD_MIN_GATHERED:
                 self._pad_from = D0
                 input_placeholders = [common.placeholder((given[0].shape[0], want)), common.placeholder((given[1].shape[0], want))]
+        elif len(given) == 2 and len(given[0].shape) == 3 and tuple(given[0].shape[1:]) == tuple(given[1].shape[1:]) \
+                and schedule_args.get('pad_features', True) and not compute_args.get('num_feat_partitions') \
+                and not any(schedule_args.get(k) for k in ('num_feat_partitions', 'num_feat_tiles')):
+            # several heads: every head padded to a length that fills whole lane groups (tuning.padded_head_len)
+            H0, D0 = given[0].shape[1], given[0].shape[2]
+            want = tuning.padded_head_len(D0)
+            if want != D0 and self._adj_row_indices.shape[0] * H0 * D0 >= tuning.PAD_MIN_GATHERED:
+                self._pad_from = D0
+                input_placeholders = [common.placeholder((given[0].shape[0], H0, want)), common.placeholder((given[1].shape[0], H0, want))]
         schedule_args = {k: v for k, v in schedule_args.items() if k != 'pad_features'}
         phs, H, D, use_csr, tiled, notes = self._resolve(input_placeholders, compute_args, schedule_args)
         self._src_pad = self._dst_pad = None
         if self._pad_from is not None:
             notes.append("rows of %d floats run as rows of %d on zero-padded copies" % (self._pad_from, D))
             phs = given
-            self._src_pad = torch.zeros((self._num_cols, D), dtype=torch.float32, device=self._ctx)
-            self._dst_pad = torch.zeros((self._num_rows, D), dtype=torch.float32, device=self._ctx)
+            tail = (D,) if len(given[0].shape) == 2 else (H, D)
+            self._src_pad = torch.zeros((self._num_cols,) + tail, dtype=torch.float32, device=self._ctx)
+            self._dst_pad = torch.zeros((self._num_rows,) + tail, dtype=torch.float32, device=self._ctx)
         self._placeholders = phs
         self._heads, self._head_len, self._use_csr, self._notes = H, D, use_csr, notes
         self._tiled = None
@@ -315,8 +325,8 @@ class SDDMMbase(object):
     def _launch(self, src_feat, dst_feat):
         s = common.stream_ptr()
         if getattr(self, '_pad_from', None) is not None:
-            self._src_pad[:, :self._pad_from].copy_(src_feat)       # the padding columns stay zero
-            self._dst_pad[:, :self._pad_from].copy_(dst_feat)
+            self._src_pad[..., :self._pad_from].copy_(src_feat)     # the padding columns stay zero
+            self._dst_pad[..., :self._pad_from].copy_(dst_feat)
             src_feat, dst_feat = self._src_pad, self._dst_pad
         if self._tiled is not None:
             d, T = self._tiled

@@ -121,8 +121,10 @@ def test_gspmm_errors(torch_cuda):
         m.build([placeholder((200, 8)), placeholder((7,))], {}, {})          # wrong weight shape
     with pytest.raises(ValueError):
         GSpMMhip(adj, 2).build([placeholder((200, 8))], {'reduce': 'max'}, {})
-    with pytest.raises(ValueError):                                          # head length 6: no kernel tile;
-        m.build([placeholder((200, 4, 6)), placeholder((adj.nnz, 4))], {}, {})   # refused when the scratch is sized
+    with pytest.raises(ValueError):                                          # head length 6 with a tiling of the caller's:
+        m.build([placeholder((200, 4, 6)), placeholder((adj.nnz, 4))], {'num_feat_partitions': 2}, {})   # no kernel tile
+    m.build([placeholder((200, 4, 6)), placeholder((adj.nnz, 4))], {}, {})       # left alone, the heads are padded to 8
+    assert m._pad_from == 6 and m._feat_len == 32
 
 
 @pytest.mark.parametrize("feat_len", [1, 3, 4, 20, 64, 256, 300, 1024])
@@ -240,3 +242,24 @@ def test_weights_given_at_run_with_an_awkward_feature_length(torch_cuda, oracle,
         ref, mass = ref / deg, mass / deg
     assert out.shape == (2500, F)
     assert_sum_close(out, ref, mass, "padded weighted %s" % reduce)
+
+
+@pytest.mark.parametrize("H,D", [(4, 6), (3, 20), (8, 48), (2, 100)])
+def test_per_head_weights_with_awkward_head_lengths(torch_cuda, oracle, H, D):
+    """Head lengths the kernels have no tile for are zero-padded to the next one they have."""
+    from featgraph_amd.module import GSpMMhip, placeholder
+    torch = torch_cuda
+    rng = np.random.default_rng(H * 100 + D)
+    adj = _graph(rng, 200, 1500, 1300)
+    x = rng.standard_normal((1500, H, D)).astype("float32")
+    w = rng.standard_normal((adj.nnz, H)).astype("float32")
+    m = GSpMMhip(adj)
+    m.build([placeholder(x.shape), placeholder(w.shape)], {}, {})
+    assert m._pad_from == D
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()]).cpu().numpy()
+    assert out.shape == (200, H, D)
+    for h in range(H):
+        ah = sp.csr_matrix((w[:, h], adj.indices, adj.indptr), shape=adj.shape)
+        mass = np.asarray(abs(ah).astype(np.float64).dot(np.abs(x[:, h]).astype(np.float64)))
+        assert_sum_close(out[:, h], oracle.spmm_f64(ah, x[:, h]), mass, "head %d of %dx%d" % (h, H, D))

@@ -351,3 +351,23 @@ def test_awkward_feature_lengths_run_on_padded_copies(torch_cuda, oracle, feat_l
     assert_sum_close(out2.cpu().numpy(), ref, mass, "unpadded F=%d" % feat_len)
     m.out_tvm.fill_(float("nan"))
     assert np.array_equal(m.run([torch_cuda.from_numpy(src).cuda(), torch_cuda.from_numpy(dst).cuda()]).cpu().numpy(), got)
+
+
+@pytest.mark.parametrize("H,D", [(3, 20), (8, 48), (2, 100)])
+def test_awkward_head_lengths_run_on_padded_copies(torch_cuda, oracle, H, D):
+    """Heads whose length is neither a power of two nor a multiple of 64 are zero-padded to the next such length."""
+    from featgraph_amd import tuning
+    from featgraph_amd.module import MultiHeadSDDMMhip
+    rng = np.random.default_rng(H * 1000 + D)
+    coo = _rand_coo(rng, 2500, 4000, 0.07)
+    assert coo.nnz * H * D >= tuning.PAD_MIN_GATHERED
+    src = rng.standard_normal((4000, H, D)).astype("float32")
+    dst = rng.standard_normal((2500, H, D)).astype("float32")
+    m, out = _run(torch_cuda, MultiHeadSDDMMhip, coo, src, dst, {}, {})
+    assert m._pad_from == D and m._head_len == tuning.padded_head_len(D) and tuple(out.shape) == (coo.nnz, H)
+    assert_sum_close(out.cpu().numpy(), oracle.sddmm_multihead_f64(coo.row, coo.col, src, dst),
+                     sddmm_mass(coo.row, coo.col, src, dst), "padded heads %dx%d" % (H, D))
+    plain, out2 = _run(torch_cuda, MultiHeadSDDMMhip, coo, src, dst, {}, {'pad_features': False})
+    assert plain._pad_from is None
+    assert_sum_close(out2.cpu().numpy(), oracle.sddmm_multihead_f64(coo.row, coo.col, src, dst),
+                     sddmm_mass(coo.row, coo.col, src, dst), "unpadded heads %dx%d" % (H, D))
