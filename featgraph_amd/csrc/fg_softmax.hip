@@ -37,6 +37,7 @@ struct SoftmaxArgs {
     float *y;
     float2 *stats;        // per (piece, head): forward (max, sum of exp); backward (sum of a * g, 0)
     int H;
+    int W;                // lanes of a wavefront in use when lanes are tied to heads: the largest multiple of H <= 64
 };
 
 // Combines `v` over the lanes that hold the same head (lane % H, H a power of two <= 64), or over
@@ -50,52 +51,72 @@ __device__ __forceinline__ float head_reduce(float v, int H) {
     return v;
 }
 
+// The same for any H <= 64: the lanes below W (the largest multiple of H that a wavefront holds) carry head
+// lane % H, the others carry nothing.  Windows of doubling length are folded towards the lanes below H, which
+// then hand every lane the result of its head.
+template <bool IS_MAX>
+__device__ __forceinline__ float head_reduce_any(float v, int H, int W, int lane) {
+    for (int off = H; off < W; off <<= 1) {
+        const float o = __shfl_down(v, off);
+        if (lane + off < W) v = IS_MAX ? fmaxf(v, o) : v + o;
+    }
+    return __shfl(v, lane % H);
+}
+
+// MODE 1: H a power of two, all 64 lanes in use; MODE 2: any H <= 64, W lanes in use.
+template <bool IS_MAX, int MODE>
+__device__ __forceinline__ float lanes_reduce(float v, int H, int W, int lane) {
+    return MODE == 2 ? head_reduce_any<IS_MAX>(v, H, W, lane) : head_reduce<IS_MAX>(v, H);
+}
+
 
 // A whole row of n <= 64 * R floats (H a power of two <= 64, so lane i always meets head i % H):
 // every lane's R loads are issued back to back, the row is read from memory once and the result
 // is formed in registers.  No load sits under a branch: lanes past the end re-read the last float.
-template <bool BWD, int R>
-__device__ __forceinline__ void row_in_registers(const float *x, const float *g, float *y, int n, int lane, int H) {
+// l0: the lane's first index (its lane number; past every run for a lane that is not in use), W: lanes in use.
+template <bool BWD, int R, int MODE>
+__device__ __forceinline__ void row_in_registers(const float *x, const float *g, float *y, int n, int lane, int l0, int W, int H) {
     float v[R], w[BWD ? R : 1];
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-        const int i = min(lane + 64 * k, n - 1);
+        const int i = min(l0 + W * k, n - 1);
         v[k] = x[i];
         if (BWD) w[k] = g[i];
     }
     if (!BWD) {
         float m = -INFINITY;
 #pragma unroll
-        for (int k = 0; k < R; ++k) m = (lane + 64 * k < n) ? fmaxf(m, v[k]) : m;
-        m = head_reduce<true>(m, H);
+        for (int k = 0; k < R; ++k) m = (l0 + W * k < n) ? fmaxf(m, v[k]) : m;
+        m = lanes_reduce<true, MODE>(m, H, W, lane);
         float s = 0.f;
 #pragma unroll
         for (int k = 0; k < R; ++k) {
-            v[k] = (lane + 64 * k < n) ? __expf(v[k] - m) : 0.f;
+            v[k] = (l0 + W * k < n) ? __expf(v[k] - m) : 0.f;
             s += v[k];
         }
-        s = head_reduce<false>(s, H);
+        s = lanes_reduce<false, MODE>(s, H, W, lane);
         const float inv = 1.0f / s;
 #pragma unroll
         for (int k = 0; k < R; ++k)
-            if (lane + 64 * k < n) y[lane + 64 * k] = v[k] * inv;
+            if (l0 + W * k < n) y[l0 + W * k] = v[k] * inv;
     } else {
         float d = 0.f;
 #pragma unroll
-        for (int k = 0; k < R; ++k) d += (lane + 64 * k < n) ? v[k] * w[k] : 0.f;
-        d = head_reduce<false>(d, H);
+        for (int k = 0; k < R; ++k) d += (l0 + W * k < n) ? v[k] * w[k] : 0.f;
+        d = lanes_reduce<false, MODE>(d, H, W, lane);
 #pragma unroll
         for (int k = 0; k < R; ++k)
-            if (lane + 64 * k < n) y[lane + 64 * k] = v[k] * (w[k] - d);
+            if (l0 + W * k < n) y[l0 + W * k] = v[k] * (w[k] - d);
     }
 }
 
 // One run of `len` elements starting at element e0, all lanes together.
-//   LANEHEAD: H divides 64, lane i always meets head i % H, values are read as one coalesced run.
-//   otherwise: one head at a time, lanes stride over the elements.
+//   LANEHEAD 1: H divides 64, lane i always meets head i % H, values are read as one coalesced run.
+//   LANEHEAD 2: any H <= 64: the same with the first W lanes (the largest multiple of H), the rest idle.
+//   LANEHEAD 0: one head at a time, lanes stride over the elements.
 // STATS_ONLY: write (max, sum) / (dot, 0) to stats[slot * H + h] instead of the result.
 // NORMALISE : the row statistics come from stats[slot * H + h] (merged over the row's pieces).
-template <bool BWD, bool LANEHEAD, bool STATS_ONLY, bool NORMALISE>
+template <bool BWD, int LANEHEAD, bool STATS_ONLY, bool NORMALISE>
 __device__ __forceinline__ void run_together(const SoftmaxArgs &a, int64_t e0, int len, int lane, int slot) {
     const int H = a.H;
     const int64_t base = e0 * H;
@@ -104,15 +125,17 @@ __device__ __forceinline__ void run_together(const SoftmaxArgs &a, int64_t e0, i
     float *y = a.y + base;
     if (LANEHEAD) {
         const int n = len * H;
+        const int W = LANEHEAD == 2 ? a.W : 64;
+        const int l0 = (LANEHEAD == 2 && lane >= W) ? (1 << 29) : lane;
         if (!STATS_ONLY && !NORMALISE) {
-            if (n <= 64 * 2) { row_in_registers<BWD, 2>(x, g, y, n, lane, H); return; }
-            if (n <= 64 * 4) { row_in_registers<BWD, 4>(x, g, y, n, lane, H); return; }
-            if (n <= 64 * 8) { row_in_registers<BWD, 8>(x, g, y, n, lane, H); return; }
+            if (n <= W * 2) { row_in_registers<BWD, 2, LANEHEAD>(x, g, y, n, lane, l0, W, H); return; }
+            if (n <= W * 4) { row_in_registers<BWD, 4, LANEHEAD>(x, g, y, n, lane, l0, W, H); return; }
+            if (n <= W * 8) { row_in_registers<BWD, 8, LANEHEAD>(x, g, y, n, lane, l0, W, H); return; }
         }
         // longer runs: sweeps of 8 loads per lane issued back to back (lanes past the end re-read
         // the last float, so no load sits under a branch)
         constexpr int U = 8;
-        const int h = lane & (H - 1);
+        const int h = LANEHEAD == 2 ? lane % H : lane & (H - 1);
         float m = 0.f, s = 0.f;
         if (NORMALISE) {
             const float2 st = a.stats[(int64_t)slot * H + h];
@@ -120,31 +143,31 @@ __device__ __forceinline__ void run_together(const SoftmaxArgs &a, int64_t e0, i
         } else if (!BWD) {
             // one sweep: running maximum, the sum rescaled whenever the maximum grows
             m = -INFINITY;
-            for (int i0 = lane; i0 < n + lane; i0 += 64 * U) {
+            for (int i0 = l0, b0 = 0; b0 < n; i0 += W * U, b0 += W * U) {
                 float v[U];
 #pragma unroll
-                for (int k = 0; k < U; ++k) v[k] = x[min(i0 + 64 * k, n - 1)];
+                for (int k = 0; k < U; ++k) v[k] = x[min(i0 + W * k, n - 1)];
 #pragma unroll
                 for (int k = 0; k < U; ++k) {
-                    const float vk = (i0 + 64 * k < n) ? v[k] : -INFINITY;
+                    const float vk = (i0 + W * k < n) ? v[k] : -INFINITY;
                     const float mn = fmaxf(m, vk);
                     s = (m == mn ? s : s * __expf(m - mn)) + (vk == -INFINITY ? 0.f : __expf(vk - mn));
                     m = mn;
                 }
             }
-            const float mw = head_reduce<true>(m, H);
+            const float mw = lanes_reduce<true, LANEHEAD>(m, H, W, lane);
             s = (m == -INFINITY) ? 0.f : s * __expf(m - mw);
             m = mw;
-            s = head_reduce<false>(s, H);
+            s = lanes_reduce<false, LANEHEAD>(s, H, W, lane);
         } else {
-            for (int i0 = lane; i0 < n + lane; i0 += 64 * U) {
+            for (int i0 = l0, b0 = 0; b0 < n; i0 += W * U, b0 += W * U) {
                 float v[U], w[U];
 #pragma unroll
-                for (int k = 0; k < U; ++k) { const int i = min(i0 + 64 * k, n - 1); v[k] = x[i]; w[k] = g[i]; }
+                for (int k = 0; k < U; ++k) { const int i = min(i0 + W * k, n - 1); v[k] = x[i]; w[k] = g[i]; }
 #pragma unroll
-                for (int k = 0; k < U; ++k) m += (i0 + 64 * k < n) ? v[k] * w[k] : 0.f;
+                for (int k = 0; k < U; ++k) m += (i0 + W * k < n) ? v[k] * w[k] : 0.f;
             }
-            m = head_reduce<false>(m, H);
+            m = lanes_reduce<false, LANEHEAD>(m, H, W, lane);
         }
         if (STATS_ONLY) {
             if (lane < H) a.stats[(int64_t)slot * H + lane] = make_float2(m, s);
@@ -152,22 +175,22 @@ __device__ __forceinline__ void run_together(const SoftmaxArgs &a, int64_t e0, i
         }
         if (!BWD) {
             const float inv = 1.0f / s;
-            for (int i0 = lane; i0 < n + lane; i0 += 64 * U) {
+            for (int i0 = l0, b0 = 0; b0 < n; i0 += W * U, b0 += W * U) {
                 float v[U];
 #pragma unroll
-                for (int k = 0; k < U; ++k) v[k] = x[min(i0 + 64 * k, n - 1)];
+                for (int k = 0; k < U; ++k) v[k] = x[min(i0 + W * k, n - 1)];
 #pragma unroll
                 for (int k = 0; k < U; ++k)
-                    if (i0 + 64 * k < n) y[i0 + 64 * k] = __expf(v[k] - m) * inv;
+                    if (i0 + W * k < n) y[i0 + W * k] = __expf(v[k] - m) * inv;
             }
         } else {
-            for (int i0 = lane; i0 < n + lane; i0 += 64 * U) {
+            for (int i0 = l0, b0 = 0; b0 < n; i0 += W * U, b0 += W * U) {
                 float v[U], w[U];
 #pragma unroll
-                for (int k = 0; k < U; ++k) { const int i = min(i0 + 64 * k, n - 1); v[k] = x[i]; w[k] = g[i]; }
+                for (int k = 0; k < U; ++k) { const int i = min(i0 + W * k, n - 1); v[k] = x[i]; w[k] = g[i]; }
 #pragma unroll
                 for (int k = 0; k < U; ++k)
-                    if (i0 + 64 * k < n) y[i0 + 64 * k] = v[k] * (w[k] - m);
+                    if (i0 + W * k < n) y[i0 + W * k] = v[k] * (w[k] - m);
             }
         }
         return;
@@ -202,7 +225,7 @@ __device__ __forceinline__ void run_together(const SoftmaxArgs &a, int64_t e0, i
 
 // PIECES == false: rows held whole by an item are finished, pieces write their statistics.
 // PIECES == true : pieces only, normalised with the merged statistics of their row.
-template <bool BWD, bool LANEHEAD, bool PIECES>
+template <bool BWD, int LANEHEAD, bool PIECES>
 __device__ __forceinline__ void edge_softmax_body(const SoftmaxArgs &a) {
     __shared__ float s_x[kWavesPerBlock][kStage];
     __shared__ float s_g[BWD ? kWavesPerBlock : 1][BWD ? kStage : 1];
@@ -317,11 +340,11 @@ __device__ __forceinline__ void edge_softmax_body(const SoftmaxArgs &a) {
 
 // The forward kernel is held to 64 registers (8 wavefronts per SIMD); the gradient kernel is bound
 // by its two LDS staging rows per wavefront instead.
-template <bool LANEHEAD, bool PIECES>
+template <int LANEHEAD, bool PIECES>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void edge_softmax_kernel(const SoftmaxArgs a) {
     edge_softmax_body<false, LANEHEAD, PIECES>(a);
 }
-template <bool LANEHEAD, bool PIECES>
+template <int LANEHEAD, bool PIECES>
 __global__ __launch_bounds__(kBlock) void edge_softmax_backward_kernel(const SoftmaxArgs a) {
     edge_softmax_body<true, LANEHEAD, PIECES>(a);
 }
@@ -354,7 +377,7 @@ __global__ __launch_bounds__(256) void edge_softmax_merge_kernel(const Fixup *fi
 // edge_softmax_head_major_kernel writes exp(x - max) / sum straight into the head-major, traversal-ordered
 // weight array that the per-head SpMM streams -- the [nnz, H] softmax array is never written or re-read.
 
-template <bool LANEHEAD>
+template <int LANEHEAD>
 __global__ __launch_bounds__(kBlock) void edge_softmax_stats_kernel(const SoftmaxArgs a, float2 *row_stats) {
     const int lane = threadIdx.x & 63;
     const int64_t item_id = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
@@ -441,7 +464,7 @@ __global__ __launch_bounds__(256) void edge_softmax_head_major_vec_kernel(const 
     }
 }
 
-template <bool BWD, bool LANEHEAD>
+template <bool BWD, int LANEHEAD>
 void launch_both(const fg_spmm_plan *pl, const SoftmaxArgs &a, hipStream_t st) {
     const dim3 grid((unsigned)((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock));
     if (BWD) hipLaunchKernelGGL((edge_softmax_backward_kernel<LANEHEAD, false>), grid, dim3(kBlock), 0, st, a);
@@ -454,6 +477,10 @@ void launch_both(const fg_spmm_plan *pl, const SoftmaxArgs &a, hipStream_t st) {
         else hipLaunchKernelGGL((edge_softmax_kernel<LANEHEAD, true>), grid, dim3(kBlock), 0, st, a);
     }
 }
+
+// How a wavefront's lanes meet the heads: 1: H divides 64; 2: any other H <= 64 (the lanes past the largest multiple of
+// H stay idle); 0: more heads than lanes, one head at a time.
+int lane_mode(int H) { return H > 64 ? 0 : (H & (H - 1)) == 0 ? 1 : 2; }
 
 int softmax_run(fg_spmm_plan *pl, const int32_t *indptr, const float *x, const float *g, float *y,
                 int H, void *stream, bool bwd) {
@@ -473,9 +500,17 @@ int softmax_run(fg_spmm_plan *pl, const int32_t *indptr, const float *x, const f
     a.items = pl->items_dev; a.n_items = pl->n_items; a.indptr = indptr;
     a.x = x; a.g = g; a.y = y; a.stats = reinterpret_cast<float2 *>(pl->partial_dev); a.H = H;
     hipStream_t st = (hipStream_t)stream;
-    const bool lanehead = H <= 64 && (H & (H - 1)) == 0;
-    if (bwd) { if (lanehead) launch_both<true, true>(pl, a, st); else launch_both<true, false>(pl, a, st); }
-    else { if (lanehead) launch_both<false, true>(pl, a, st); else launch_both<false, false>(pl, a, st); }
+    const int mode = lane_mode(H);
+    a.W = H <= 64 ? 64 / H * H : 64;
+    if (bwd) {
+        if (mode == 1) launch_both<true, 1>(pl, a, st);
+        else if (mode == 2) launch_both<true, 2>(pl, a, st);
+        else launch_both<true, 0>(pl, a, st);
+    } else {
+        if (mode == 1) launch_both<false, 1>(pl, a, st);
+        else if (mode == 2) launch_both<false, 2>(pl, a, st);
+        else launch_both<false, 0>(pl, a, st);
+    }
     FG_HIP_TRY(hipGetLastError());
     return FG_OK;
 }
@@ -516,8 +551,11 @@ extern "C" int fg_edge_softmax_stats_f32(fg_spmm_plan *pl, const int32_t *indptr
     hipStream_t st = (hipStream_t)stream;
     float2 *row_stats = reinterpret_cast<float2 *>(row_stats_dev);
     const dim3 grid((unsigned)((pl->n_items + kWavesPerBlock - 1) / kWavesPerBlock));
-    if (heads <= 64 && (heads & (heads - 1)) == 0) hipLaunchKernelGGL(edge_softmax_stats_kernel<true>, grid, dim3(kBlock), 0, st, a, row_stats);
-    else hipLaunchKernelGGL(edge_softmax_stats_kernel<false>, grid, dim3(kBlock), 0, st, a, row_stats);
+    a.W = heads <= 64 ? 64 / heads * heads : 64;
+    const int mode = lane_mode(heads);
+    if (mode == 1) hipLaunchKernelGGL(edge_softmax_stats_kernel<1>, grid, dim3(kBlock), 0, st, a, row_stats);
+    else if (mode == 2) hipLaunchKernelGGL(edge_softmax_stats_kernel<2>, grid, dim3(kBlock), 0, st, a, row_stats);
+    else hipLaunchKernelGGL(edge_softmax_stats_kernel<0>, grid, dim3(kBlock), 0, st, a, row_stats);
     if (pl->n_fixups > 0) {
         const int64_t threads = pl->n_fixups * heads;
         hipLaunchKernelGGL(edge_softmax_stats_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,

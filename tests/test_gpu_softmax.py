@@ -39,7 +39,7 @@ def _ragged(rng, kind):
 
 
 @pytest.mark.parametrize("kind", ["short", "medium", "hub"])
-@pytest.mark.parametrize("H", [1, 2, 3, 4, 8, 64])
+@pytest.mark.parametrize("H", [1, 2, 3, 4, 6, 8, 12, 33, 64, 65])   # 3, 6, 12, 33: lanes past the largest multiple of H idle; 65: one head at a time
 def test_edge_softmax_matches_oracle(torch_cuda, oracle, kind, H):
     from featgraph_amd.module import EdgeSoftmaxhip, placeholder
     torch = torch_cuda
