@@ -363,8 +363,11 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: weighted CSR SpMM + SDDMM over the same edges, F=%d, fp32, int32 indices" % (args.workload, F),
                    "nodes": n, "edges": nnz, "max_in_degree": int(deg.max()), "median_in_degree": float(np.median(deg)),
-                   "feat_len": F, "num_feat_partitions": args.num_feat_partitions,
-                   "num_col_partitions": args.num_col_partitions, "seeds": {"graph": 0xFEA7, "weights": 1, "features": 2}},
+                   "feat_len": F,
+                   # what ran (the library's own choice where the command line left the default: 0 tiles / 1 partition)
+                   "num_feat_partitions": spmm._num_feat_partitions, "num_col_partitions": spmm._active['P'],
+                   "requested": {"num_feat_partitions": args.num_feat_partitions, "num_col_partitions": args.num_col_partitions},
+                   "seeds": {"graph": 0xFEA7, "weights": 1, "features": 2}},
         "roofline": roofline,
         "verified": not failures,
         "gpu_mean_of_5_runs": runs5,
