@@ -27,6 +27,15 @@ def device():
     return torch.device("cuda", torch.cuda.current_device())
 
 
+def check_int32_sizes(num_rows, num_cols, nnz):
+    """The kernels address vertices and stored elements with int32 (every benchmark configuration fits); a larger
+    matrix would wrap around silently when its index arrays are narrowed, so it is refused here."""
+    limit = 2 ** 31 - 1
+    if num_rows >= limit or num_cols >= limit or nnz >= limit:
+        raise ValueError("a %d x %d adjacency with %d stored elements does not fit the kernels' int32 indices"
+                         % (num_rows, num_cols, nnz))
+
+
 def to_device_i32(a, dev):
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(dev)
 

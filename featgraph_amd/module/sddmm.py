@@ -36,6 +36,7 @@ class SDDMMbase(object):
             adj_scipy_coo = adj_scipy
         self._num_rows = adj_scipy_coo.shape[0]
         self._num_cols = adj_scipy_coo.shape[1]
+        common.check_int32_sizes(self._num_rows, self._num_cols, adj_scipy_coo.nnz)
         assert num_row_partitions >= 1, "num_row_partitions should be larger than or equal to 1"
         assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
         self._num_row_partitions = num_row_partitions

@@ -34,6 +34,7 @@ class SpMMbase(object):
             adj_scipy_csr = adj_scipy_csr.astype(np.float32)
         self._num_rows = adj_scipy_csr.shape[0]
         self._num_cols = adj_scipy_csr.shape[1]
+        common.check_int32_sizes(self._num_rows, self._num_cols, adj_scipy_csr.nnz)
         assert num_col_partitions >= 1, "num_col_partitions should be larger than or equal to 1"
         self._num_col_partitions = num_col_partitions
         self._target = None

@@ -296,3 +296,12 @@ def test_edge_mapping_restores_stored_order_for_unequal_partition_counts(fg, ora
     rb = row // -(-50 // R)
     cb = col // -(-70 // C)
     assert (np.diff(rb * C + cb) >= 0).all()
+
+
+def test_sizes_beyond_int32_are_refused():
+    """Index arrays are narrowed to int32 at construction; a matrix that does not fit must raise, not wrap."""
+    from featgraph_amd.module import common
+    common.check_int32_sizes(232965, 232965, 114766039)
+    for shape in [(2 ** 31, 10, 5), (10, 2 ** 31 - 1, 5), (10, 10, 2 ** 31 - 1)]:
+        with pytest.raises(ValueError, match="int32"):
+            common.check_int32_sizes(*shape)
