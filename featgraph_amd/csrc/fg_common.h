@@ -69,6 +69,10 @@ struct fg_spmm_plan {
     // tile-by-tile copy of the gathered operand(s) of the call in progress; grown the same way
     float *tiled_dev = nullptr;
     size_t tiled_floats = 0;
+    // 16-bit copy of the layout's (partition-local) column ids, made by fg_spmm_plan_narrow_indices and owned by the
+    // plan: the kernels that can read it do so whenever a call hands them the int32 array it was made from.
+    uint16_t *idx16_dev = nullptr;
+    const int32_t *idx16_src = nullptr;
     // statistics for fg_spmm_plan_describe
     int64_t max_len = 0, n_empty = 0, n_split_rows = 0, n_multi_items = 0;
 };
@@ -93,6 +97,10 @@ bool wants_tile_major(const fg_spmm_plan *plan, int n_tiles, uint64_t x_bytes);
 // the call fills copy `slot`.  The buffer must already be large enough (ensure_scratch).
 int make_tile_major(const fg_spmm_plan *plan, const float *x, int64_t n_rows, int F, int tile, void *stream,
                     int slot = 0, int n_slots = 1);
+// The plan's 16-bit copy of `idx` when it has one of exactly this array, else null.
+inline const uint16_t *narrow_indices(const fg_spmm_plan *plan, const int32_t *idx) {
+    return (plan->idx16_dev && idx && idx == plan->idx16_src) ? plan->idx16_dev : nullptr;
+}
 // FG_OK when the calling thread's current device is the one the plan was created on.
 int check_device(const fg_spmm_plan *plan);
 

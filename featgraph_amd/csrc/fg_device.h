@@ -7,8 +7,9 @@
 
 namespace fg {
 
-// Four consecutive words that are only known to be 4-byte aligned: read with one 128-bit load.
-template <typename T> struct __attribute__((packed, aligned(4))) Words4 { T v[4]; };
+// Four consecutive elements that are only known to be aligned like one of them (4 bytes for 32-bit words, 2 for
+// 16-bit ones): read with one 128-bit or 64-bit load.
+template <typename T> struct __attribute__((packed, aligned(sizeof(T) < 4 ? sizeof(T) : 4))) Words4 { T v[4]; };
 
 // o[i] = p[min(4 * lane + i, n - 1) * stride], n >= 1: the lane's four consecutive elements of a
 // stream of n, lanes past the end repeating the last element so that no load is conditional.

@@ -132,6 +132,7 @@ extern "C" void fg_spmm_plan_destroy(fg_spmm_plan *pl) {
     if (pl->fixups_dev) (void)hipFree(pl->fixups_dev);
     if (pl->partial_dev) (void)hipFree(pl->partial_dev);
     if (pl->tiled_dev) (void)hipFree(pl->tiled_dev);
+    if (pl->idx16_dev) (void)hipFree(pl->idx16_dev);
     delete pl;
 }
 
@@ -206,6 +207,41 @@ int ensure_scratch(fg_spmm_plan *pl, const ScratchNeed &need, void *stream) {
 std::string spmm_launch_text(const fg_spmm_plan *plan, int F, int num_feat_partitions);
 }
 
+namespace {
+// dst[i] = (uint16_t)src[i], four elements per lane (the tail one by one).
+__global__ __launch_bounds__(256) void narrow_indices_kernel(const int32_t *src, uint16_t *dst, int64_t n) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n) return;
+    for (int k = 0; k < 4 && i + k < n; ++k) dst[i + k] = (uint16_t)src[i + k];
+}
+}  // namespace
+
+extern "C" int fg_spmm_plan_narrow_indices(fg_spmm_plan *pl, const int32_t *idx_dev, void *stream) {
+    if (!pl) return fail(FG_ERR_ARG, "plan is null");
+    if (int drc = fg::check_device(pl)) return drc;
+    if (!idx_dev) {                                  // forget the copy
+        if (pl->idx16_dev) FG_HIP_TRY(hipFree(pl->idx16_dev));
+        pl->idx16_dev = nullptr; pl->idx16_src = nullptr;
+        return FG_OK;
+    }
+    const int64_t width = (pl->n_src + pl->num_col_partitions - 1) / pl->num_col_partitions;
+    if (width > 65536)
+        return fail(FG_ERR_SHAPE, "column ids of partitions %lld columns wide do not fit 16 bits", (long long)width);
+    if (pl->idx16_dev) FG_HIP_TRY(hipFree(pl->idx16_dev));
+    pl->idx16_dev = nullptr; pl->idx16_src = nullptr;
+    if (pl->nnz == 0) return FG_OK;
+    if (hipMalloc((void **)&pl->idx16_dev, (size_t)pl->nnz * sizeof(uint16_t)) != hipSuccess) {
+        (void)hipGetLastError();
+        pl->idx16_dev = nullptr;
+        return fail(FG_ERR_NOMEM, "cannot allocate %zu bytes for the 16-bit column ids", (size_t)pl->nnz * sizeof(uint16_t));
+    }
+    const int64_t blocks = (pl->nnz + 1023) / 1024;
+    hipLaunchKernelGGL(narrow_indices_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, idx_dev, pl->idx16_dev, pl->nnz);
+    FG_HIP_TRY(hipGetLastError());
+    pl->idx16_src = idx_dev;
+    return FG_OK;
+}
+
 extern "C" int fg_spmm_plan_reserve(fg_spmm_plan *pl, int op, int heads, int head_len, int num_feat_partitions) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (int drc = fg::check_device(pl)) return drc;
@@ -241,6 +277,7 @@ extern "C" int fg_spmm_plan_describe(const fg_spmm_plan *pl, int F, int T, char 
              (long long)pl->n_items, (long long)pl->n_multi_items, pl->item_edges, pl->split_threshold, (long long)pl->n_split_rows,
              (long long)pl->n_slots, (long long)pl->max_len, (long long)pl->n_empty);
     std::string s = head;
+    if (pl->idx16_dev) s += "  column ids       : a 16-bit copy is streamed by the sum SpMM and the tiled SDDMM\n";
     if (F > 0) s += fg::spmm_launch_text(pl, F, T);
     const size_t n = std::min(s.size(), buf_len - 1);
     memcpy(buf, s.data(), n);

@@ -248,6 +248,7 @@ struct SddmmTiledArgs {
     const int32_t *pos;       // row boundaries, one array of pos_stride entries per partition
     int64_t pos_stride;
     const int32_t *col;       // partition-local column ids, DDS order
+    const uint16_t *col16;    // the plan's 16-bit copy of `col`, read instead of it (null: none)
     const int32_t *edge_pos;  // DDS position -> position in the caller's edge order
     const float *src;         // partition p's first src row is src + p * src_stride
     int64_t src_stride;
@@ -413,7 +414,14 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     auto stage = [&](int64_t base, int n) {
         // lane l holds edges 4l .. 4l + 3 (past the end: the last edge again)
         int32_t c[4], at[4] = {0, 0, 0, 0};
-        fg::load_four(a.col + base, n, lane, 1, c);
+        if (a.col16) {
+            uint16_t c16[4];
+            fg::load_four(a.col16 + base, n, lane, 1, c16);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) c[i] = c16[i];
+        } else {
+            fg::load_four(a.col + base, n, lane, 1, c);
+        }
         if (SCATTER) fg::load_four(a.edge_pos + base, n, lane, 1, at);
 #pragma unroll
         for (int i = 0; i < 4; ++i) c[i] = (int)((uint32_t)c[i] * scale);
@@ -881,7 +889,7 @@ extern "C" int fg_sddmm_dds_f32(fg_spmm_plan *pl, const int32_t *s1_pos_dev, con
     const bool tile_sum = ts.tile_sum, staged = ts.staged, off32 = ts.off32;
     hipStream_t st = (hipStream_t)stream;
     SddmmTiledArgs a;
-    a.col = s1_idx_dev; a.edge_pos = edge_pos_dev; a.dst = dst_dev; a.F = F; a.n_tiles = T;
+    a.col = s1_idx_dev; a.col16 = fg::narrow_indices(pl, s1_idx_dev); a.edge_pos = edge_pos_dev; a.dst = dst_dev; a.F = F; a.n_tiles = T;
     if (tile_sum) {
         a.out = pl->partial_dev; a.out_edge_stride = 1; a.out_tile_stride = (pl->nnz + 3) & ~(int64_t)3;
     } else if (staged) {

@@ -56,6 +56,7 @@ struct SpmmArgs {
     int64_t n_items;
     const int32_t *pos;    // this partition's position array (row boundaries), n_dst + 1 entries
     const int32_t *indices;
+    const uint16_t *indices16 = nullptr;   // the plan's 16-bit copy of `indices` (null: none), read by the sum kernel
     const float *vals;
     const float *x;        // already offset to the partition's first source row
     // Sum, max and min kernels, 32-bit offsets only.  Bytes between consecutive source rows, and, when the
@@ -198,11 +199,19 @@ __device__ __forceinline__ void finish_row(typename Vec<V>::type (&acc)[K], cons
 // elements 4l .. 4l + 3.  n >= 1.
 // `scale` turns a column id into the staged word: the row's byte size (OFF32) or 1.  The weight of
 // element t is vals[t * vstride + voff] (one weight per head), or 1 when there are no weights.
-__device__ __forceinline__ void stage_load(const int32_t *indices, const float *vals, int64_t base, int n,
+// indices16 (uniform; null: none): the same ids as 16-bit words, read instead of `indices`.
+__device__ __forceinline__ void stage_load(const int32_t *indices, const uint16_t *indices16, const float *vals, int64_t base, int n,
                                            int lane, uint32_t scale, int vstride, int64_t voff, int2 (&r)[4]) {
     int32_t c[4];
     float w[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-    fg::load_four(indices + base, n, lane, 1, c);
+    if (indices16) {
+        uint16_t c16[4];
+        fg::load_four(indices16 + base, n, lane, 1, c16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) c[i] = c16[i];
+    } else {
+        fg::load_four(indices + base, n, lane, 1, c);
+    }
     if (vals) fg::load_four(vals + base * vstride + voff, n, lane, vstride, w);
 #pragma unroll
     for (int i = 0; i < 4; ++i) r[i] = make_int2((int)((uint32_t)c[i] * scale), __float_as_int(w[i]));
@@ -318,7 +327,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
             }
         }
         if (it.len > 0) {
-            stage_load(a.indices, col_vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
+            stage_load(a.indices, a.indices16, col_vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
             if (HPT > 1) stage_load_w<HPT>(a.vals, it.start, it.len, lane, a.vstride, voff, a.head_stride, wregs);
             stage_store(edge, lane, regs);
             if (HPT > 1) stage_store_w<HPT>(s_w[wave], lane, wregs);
@@ -427,7 +436,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
 #pragma unroll
     for (int k = 0; k < K; ++k) acc[k] = vzero(vec());
     if (it.len > 0) {
-        stage_load(a.indices, col_vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
+        stage_load(a.indices, a.indices16, col_vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
         if (HPT > 1) stage_load_w<HPT>(a.vals, it.start, it.len, lane, a.vstride, voff, a.head_stride, wregs);
     }
     if (ACC) {
@@ -442,7 +451,7 @@ __device__ __forceinline__ void spmm_items_body(const SpmmArgs &a) {
         if (HPT > 1) stage_store_w<HPT>(s_w[wave], lane, wregs);
         wave_lds_sync();
         if (base + fg::kItemEdges < it.len) {
-            stage_load(a.indices, col_vals, (int64_t)it.start + base + fg::kItemEdges,
+            stage_load(a.indices, a.indices16, col_vals, (int64_t)it.start + base + fg::kItemEdges,
                        it.len - base - fg::kItemEdges, lane, scale, a.vstride, voff, regs);
             if (HPT > 1)
                 stage_load_w<HPT>(a.vals, (int64_t)it.start + base + fg::kItemEdges, it.len - base - fg::kItemEdges,
@@ -568,7 +577,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_extreme_kernel(const SpmmArgs a)
     if (it.info < -1) {
         const int nrows = -it.info;
         if (it.len > 0) {
-            stage_load(a.indices, a.vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
+            stage_load(a.indices, nullptr, a.vals, it.start, it.len, lane, scale, a.vstride, voff, regs);
             stage_store(edge, lane, regs);
         }
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
@@ -587,7 +596,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_extreme_kernel(const SpmmArgs a)
     for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
         const int n = min(fg::kItemEdges, it.len - base);
         wave_lds_sync();
-        stage_load(a.indices, a.vals, (int64_t)it.start + base, n, lane, scale, a.vstride, voff, regs);
+        stage_load(a.indices, nullptr, a.vals, (int64_t)it.start + base, n, lane, scale, a.vstride, voff, regs);
         stage_store(edge, lane, regs);
         wave_lds_sync();
         walk(0, n);
@@ -720,7 +729,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_arg_kernel(const SpmmArgs a) {
     if (it.info < -1) {
         const int nrows = -it.info;
         if (it.len > 0) {
-            stage_load(a.indices, a.vals, it.start, it.len, lane, 1u, a.vstride, voff, regs);
+            stage_load(a.indices, nullptr, a.vals, it.start, it.len, lane, 1u, a.vstride, voff, regs);
             stage_store(edge, lane, regs);
         }
         s_end[wave][lane] = a.pos[it.row + min(lane, nrows - 1) + 1] - it.start;
@@ -745,7 +754,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_arg_kernel(const SpmmArgs a) {
     for (int32_t base = 0; base < it.len; base += fg::kItemEdges) {
         const int n = min(fg::kItemEdges, it.len - base);
         wave_lds_sync();
-        stage_load(a.indices, a.vals, (int64_t)it.start + base, n, lane, 1u, a.vstride, voff, regs);
+        stage_load(a.indices, nullptr, a.vals, (int64_t)it.start + base, n, lane, 1u, a.vstride, voff, regs);
         stage_store(edge, lane, regs);
         wave_lds_sync();
         walk(0, n, it.start + base);
@@ -1078,7 +1087,7 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
         a.items = pl->items_dev; a.n_items = pl->n_items;
         a.item_off = pl->item_off_dev; a.n_parts = P;
         a.pos = pos; a.pos_stride = pl->n_dst + 1;
-        a.indices = idx; a.vals = vals;
+        a.indices = idx; a.indices16 = fg::narrow_indices(pl, idx); a.vals = vals;
         a.x = tiled ? pl->tiled_dev : x; a.x_stride = width * (tiled ? ft : F);
         a.x_row_bytes = (uint32_t)(tiled ? ft : F) * 4u;
         a.x_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * ft * 4u) : 0u;
@@ -1111,7 +1120,7 @@ int spmm_run(fg_spmm_plan *pl, const int32_t *pos, const int32_t *idx, const flo
             SpmmArgs a;
             a.items = pl->items_dev + i0; a.n_items = i1 - i0;
             a.pos = pos + (int64_t)p * (pl->n_dst + 1);
-            a.indices = idx; a.vals = vals;
+            a.indices = idx; a.indices16 = fg::narrow_indices(pl, idx); a.vals = vals;
             a.x = tiled ? pl->tiled_dev + (int64_t)p * width * ft : x + (int64_t)p * width * F;
             a.x_row_bytes = (uint32_t)(tiled ? ft : F) * 4u;
             a.x_tile_bytes = tiled ? (uint32_t)((uint64_t)pl->n_src * ft * 4u) : 0u;

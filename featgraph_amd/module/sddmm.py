@@ -123,6 +123,7 @@ class SDDMMbase(object):
         with torch.cuda.device(self._ctx):
             _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(s1_pos), self._num_rows, self._num_cols, P, _lib.plan_opts_ptr(),
                                                       ctypes.byref(d['plan'])))
+        common.narrow_indices(d['plan'], d['idx'], self._num_cols, P, self._ctx)
         self._dds[P] = d
         return d
 

@@ -85,6 +85,7 @@ class SpMMbase(object):
         with torch.cuda.device(self._ctx):
             _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(pos), self._num_rows, self._num_cols, P, _lib.plan_opts_ptr(),
                                                       ctypes.byref(lay['plan'])))
+        common.narrow_indices(lay['plan'], lay['idx'], self._num_cols, P, self._ctx)
         self._layouts[P] = lay
         return lay
 

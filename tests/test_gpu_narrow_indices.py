@@ -1,0 +1,149 @@
+"""16-bit copy of a layout's column ids (fg_spmm_plan_narrow_indices): the sum SpMM and the tiled SDDMM read it
+instead of the int32 array whenever a partition is at most 65,536 columns wide.  The ids are the same, so every
+result must agree bit for bit with the int32 stream -- on graphs with empty rows, rows split over wavefronts,
+item starts at odd element positions (a 16-bit word is only 2-byte aligned there) and ids up to 65,535."""
+import ctypes
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+from helpers import assert_sum_close, spmm_mass
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph(rng, n_rows=500, n_cols=4000, long_len=2700):
+    a = sp.random(n_rows, n_cols, density=0.012, format="csr", random_state=rng,
+                  data_rvs=lambda k: rng.standard_normal(k)).astype("float32").tolil()
+    a[[0, 1, n_rows // 2, n_rows - 1], :] = 0
+    a[3, :] = 0
+    a[3, [n_cols - 1]] = 2.0                                            # one element: later rows start at odd positions
+    a[7, rng.choice(n_cols, size=long_len, replace=False)] = 1.5       # longer than the split threshold
+    a = a.tocsr().astype("float32"); a.eliminate_zeros(); a.sort_indices()
+    return a
+
+
+def _with(narrow, fn):
+    from featgraph_amd.module import common
+    old = common.NARROW_INDICES
+    common.NARROW_INDICES = narrow
+    try:
+        return fn()
+    finally:
+        common.NARROW_INDICES = old
+
+
+@pytest.mark.parametrize("feat_len,P,T", [(128, 1, 0), (128, 2, 2), (64, 8, 0), (512, 4, 8), (96, 3, 3), (32, 5, 1), (7, 3, 1)])
+def test_spmm_bit_identical(oracle, feat_len, P, T):
+    import torch
+    from featgraph_amd.module import VanillaSpMMhip, placeholder
+    rng = np.random.default_rng(100 + feat_len + P)
+    adj = _graph(rng)
+    x = rng.standard_normal((adj.shape[1], feat_len)).astype("float32")
+    xd = torch.from_numpy(x).cuda()
+
+    def run():
+        m = VanillaSpMMhip(adj, P)
+        m.build([placeholder(x.shape)], {'num_feat_partitions': T}, {'num_src_partitions': None})
+        m.out_tvm.fill_(float("nan"))
+        return m.run([xd]).cpu().numpy().copy()
+
+    wide, narrow = _with(False, run), _with(True, run)
+    assert np.array_equal(wide, narrow)
+    assert_sum_close(narrow, oracle.spmm_f64(adj, x), spmm_mass(adj, x), "F=%d P=%d T=%d" % (feat_len, P, T))
+
+
+def test_per_head_weights_bit_identical():
+    import torch
+    from featgraph_amd.module import GSpMMhip, placeholder
+    rng = np.random.default_rng(5)
+    adj = _graph(rng)
+    H, D = 4, 32
+    x = rng.standard_normal((adj.shape[1], H, D)).astype("float32")
+    w = rng.random((adj.nnz, H)).astype("float32")
+
+    def run():
+        m = GSpMMhip(adj, 3)
+        m.build([placeholder(x.shape), placeholder(w.shape)], {}, {'num_src_partitions': None})
+        return m.run([torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()]).cpu().numpy().copy()
+
+    assert np.array_equal(_with(False, run), _with(True, run))
+
+
+@pytest.mark.parametrize("H,D,P,T", [(1, 128, 2, 2), (1, 512, 3, 8), (1, 64, 4, 1), (4, 32, 2, 2), (8, 64, 2, 8)])
+def test_sddmm_tiled_bit_identical(H, D, P, T):
+    import torch
+    from featgraph_amd.module import VanillaSDDMMhip, MultiHeadSDDMMhip, placeholder
+    rng = np.random.default_rng(200 + H * D + P)
+    adj = _graph(rng)
+    shape_s = (adj.shape[1], D) if H == 1 else (adj.shape[1], H, D)
+    shape_d = (adj.shape[0], D) if H == 1 else (adj.shape[0], H, D)
+    src = rng.standard_normal(shape_s).astype("float32")
+    dst = rng.standard_normal(shape_d).astype("float32")
+
+    def run():
+        m = (VanillaSDDMMhip if H == 1 else MultiHeadSDDMMhip)(adj)
+        m.build([placeholder(shape_s), placeholder(shape_d)], {}, {'order': 'tiled', 'num_src_partitions': P, 'num_feat_tiles': T})
+        m.out_tvm.fill_(float("nan"))
+        return m.run([torch.from_numpy(src).cuda(), torch.from_numpy(dst).cuda()]).cpu().numpy().copy()
+
+    wide, narrow = _with(False, run), _with(True, run)
+    assert np.array_equal(wide, narrow)
+    coo = adj.tocoo()
+    ref = np.einsum('e...d,e...d->e...', src[coo.col].astype(np.float64), dst[coo.row].astype(np.float64))
+    np.testing.assert_allclose(narrow, ref, rtol=1e-4, atol=1e-3)
+
+
+def test_ids_up_to_65535_and_other_arrays():
+    """C ABI directly: a 65,536-column partition's largest id survives the narrowing; a call that hands the kernels
+    another index array than the one that was narrowed reads that array (as int32); releasing the copy works."""
+    import torch
+    from featgraph_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(9)
+    n_dst, n_src, F = 300, 65536, 64
+    rows = []
+    for r in range(n_dst):
+        cols = np.unique(np.concatenate([rng.integers(0, n_src, size=rng.integers(0, 40)), [65535] if r % 3 == 0 else []])).astype(np.int32)
+        rows.append(cols)
+    indptr = np.zeros(n_dst + 1, np.int32)
+    indptr[1:] = np.cumsum([len(c) for c in rows])
+    indices = np.concatenate(rows).astype(np.int32)
+    vals = rng.random(indices.shape[0]).astype("float32")
+    x = rng.standard_normal((n_src, F)).astype("float32")
+    ref = sp.csr_matrix((vals.astype(np.float64), indices, indptr), shape=(n_dst, n_src)).dot(x.astype(np.float64))
+    plan = ctypes.c_void_p()
+    _lib.check(L.fg_spmm_plan_create(_lib.host_ptr(indptr), n_dst, n_src, 1, None, ctypes.byref(plan)))
+    try:
+        ip, ix, vl, xd = (torch.from_numpy(a).cuda() for a in (indptr, indices, vals, x))
+        ix_other = ix.clone()
+        out = torch.empty((n_dst, F), device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def spmm(idx):
+            out.fill_(float("nan"))
+            _lib.check(L.fg_spmm_csr_f32(plan, _lib.dev_ptr(ip), _lib.dev_ptr(idx), _lib.dev_ptr(vl), _lib.dev_ptr(xd),
+                                         _lib.dev_ptr(out), F, 0, stream))
+            return out.cpu().numpy().copy()
+
+        base = spmm(ix)
+        _lib.check(L.fg_spmm_plan_narrow_indices(plan, _lib.dev_ptr(ix), stream))
+        assert np.array_equal(spmm(ix), base)
+        np.testing.assert_allclose(base, ref, rtol=1e-4, atol=1e-4)
+        # the narrowed array's contents no longer matter to a call that passes another array
+        assert np.array_equal(spmm(ix_other), base)
+        _lib.check(L.fg_spmm_plan_narrow_indices(plan, None, stream))
+        assert np.array_equal(spmm(ix), base)
+    finally:
+        L.fg_spmm_plan_destroy(plan)
+    # partitions wider than 65,536 columns are refused
+    indptr2 = np.zeros(3, np.int32)
+    plan2 = ctypes.c_void_p()
+    _lib.check(L.fg_spmm_plan_create(_lib.host_ptr(indptr2), 2, 65537, 1, None, ctypes.byref(plan2)))
+    try:
+        dummy = torch.zeros(4, dtype=torch.int32, device="cuda")
+        assert L.fg_spmm_plan_narrow_indices(plan2, _lib.dev_ptr(dummy), None) == -2
+        assert b"16 bits" in L.fg_last_error()
+    finally:
+        L.fg_spmm_plan_destroy(plan2)
