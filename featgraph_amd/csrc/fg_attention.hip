@@ -37,6 +37,7 @@ struct AttnArgs {
     int64_t n_items;
     const int32_t *pos;       // this partition's row boundaries
     const int32_t *indices;   // partition-local column ids
+    const uint16_t *indices16 = nullptr;   // the plan's 16-bit copy of them, read instead (null: none)
     const float *q;           // [n_dst, F]
     const float *k, *v;       // offset to the partition's first source row
     uint32_t kv_row_bytes;    // bytes between consecutive rows of k / v
@@ -253,7 +254,7 @@ __global__ __launch_bounds__(kBlock) void attention_items_kernel(const AttnArgs 
 
     auto stage = [&](int64_t base, int n) {
         int32_t c[4];
-        fg::load_four(a.indices + base, n, lane, 1, c);
+        fg::load_four_ids(a.indices, a.indices16, base, n, lane, c);
         uint32_t b[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) b[i] = (uint32_t)c[i] * a.kv_row_bytes;
@@ -467,7 +468,7 @@ int run_forward(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev
         AttnArgs a;
         a.items = pl->items_dev; a.n_items = pl->n_items; a.item_off = pl->item_off_dev; a.n_parts = P;
         a.pos = pos_dev; a.pos_stride = pl->n_dst + 1;
-        a.indices = idx_dev; a.q = q_dev;
+        a.indices = idx_dev; a.indices16 = fg::narrow_indices(pl, idx_dev); a.q = q_dev;
         a.k = k; a.k_stride = ADD ? width : width * row_floats;
         a.v = v; a.v_stride = width * row_floats;
         a.kv_row_bytes = (uint32_t)row_floats * 4u;
@@ -499,7 +500,7 @@ int run_forward(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_dev
         AttnArgs a;
         a.items = pl->items_dev + i0; a.n_items = i1 - i0;
         a.pos = pos_dev + (int64_t)p * (pl->n_dst + 1);
-        a.indices = idx_dev; a.q = q_dev;
+        a.indices = idx_dev; a.indices16 = fg::narrow_indices(pl, idx_dev); a.q = q_dev;
         a.k = ADD ? k + (int64_t)p * width : k + (int64_t)p * width * row_floats;
         a.v = v + (int64_t)p * width * row_floats;
         a.kv_row_bytes = (uint32_t)row_floats * 4u;

@@ -62,6 +62,7 @@ struct BwdArgs {
     int64_t n_items;
     const int32_t *pos;
     const int32_t *indices;   // partition-local ids of the far side
+    const uint16_t *indices16 = nullptr;   // the plan's 16-bit copy of them, read instead (null: none)
     const float *own0, *own1; // [n_own, F]: (Q, dout) or (K, V)
     const float *far0, *far1; // offset to the partition's first far row: (K, V) or (Q, dout)
     uint32_t far_row_bytes, far_tile_bytes;
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(kBlock) void attention_backward_kernel(const BwdArg
 
     auto stage = [&](int64_t base, int n) {
         int32_t c[4];
-        fg::load_four(a.indices + base, n, lane, 1, c);
+        fg::load_four_ids(a.indices, a.indices16, base, n, lane, c);
         W w[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -369,7 +370,7 @@ int run_backward(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx_de
         BwdArgs a;
         a.items = pl->items_dev + i0; a.n_items = i1 - i0;
         a.pos = pos_dev + (int64_t)p * (pl->n_dst + 1);
-        a.indices = idx_dev;
+        a.indices = idx_dev; a.indices16 = fg::narrow_indices(pl, idx_dev);
         a.own0 = own0; a.own1 = own1;
         a.far0 = ADD ? nullptr : far0 + (int64_t)p * width * row_floats; a.far1 = far1 + (int64_t)p * width * row_floats;
         a.far_row_bytes = (uint32_t)row_floats * 4u;

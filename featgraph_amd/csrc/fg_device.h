@@ -31,6 +31,20 @@ __device__ __forceinline__ void load_four(const T *p, int n, int lane, int strid
     }
 }
 
+// The lane's four column ids of a stream of n (as load_four): from the 16-bit copy `ids16` when there is one
+// (uniform over the wavefront), else from `ids`.
+__device__ __forceinline__ void load_four_ids(const int32_t *ids, const uint16_t *ids16, int64_t base, int n, int lane,
+                                              int32_t (&c)[4]) {
+    if (ids16) {
+        uint16_t c16[4];
+        load_four(ids16 + base, n, lane, 1, c16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) c[i] = c16[i];
+    } else {
+        load_four(ids + base, n, lane, 1, c);
+    }
+}
+
 // Orders this wavefront's LDS writes before its later LDS reads (and the reverse); for staging buffers
 // that are private to one wavefront, so no workgroup barrier is involved.
 __device__ __forceinline__ void wave_lds_sync() {

@@ -414,14 +414,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     auto stage = [&](int64_t base, int n) {
         // lane l holds edges 4l .. 4l + 3 (past the end: the last edge again)
         int32_t c[4], at[4] = {0, 0, 0, 0};
-        if (a.col16) {
-            uint16_t c16[4];
-            fg::load_four(a.col16 + base, n, lane, 1, c16);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) c[i] = c16[i];
-        } else {
-            fg::load_four(a.col + base, n, lane, 1, c);
-        }
+        fg::load_four_ids(a.col, a.col16, base, n, lane, c);
         if (SCATTER) fg::load_four(a.edge_pos + base, n, lane, 1, at);
 #pragma unroll
         for (int i = 0; i < 4; ++i) c[i] = (int)((uint32_t)c[i] * scale);

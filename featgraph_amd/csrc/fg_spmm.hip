@@ -204,14 +204,7 @@ __device__ __forceinline__ void stage_load(const int32_t *indices, const uint16_
                                            int lane, uint32_t scale, int vstride, int64_t voff, int2 (&r)[4]) {
     int32_t c[4];
     float w[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-    if (indices16) {
-        uint16_t c16[4];
-        fg::load_four(indices16 + base, n, lane, 1, c16);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) c[i] = c16[i];
-    } else {
-        fg::load_four(indices + base, n, lane, 1, c);
-    }
+    fg::load_four_ids(indices, indices16, base, n, lane, c);
     if (vals) fg::load_four(vals + base * vstride + voff, n, lane, vstride, w);
 #pragma unroll
     for (int i = 0; i < 4; ++i) r[i] = make_int2((int)((uint32_t)c[i] * scale), __float_as_int(w[i]));

@@ -57,6 +57,7 @@ class GraphAttentionhip(object):
             _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(np.ascontiguousarray(pos, dtype=np.int32)),
                                                       self._num_rows, self._num_cols, P, ctypes.byref(opts),
                                                       ctypes.byref(lay['plan'])))
+        common.narrow_indices(lay['plan'], lay['idx'], self._num_cols, P, self._ctx)
         self._layouts[P] = lay
         return lay
 
@@ -186,6 +187,7 @@ class GraphAttentionhip(object):
         with torch.cuda.device(self._ctx):
             _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(pos), self._num_cols, self._num_rows, P,
                                                       ctypes.byref(opts), ctypes.byref(lay['plan'])))
+        common.narrow_indices(lay['plan'], lay['idx'], self._num_rows, P, self._ctx)      # the transposed graph gathers from the rows
         self._layouts[key] = lay
         return lay
 

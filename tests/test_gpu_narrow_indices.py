@@ -147,3 +147,31 @@ def test_ids_up_to_65535_and_other_arrays():
         assert b"16 bits" in L.fg_last_error()
     finally:
         L.fg_spmm_plan_destroy(plan2)
+
+
+@pytest.mark.parametrize("additive", [False, True])
+@pytest.mark.parametrize("P", [1, 3])
+def test_attention_bit_identical(additive, P):
+    """Forward pass and both gradient sweeps (the second one over the transposed adjacency's own layout)."""
+    import torch
+    from featgraph_amd.module import GraphAttentionhip, placeholder
+    rng = np.random.default_rng(31 + P)
+    adj = _graph(rng, n_rows=600, n_cols=600, long_len=500)
+    n, H, D = 600, 2, 64
+    q = torch.from_numpy(rng.standard_normal((n, H) if additive else (n, H, D)).astype("float32")).cuda()
+    k = torch.from_numpy(rng.standard_normal((n, H) if additive else (n, H, D)).astype("float32")).cuda()
+    v = torch.from_numpy(rng.standard_normal((n, H, D)).astype("float32")).cuda()
+    g = torch.from_numpy(rng.standard_normal((n, H, D)).astype("float32")).cuda()
+
+    def run():
+        m = GraphAttentionhip(adj)
+        m.build([placeholder(tuple(q.shape)), placeholder(tuple(k.shape)), placeholder(tuple(v.shape))],
+                {'scores': 'additive'} if additive else {}, {'num_src_partitions': P, 'num_dst_partitions': P})
+        out = m.run([q, k, v]).clone()
+        grads = m.backward(q, k, v, m.out_tvm, m.state_tvm, g)
+        return [out.cpu().numpy()] + [t.cpu().numpy() for t in grads]
+
+    wide, narrow = _with(False, run), _with(True, run)
+    for a, b in zip(wide, narrow):
+        assert np.isfinite(b).all()
+        assert np.array_equal(a, b)
