@@ -42,10 +42,10 @@ MEASURED_TRAFFIC = {
     # (operator, workload, F, partitions, tiles): (bytes, summary); tiles 0 = the kernel's own single tile
     ("spmm", "powerlaw-233k", 512, 8, 8): (60.7e9, _PROFILES % "powerlaw233k_f512"),     # spmm_items_kernel (copy: +0.95e9, sum of the passes: +4.3e9)
     ("sddmm", "powerlaw-233k", 512, 8, 8): (64.2e9, _PROFILES % "powerlaw233k_f512"),    # sddmm_tiled_kernel (copy: +0.95e9, tile sum: +4.7e9)
-    ("spmm", "powerlaw-233k", 64, 8, 0): (8.50e9, _PROFILES % "powerlaw233k_f64"),
-    ("sddmm", "powerlaw-233k", 64, 8, 1): (9.30e9, _PROFILES % "powerlaw233k_f64"),
-    ("spmm", "powerlaw-233k", 32, 4, 0): (4.72e9, _PROFILES % "powerlaw233k_f32"),
-    ("sddmm", "powerlaw-233k", 32, 4, 1): (5.44e9, _PROFILES % "powerlaw233k_f32"),
+    ("spmm", "powerlaw-233k", 64, 8, 0): (8.14e9, _PROFILES % "powerlaw233k_f64"),
+    ("sddmm", "powerlaw-233k", 64, 8, 1): (8.94e9, _PROFILES % "powerlaw233k_f64"),
+    ("spmm", "powerlaw-233k", 32, 4, 0): (4.37e9, _PROFILES % "powerlaw233k_f32"),
+    ("sddmm", "powerlaw-233k", 32, 4, 1): (5.10e9, _PROFILES % "powerlaw233k_f32"),
     ("spmm", "powerlaw-2.45M", 128, 1, 1): (33.15e9, _PROFILES % "powerlaw2450k_f128"),
     ("sddmm", "powerlaw-2.45M", 128, 1, 1): (33.41e9, _PROFILES % "powerlaw2450k_f128"),
 }
@@ -331,7 +331,7 @@ def main():
                   "kernel": "sddmm_tiled_kernel" if sddmm._tiled else plain_sddmm,
                   "launches": sddmm_launches(),
                   "kernels": ({"tile_major_kernel": copies(sddmm._tiled[1]), "sddmm_tiled_kernel": sddmm_launches(),
-                               "sddmm_tile_sum_kernel": 1}
+                               "sddmm_tile_sum_kernel": 1 if sddmm._tiled[1] > 1 else 0}
                               if sddmm._tiled else {plain_sddmm: 1}),
                   "num_src_partitions": sddmm._tiled[0]['P'] if sddmm._tiled else 1,
                   "num_feat_tiles": sddmm._tiled[1] if sddmm._tiled else 1},
