@@ -437,11 +437,23 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
             // and one that was only touched here has left the L2 again by the time a later row of the item needs it.
             constexpr int RV = L * K;                    // 128-bit words per row slice
             float4 held[2 * K];
+            // With one partition in flight nobody else reads these slices before they have left the caches: non-temporal
+            // loads then keep them from displacing the gathered operand's rows (232,965-node graph, F=512, 8 tiles: 13.22 ->
+            // 13.03 ms).  With several partitions in flight (fewer than 8 tiles) the other partitions' workgroups read the same
+            // rows at about the same time, through the memory-side cache, and plain loads are 1-2.5 % faster.
+            const bool stream_dst = a.conc == 1;
+            typedef float f4 __attribute__((ext_vector_type(4)));
 #pragma unroll
             for (int i = 0; i < 2 * K; ++i) {
                 const int t = lane + 64 * i;
                 const int r = min(t / RV, nrows - 1);
-                held[i] = *reinterpret_cast<const float4 *>(a.dst + (int64_t)(it.row + r) * F + tile * (RV * 4) + (t % RV) * 4);
+                const float *at = a.dst + (int64_t)(it.row + r) * F + tile * (RV * 4) + (t % RV) * 4;
+                if (stream_dst) {
+                    const f4 hv = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(at));
+                    held[i] = make_float4(hv.x, hv.y, hv.z, hv.w);
+                } else {
+                    held[i] = *reinterpret_cast<const float4 *>(at);
+                }
             }
             stage(it.start, it.len);
             s_end[wave][lane] = pos[it.row + min(lane, nrows - 1) + 1] - it.start;
