@@ -208,7 +208,14 @@ __device__ __forceinline__ void finish_row(Running r, const Running &old, int g,
     }
     if (g != 0) return;
     if (!FIRST) running_merge(r, old);
-    *reinterpret_cast<float4 *>(out_row) = r.acc;
+    if constexpr (FIRST) {
+        // written once and read back by another kernel (or a later pass): a non-temporal store leaves the L2 to the gathered rows
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        f4 t; t.x = r.acc.x; t.y = r.acc.y; t.z = r.acc.z; t.w = r.acc.w;
+        __builtin_nontemporal_store(t, reinterpret_cast<f4 *>(out_row));
+    } else {
+        *reinterpret_cast<float4 *>(out_row) = r.acc;
+    }
     if (li == 0) { state_row[0] = r.m; state_row[1] = r.l; }
 }
 
@@ -400,7 +407,8 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(float4 *out, float
 #pragma unroll 4
         for (int p = 0; p < P; ++p) {
             const float f = __expf(buf_state[p * sstride + srow] - m);      // exp(-inf) = 0 for a partition without elements
-            const float4 a = buf_out[(uint64_t)p * n_words + i];
+            typedef float f4 __attribute__((ext_vector_type(4)));
+            const f4 a = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(buf_out) + (uint64_t)p * n_words + i);   // read once
             run.acc.x += a.x * f; run.acc.y += a.y * f; run.acc.z += a.z * f; run.acc.w += a.w * f;
             run.l += buf_state[p * sstride + srow + 1] * f;
         }
