@@ -276,7 +276,9 @@ struct SddmmTiledArgs {
 // head's U results end up one per lane (lane position u of the head segment keeps result u) and
 // are stored by those lanes.
 constexpr int kTilePad = 8;   // staging slots past the last edge that the unclamped walk may read
-template <int L, int K, int RW, int KH, int U, bool SCATTER, bool OFF32, bool CLAMP, bool ALLVALID = false>
+// STAGE: a result goes to the .y word of its edge's staging slot instead of to `out` (the kernel writes the item's results
+// from there in whole runs).
+template <int L, int K, int RW, int KH, int U, bool SCATTER, bool OFF32, bool CLAMP, bool ALLVALID = false, bool STAGE = false>
 __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int jstride, int e, const float *src,
                                                  uint32_t lane_bytes, int64_t F, const float4 (&dv)[K], float *out,
                                                  int64_t estride, int64_t e_base, int seg_pos) {
@@ -318,8 +320,12 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
         const int u_mine = seg_pos >> 1;
         const int ju = j0 + u_mine * jstride;
         if ((seg_pos & 1) == 0 && (ALLVALID || ju < e)) {
-            const int64_t at = SCATTER ? (int64_t)edge[ju].y : e_base + ju;
-            out[at * estride] = t;
+            if constexpr (STAGE) {
+                const_cast<int2 *>(edge)[ju].y = __float_as_int(t);
+            } else {
+                const int64_t at = SCATTER ? (int64_t)edge[ju].y : e_base + ju;
+                out[at * estride] = t;
+            }
         }
         return;
     }
@@ -341,26 +347,31 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
     }
     const int ju = j0 + seg_pos * jstride;
     if (seg_pos < U && (ALLVALID || ju < e)) {
-        const int64_t at = SCATTER ? (int64_t)my_pos : e_base + ju;
+        if constexpr (STAGE) {
+            static_assert(!STAGE || (NH == 1 && HPL == 1 && !SCATTER), "one result per edge and tile");
+            const_cast<int2 *>(edge)[ju].y = __float_as_int(mine[0]);
+        } else {
+            const int64_t at = SCATTER ? (int64_t)my_pos : e_base + ju;
 #pragma unroll
-        for (int kk = 0; kk < NH; ++kk) out[at * estride + kk * HPL] = mine[kk];
+            for (int kk = 0; kk < NH; ++kk) out[at * estride + kk * HPL] = mine[kk];
+        }
     }
 }
 
 // The last, partly filled batch of a row: exactly `nu` steps (1 <= nu <= U, uniform over the
 // wavefront) are loaded and reduced, instead of U steps padded with re-reads of the last edge --
 // a re-read costs the same cache bandwidth as a gather.
-template <int L, int K, int RW, int KH, int NU, bool SCATTER, bool OFF32>
+template <int L, int K, int RW, int KH, int NU, bool SCATTER, bool OFF32, bool STAGE = false>
 __device__ __forceinline__ void sddmm_tile_tail(int nu, const int2 *edge, int j0, int jstride, int e, const float *src,
                                                 uint32_t lane_bytes, int64_t F, const float4 (&dv)[K], float *out,
                                                 int64_t estride, int64_t e_base, int seg_pos) {
     if (nu >= NU) {
-        sddmm_tile_batch<L, K, RW, KH, NU, SCATTER, OFF32, true>(edge, j0, jstride, e, src, lane_bytes, F, dv, out, estride,
+        sddmm_tile_batch<L, K, RW, KH, NU, SCATTER, OFF32, true, false, STAGE>(edge, j0, jstride, e, src, lane_bytes, F, dv, out, estride,
                                                                   e_base, seg_pos);
         return;
     }
     if constexpr (NU > 1)
-        sddmm_tile_tail<L, K, RW, KH, NU - 1, SCATTER, OFF32>(nu, edge, j0, jstride, e, src, lane_bytes, F, dv, out, estride,
+        sddmm_tile_tail<L, K, RW, KH, NU - 1, SCATTER, OFF32, STAGE>(nu, edge, j0, jstride, e, src, lane_bytes, F, dv, out, estride,
                                                               e_base, seg_pos);
 }
 
@@ -370,6 +381,10 @@ template <int L, int K, int RW, int KH, bool SCATTER, bool OFF32>
 __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArgs a) {
     constexpr int G = 64 / L;
     constexpr int U = (RW < 8 ? RW : 8) / (K >= 2 ? 2 : 1) > 0 ? (RW < 8 ? RW : 8) / (K >= 2 ? 2 : 1) : 1;
+    // One result per edge and tile, written in traversal order: the results of an item (or of 256 elements of a long row)
+    // are collected in the staging row's unused position words and written from there as whole runs of consecutive floats,
+    // instead of 4 bytes per lane from every batch (which reached memory as partly filled 64-byte blocks).
+    constexpr bool STAGE = !SCATTER && K == KH && RW == L;
     static_assert(U <= kTilePad, "unclamped reads must stay inside the padded staging row");
     __shared__ __align__(16) int2 s_edge[kWavesPerBlock][fg::kItemEdges + kTilePad];     // x = column word, y = edge_pos
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
@@ -423,6 +438,15 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         e4[2 * lane + 1] = make_int4(c[2], at[2], c[3], at[3]);
         if (lane < kTilePad) edge[fg::kItemEdges + lane] = make_int2(c[3], at[3]);
     };
+    // the staged results of elements [0, n) of the staging row go to out[e_base ..]
+    auto flush = [&](int64_t e_base, int n) {
+        wave_lds_sync();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int j = lane + 64 * i;
+            if (j < n) out[(e_base + j) * a.out_edge_stride] = __int_as_float(edge[j].y);
+        }
+    };
     auto load_dst = [&](int64_t row) {
 #pragma unroll
         for (int k = 0; k < K; ++k) dv[k] = *reinterpret_cast<const float4 *>(db + row * F + k * L * 4);
@@ -468,14 +492,15 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
                     for (int k = 0; k < K; ++k) dv[k] = s_dst[wave][q * RV + k * L + li];
                     int s0 = b;
                     for (; s0 + G * U <= e; s0 += G * U)
-                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, e, src, lane_bytes, F, dv,
+                        sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true, STAGE>(edge, s0 + g, G, e, src, lane_bytes, F, dv,
                                                                                  out, a.out_edge_stride, it.start, seg_pos);
                     if (s0 < e)
-                        sddmm_tile_tail<L, K, RW, KH, U, SCATTER, OFF32>((e - s0 + G - 1) / G, edge, s0 + g, G, e, src, lane_bytes,
+                        sddmm_tile_tail<L, K, RW, KH, U, SCATTER, OFF32, STAGE>((e - s0 + G - 1) / G, edge, s0 + g, G, e, src, lane_bytes,
                                                                          F, dv, out, a.out_edge_stride, it.start, seg_pos);
                 }
                 b = e;
             }
+            if constexpr (STAGE) flush(it.start, it.len);
             return;
         }
         // Many short rows.  Their destination slices are touched once here, one word per 128 bytes, while the
@@ -517,11 +542,12 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
             }
             if (__all(done)) break;
             if (!done && j < e) {
-                sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false>(edge, j, 1, e, src, lane_bytes, F, dv, out,
+                sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, false, STAGE>(edge, j, 1, e, src, lane_bytes, F, dv, out,
                                                                   a.out_edge_stride, it.start, seg_pos);
                 j += U;
             }
         }
+        if constexpr (STAGE) flush(it.start, it.len);
         return;
     }
     // one row, or one piece of a long row
@@ -533,11 +559,12 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         wave_lds_sync();
         int s0 = 0;
         for (; s0 + G * U <= n; s0 += G * U)
-            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true>(edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
+            sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, true, STAGE>(edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
                                                                      a.out_edge_stride, (int64_t)it.start + base, seg_pos);
         if (s0 < n)
-            sddmm_tile_tail<L, K, RW, KH, U, SCATTER, OFF32>((n - s0 + G - 1) / G, edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
+            sddmm_tile_tail<L, K, RW, KH, U, SCATTER, OFF32, STAGE>((n - s0 + G - 1) / G, edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
                                                              a.out_edge_stride, (int64_t)it.start + base, seg_pos);
+        if constexpr (STAGE) flush((int64_t)it.start + base, n);
     }
 }
 
