@@ -276,9 +276,10 @@ struct SddmmTiledArgs {
 // head's U results end up one per lane (lane position u of the head segment keeps result u) and
 // are stored by those lanes.
 constexpr int kTilePad = 8;   // staging slots past the last edge that the unclamped walk may read
-// STAGE: a result goes to the .y word of its edge's staging slot instead of to `out` (the kernel writes the item's results
-// from there in whole runs).
-template <int L, int K, int RW, int KH, int U, bool SCATTER, bool OFF32, bool CLAMP, bool ALLVALID = false, bool STAGE = false>
+// STAGE: a result goes to a word of its edge's staging slot instead of to `out`, and the kernel writes the item's results
+// from there in whole runs: 1 = the .y word (results in traversal order; the positions are not needed), 2 = the .x word
+// (the column word, which is dead once the batch's gathers are issued; .y keeps the position the result goes to).
+template <int L, int K, int RW, int KH, int U, bool SCATTER, bool OFF32, bool CLAMP, bool ALLVALID = false, int STAGE = 0>
 __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int jstride, int e, const float *src,
                                                  uint32_t lane_bytes, int64_t F, const float4 (&dv)[K], float *out,
                                                  int64_t estride, int64_t e_base, int seg_pos) {
@@ -320,8 +321,10 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
         const int u_mine = seg_pos >> 1;
         const int ju = j0 + u_mine * jstride;
         if ((seg_pos & 1) == 0 && (ALLVALID || ju < e)) {
-            if constexpr (STAGE) {
+            if constexpr (STAGE == 1) {
                 const_cast<int2 *>(edge)[ju].y = __float_as_int(t);
+            } else if constexpr (STAGE == 2) {
+                const_cast<int2 *>(edge)[ju].x = __float_as_int(t);
             } else {
                 const int64_t at = SCATTER ? (int64_t)edge[ju].y : e_base + ju;
                 out[at * estride] = t;
@@ -347,9 +350,12 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
     }
     const int ju = j0 + seg_pos * jstride;
     if (seg_pos < U && (ALLVALID || ju < e)) {
-        if constexpr (STAGE) {
-            static_assert(!STAGE || (NH == 1 && HPL == 1 && !SCATTER), "one result per edge and tile");
+        if constexpr (STAGE == 1) {
+            static_assert(STAGE != 1 || (NH == 1 && HPL == 1 && !SCATTER), "one result per edge and tile");
             const_cast<int2 *>(edge)[ju].y = __float_as_int(mine[0]);
+        } else if constexpr (STAGE == 2) {
+            static_assert(STAGE != 2 || (NH == 1 && HPL == 1 && SCATTER), "one result per edge");
+            const_cast<int2 *>(edge)[ju].x = __float_as_int(mine[0]);
         } else {
             const int64_t at = SCATTER ? (int64_t)my_pos : e_base + ju;
 #pragma unroll
@@ -361,7 +367,7 @@ __device__ __forceinline__ void sddmm_tile_batch(const int2 *edge, int j0, int j
 // The last, partly filled batch of a row: exactly `nu` steps (1 <= nu <= U, uniform over the
 // wavefront) are loaded and reduced, instead of U steps padded with re-reads of the last edge --
 // a re-read costs the same cache bandwidth as a gather.
-template <int L, int K, int RW, int KH, int NU, bool SCATTER, bool OFF32, bool STAGE = false>
+template <int L, int K, int RW, int KH, int NU, bool SCATTER, bool OFF32, int STAGE = 0>
 __device__ __forceinline__ void sddmm_tile_tail(int nu, const int2 *edge, int j0, int jstride, int e, const float *src,
                                                 uint32_t lane_bytes, int64_t F, const float4 (&dv)[K], float *out,
                                                 int64_t estride, int64_t e_base, int seg_pos) {
@@ -384,7 +390,12 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
     // One result per edge and tile, written in traversal order: the results of an item (or of 256 elements of a long row)
     // are collected in the staging row's unused position words and written from there as whole runs of consecutive floats,
     // instead of 4 bytes per lane from every batch (which reached memory as partly filled 64-byte blocks).
-    constexpr bool STAGE = !SCATTER && K == KH && RW == L;
+    // Results that are scattered to stored positions take the column words instead, where the whole wavefront walks one row
+    // at a time; where lane groups walk rows of their own a group may still read a later row's column words, so those items
+    // keep storing 4 bytes per lane.
+    constexpr bool ONE = K == KH && RW == L;
+    constexpr int STAGE = ONE ? (SCATTER ? 2 : 1) : 0;
+    constexpr int STAGE_OWN_ROWS = STAGE == 1 ? 1 : 0;
     static_assert(U <= kTilePad, "unclamped reads must stay inside the padded staging row");
     __shared__ __align__(16) int2 s_edge[kWavesPerBlock][fg::kItemEdges + kTilePad];     // x = column word, y = edge_pos
     __shared__ int32_t s_end[kWavesPerBlock][fg::kItemRows];
@@ -444,7 +455,11 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int j = lane + 64 * i;
-            if (j < n) out[(e_base + j) * a.out_edge_stride] = __int_as_float(edge[j].y);
+            if (j < n) {
+                const int2 w = edge[j];
+                if (STAGE == 2) out[(int64_t)w.y * a.out_edge_stride] = __int_as_float(w.x);
+                else out[(e_base + j) * a.out_edge_stride] = __int_as_float(w.y);
+            }
         }
     };
     auto load_dst = [&](int64_t row) {
@@ -500,7 +515,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
                 }
                 b = e;
             }
-            if constexpr (STAGE) flush(it.start, it.len);
+            if constexpr (STAGE != 0) flush(it.start, it.len);
             return;
         }
         // Many short rows.  Their destination slices are touched once here, one word per 128 bytes, while the
@@ -542,12 +557,12 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
             }
             if (__all(done)) break;
             if (!done && j < e) {
-                sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, false, STAGE>(edge, j, 1, e, src, lane_bytes, F, dv, out,
+                sddmm_tile_batch<L, K, RW, KH, U, SCATTER, OFF32, false, false, STAGE_OWN_ROWS>(edge, j, 1, e, src, lane_bytes, F, dv, out,
                                                                   a.out_edge_stride, it.start, seg_pos);
                 j += U;
             }
         }
-        if constexpr (STAGE) flush(it.start, it.len);
+        if constexpr (STAGE_OWN_ROWS != 0) flush(it.start, it.len);
         return;
     }
     // one row, or one piece of a long row
@@ -564,7 +579,7 @@ __global__ __launch_bounds__(kBlock) void sddmm_tiled_kernel(const SddmmTiledArg
         if (s0 < n)
             sddmm_tile_tail<L, K, RW, KH, U, SCATTER, OFF32, STAGE>((n - s0 + G - 1) / G, edge, s0 + g, G, n, src, lane_bytes, F, dv, out,
                                                              a.out_edge_stride, (int64_t)it.start + base, seg_pos);
-        if constexpr (STAGE) flush((int64_t)it.start + base, n);
+        if constexpr (STAGE != 0) flush((int64_t)it.start + base, n);
     }
 }
 
