@@ -41,11 +41,11 @@ _PROFILES = "profiles/bench_%s_rocprofv3.txt"
 MEASURED_TRAFFIC = {
     # (operator, workload, F, partitions, tiles): (bytes, summary); tiles 0 = the kernel's own single tile
     ("spmm", "powerlaw-233k", 512, 8, 8): (59.2e9, _PROFILES % "powerlaw233k_f512"),     # spmm_items_kernel (copy: +0.95e9, sum of the passes: +4.3e9)
-    ("sddmm", "powerlaw-233k", 512, 8, 8): (62.8e9, _PROFILES % "powerlaw233k_f512"),    # sddmm_tiled_kernel (copy: +0.95e9, tile sum: +4.7e9)
-    ("spmm", "powerlaw-233k", 64, 8, 0): (8.14e9, _PROFILES % "powerlaw233k_f64"),
-    ("sddmm", "powerlaw-233k", 64, 8, 1): (8.94e9, _PROFILES % "powerlaw233k_f64"),
-    ("spmm", "powerlaw-233k", 32, 4, 0): (4.37e9, _PROFILES % "powerlaw233k_f32"),
-    ("sddmm", "powerlaw-233k", 32, 4, 1): (5.10e9, _PROFILES % "powerlaw233k_f32"),
+    ("sddmm", "powerlaw-233k", 512, 8, 8): (61.2e9, _PROFILES % "powerlaw233k_f512"),    # sddmm_tiled_kernel (copy: +0.95e9, tile sum: +4.7e9)
+    ("spmm", "powerlaw-233k", 64, 8, 0): (7.96e9, _PROFILES % "powerlaw233k_f64"),
+    ("sddmm", "powerlaw-233k", 64, 8, 1): (8.83e9, _PROFILES % "powerlaw233k_f64"),
+    ("spmm", "powerlaw-233k", 32, 4, 0): (4.31e9, _PROFILES % "powerlaw233k_f32"),
+    ("sddmm", "powerlaw-233k", 32, 4, 1): (5.07e9, _PROFILES % "powerlaw233k_f32"),
     ("spmm", "powerlaw-2.45M", 128, 1, 1): (33.15e9, _PROFILES % "powerlaw2450k_f128"),
     ("sddmm", "powerlaw-2.45M", 128, 1, 1): (33.41e9, _PROFILES % "powerlaw2450k_f128"),
 }
