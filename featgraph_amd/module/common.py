@@ -107,6 +107,8 @@ def narrow_indices(plan, idx_dev, num_cols, num_partitions, dev):
         return
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().fg_spmm_plan_narrow_indices(plan, _lib.dev_ptr(idx_dev), stream_ptr()))
+        # the copy is made on the current stream, once, at construction; run() may be called under any other stream
+        torch.cuda.current_stream().synchronize()
 
 
 def take_args(args, allowed, what):
