@@ -58,6 +58,7 @@ struct GenArgs {
     int64_t n_items;
     const int32_t *indptr;
     const int32_t *indices;
+    const uint16_t *indices16;   // the plan's 16-bit copy of `indices`, read instead of it (null: none)
     const float *lhs, *rhs;
     const int32_t *lhs_off, *rhs_off;
     int lhs_len, rhs_len;
@@ -162,8 +163,10 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
     __shared__ int2 s_el[kWavesPerBlock][kStage];
     int2 *const el = s_el[wave];
     auto stage = [&](int64_t c0, int n) {
-        for (int t = lane; t < n; t += 64)
-            el[t] = make_int2((int)(a.indices[c0 + t] + ubase), PART ? a.edge_pos[c0 + t] : (int)(c0 + t));
+        for (int t = lane; t < n; t += 64) {
+            const int col = a.indices16 ? (int)a.indices16[c0 + t] : a.indices[c0 + t];      // uniform choice
+            el[t] = make_int2(col + (int)ubase, PART ? a.edge_pos[c0 + t] : (int)(c0 + t));
+        }
         wave_lds_sync();
     };
 
@@ -623,7 +626,7 @@ int gspmm_bcast_run(fg_spmm_plan *pl, const int32_t *pos_dev, const int32_t *idx
     int32_t *const abuf = positions + (size_t)P * b.pieces;
     GenArgs a;
     a.items = pl->items_dev; a.n_items = pl->n_items;
-    a.indptr = pos_dev; a.indices = idx_dev;
+    a.indptr = pos_dev; a.indices = idx_dev; a.indices16 = fg::narrow_indices(pl, idx_dev);
     a.lhs = lhs_dev; a.rhs = rhs_dev; a.lhs_off = lhs_off_dev; a.rhs_off = rhs_off_dev;
     a.lhs_len = lhs_len; a.rhs_len = rhs_len; a.lhs_target = lhs_target; a.rhs_target = rhs_target;
     a.sign = reduce == FG_REDUCE_MIN ? -1.f : 1.f;

@@ -175,3 +175,25 @@ def test_attention_bit_identical(additive, P):
     for a, b in zip(wide, narrow):
         assert np.isfinite(b).all()
         assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("msg,reduce,P", [("u_add_e", "sum", None), ("u_mul_e", "max", None), ("u_add_e", "sum", 3), ("copy_u", "min", 2)])
+def test_broadcasting_spmm_bit_identical(msg, reduce, P):
+    import torch
+    from featgraph_amd.module import GSpMMhip, placeholder
+    rng = np.random.default_rng(77)
+    adj = _graph(rng)
+    F = 64
+    x = rng.standard_normal((adj.shape[1], F)).astype("float32")
+    e = rng.standard_normal((adj.nnz, 1)).astype("float32")
+
+    def run():
+        m = GSpMMhip(adj)
+        phs = [placeholder(x.shape)] + ([placeholder(e.shape)] if msg != "copy_u" else [])
+        m.build(phs, {'msg': msg, 'reduce': reduce}, {'num_src_partitions': P})
+        ins = [torch.from_numpy(x).cuda()] + ([torch.from_numpy(e).cuda()] if msg != "copy_u" else [])
+        return m.run(ins).cpu().numpy().copy()
+
+    wide, narrow = _with(False, run), _with(True, run)
+    assert np.isfinite(narrow).all()
+    assert np.array_equal(wide, narrow)
