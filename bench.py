@@ -168,42 +168,107 @@ def cpu_baseline(indptr, indices, vals, x, y, F, spmm_run_s=0.25, sddmm_run_s=0.
 
 
 def verify(torch, spmm, sddmm, indptr, indices_d, vals_d, x_d, y_d):
-    """Checks the operators' outputs for the benchmark inputs without a CPU product: the SpMM's column
-    sums against the weighted out-degree contraction of X, five of its rows (largest, smallest, first,
-    middle, last) and 200,000 sampled SDDMM edges against float64 formed on the device.
-    Returns a list of failures (empty: verified)."""
+    """Checks the operators' outputs for the benchmark inputs without a CPU product (the checks of
+    featgraph_amd/benchmark/verify.py): the SpMM's column sums against the weighted out-degree contraction
+    of X, five of its rows (largest, smallest, first, middle, last) and 200,000 sampled SDDMM edges against
+    float64 formed on the device.  Returns a list of failures (empty: verified)."""
+    from featgraph_amd.benchmark import verify as chk
+    failures = chk.spmm_failures(spmm.run([x_d]), indptr, indices_d, vals_d, x_d)
+    rows_d = torch.repeat_interleave(torch.arange(indptr.shape[0] - 1, device="cuda"),
+                                     torch.from_numpy(indptr[1:] - indptr[:-1]).cuda().long())
+    return failures + chk.sddmm_failures(sddmm.run([x_d, y_d]), rows_d, indices_d, x_d, y_d)
+
+
+VALU_PEAK_GFLOPS = 157300.0      # fp32 vector peak of the part
+
+
+def config_entry(config, workload, op, shape, tiling, seconds, flops, bytes_model, failures):
+    gflops = flops / seconds / 1e9
+    return {"config": config, "workload": workload, "op": op, "shape": shape, "tiling": tiling,
+            "ms_mean_of_5": round(seconds * 1e3, 4), "gflops": round(gflops, 1),
+            "compulsory_gb": round(bytes_model / 1e9, 4), "hbm_gbs": round(bytes_model / seconds / 1e9, 1),
+            "pct_hbm_roofline": round(100.0 * bytes_model / seconds / 1e9 / HBM_PEAK_GBS, 3),
+            "valu_frac": round(gflops / VALU_PEAK_GFLOPS, 4),
+            "verified": not failures, **({"failures": failures} if failures else {})}
+
+
+def sddmm_tiling(m):
+    if m._tiled:
+        return "%d partitions x %d tiles" % (m._tiled[0]['P'], m._tiled[1])
+    return "stored order (%s)" % ("sddmm_csr_kernel" if m._use_csr else "sddmm_coo_kernel")
+
+
+def run_configs(torch, workload, indptr, indices, vals_d, spmm, sddmm, headline_F, skip_low_degree=False):
+    """Every other benchmark configuration at the library's defaults, outside the headline's timed region: the
+    reference's protocol (mean of 5 back-to-back runs after a warm-up, python/featgraph/module/spmm.py:179-186;
+    check of the output, tests/test_module_sddmm.py:34-37) per entry.  cfg2: SpMM at the other feature lengths;
+    cfg3: SDDMM at the other feature lengths (edges stored in CSR order, the library's choice of kernel) and at the
+    headline length with the kernel that walks the stored row / col arrays (`order='coo'`); cfg4: multi-head SDDMM;
+    cfg5: SpMM then SDDMM on the 2.45M-node low-degree graph."""
     import numpy as np
-    eps8 = 8 * float(np.finfo(np.float32).eps)
-    failures = []
+    import scipy.sparse as sp
+    from featgraph_amd import synthetic
+    from featgraph_amd.benchmark import verify as chk
+    from featgraph_amd.module import VanillaSpMMhip, VanillaSDDMMhip, MultiHeadSDDMMhip, placeholder
+    entries = []
+    gen = torch.Generator(device="cuda")
+
+    def graph_side(indptr, indices):
+        idx_d = torch.from_numpy(indices).cuda().long()
+        rows_d = torch.repeat_interleave(torch.arange(indptr.shape[0] - 1, device="cuda"),
+                                         torch.from_numpy(np.diff(indptr)).cuda().long())
+        return idx_d, rows_d
+
+    def pair(config, name, indptr, idx_d, rows_d, vals_d, spmm, sddmm, F, sddmm_only_order=None):
+        n = indptr.shape[0] - 1
+        nnz = idx_d.shape[0]
+        gen.manual_seed(2)
+        x = torch.randn((n, F), generator=gen, device="cuda")
+        y = torch.randn((n, F), generator=gen, device="cuda")
+        if sddmm_only_order is None:
+            spmm.build([placeholder((n, F))], {}, {})
+            t = spmm.measure_average_time([x], 5)
+            entries.append(config_entry(config.split("/")[0], name, "spmm", "F=%d" % F,
+                                        "%d partitions x %d tiles" % (spmm._active['P'], spmm._num_feat_partitions or 1),
+                                        t, 2.0 * nnz * F, spmm_bytes(n, n, nnz, F),
+                                        chk.spmm_failures(spmm.run([x]), indptr, idx_d, vals_d, x)))
+        sa = {} if sddmm_only_order is None else {'order': sddmm_only_order}
+        sddmm.build([placeholder((n, F)), placeholder((n, F))], {}, sa)
+        t = sddmm.measure_average_time([x, y], 5)
+        csr = sddmm_only_order != 'coo'
+        entries.append(config_entry(config.split("/")[-1], name, "sddmm" if csr else "sddmm_coo_order", "F=%d" % F,
+                                    sddmm_tiling(sddmm), t, 2.0 * nnz * F, sddmm_bytes(n, nnz, F, 1, csr=csr),
+                                    chk.sddmm_failures(sddmm.run([x, y]), rows_d, idx_d, x, y)))
+
     n = indptr.shape[0] - 1
-    out = spmm.run([x_d])
-    col_w = torch.zeros(x_d.shape[0], device="cuda", dtype=torch.float64)
-    col_w.index_add_(0, indices_d, vals_d.double())
-    expect = (col_w[:, None] * x_d.double()).sum(0)
-    scale = (col_w[:, None] * x_d.double().abs()).sum(0)
-    if not ((out.double().sum(0) - expect).abs() <= 1e-5 * scale).all().item():
-        failures.append("spmm: column sums differ from the out-degree contraction of X")
-    deg = np.diff(indptr)
-    for v in (int(np.argmax(deg)), int(np.argmin(deg)), 0, n // 2, n - 1):
-        e = slice(int(indptr[v]), int(indptr[v + 1]))
-        terms = vals_d[e].double()[:, None] * x_d[indices_d[e]].double()
-        tol = 1e-5 + 1e-4 * terms.sum(0).abs() + eps8 * terms.abs().sum(0)
-        if not ((out[v].double() - terms.sum(0)).abs() <= tol).all().item():
-            failures.append("spmm: row %d differs from its float64 sum" % v)
-    scores = sddmm.run([x_d, y_d])
-    g = torch.Generator(device="cuda")
-    g.manual_seed(7)
-    nnz = indices_d.shape[0]
-    pick = torch.randint(0, nnz, (200000,), generator=g, device="cuda")
-    pick[0], pick[1] = 0, nnz - 1
-    rows = torch.searchsorted(torch.from_numpy(indptr).cuda().long(), pick, right=True) - 1
-    prod = x_d[indices_d[pick]].double() * y_d[rows].double()
-    tol = 1e-5 + 1e-4 * prod.sum(1).abs() + eps8 * prod.abs().sum(1)
-    if not torch.isfinite(scores).all().item():
-        failures.append("sddmm: non-finite scores")
-    if not ((scores[pick].double() - prod.sum(1)).abs() <= tol).all().item():
-        failures.append("sddmm: sampled edges differ from their float64 dot products")
-    return failures
+    nnz = indices.shape[0]
+    idx_d, rows_d = graph_side(indptr, indices)
+    for F in (32, 64, 128, 256, 512):
+        if F != headline_F:
+            pair("cfg2/cfg3", workload, indptr, idx_d, rows_d, vals_d, spmm, sddmm, F)
+    pair("cfg3", workload, indptr, idx_d, rows_d, vals_d, spmm, sddmm, headline_F, sddmm_only_order='coo')
+    mh = MultiHeadSDDMMhip(sp.csr_matrix((np.ones(nnz, np.float32), indices, indptr), shape=(n, n)))
+    for H, D in ((4, 32), (4, 64), (8, 32), (8, 64)):
+        gen.manual_seed(2)
+        x = torch.randn((n, H, D), generator=gen, device="cuda")
+        y = torch.randn((n, H, D), generator=gen, device="cuda")
+        mh.build([placeholder((n, H, D)), placeholder((n, H, D))], {}, {})
+        t = mh.measure_average_time([x, y], 5)
+        entries.append(config_entry("cfg4", workload, "sddmm_multihead", "H=%d D=%d" % (H, D), sddmm_tiling(mh), t,
+                                    2.0 * nnz * H * D, sddmm_bytes(n, nnz, H * D, H, csr=True),
+                                    chk.sddmm_failures(mh.run([x, y]), rows_d, idx_d, x, y)))
+    del mh, x, y, idx_d, rows_d
+    torch.cuda.empty_cache()
+    if not skip_low_degree:
+        name = "powerlaw-2.45M"
+        ip5, ix5 = synthetic.make_workload(name)
+        n5, nnz5 = ip5.shape[0] - 1, ix5.shape[0]
+        gen.manual_seed(1)
+        v5 = torch.rand(nnz5, generator=gen, device="cuda", dtype=torch.float32)
+        adj5 = sp.csr_matrix((v5.cpu().numpy(), ix5, ip5), shape=(n5, n5))
+        idx_d, rows_d = graph_side(ip5, ix5)
+        pair("cfg5", name, ip5, idx_d, rows_d, v5, VanillaSpMMhip(adj5), VanillaSDDMMhip(adj5), 128)
+    return entries
 
 
 def main():
@@ -216,6 +281,8 @@ def main():
     ap.add_argument("--num-feat-partitions", type=int, default=0, help="SpMM feature tiles (0 = library default)")
     ap.add_argument("--num-col-partitions", type=int, default=1, help="SpMM source-column partitions")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the block that times and checks the other benchmark configurations after the headline")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: both ops are single-device kernels with no collective; "
@@ -338,6 +405,7 @@ def main():
     }
     for o in ops.values():
         o["pct_hbm_roofline"] = 100.0 * o["hbm_gbs"] / HBM_PEAK_GBS
+        o["valu_frac"] = o["gflops"] / VALU_PEAK_GFLOPS          # share of the fp32 vector peak (157.3 TFLOP/s)
     dom = "spmm" if t_spmm >= t_sddmm else "sddmm"
     key = (dom, args.workload, F, ops[dom].get("num_col_partitions", ops[dom].get("num_src_partitions")),
            ops[dom].get("num_feat_partitions", ops[dom].get("num_feat_tiles")))
@@ -348,6 +416,7 @@ def main():
     # ratio as for the whole operator; `traffic` is the measured fabric-side bytes of one such launch
     roofline = {"bound": "hbm", "kernel": ops[dom]["kernel"], "achieved": round(ops[dom]["hbm_gbs"], 2),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ops[dom]["hbm_gbs"] / HBM_PEAK_GBS, 5),
+                "valu_frac": round(ops[dom]["valu_frac"], 5),
                 "traffic": (round(op_traffic[0] / n_launch) if op_traffic else None),
                 "op_traffic": (op_traffic[0] if op_traffic else None),
                 # `traffic` is a stored figure from the named rocprofv3 summary (same workload, feature length and
@@ -377,6 +446,15 @@ def main():
         line["cpu_baseline"] = cpu_baseline(indptr, indices, vals, x_d.cpu().numpy(), y_d.cpu().numpy(), F)
     if failures:
         line["verification_failures"] = failures
+    if not args.no_configs and args.workload == "powerlaw-233k":
+        del x_d, y_d
+        torch.cuda.empty_cache()
+        t0 = time.perf_counter()
+        line["configs"] = run_configs(torch, args.workload, indptr, indices, vals_d, spmm, sddmm, F)
+        line["configs_verified"] = sum(1 for e in line["configs"] if e["verified"])
+        line["configs_seconds"] = round(time.perf_counter() - t0, 1)
+        failures = failures + ["%s %s %s: %s" % (e["workload"], e["op"], e["shape"], "; ".join(e["failures"]))
+                               for e in line["configs"] if not e["verified"]]
     print(json.dumps(line))
     if failures:
         sys.exit("bench.py: output verification failed: " + "; ".join(failures))

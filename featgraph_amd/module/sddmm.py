@@ -111,7 +111,10 @@ class SDDMMbase(object):
             indices = self._adj_col_indices
             positions = np.arange(nnz, dtype=np.int32)
         else:
-            order = np.lexsort((self._adj_col_indices, self._adj_row_indices)).astype(np.int32)
+            # stable sort by (row, col), i.e. np.lexsort((col, row)), on the device: seconds instead of a minute at 1e8 edges
+            key = self._adj_row_indices_dev.long() * self._num_cols + self._adj_col_indices_dev.long()
+            order = torch.sort(key, stable=True).indices.to(torch.int32).cpu().numpy()
+            del key
             indptr = np.zeros(self._num_rows + 1, dtype=np.int32)
             np.cumsum(np.bincount(self._adj_row_indices, minlength=self._num_rows), out=indptr[1:])
             indices = self._adj_col_indices[order]

@@ -31,6 +31,123 @@ def _close(got, ref64, mass):
     return ((got.double() - ref64).abs() <= ATOL + RTOL * ref64.abs() + MASS_FACTOR * mass).all().item()
 
 
+@pytest.fixture(scope="module")
+def weighted(graph):
+    """The benchmark's weighted adjacency (weights U[0, 1), seed 1), one SpMM and one SDDMM module that every
+    feature length re-builds, and the graph's arrays on the device."""
+    import torch
+    from featgraph_amd.module import VanillaSpMMhip, VanillaSDDMMhip
+    adj, n, nnz = graph
+    g = torch.Generator(device="cuda"); g.manual_seed(1)
+    vals_d = torch.rand(nnz, generator=g, device="cuda", dtype=torch.float32)
+    wadj = sp.csr_matrix((vals_d.cpu().numpy(), adj.indices, adj.indptr), shape=adj.shape)
+    idx_d = torch.from_numpy(adj.indices).cuda().long()
+    rows_d = torch.repeat_interleave(torch.arange(n, device="cuda"), torch.from_numpy(np.diff(adj.indptr)).cuda().long())
+    return dict(adj=wadj, n=n, nnz=nnz, vals_d=vals_d, idx_d=idx_d, rows_d=rows_d,
+                spmm=VanillaSpMMhip(wadj), sddmm=VanillaSDDMMhip(wadj))
+
+
+# what the cost model picks on this graph (partitions, tiles; SpMM tiles 0 = the kernel's own single tile):
+# 16-bit ids and several partitions in flight at F <= 128, the tile-by-tile copy of X from F = 256 on
+SPMM_DEFAULTS = {32: (4, 0), 64: (8, 0), 128: (8, 2), 256: (8, 4), 512: (8, 8)}
+SDDMM_DEFAULTS = {32: (4, 1), 64: (8, 1), 128: (16, 1), 256: (8, 4), 512: (8, 8)}
+
+
+@pytest.mark.parametrize("F", [32, 64, 128, 256, 512])
+def test_spmm_default_tiling_at_every_benchmark_length(weighted, F):
+    """Weighted CSR SpMM at every feature length the benchmark names, in the tiling the library picks there:
+    all-ones features give the rows' weight sums in every column, the output's column sums equal the weighted
+    out-degree contraction of X (a checksum every stored element enters once), five rows against float64."""
+    import torch
+    from featgraph_amd.benchmark import verify as chk
+    from featgraph_amd.module import placeholder
+    w = weighted
+    n, m = w['n'], w['spmm']
+    m.build([placeholder((n, F))], {}, {})
+    assert (m._active['P'], m._num_feat_partitions) == SPMM_DEFAULTS[F], m.lower_to_ir([placeholder((n, F))], {}, {})
+    indptr = w['adj'].indptr
+    m.out_tvm.fill_(float("nan"))
+    assert chk.spmm_ones_failures(m.run([torch.ones((n, F), device="cuda")]), indptr, w['vals_d']) == []
+    g = torch.Generator(device="cuda"); g.manual_seed(2)
+    x = torch.randn((n, F), generator=g, device="cuda")
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([x])
+    assert chk.spmm_failures(out, indptr, w['idx_d'], w['vals_d'], x) == []
+    first = out.clone()
+    assert torch.equal(m.run([x]), first)                     # repeatable bit for bit
+
+
+@pytest.mark.parametrize("F", [32, 64, 128, 256, 512])
+def test_sddmm_default_tiling_at_every_benchmark_length(weighted, F):
+    """SDDMM over the CSR-ordered edges at every feature length the benchmark names, in the traversal the library
+    picks there: dst = ones gives the gathered rows' sums on every edge, 200,000 sampled edges against float64."""
+    import torch
+    from featgraph_amd.benchmark import verify as chk
+    from featgraph_amd.module import placeholder
+    w = weighted
+    n, m = w['n'], w['sddmm']
+    phs = [placeholder((n, F)), placeholder((n, F))]
+    m.build(phs, {}, {})
+    assert m._tiled is not None and (m._tiled[0]['P'], m._tiled[1]) == SDDMM_DEFAULTS[F], m.lower_to_ir(phs, {}, {})
+    g = torch.Generator(device="cuda"); g.manual_seed(5)
+    src = torch.randn((n, F), generator=g, device="cuda")
+    dst = torch.randn((n, F), generator=g, device="cuda")
+    m.out_tvm.fill_(float("nan"))
+    assert chk.sddmm_ones_failures(m.run([src, torch.ones((n, F), device="cuda")]), w['idx_d'], src) == []
+    m.out_tvm.fill_(float("nan"))
+    assert chk.sddmm_failures(m.run([src, dst]), w['rows_d'], w['idx_d'], src, dst) == []
+
+
+def test_sddmm_coo_order_at_feat_512(weighted):
+    """The kernel that walks the stored row / col arrays (`order='coo'`), at the headline feature length."""
+    import torch
+    from featgraph_amd.benchmark import verify as chk
+    from featgraph_amd.module import placeholder
+    w = weighted
+    n, m, F = w['n'], w['sddmm'], 512
+    m.build([placeholder((n, F)), placeholder((n, F))], {}, {'order': 'coo'})
+    assert m._tiled is None and not m._use_csr
+    g = torch.Generator(device="cuda"); g.manual_seed(6)
+    src = torch.randn((n, F), generator=g, device="cuda")
+    dst = torch.randn((n, F), generator=g, device="cuda")
+    m.out_tvm.fill_(float("nan"))
+    assert chk.sddmm_ones_failures(m.run([src, torch.ones((n, F), device="cuda")]), w['idx_d'], src) == []
+    m.out_tvm.fill_(float("nan"))
+    assert chk.sddmm_failures(m.run([src, dst]), w['rows_d'], w['idx_d'], src, dst) == []
+
+
+def test_sddmm_shuffled_coo_at_feat_128(weighted):
+    """The same edges stored in a random order: `order='auto'` sorts them into the tiled traversal and scatters
+    every result back to its stored position; checked against float64 on a sample and, edge by edge, against
+    the CSR-ordered module's results permuted the same way."""
+    import torch
+    from featgraph_amd.benchmark import verify as chk
+    from featgraph_amd.module import VanillaSDDMMhip, placeholder
+    w = weighted
+    n, nnz, F = w['n'], w['nnz'], 128
+    perm = torch.randperm(nnz, generator=torch.Generator().manual_seed(3))
+    perm_d = perm.cuda()
+    rows_s, cols_s = w['rows_d'][perm_d], w['idx_d'][perm_d]
+    coo = sp.coo_matrix((np.ones(nnz, np.float32), (rows_s.cpu().numpy().astype(np.int32), cols_s.cpu().numpy().astype(np.int32))),
+                        shape=(n, n))
+    m = VanillaSDDMMhip(coo)
+    del coo
+    phs = [placeholder((n, F)), placeholder((n, F))]
+    m.build(phs, {}, {})
+    assert not m._row_sorted and m._tiled is not None and (m._tiled[0]['P'], m._tiled[1]) == SDDMM_DEFAULTS[F]
+    g = torch.Generator(device="cuda"); g.manual_seed(8)
+    src = torch.randn((n, F), generator=g, device="cuda")
+    dst = torch.randn((n, F), generator=g, device="cuda")
+    m.out_tvm.fill_(float("nan"))
+    out = m.run([src, dst])
+    assert chk.sddmm_failures(out, rows_s, cols_s, src, dst) == []
+    ordered = w['sddmm']
+    ordered.build(phs, {}, {})
+    ref = ordered.run([src, dst])
+    # the tiled traversal visits an edge's features in the same order whichever way the edges are stored
+    assert torch.equal(out, ref[perm_d])
+
+
 def test_sddmm_default_at_feat_512(graph):
     """What bench.py times: the tile-by-tile copy of Src, 8 partitions x 8 tiles, the sum over tiles."""
     import torch
