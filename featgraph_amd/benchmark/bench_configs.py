@@ -152,12 +152,48 @@ def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):
             del x, y
 
 
+def run_multihead_only(name, H, D, partitions, tiles, runs):
+    """One multi-head SDDMM shape on one workload (for profiler runs): a plain device copy of the source operand first
+    (the reference point that byte counters are scaled by), then `runs` launches after a warm-up."""
+    indptr, indices = synthetic.make_workload(name)
+    n = indptr.shape[0] - 1
+    nnz = int(indptr[-1])
+    adj = sp.csr_matrix((np.ones(nnz, np.float32), indices, indptr), shape=(n, n))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(2)
+    x = torch.randn((n, H, D), generator=gen, device="cuda")
+    y = torch.randn((n, H, D), generator=gen, device="cuda")
+    x_copy = torch.empty_like(x)
+    x_copy.copy_(x)
+    del x_copy
+    mh = MultiHeadSDDMMhip(adj)
+    sched = {}
+    if partitions:
+        sched['num_src_partitions'] = partitions
+    if tiles:
+        sched['num_feat_tiles'] = tiles
+    mh.build([placeholder((n, H, D)), placeholder((n, H, D))], {}, sched)
+    t = mh.measure_average_time([x, y], runs)
+    tiled = (mh._tiled[0]['P'], mh._tiled[1]) if mh._tiled else None
+    _line(name, "sddmm_multihead", {"heads": H, "head_len": D, "tiled": tiled, "copy_bytes": 4 * n * H * D}, t, nnz, H * D,
+          4 * (n + 1) + 4 * nnz + 8 * n * H * D + 4 * nnz * H)
+
+
 if __name__ == '__main__':
     ap = argparse.ArgumentParser()
     ap.add_argument("--quick", action="store_true", help="small graphs only")
+    ap.add_argument("--multihead", type=int, nargs=2, metavar=("H", "D"),
+                    help="only the multi-head SDDMM of this shape (see --workload, --partitions, --tiles, --runs)")
+    ap.add_argument("--workload", default="powerlaw-233k")
+    ap.add_argument("--partitions", type=int, default=0, help="source-column partitions (0: the library's choice)")
+    ap.add_argument("--tiles", type=int, default=0, help="feature tiles (0: the library's choice)")
+    ap.add_argument("--runs", type=int, default=5)
     ap.add_argument("--attention-only", action="store_true",
                     help="only the edge softmax / per-head SpMM steps on the 232,965-node graph")
     args = ap.parse_args()
+    if args.multihead:
+        run_multihead_only(args.workload, args.multihead[0], args.multihead[1], args.partitions, args.tiles, args.runs)
+        raise SystemExit(0)
     if args.attention_only:
         indptr, indices = synthetic.make_workload("powerlaw-233k")
         n = indptr.shape[0] - 1

@@ -333,33 +333,41 @@ def _partitions(n_src, row_bytes, nnz, n_rows, slice_bytes, min_segment):
 
 
 def _choose_sddmm_heads(n_rows, n_cols, nnz, heads, head_len):
-    """Several heads per edge: a tile's results are scattered per edge, so wider tiles (more heads per
-    write) win (232,965-node graph, H=8, D=32: 8.8 ms with 128-float tiles, 9.3 ms with 64; H=8, D=64: 16.0
-    against 16.8 ms) unless that leaves fewer than 4 tiles of whole 64-float heads (H=4, D=64: 7.7 ms, 7.3 ms
-    with 64-float tiles).  Partitions: two L2s' worth of slices per XCD, segments of 24 elements or more."""
+    """Several heads per edge.  What an (edge, tile) pair writes decides the tile: the memory system writes whole 32-byte
+    sectors, so a tile that holds fewer than 8 heads and scatters them to `out` pays a sector for its 8 or 16 bytes
+    (232,965-node graph, counted at the fabric: 8.0 GB written for 3.67 GB of results at H=8, D=32 with 128-float tiles,
+    16.2 GB at H=8, D=64).  Hence
+      * heads of up to 32 floats, 8 or more of them: 256-float tiles (8 or more heads, 32 bytes or more per edge and
+        tile, written where they belong) -- H=8, D=32: 8.64 -> 7.71 ms with one tile x 32 partitions;
+      * longer heads: one head per tile, each tile's results kept in traversal order (whole runs) and every edge's H
+        results written as one run by a last kernel -- H=8, D=64: 15.2 -> 13.4 ms with 8 tiles x 8 partitions;
+      * fewer than 8 short heads: 64-float tiles as before (H=4, D=32: one 128-float tile is no faster).
+    Partitions: two L2s' worth of slices per XCD, segments of 24 elements or more (12 for the 256-float tiles, whose
+    slices need four times the partitions: 7.7 ms at 32 partitions against 8.4 at 16)."""
     feat_len = heads * head_len
-    tile = None
-    if feat_len >= 256 and not (head_len >= 64 and feat_len // 128 < 4):
-        order = (128, 64, 256, 32, 16)
-    else:
-        order = (64, 128, 256, 32, 16)
-    for cand in order:
-        if feat_len % cand != 0:
-            continue
-        if cand % head_len == 0 or head_len == cand:
-            if head_len % 4 != 0 or head_len < 8 or (head_len & (head_len - 1)) != 0:
-                continue
-            tile = cand
-            break
-    if tile is None:
+    if head_len % 4 != 0 or head_len < 8 or (head_len & (head_len - 1)) != 0:
         return None
+    min_segment = 24
+    if head_len <= 32 and heads >= 8 and feat_len % 256 == 0:
+        tile, min_segment = 256, 12
+    elif head_len in (64, 128) and feat_len >= 256:
+        tile = head_len
+    else:
+        tile = None
+        for cand in (64, 128, 256, 32, 16):
+            if feat_len % cand == 0 and (cand % head_len == 0 or head_len == cand):
+                tile = cand
+                break
+        if tile is None:
+            return None
     t = feat_len // tile
     row_bytes = 4 * feat_len / t          # more than 8 tiles are launched 8 at a time: one tile's slice per XCD
     if n_cols * row_bytes <= SDDMM_SLICE_BYTES:
         return None
-    p = _partitions(n_cols, row_bytes, nnz, n_rows, SDDMM_SLICE_BYTES, min_segment=24)
-    if p > 1 and t < 8 and 8 % t == 0:
-        p = max(p, 8 // t)          # at least one partition per XCD: a single launch covers them all
+    p = _partitions(n_cols, row_bytes, nnz, n_rows, SDDMM_SLICE_BYTES, min_segment=min_segment)
+    if p > 1 and t < 8 and 8 % t == 0 and p < 8 // t:
+        # at least one partition per XCD (a single launch covers them all) -- unless that leaves the segments too short
+        p = 8 // t if nnz / max(1, n_rows) / (8 // t) >= min_segment else 1
     if p == 1:
         if feat_len <= 256 and (feat_len & (feat_len - 1)) == 0 and feat_len >= 16 and feat_len % head_len == 0:
             return 1, 1

@@ -179,9 +179,9 @@ def test_default_tilings():
     assert tuning.choose_sddmm(2450000, 2450000, 61903880, 1, 128) is None    # stored-order kernels
     assert tuning.choose_sddmm(2450000, 2450000, 61903880, 1, 512) is None    # no source partitions: stored order, not 1 x 2 tiles
     assert tuning.choose_sddmm(1000000, 1000000, 64998031, 1, 512) is None
-    assert tuning.choose_sddmm(n, n, nnz, 8, 64) == (16, 4)
+    assert tuning.choose_sddmm(n, n, nnz, 8, 64) == (8, 8)                     # one head per tile, results staged per tile
     assert tuning.choose_sddmm(n, n, nnz, 4, 64) == (8, 4)
-    assert tuning.choose_sddmm(n, n, nnz, 8, 32) == (16, 2)
+    assert tuning.choose_sddmm(n, n, nnz, 8, 32) == (32, 1)                    # all 8 heads in one 256-float tile: whole 32-byte runs
     assert tuning.choose_sddmm(n, n, nnz, 4, 32) == (8, 2)
     assert tuning.choose_sddmm(10000, 10000, 170000, 1, 32) is None           # fits the caches: plain kernels
     for F in (32, 64, 96, 128, 256, 512, 2048):
