@@ -36,16 +36,17 @@ HBM_PEAK_GBS = 8000.0
 # Fabric-side bytes (rocprofv3 FETCH_SIZE x2 + WRITE_SIZE, scaled by the X copy of the same run) moved
 # by all launches of the gather kernel in one operator call, at the default tiling (the JSON reports
 # them per launch as `traffic` and per operator as `op_traffic`, and names the summary they come from as
-# `traffic_source`).  Configurations without a committed summary: null.
+# `traffic_source`).  Configurations without a committed summary: null.  tests/test_bench_records.py holds every figure
+# to the "Per launch, after calibration" table of the summary it names (read + write GB of the gather kernel, within 1 %).
 _PROFILES = "profiles/bench_%s_rocprofv3.txt"
 MEASURED_TRAFFIC = {
     # (operator, workload, F, partitions, tiles): (bytes, summary); tiles 0 = the kernel's own single tile
     ("spmm", "powerlaw-233k", 512, 8, 8): (59.2e9, _PROFILES % "powerlaw233k_f512"),     # spmm_items_kernel (copy: +0.95e9, sum of the passes: +4.3e9)
     ("sddmm", "powerlaw-233k", 512, 8, 8): (61.2e9, _PROFILES % "powerlaw233k_f512"),    # sddmm_tiled_kernel (copy: +0.95e9, tile sum: +4.7e9)
-    ("spmm", "powerlaw-233k", 64, 8, 0): (7.96e9, _PROFILES % "powerlaw233k_f64"),
-    ("sddmm", "powerlaw-233k", 64, 8, 1): (8.83e9, _PROFILES % "powerlaw233k_f64"),
-    ("spmm", "powerlaw-233k", 32, 4, 0): (4.31e9, _PROFILES % "powerlaw233k_f32"),
-    ("sddmm", "powerlaw-233k", 32, 4, 1): (5.07e9, _PROFILES % "powerlaw233k_f32"),
+    ("spmm", "powerlaw-233k", 64, 8, 0): (8.50e9, _PROFILES % "powerlaw233k_f64"),
+    ("sddmm", "powerlaw-233k", 64, 8, 1): (9.30e9, _PROFILES % "powerlaw233k_f64"),
+    ("spmm", "powerlaw-233k", 32, 4, 0): (4.72e9, _PROFILES % "powerlaw233k_f32"),
+    ("sddmm", "powerlaw-233k", 32, 4, 1): (5.44e9, _PROFILES % "powerlaw233k_f32"),
     ("spmm", "powerlaw-2.45M", 128, 1, 1): (33.15e9, _PROFILES % "powerlaw2450k_f128"),
     ("sddmm", "powerlaw-2.45M", 128, 1, 1): (33.41e9, _PROFILES % "powerlaw2450k_f128"),
 }

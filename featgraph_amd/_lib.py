@@ -72,6 +72,7 @@ SIGNATURES = {
     "fg_graph_attention_additive_backward_er_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),
     "fg_graph_attention_additive_backward_elv_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, _vp]),
     "fg_synth_powerlaw_csr": (_int, [_i64, _vp, _vp, _vp, ctypes.c_uint64, _int, _vp, _vp]),
+    "fg_synth_community_csr": (_int, [_i64, _vp, _vp, _vp, _int, _vp, _vp, _vp, _vp, ctypes.c_double, ctypes.c_uint64, _int, _vp, _vp]),
 }
 
 

@@ -204,20 +204,55 @@ void draw_row(int64_t v, int64_t n, int32_t deg, const double *cdf, const int32_
     buf.erase(std::unique(buf.begin(), buf.end()), buf.end());
 }
 
-}  // namespace
+// The same with planted communities: each draw stays inside the row's own community with probability p_in (its
+// sources then come from that community's own distribution) and is a draw from the whole graph otherwise.
+struct Communities {
+    const int32_t *of_vertex;   // [n]
+    const int64_t *off;         // [n_comm + 1] into member / cdf
+    const int32_t *member;      // vertex ids, community by community
+    const double *cdf;          // per community, non-decreasing, last element 1
+    double p_in;
+};
 
-extern "C" int fg_synth_powerlaw_csr(int64_t n, const int32_t *in_degree, const double *cdf,
-                                     const int32_t *perm, uint64_t seed, int num_threads,
-                                     int32_t *indptr, int32_t *indices) {
-    if (n < 1 || !in_degree || !cdf || !perm || !indptr)
-        return fail(FG_ERR_ARG, "fg_synth_powerlaw_csr: bad argument");
+void draw_row_communities(int64_t v, int64_t n, int32_t deg, const double *cdf, const int32_t *perm, const Communities &cm,
+                          uint64_t seed, std::vector<int32_t> &buf) {
+    buf.clear();
+    buf.push_back((int32_t)v);                               // self-loop
+    const uint64_t key = mix64(seed ^ mix64((uint64_t)v));
+    const int32_t c = cm.of_vertex[v];
+    const double *ccdf = cm.cdf + cm.off[c];
+    const int64_t csize = cm.off[c + 1] - cm.off[c];
+    // a row that asks for more than half of its community keeps that many draws inside and takes the rest from the
+    // whole graph (a hub's neighbours are not confined to its community, and repeated draws would merge)
+    const double p_in = (double)deg * 2.0 <= (double)csize ? cm.p_in : cm.p_in * ((double)csize / 2.0) / (double)deg;
+    for (int32_t k = 0; k < deg; ++k) {
+        const uint64_t bits = mix64(key + (uint64_t)k * 0xd1342543de82ef95ull);
+        const double u = (double)(bits >> 11) * (1.0 / 9007199254740992.0);   // [0, 1)
+        const uint64_t bits2 = mix64(bits ^ 0xa0761d6478bd642full);
+        const double where = (double)(bits2 >> 11) * (1.0 / 9007199254740992.0);
+        if (where < p_in && csize > 0) {
+            int64_t at = std::upper_bound(ccdf, ccdf + csize, u) - ccdf;
+            if (at >= csize) at = csize - 1;
+            buf.push_back(cm.member[cm.off[c] + at]);
+        } else {
+            int64_t rank = std::upper_bound(cdf, cdf + n, u) - cdf;
+            if (rank >= n) rank = n - 1;
+            buf.push_back(perm[rank]);
+        }
+    }
+    std::sort(buf.begin(), buf.end());
+    buf.erase(std::unique(buf.begin(), buf.end()), buf.end());
+}
+
+template <typename Draw>
+int synth_csr(int64_t n, int num_threads, int32_t *indptr, int32_t *indices, const char *what, Draw draw) {
     const int nt = num_threads > 0 ? num_threads : fg::default_threads();
     if (!indices) {
         // first call: row lengths only
         fg::parallel_ranges(n, nt, [&](int, int64_t v0, int64_t v1) {
             std::vector<int32_t> buf;
             for (int64_t v = v0; v < v1; ++v) {
-                draw_row(v, n, in_degree[v], cdf, perm, seed, buf);
+                draw(v, buf);
                 indptr[v + 1] = (int32_t)buf.size();
             }
         });
@@ -234,11 +269,41 @@ extern "C" int fg_synth_powerlaw_csr(int64_t n, const int32_t *in_degree, const 
     fg::parallel_ranges(n, nt, [&](int, int64_t v0, int64_t v1) {
         std::vector<int32_t> buf;
         for (int64_t v = v0; v < v1; ++v) {
-            draw_row(v, n, in_degree[v], cdf, perm, seed, buf);
+            draw(v, buf);
             if ((int64_t)buf.size() != indptr[v + 1] - indptr[v]) { bad.store(true, std::memory_order_relaxed); continue; }
             std::copy(buf.begin(), buf.end(), indices + indptr[v]);
         }
     });
-    if (bad.load()) return fail(FG_ERR_ARG, "fg_synth_powerlaw_csr: indptr does not match this seed");
+    if (bad.load()) return fail(FG_ERR_ARG, "%s: indptr does not match this seed", what);
     return FG_OK;
+}
+
+}  // namespace
+
+extern "C" int fg_synth_community_csr(int64_t n, const int32_t *in_degree, const double *cdf, const int32_t *perm,
+                                      int n_comm, const int32_t *comm_of_vertex, const int64_t *comm_off,
+                                      const int32_t *comm_member, const double *comm_cdf, double p_in, uint64_t seed,
+                                      int num_threads, int32_t *indptr, int32_t *indices) {
+    if (n < 1 || !in_degree || !cdf || !perm || !indptr || n_comm < 1 || !comm_of_vertex || !comm_off || !comm_member ||
+        !comm_cdf || !(p_in >= 0.0 && p_in <= 1.0))
+        return fail(FG_ERR_ARG, "fg_synth_community_csr: bad argument");
+    if (comm_off[0] != 0 || comm_off[n_comm] != n) return fail(FG_ERR_ARG, "fg_synth_community_csr: communities must cover the n vertices");
+    for (int64_t v = 0; v < n; ++v)
+        if (comm_of_vertex[v] < 0 || comm_of_vertex[v] >= n_comm) return fail(FG_ERR_ARG, "fg_synth_community_csr: community id out of range");
+    for (int64_t i = 0; i < n; ++i)
+        if (comm_member[i] < 0 || comm_member[i] >= n) return fail(FG_ERR_ARG, "fg_synth_community_csr: member id out of range");
+    const Communities cm{comm_of_vertex, comm_off, comm_member, comm_cdf, p_in};
+    return synth_csr(n, num_threads, indptr, indices, "fg_synth_community_csr", [&](int64_t v, std::vector<int32_t> &buf) {
+        draw_row_communities(v, n, in_degree[v], cdf, perm, cm, seed, buf);
+    });
+}
+
+extern "C" int fg_synth_powerlaw_csr(int64_t n, const int32_t *in_degree, const double *cdf,
+                                     const int32_t *perm, uint64_t seed, int num_threads,
+                                     int32_t *indptr, int32_t *indices) {
+    if (n < 1 || !in_degree || !cdf || !perm || !indptr)
+        return fail(FG_ERR_ARG, "fg_synth_powerlaw_csr: bad argument");
+    return synth_csr(n, num_threads, indptr, indices, "fg_synth_powerlaw_csr", [&](int64_t v, std::vector<int32_t> &buf) {
+        draw_row(v, n, in_degree[v], cdf, perm, seed, buf);
+    });
 }

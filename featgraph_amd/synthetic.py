@@ -75,6 +75,52 @@ def uniform_csr(n, avg_degree, seed, num_threads=0):
     return _draw(n, in_degree, cdf, perm, seed, num_threads)
 
 
+def community_csr(n, total_edges, exponent, max_degree, n_comm, p_in, contiguous, seed, num_threads=0):
+    """Power-law graph with planted communities (rows = destinations): the degrees and the whole-graph source
+    distribution of powerlaw_csr, but every draw of a row stays inside the row's community with probability `p_in`
+    (sources then follow the community's own share of the same weights; rows whose degree exceeds half the
+    community's size keep that many draws inside it and take the rest from the whole graph).  Rank r belongs to community r % n_comm, so
+    every community has its hubs.  `contiguous`: vertex ids are community-major (a community's vertices are
+    consecutive ids, in a seeded order inside it), so consecutive rows share their hot columns; otherwise ranks are
+    mapped to ids by a seeded permutation of all vertices (the same graph up to relabelling).  The stand-in for the
+    Reddit adjacency of benchmark/bench_vanilla_spmm.py:78-79 (41 subreddit communities), which needs a network."""
+    w = powerlaw_weights(n, float(total_edges - n), exponent, float(max_degree))
+    ranks = np.arange(n, dtype=np.int64)
+    comm_of_rank = (ranks % n_comm).astype(np.int32)
+    if contiguous:
+        keys = _mix64(ranks.astype(np.uint64) ^ _mix64(np.full(n, seed, dtype=np.uint64)))
+        order = np.lexsort((keys, comm_of_rank))               # ranks, community by community, seeded order inside
+        perm = np.empty(n, dtype=np.int32)
+        perm[order] = np.arange(n, dtype=np.int32)             # rank -> vertex id
+    else:
+        perm = seeded_permutation(n, seed)
+    in_degree = np.empty(n, dtype=np.int32)
+    in_degree[perm] = np.maximum(np.rint(w), 0).astype(np.int32)
+    cdf = np.cumsum(w)
+    cdf /= cdf[-1]
+    cdf[-1] = 1.0
+    comm_of_vertex = np.empty(n, dtype=np.int32)
+    comm_of_vertex[perm] = comm_of_rank
+    by_comm = np.argsort(comm_of_rank, kind="stable")          # ranks, community by community, ascending rank inside
+    comm_off = np.zeros(n_comm + 1, dtype=np.int64)
+    np.cumsum(np.bincount(comm_of_rank, minlength=n_comm), out=comm_off[1:])
+    comm_member = np.ascontiguousarray(perm[by_comm], dtype=np.int32)
+    comm_cdf = np.empty(n, dtype=np.float64)
+    for c in range(n_comm):
+        part = np.cumsum(w[by_comm[comm_off[c]:comm_off[c + 1]]])
+        part /= part[-1]
+        part[-1] = 1.0
+        comm_cdf[comm_off[c]:comm_off[c + 1]] = part
+    L = _lib.lib()
+    args = (n, _lib.host_ptr(in_degree), _lib.host_ptr(cdf), _lib.host_ptr(perm), int(n_comm), _lib.host_ptr(comm_of_vertex),
+            _lib.host_ptr(comm_off), _lib.host_ptr(comm_member), _lib.host_ptr(comm_cdf), float(p_in), int(seed), int(num_threads))
+    indptr = np.zeros(n + 1, dtype=np.int32)
+    _lib.check(L.fg_synth_community_csr(*args, _lib.host_ptr(indptr), None))
+    indices = np.zeros(int(indptr[-1]), dtype=np.int32)
+    _lib.check(L.fg_synth_community_csr(*args, _lib.host_ptr(indptr), _lib.host_ptr(indices)))
+    return indptr, indices
+
+
 def _draw(n, in_degree, cdf, perm, seed, num_threads):
     L = _lib.lib()
     in_degree = np.ascontiguousarray(in_degree, dtype=np.int32)
@@ -106,6 +152,14 @@ WORKLOADS = {
     # graphs of other shapes, for checking that the tiling defaults carry over (seeds of their own)
     "uniform-1M-deg64": dict(kind="uniform", n=1_000_000, avg_degree=64, seed=11),
     "powerlaw-1M-deg100-g2.5": dict(kind="powerlaw", n=1_000_000, total_edges=100_000_000, exponent=2.5, max_degree=30000, seed=12),
+    # planted communities at the benchmark graph's size (41, like Reddit's subreddits; 80 % of a row's draws stay inside
+    # its community): once with community-contiguous vertex ids, once with the same kind of graph randomly relabelled
+    "communities-233k": dict(kind="community", n=232965, total_edges=139_600_000, exponent=2.1, max_degree=26500,
+                             n_comm=41, p_in=0.8, contiguous=True, seed=14),
+    "communities-233k-relabelled": dict(kind="community", n=232965, total_edges=139_600_000, exponent=2.1, max_degree=26500,
+                                        n_comm=41, p_in=0.8, contiguous=False, seed=14),
+    "communities-23k": dict(kind="community", n=23296, total_edges=1_300_000, exponent=2.1, max_degree=2000,
+                            n_comm=8, p_in=0.8, contiguous=True, seed=15),
     # non-square: the first 100,000 destination rows of a 1M-node graph, all 1M sources
     "nonsquare-100k-x-1M": dict(kind="powerlaw", n=1_000_000, total_edges=80_000_000, exponent=2.2, max_degree=20000, seed=13,
                                 rows=100_000),
@@ -119,6 +173,9 @@ def make_workload(name, seed=None, num_threads=0):
         seed = spec.get("seed", 0xFEA7)
     if spec["kind"] == "uniform":
         indptr, indices = uniform_csr(spec["n"], spec["avg_degree"], seed, num_threads)
+    elif spec["kind"] == "community":
+        indptr, indices = community_csr(spec["n"], spec["total_edges"], spec["exponent"], spec["max_degree"], spec["n_comm"],
+                                        spec["p_in"], spec["contiguous"], seed, num_threads)
     else:
         indptr, indices = powerlaw_csr(spec["n"], spec["total_edges"], spec["exponent"], spec["max_degree"], seed, num_threads)
     if "rows" in spec:
