@@ -45,6 +45,8 @@ SIGNATURES = {
     "fg_spmm_plan_destroy": (None, [_vp]),
     "fg_spmm_plan_reserve": (_int, [_vp, _int, _int, _int, _int]),
     "fg_spmm_plan_narrow_indices": (_int, [_vp, _vp, _vp]),
+    "fg_debug_checks": (_int, [_int]),
+    "fg_spmm_plan_bytes": (_i64, [_vp]),
     "fg_spmm_plan_describe": (_int, [_vp, _int, _int, ctypes.c_char_p, ctypes.c_size_t]),
     "fg_spmm_csr_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),
     "fg_spmm_csr_noalloc_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _vp]),

@@ -73,6 +73,8 @@ struct fg_spmm_plan {
     // plan: the kernels that can read it do so whenever a call hands them the int32 array it was made from.
     uint16_t *idx16_dev = nullptr;
     const int32_t *idx16_src = nullptr;
+    uint64_t idx16_fingerprint = 0;               // of idx16_src's contents when the copy was made (fg_debug_checks re-checks it)
+    unsigned long long *idx16_words_dev = nullptr; // two device words: the range flag and the fingerprint under construction
     // statistics for fg_spmm_plan_describe
     int64_t max_len = 0, n_empty = 0, n_split_rows = 0, n_multi_items = 0;
 };
@@ -97,10 +99,12 @@ bool wants_tile_major(const fg_spmm_plan *plan, int n_tiles, uint64_t x_bytes);
 // the call fills copy `slot`.  The buffer must already be large enough (ensure_scratch).
 int make_tile_major(const fg_spmm_plan *plan, const float *x, int64_t n_rows, int F, int tile, void *stream,
                     int slot = 0, int n_slots = 1);
-// The plan's 16-bit copy of `idx` when it has one of exactly this array, else null.
-inline const uint16_t *narrow_indices(const fg_spmm_plan *plan, const int32_t *idx) {
-    return (plan->idx16_dev && idx && idx == plan->idx16_src) ? plan->idx16_dev : nullptr;
-}
+// The plan's 16-bit copy of `idx` when it has one of exactly this array (same address), else null.  With
+// fg_debug_checks(1) the array's fingerprint is compared as well (a device round trip per call): an array that was
+// rewritten or replaced at the same address is then read as int32 and the mismatch is left in fg_last_error().
+const uint16_t *narrow_indices(const fg_spmm_plan *plan, const int32_t *idx);
+// Looks up, once per device, the address of the fixed array that fg_spmm_csr_noalloc_f32 keeps its partial sums in.
+void prepare_fixed_scratch(int dev);
 // FG_OK when the calling thread's current device is the one the plan was created on.
 int check_device(const fg_spmm_plan *plan);
 

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <string>
 
@@ -108,6 +109,7 @@ extern "C" int fg_spmm_plan_create(const int32_t *pos, int64_t n_dst, int64_t n_
     pl->n_fixups = (int64_t)fixups.size();
 
     hipError_t e = hipGetDevice(&pl->device);
+    if (e == hipSuccess && P == 1) fg::prepare_fixed_scratch(pl->device);
     if (e == hipSuccess && pl->n_items) e = hipMalloc((void **)&pl->items_dev, sizeof(Item) * items.size());
     if (e == hipSuccess && pl->n_items)
         e = hipMemcpy(pl->items_dev, items.data(), sizeof(Item) * items.size(), hipMemcpyHostToDevice);
@@ -133,6 +135,7 @@ extern "C" void fg_spmm_plan_destroy(fg_spmm_plan *pl) {
     if (pl->partial_dev) (void)hipFree(pl->partial_dev);
     if (pl->tiled_dev) (void)hipFree(pl->tiled_dev);
     if (pl->idx16_dev) (void)hipFree(pl->idx16_dev);
+    if (pl->idx16_words_dev) (void)hipFree(pl->idx16_words_dev);
     delete pl;
 }
 
@@ -208,38 +211,135 @@ std::string spmm_launch_text(const fg_spmm_plan *plan, int F, int num_feat_parti
 }
 
 namespace {
-// dst[i] = (uint16_t)src[i], four elements per lane (the tail one by one).
-__global__ __launch_bounds__(256) void narrow_indices_kernel(const int32_t *src, uint16_t *dst, int64_t n) {
+// dst[i] = (uint16_t)src[i], four elements per lane (the tail one by one); *bad is set when an id lies outside [0, width).
+__global__ __launch_bounds__(256) void narrow_indices_kernel(const int32_t *src, uint16_t *dst, int64_t n, int32_t width, int32_t *bad) {
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= n) return;
-    for (int k = 0; k < 4 && i + k < n; ++k) dst[i + k] = (uint16_t)src[i + k];
+    bool out_of_range = false;
+    for (int k = 0; k < 4 && i + k < n; ++k) {
+        const int32_t c = src[i + k];
+        out_of_range |= (c < 0 || c >= width);
+        dst[i + k] = (uint16_t)c;
+    }
+    if (out_of_range) atomicOr(bad, 1);
 }
+
+__device__ __forceinline__ uint64_t mix64_dev(uint64_t z) {          // splitmix64 finaliser
+    z += 0x9e3779b97f4a7c15ull;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+// A cheap fingerprint of an id array: the sum of a hash of (position, id) over the first and the last kPrintIds ids.
+constexpr int kPrintIds = 1024;
+__global__ __launch_bounds__(256) void fingerprint_kernel(const int32_t *src, int64_t n, unsigned long long *out) {
+    unsigned long long h = 0;
+    for (int64_t j = threadIdx.x; j < 2 * kPrintIds; j += 256) {
+        const int64_t i = j < kPrintIds ? j : n - 2 * kPrintIds + j;      // the last kPrintIds positions
+        if (i < 0 || i >= n || (j >= kPrintIds && i < kPrintIds)) continue;
+        h += mix64_dev(((uint64_t)i << 32) ^ (uint32_t)src[i]);
+    }
+    if (h) atomicAdd(out, h);
+}
+
+// words_dev[0] holds the range flag of narrow_indices_kernel, words_dev[1] the fingerprint; read back synchronously
+int fingerprint(const int32_t *idx_dev, int64_t n, hipStream_t st, unsigned long long *words_dev, uint64_t *out) {
+    FG_HIP_TRY(hipMemsetAsync(words_dev + 1, 0, sizeof(unsigned long long), st));
+    hipLaunchKernelGGL(fingerprint_kernel, dim3(1), dim3(256), 0, st, idx_dev, n, words_dev + 1);
+    FG_HIP_TRY(hipGetLastError());
+    unsigned long long h = 0;
+    FG_HIP_TRY(hipMemcpyAsync(&h, words_dev + 1, sizeof(h), hipMemcpyDeviceToHost, st));
+    FG_HIP_TRY(hipStreamSynchronize(st));
+    *out = (uint64_t)h + (uint64_t)n;
+    return FG_OK;
+}
+
+std::atomic<int> g_debug_checks{0};
 }  // namespace
+
+extern "C" int fg_debug_checks(int on) { return g_debug_checks.exchange(on ? 1 : 0); }
+
+namespace fg {
+const uint16_t *narrow_indices(const fg_spmm_plan *plan, const int32_t *idx) {
+    if (!plan->idx16_dev || !idx || idx != plan->idx16_src) return nullptr;
+    if (g_debug_checks.load(std::memory_order_relaxed)) {
+        // the array at this address must still be the one the copy was made from
+        uint64_t now = 0;
+        if (fingerprint(idx, plan->nnz, nullptr, plan->idx16_words_dev, &now) != FG_OK) return nullptr;
+        if (now != plan->idx16_fingerprint) {
+            fail(FG_ERR_ARG, "the int32 column ids at %p changed after fg_spmm_plan_narrow_indices copied them; the int32 array is read instead",
+                 (const void *)idx);
+            return nullptr;
+        }
+    }
+    return plan->idx16_dev;
+}
+}  // namespace fg
 
 extern "C" int fg_spmm_plan_narrow_indices(fg_spmm_plan *pl, const int32_t *idx_dev, void *stream) {
     if (!pl) return fail(FG_ERR_ARG, "plan is null");
     if (int drc = fg::check_device(pl)) return drc;
+    auto forget = [&]() {
+        if (pl->idx16_dev) (void)hipFree(pl->idx16_dev);
+        pl->idx16_dev = nullptr; pl->idx16_src = nullptr; pl->idx16_fingerprint = 0;
+    };
     if (!idx_dev) {                                  // forget the copy
-        if (pl->idx16_dev) FG_HIP_TRY(hipFree(pl->idx16_dev));
-        pl->idx16_dev = nullptr; pl->idx16_src = nullptr;
+        forget();
         return FG_OK;
     }
     const int64_t width = (pl->n_src + pl->num_col_partitions - 1) / pl->num_col_partitions;
     if (width > 65536)
         return fail(FG_ERR_SHAPE, "column ids of partitions %lld columns wide do not fit 16 bits", (long long)width);
-    if (pl->idx16_dev) FG_HIP_TRY(hipFree(pl->idx16_dev));
-    pl->idx16_dev = nullptr; pl->idx16_src = nullptr;
+    forget();
     if (pl->nnz == 0) return FG_OK;
+    if (!pl->idx16_words_dev && hipMalloc((void **)&pl->idx16_words_dev, 2 * sizeof(unsigned long long)) != hipSuccess) {
+        (void)hipGetLastError();
+        pl->idx16_words_dev = nullptr;
+        return fail(FG_ERR_NOMEM, "cannot allocate the 16-bit column ids' check words");
+    }
     if (hipMalloc((void **)&pl->idx16_dev, (size_t)pl->nnz * sizeof(uint16_t)) != hipSuccess) {
         (void)hipGetLastError();
         pl->idx16_dev = nullptr;
         return fail(FG_ERR_NOMEM, "cannot allocate %zu bytes for the 16-bit column ids", (size_t)pl->nnz * sizeof(uint16_t));
     }
-    const int64_t blocks = (pl->nnz + 1023) / 1024;
-    hipLaunchKernelGGL(narrow_indices_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, idx_dev, pl->idx16_dev, pl->nnz);
-    FG_HIP_TRY(hipGetLastError());
+    hipStream_t st = (hipStream_t)stream;
+    int32_t *bad_dev = reinterpret_cast<int32_t *>(pl->idx16_words_dev);
+    hipError_t e = hipMemsetAsync(bad_dev, 0, sizeof(int32_t), st);
+    if (e == hipSuccess) {
+        const int64_t blocks = (pl->nnz + 1023) / 1024;
+        hipLaunchKernelGGL(narrow_indices_kernel, dim3((unsigned)blocks), dim3(256), 0, st, idx_dev, pl->idx16_dev, pl->nnz,
+                           (int32_t)std::max<int64_t>(width, 1), bad_dev);
+        e = hipGetLastError();
+    }
+    int32_t bad = 0;
+    if (e == hipSuccess) e = hipMemcpyAsync(&bad, bad_dev, sizeof(bad), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) {
+        forget();
+        return fail(FG_ERR_HIP, "fg_spmm_plan_narrow_indices: %s", hipGetErrorString(e));
+    }
+    if (bad) {
+        forget();
+        return fail(FG_ERR_GRAPH, "fg_spmm_plan_narrow_indices: a column id lies outside [0, %lld)", (long long)width);
+    }
+    if (int rc = fingerprint(idx_dev, pl->nnz, st, pl->idx16_words_dev, &pl->idx16_fingerprint)) {
+        forget();
+        return rc;
+    }
     pl->idx16_src = idx_dev;
     return FG_OK;
+}
+
+extern "C" int64_t fg_spmm_plan_bytes(const fg_spmm_plan *pl) {
+    if (!pl) return 0;
+    int64_t b = 0;
+    b += (int64_t)pl->n_items * (int64_t)sizeof(Item) + (int64_t)pl->n_fixups * (int64_t)sizeof(Fixup);
+    b += (int64_t)(pl->num_col_partitions + 1) * (int64_t)sizeof(int64_t);
+    b += (int64_t)pl->partial_floats * 4 + (int64_t)pl->tiled_floats * 4;
+    if (pl->idx16_dev) b += pl->nnz * 2;
+    if (pl->idx16_words_dev) b += 16;
+    return b;
 }
 
 extern "C" int fg_spmm_plan_reserve(fg_spmm_plan *pl, int op, int heads, int head_len, int num_feat_partitions) {

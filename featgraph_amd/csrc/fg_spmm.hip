@@ -1267,6 +1267,15 @@ int fixed_scratch(int dev, float **ptr) {
 }
 }  // namespace
 
+namespace fg {
+// Called by fg_spmm_plan_create (never under stream capture), so that fg_spmm_csr_noalloc_f32 finds the address known
+// when its first call on this device is being recorded into a graph.  A failure here is reported by that call instead.
+void prepare_fixed_scratch(int dev) {
+    float *ptr = nullptr;
+    (void)fixed_scratch(dev, &ptr);
+}
+}  // namespace fg
+
 extern "C" int fg_spmm_csr_noalloc_f32(const fg_spmm_plan *plan, const int32_t *indptr_dev,
                                        const int32_t *indices_dev, const float *vals_dev, const float *x_dev,
                                        float *out_dev, int F, int num_feat_partitions, void *stream) {

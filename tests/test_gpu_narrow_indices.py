@@ -197,3 +197,85 @@ def test_broadcasting_spmm_bit_identical(msg, reduce, P):
     wide, narrow = _with(False, run), _with(True, run)
     assert np.isfinite(narrow).all()
     assert np.array_equal(wide, narrow)
+
+
+def _small_csr(rng, n_dst, n_src, per_row):
+    rows = [np.unique(rng.integers(0, n_src, size=per_row)).astype(np.int32) for _ in range(n_dst)]
+    indptr = np.zeros(n_dst + 1, np.int32)
+    indptr[1:] = np.cumsum([len(c) for c in rows])
+    return indptr, np.concatenate(rows).astype(np.int32)
+
+
+def test_rewritten_ids_need_a_new_copy_and_the_debug_check_sees_stale_ones():
+    """C ABI directly.  The 16-bit copy is bound to the int32 array by address: after the array has been overwritten in
+    place with other ids (what an allocator that hands the same address out again amounts to), narrowing again gives
+    the new product; without it the stale copy would be gathered through -- which fg_debug_checks(1) detects by the
+    array's fingerprint, reading the int32 array instead and leaving a message."""
+    import torch
+    from featgraph_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(12)
+    n_dst, n_src, F = 400, 3000, 32
+    indptr, idx_a = _small_csr(rng, n_dst, n_src, 20)
+    # other ids with the same row lengths (sorted inside each row), different in the first and the last rows as well
+    idx_b = np.concatenate([np.sort(rng.choice(n_src, size=indptr[r + 1] - indptr[r], replace=False)) for r in range(n_dst)]).astype(np.int32)
+    assert (idx_a[:64] != idx_b[:64]).any() and (idx_a[-64:] != idx_b[-64:]).any()
+    vals = rng.random(idx_a.shape[0]).astype("float32")
+    x = rng.standard_normal((n_src, F)).astype("float32")
+    ref = {k: sp.csr_matrix((vals.astype(np.float64), ix, indptr), shape=(n_dst, n_src)).dot(x.astype(np.float64))
+           for k, ix in (("a", idx_a), ("b", idx_b))}
+    plan = ctypes.c_void_p()
+    _lib.check(L.fg_spmm_plan_create(_lib.host_ptr(indptr), n_dst, n_src, 1, None, ctypes.byref(plan)))
+    was = L.fg_debug_checks(0)
+    try:
+        ip, ix, vl, xd = (torch.from_numpy(a).cuda() for a in (indptr, idx_a, vals, x))
+        out = torch.empty((n_dst, F), device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def spmm():
+            out.fill_(float("nan"))
+            _lib.check(L.fg_spmm_csr_f32(plan, _lib.dev_ptr(ip), _lib.dev_ptr(ix), _lib.dev_ptr(vl), _lib.dev_ptr(xd),
+                                         _lib.dev_ptr(out), F, 0, stream))
+            return out.cpu().numpy().copy()
+
+        _lib.check(L.fg_spmm_plan_narrow_indices(plan, _lib.dev_ptr(ix), stream))
+        np.testing.assert_allclose(spmm(), ref["a"], rtol=1e-4, atol=1e-4)
+        ix.copy_(torch.from_numpy(idx_b).cuda())                # same address, other ids
+        # the debug check notices, the call reads the int32 array and is right; the message says why
+        L.fg_debug_checks(1)
+        np.testing.assert_allclose(spmm(), ref["b"], rtol=1e-4, atol=1e-4)
+        assert b"changed after fg_spmm_plan_narrow_indices" in L.fg_last_error()
+        L.fg_debug_checks(0)
+        # narrowing again binds the copy to the new contents
+        _lib.check(L.fg_spmm_plan_narrow_indices(plan, _lib.dev_ptr(ix), stream))
+        narrow_b = spmm()
+        np.testing.assert_allclose(narrow_b, ref["b"], rtol=1e-4, atol=1e-4)
+        L.fg_debug_checks(1)
+        assert np.array_equal(spmm(), narrow_b)                  # fingerprint matches: the copy is used, same bits
+        L.fg_debug_checks(0)
+        _lib.check(L.fg_spmm_plan_narrow_indices(plan, None, stream))
+        assert np.array_equal(spmm(), narrow_b)                  # and the int32 stream gives the same bits
+    finally:
+        L.fg_debug_checks(was)
+        L.fg_spmm_plan_destroy(plan)
+
+
+def test_ids_outside_the_partition_are_refused():
+    """An id that would not survive the cast to 16 bits (or lies outside the partition's width) fails the narrowing
+    instead of being truncated."""
+    import torch
+    from featgraph_amd import _lib
+    L = _lib.lib()
+    indptr = np.array([0, 2, 3], np.int32)
+    plan = ctypes.c_void_p()
+    _lib.check(L.fg_spmm_plan_create(_lib.host_ptr(indptr), 2, 1000, 1, None, ctypes.byref(plan)))
+    try:
+        for bad in (70000, 1000, -1):
+            ix = torch.tensor([1, bad, 5], dtype=torch.int32, device="cuda")
+            assert L.fg_spmm_plan_narrow_indices(plan, _lib.dev_ptr(ix), None) == -3      # FG_ERR_GRAPH
+            assert b"outside [0, 1000)" in L.fg_last_error()
+        ix = torch.tensor([1, 999, 5], dtype=torch.int32, device="cuda")
+        _lib.check(L.fg_spmm_plan_narrow_indices(plan, _lib.dev_ptr(ix), None))
+        assert L.fg_spmm_plan_bytes(plan) >= 3 * 2
+    finally:
+        L.fg_spmm_plan_destroy(plan)

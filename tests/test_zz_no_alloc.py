@@ -88,3 +88,58 @@ def test_noalloc_refuses_what_does_not_fit():
         assert L.fg_spmm_csr_noalloc_f32(None, p(x), p(x), p(x), p(x), p(x), 8, 0, None) == -1
     finally:
         L.fg_spmm_plan_destroy(plan2)
+
+
+def test_noalloc_allocates_nothing_and_can_be_the_recorded_call():
+    """The entry point on a plan whose scratch was never reserved: the plan's device memory and the device's free memory
+    are the same before and after, and its very first call may be the one recorded into a HIP graph (the fixed array's
+    address is looked up when the plan is created); replays between eager work reproduce the eager result bit for bit."""
+    import torch
+    from featgraph_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(73)
+    adj = _graph(rng, 300, 4000, (3, 40, 250), 3500, 0.01)
+    F = 128
+    indptr = np.ascontiguousarray(adj.indptr, dtype=np.int32)
+    p = _lib.dev_ptr
+    x = torch.from_numpy(rng.standard_normal((4000, F)).astype("float32")).cuda()
+    ip, ix, vals = (torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (indptr, adj.indices, adj.data))
+    ref = torch.full((300, F), float("nan"), device="cuda")
+    got = torch.full((300, F), float("nan"), device="cuda")
+    plan = ctypes.c_void_p()
+    assert L.fg_spmm_plan_create(_lib.host_ptr(indptr), 300, 4000, 1, None, ctypes.byref(plan)) == 0
+    plan_ref = ctypes.c_void_p()
+    assert L.fg_spmm_plan_create(_lib.host_ptr(indptr), 300, 4000, 1, None, ctypes.byref(plan_ref)) == 0
+    try:
+        assert L.fg_spmm_csr_f32(plan_ref, p(ip), p(ix), p(vals), p(x), p(ref), F, 2, None) == 0
+        torch.cuda.synchronize()
+        bytes_before = L.fg_spmm_plan_bytes(plan)
+        free_before = torch.cuda.mem_get_info()[0]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            rc = L.fg_spmm_csr_noalloc_f32(plan, p(ip), p(ix), p(vals), p(x), p(got), F, 2, s)
+        assert rc == 0, L.fg_last_error()
+        for k in range(3):
+            got.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(got, ref), "replay %d differs" % k
+            # eager work of another shape between the replays shares the fixed array
+            small = _graph(rng, 40, 1500, (7,), 1300, 0.02)
+            x2 = torch.from_numpy(rng.standard_normal((1500, 32)).astype("float32")).cuda()
+            r2, g2, rc2 = _both(L, _lib, small, x2, 32, 0)
+            assert rc2 == 0 and torch.equal(r2, g2)
+        assert L.fg_spmm_plan_bytes(plan) == bytes_before              # the plan's scratch was never grown
+        x.copy_(x * 2)                                                  # new inputs through the same graph
+        graph.replay()
+        torch.cuda.synchronize()
+        assert L.fg_spmm_csr_f32(plan_ref, p(ip), p(ix), p(vals), p(x), p(ref), F, 2, None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref)
+        del graph
+        assert torch.cuda.mem_get_info()[0] >= free_before - (8 << 20)  # nothing of the operator's size was taken from the device
+    finally:
+        L.fg_spmm_plan_destroy(plan)
+        L.fg_spmm_plan_destroy(plan_ref)
