@@ -249,6 +249,7 @@ def run_configs(torch, workload, indptr, indices, vals_d, spmm, sddmm, headline_
             pair("cfg2/cfg3", workload, indptr, idx_d, rows_d, vals_d, spmm, sddmm, F)
     pair("cfg3", workload, indptr, idx_d, rows_d, vals_d, spmm, sddmm, headline_F, sddmm_only_order='coo')
     mh = MultiHeadSDDMMhip(sp.csr_matrix((np.ones(nnz, np.float32), indices, indptr), shape=(n, n)))
+    mh.share_layouts(spmm)
     for H, D in ((4, 32), (4, 64), (8, 32), (8, 64)):
         gen.manual_seed(2)
         x = torch.randn((n, H, D), generator=gen, device="cuda")
@@ -299,7 +300,10 @@ def main():
         sys.exit("bench.py needs a ROCm GPU")
     torch.cuda.set_device(0)
     F = args.feat_len
+    setup = {}
+    t0 = time.perf_counter()
     indptr, indices = synthetic.make_workload(args.workload)
+    setup["graph_generation_s"] = round(time.perf_counter() - t0, 3)
     n = indptr.shape[0] - 1
     nnz = int(indptr[-1])
     deg = np.diff(indptr)
@@ -312,10 +316,21 @@ def main():
     vals = vals_d.cpu().numpy()
     adj = sp.csr_matrix((vals, indices, indptr), shape=(n, n))
 
-    spmm = VanillaSpMMhip(adj, args.num_col_partitions)
-    spmm.build([placeholder((n, F))], {'num_feat_partitions': args.num_feat_partitions}, {})
-    sddmm = VanillaSDDMMhip(adj)
-    sddmm.build([placeholder((n, F)), placeholder((n, F))], {}, {})
+    def timed(key, fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        res = fn()
+        torch.cuda.synchronize()
+        setup[key] = round(time.perf_counter() - t0, 3)
+        return res
+
+    # construction: structure checks and host arrays; build(): the cost model's choice, the source-partitioned copy of the
+    # adjacency (converted on the host), its work plan, the upload, the 16-bit column ids and the scratch
+    spmm = timed("spmm_construct_s", lambda: VanillaSpMMhip(adj, args.num_col_partitions))
+    timed("spmm_build_s", lambda: spmm.build([placeholder((n, F))], {'num_feat_partitions': args.num_feat_partitions}, {}))
+    sddmm = timed("sddmm_construct_s", lambda: VanillaSDDMMhip(adj))
+    sddmm.share_layouts(spmm)           # same adjacency: one partitioned copy, one plan, one scratch for both operators
+    timed("sddmm_build_s", lambda: sddmm.build([placeholder((n, F)), placeholder((n, F))], {}, {}))
     del adj
 
     def step(ev=None):
@@ -346,6 +361,14 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     # outside the timed region: the operators' outputs for these inputs are checked, and the reference's own
     # protocol (mean of 5 back-to-back runs, python/featgraph/module/spmm.py:179-186) is timed as well
+    # what the two modules and their inputs hold on the device: the modules' own accounts (graph arrays; plans = the
+    # library's own allocations, fg_spmm_plan_bytes; output buffers) and the device's view of the whole process
+    free_b, total_b = torch.cuda.mem_get_info()
+    gb = lambda b: round(b / 1e9, 3)
+    device_mem = {"spmm_module_gb": {k: gb(v) for k, v in spmm.device_bytes().items()},
+                  "sddmm_module_gb": {k: gb(v) for k, v in sddmm.device_bytes().items()},
+                  "inputs_gb": gb(4 * (2 * n * F + nnz)), "torch_peak_allocated_gb": gb(torch.cuda.max_memory_allocated()),
+                  "process_total_gb": gb(total_b - free_b)}
     failures = verify(torch, spmm, sddmm, indptr, torch.from_numpy(indices).cuda().long(), vals_d, x_d, y_d)
     runs5 = {"spmm_ms": round(spmm.measure_average_time([x_d], 5) * 1e3, 4),
              "sddmm_ms": round(sddmm.measure_average_time([x_d, y_d], 5) * 1e3, 4)}
@@ -440,6 +463,8 @@ def main():
                    "seeds": {"graph": 0xFEA7, "weights": 1, "features": 2}},
         "roofline": roofline,
         "verified": not failures,
+        "setup_s": setup,
+        "device_mem_gb": device_mem,
         "gpu_mean_of_5_runs": runs5,
         "ops": {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in ops.items()},
     }

@@ -56,6 +56,12 @@ class Graph(object):
         key = ('sddmm', tail)
         if key not in self._mods:
             m = (MultiHeadSDDMMhip if len(tail) == 2 else VanillaSDDMMhip)(self._csr)
+            # one partitioned copy of the adjacency, one plan and one scratch with a forward SpMM module, if there is one
+            # (every operator of a Graph runs on the caller's one stream, one after the other)
+            for k, other in self._mods.items():
+                if k[0] == 'spmm' and not k[1]:
+                    m.share_layouts(other)
+                    break
             m.build([placeholder((self.shape[1],) + tail), placeholder((self.shape[0],) + tail)], {}, {})
             self._mods[key] = m
         return self._mods[key]

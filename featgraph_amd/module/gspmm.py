@@ -118,6 +118,8 @@ class GSpMMhip(VanillaSpMMhip):
             self._out_pad = torch.zeros((self._num_rows,) + tail, dtype=torch.float32, device=self._ctx)
         self.out_tvm = torch.zeros((self._num_rows,) + tuple(src_ph.shape[1:]), dtype=torch.float32, device=self._ctx)
         self.arg_tvm = torch.full(self.out_tvm.shape, -1, dtype=torch.int32, device=self._ctx) if return_arg else None
+        if not weights_at_run:
+            self._weights(None)          # the adjacency's own values, laid out for the kernel now: run() uploads nothing
 
     def _is_broadcast_message(self, msg, input_placeholders, reduce='sum', force=False):
         if msg not in ('u_mul_e', 'copy_u'):

@@ -60,8 +60,9 @@ class SDDMMbase(object):
                 raise ValueError("edge endpoints outside the %d x %d matrix" % (self._num_rows, self._num_cols))
         self._adj_row_indices = adj_row_indices
         self._adj_col_indices = adj_col_indices
-        self._adj_row_indices_dev = common.to_device_i32(adj_row_indices, self._ctx)
-        self._adj_col_indices_dev = common.to_device_i32(adj_col_indices, self._ctx)
+        # (the stored row / col arrays go to the device when something first needs them -- see _adj_row_indices_dev
+        # below -- so a module that only ever runs the tiled traversal holds the partitioned copy only)
+        self._share_from = None
         # Stored order with non-decreasing row ids is CSR order: row pieces from the SpMM plan
         # then replace the per-edge row array and dst rows are fetched once per piece.
         self._plan = ctypes.c_void_p()
@@ -71,6 +72,7 @@ class SDDMMbase(object):
             counts = np.bincount(adj_row_indices, minlength=self._num_rows) if nnz else np.zeros(self._num_rows, np.int64)
             indptr = np.zeros(self._num_rows + 1, dtype=np.int32)
             np.cumsum(counts, out=indptr[1:])
+            self._adj_indptr = indptr
             self._adj_indptr_dev = common.to_device_i32(indptr, self._ctx)
             with torch.cuda.device(self._ctx):
                 _lib.check(_lib.lib().fg_spmm_plan_create(_lib.host_ptr(indptr), self._num_rows, self._num_cols,
@@ -87,15 +89,70 @@ class SDDMMbase(object):
         self._notes = []
         self.out_tvm = None
 
+    # The stored edge list's device arrays (uploaded on first use).
+    @property
+    def _adj_row_indices_dev(self):
+        if '_row_dev' not in self.__dict__:
+            self.__dict__['_row_dev'] = common.to_device_i32(self._adj_row_indices, self._ctx)
+        return self.__dict__['_row_dev']
+
+    @property
+    def _adj_col_indices_dev(self):
+        if '_col_dev' not in self.__dict__:
+            self.__dict__['_col_dev'] = common.to_device_i32(self._adj_col_indices, self._ctx)
+        return self.__dict__['_col_dev']
+
+    def _upload_edge_list(self):
+        return self._adj_row_indices_dev, self._adj_col_indices_dev
+
+    def share_layouts(self, spmm_module):
+        """Lets the tiled traversal use the partitioned copies of an SpMM module built on the same adjacency -- the
+        position and column arrays, the 16-bit ids, the plan and its scratch -- instead of making its own (at the
+        benchmark size: 0.7 GB of arrays and up to 3.7 GB of scratch less per shared layout).  Needs stored edges in CSR
+        order with exactly that module's structure.  The two modules then share one scratch: their run() calls must
+        follow each other on one stream, as two calls on one module must.  Keeps `spmm_module` alive."""
+        ok = self._row_sorted and (self._num_rows, self._num_cols) == (spmm_module._num_rows, spmm_module._num_cols) \
+            and np.array_equal(self._adj_col_indices, spmm_module._adj_indices) \
+            and np.array_equal(getattr(self, '_adj_indptr', None), spmm_module._adj_indptr)
+        if not ok:
+            raise ValueError("share_layouts needs stored edges in CSR order with the same structure as the SpMM module's adjacency")
+        self._share_from = spmm_module
+
+    @staticmethod
+    def _destroy_plan(plan):
+        if plan is not None and plan.value:
+            try:
+                _lib.lib().fg_spmm_plan_destroy(plan)
+            except Exception:
+                pass
+            plan.value = None
+
+    def _drop_dds(self, P):
+        d = self._dds.pop(P)
+        if d.get('shared_with') is not None:
+            d['shared_with']['users'] = d['shared_with'].get('users', 1) - 1
+        else:
+            self._destroy_plan(d['plan'])
+
+    def device_bytes(self):
+        """Device memory this module holds: {'graph': the stored edge list and the partitioned copies it made itself,
+        'plans': work items, scratch, tile-by-tile copy and 16-bit ids of its own plans (fg_spmm_plan_bytes),
+        'buffers': output and padding}; what it shares with an SpMM module is counted there."""
+        tensors = [self.__dict__.get('_row_dev'), self.__dict__.get('_col_dev'), self._adj_indptr_dev]
+        plans = int(_lib.lib().fg_spmm_plan_bytes(self._plan)) if self._plan.value else 0
+        for d in self._dds.values():
+            tensors.append(d['edge_pos'])
+            if d.get('shared_with') is None:
+                tensors += [d['pos'], d['idx']]
+                plans += int(_lib.lib().fg_spmm_plan_bytes(d['plan']))
+        size = lambda ts: sum(t.numel() * t.element_size() for t in ts if isinstance(t, torch.Tensor))
+        return {'graph': size(tensors), 'plans': plans,
+                'buffers': size([self.out_tvm, getattr(self, '_src_pad', None), getattr(self, '_dst_pad', None)])}
+
     def __del__(self):
-        plans = [getattr(self, "_plan", None)] + [d['plan'] for d in getattr(self, "_dds", {}).values()]
-        for plan in plans:
-            if plan is not None and plan.value:
-                try:
-                    _lib.lib().fg_spmm_plan_destroy(plan)
-                except Exception:
-                    pass
-                plan.value = None
+        self._destroy_plan(getattr(self, "_plan", None))
+        for P in list(getattr(self, "_dds", {})):
+            self._drop_dds(P)
 
     def _dds_layout(self, P):
         """DDS copy of the stored edges (P source-column partitions, CSR inside each) with, per
@@ -104,6 +161,18 @@ class SDDMMbase(object):
             return self._dds[P]
         import scipy.sparse
         nnz = self._adj_row_indices.shape[0]
+        if self._share_from is not None and P > 1:
+            src = self._share_from._layout(P)
+            src['users'] = src.get('users', 0) + 1
+            # stored order is CSR order: a traversed edge's stored position is its position in the DDS copy's own CSR
+            # numbering, which the conversion of the position numbers 0 .. nnz-1 gives
+            csr = scipy.sparse.csr_matrix((np.arange(nnz, dtype=np.int32), self._adj_col_indices, self._adj_indptr),
+                                          shape=(self._num_rows, self._num_cols))
+            _, _, edge_pos = util_convert_csr_to_dds(csr, P)
+            d = {'P': P, 'pos': src['pos'], 'idx': src['idx'], 'edge_pos': common.to_device_i32(edge_pos, self._ctx),
+                 'plan': src['plan'], 'shared_with': src}
+            self._dds[P] = d
+            return d
         if self._row_sorted:
             order = None                        # stored order is already CSR order
             indptr = np.zeros(self._num_rows + 1, dtype=np.int32)
@@ -227,14 +296,18 @@ class SDDMMbase(object):
         src = torch.zeros(phs[0].shape, dtype=torch.float32, device=self._ctx)
         dst = torch.zeros(phs[1].shape, dtype=torch.float32, device=self._ctx)
         timed = []
-        for extra in cands:
-            sa = {k: v for k, v in schedule_args.items() if k != 'tune'}
-            sa.update(extra)
-            try:
-                self.build(phs, compute_args, sa)
-            except ValueError:
-                continue
-            timed.append((self.measure_average_time([src, dst], 3), sa))
+        self._tuning = True             # candidates' layouts are kept until the choice is built
+        try:
+            for extra in cands:
+                sa = {k: v for k, v in schedule_args.items() if k != 'tune'}
+                sa.update(extra)
+                try:
+                    self.build(phs, compute_args, sa)
+                except ValueError:
+                    continue
+                timed.append((self.measure_average_time([src, dst], 3), sa))
+        finally:
+            self._tuning = False
         timed.sort(key=lambda e: e[0])
         self._tuned = [(round(s * 1e3, 4), sa) for s, sa in timed]
         return timed[0][1]
@@ -301,8 +374,13 @@ class SDDMMbase(object):
         self._tiled = None
         if tiled is not None:
             self._tiled = (self._dds_layout(tiled[0]), tiled[1])
+            if not getattr(self, '_tuning', False):
+                for P in [P for P in self._dds if P != tiled[0]]:
+                    self._drop_dds(P)          # partitioned copies the built configuration does not use
             common.reserve(self._tiled[0]['plan'], common.OP_SDDMM_DDS, H, D, tiled[1], self._ctx)
         self._func = _lib.lib().fg_sddmm_csr_f32 if use_csr else _lib.lib().fg_sddmm_coo_f32
+        if self._tiled is None:
+            self._upload_edge_list()           # the stored-order kernels read it; run() itself must not upload anything
         nnz = self._adj_row_indices.shape[0]
         oshape = (nnz,) if self._out_1d else (nnz, H)
         self.out_tvm = torch.zeros(oshape, dtype=torch.float32, device=self._ctx)
@@ -474,6 +552,7 @@ class GSDDMMhip(VanillaSDDMMhip):
             phs, H, D, _, _, notes = self._resolve(input_placeholders, compute_args, dict(schedule_args, order='coo'))
             self._placeholders, self._heads, self._head_len, self._notes = phs, H, D, notes
             self._tiled, self._use_csr = None, False
+            self._upload_edge_list()
             self._func = _lib.lib().fg_gsddmm_elementwise_f32
             self.out_tvm = torch.zeros((self._adj_row_indices.shape[0], H * D), dtype=torch.float32, device=self._ctx)
             return
@@ -496,6 +575,7 @@ class GSDDMMhip(VanillaSDDMMhip):
         self._heads, self._head_len = 1, bop.out_len
         self._notes = [bop.describe()]
         self._tiled, self._use_csr = None, False
+        self._upload_edge_list()
         self._func = _lib.lib().fg_gsddmm_bcast_f32
         self.out_tvm = torch.zeros((nnz,) + tuple(bop.out_shape), dtype=torch.float32, device=self._ctx)
 

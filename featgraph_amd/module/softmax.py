@@ -151,7 +151,7 @@ class EdgeSoftmaxSpMMhip(object):
         w_shape = (self._nnz,) if heads == 1 else (self._nnz, heads)
         self._agg.build([x_ph, common.placeholder(w_shape)], dict(compute_args or {}), dict(schedule_args or {}))
         self._heads = heads
-        common.reserve(self._agg._layouts[1]['plan'], common.OP_EDGE_SOFTMAX, heads, 1, 0, self._ctx)
+        common.reserve(self._agg._layout(1)['plan'], common.OP_EDGE_SOFTMAX, heads, 1, 0, self._ctx)
         self._placeholders = [s_ph, x_ph]
         self._row_stats = torch.zeros((self._num_rows, heads, 2), dtype=torch.float32, device=self._ctx)
         self._weights = torch.empty((heads, self._nnz), dtype=torch.float32, device=self._ctx)
@@ -159,7 +159,7 @@ class EdgeSoftmaxSpMMhip(object):
 
     def _launch(self, scores, x):
         agg, L, s = self._agg, _lib.lib(), common.stream_ptr()
-        csr = agg._layouts[1]
+        csr = agg._layout(1)
         lay = agg._active
         _lib.check(L.fg_edge_softmax_stats_f32(csr['plan'], _lib.dev_ptr(csr['pos']), _lib.dev_ptr(scores),
                                                _lib.dev_ptr(self._row_stats), self._heads, s))

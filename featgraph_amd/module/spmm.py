@@ -54,12 +54,12 @@ class SpMMbase(object):
         if self._num_col_partitions > 1:
             lay = self._layout(self._num_col_partitions)
             self._adj_s1_pos, self._adj_s1_idx, self._adj_vals = lay['host']
-            self._adj_s1_pos_dev, self._adj_s1_idx_dev, self._adj_vals_dev = lay['pos'], lay['idx'], lay['vals']
+            self._adj_s1_pos_dev, self._adj_s1_idx_dev = lay['pos'], lay['idx']
+            self.__dict__['_adj_vals_dev'] = lay['vals']
             self._adj_d1_size = self._num_col_partitions
             self._adj_d2_size = self._num_rows + 1
-        else:
-            lay = self._layout(1)
-            self._adj_indptr_dev, self._adj_indices_dev, self._adj_vals_dev = lay['pos'], lay['idx'], lay['vals']
+        # (one partition: the CSR arrays go to the device when something first needs them -- see _adj_indptr_dev below --
+        # so a module whose build() picks source partitions holds the partitioned copy only)
         # To be updated in self.build
         self._func = None
         self._active = None
@@ -89,15 +89,50 @@ class SpMMbase(object):
         self._layouts[P] = lay
         return lay
 
+    # The CSR layout's device arrays, for modules constructed with one partition (uploaded on first use).
+    @property
+    def _adj_indptr_dev(self):
+        return self.__dict__['_adj_indptr_dev'] if '_adj_indptr_dev' in self.__dict__ else self._layout(1)['pos']
+
+    @property
+    def _adj_indices_dev(self):
+        return self.__dict__['_adj_indices_dev'] if '_adj_indices_dev' in self.__dict__ else self._layout(1)['idx']
+
+    @property
+    def _adj_vals_dev(self):
+        return self.__dict__['_adj_vals_dev'] if '_adj_vals_dev' in self.__dict__ else self._layout(1)['vals']
+
+    @staticmethod
+    def _destroy_layout(lay):
+        plan = lay.get('plan')
+        if plan is not None and plan.value:
+            try:
+                _lib.lib().fg_spmm_plan_destroy(plan)
+            except Exception:
+                pass
+            lay['plan'] = None
+
+    def _release_unused_layouts(self):
+        """Frees the partitioned copies (device arrays, plan, scratch) that the built configuration does not use; a
+        later build() that wants one of them makes it again.  The constructor's own layout and the CSR arrays stay."""
+        keep = {1, self._num_col_partitions, self._active['P']}
+        for P in [P for P in self._layouts if P not in keep and not self._layouts[P].get('users')]:
+            self._destroy_layout(self._layouts.pop(P))
+
+    def device_bytes(self):
+        """Device memory this module holds: {'graph': the adjacency's arrays in every layout kept, 'plans': work items,
+        scratch, tile-by-tile copy and 16-bit ids of their plans (fg_spmm_plan_bytes), 'buffers': output and padding}."""
+        graph = plans = 0
+        for lay in self._layouts.values():
+            graph += sum(t.numel() * t.element_size() for t in lay.values() if isinstance(t, torch.Tensor))
+            plans += int(_lib.lib().fg_spmm_plan_bytes(lay['plan']))
+        bufs = sum(t.numel() * t.element_size() for t in (self.out_tvm, getattr(self, '_x_pad', None), getattr(self, '_out_pad', None))
+                   if isinstance(t, torch.Tensor))
+        return {'graph': graph, 'plans': plans, 'buffers': bufs}
+
     def __del__(self):
         for lay in getattr(self, "_layouts", {}).values():
-            plan = lay.get('plan')
-            if plan is not None and plan.value:
-                try:
-                    _lib.lib().fg_spmm_plan_destroy(plan)
-                except Exception:
-                    pass
-                lay['plan'] = None
+            self._destroy_layout(lay)
 
     def _preprocess_adj(self, adj_scipy_csr, num_col_partitions=1):
         return util_convert_csr_to_dds(adj_scipy_csr, num_col_partitions)
@@ -162,12 +197,16 @@ class SpMMbase(object):
         cands = tuning.rank_spmm(self._graph_stats(), feat_len)[:max(1, how_many)]
         x = torch.zeros(ph.shape, dtype=torch.float32, device=self._ctx)
         timed = []
-        for p, t in cands:
-            ca = dict(compute_args, num_feat_partitions=t)
-            sa = dict(schedule_args, num_src_partitions=(p if p > 1 else None))
-            sa.pop('tune', None)
-            self.build([ph], ca, sa)
-            timed.append((self.measure_average_time([x], 3), p, t, ca, sa))
+        self._tuning = True             # candidates' layouts are kept until the choice is built
+        try:
+            for p, t in cands:
+                ca = dict(compute_args, num_feat_partitions=t)
+                sa = dict(schedule_args, num_src_partitions=(p if p > 1 else None))
+                sa.pop('tune', None)
+                self.build([ph], ca, sa)
+                timed.append((self.measure_average_time([x], 3), p, t, ca, sa))
+        finally:
+            self._tuning = False
         timed.sort(key=lambda e: e[0])
         self._tuned = [(round(s * 1e3, 4), p, t) for s, p, t, _, _ in timed]
         return timed[0][3], timed[0][4]
@@ -216,6 +255,8 @@ class SpMMbase(object):
         self._num_feat_partitions = T
         self._notes = notes
         self._active = self._layout(P)
+        if not getattr(self, '_tuning', False):
+            self._release_unused_layouts()
         self._func = _lib.lib().fg_spmm_dds_f32 if P > 1 else _lib.lib().fg_spmm_csr_f32
         common.reserve(self._active['plan'], common.OP_SPMM_SUM, 1, feat_len, T, self._ctx)
         self._x_pad = self._out_pad = None
