@@ -112,11 +112,19 @@ template <int OP> constexpr bool kUsesRhs = OP != FG_BIN_COPY_LHS;
 template <int RED> __device__ __forceinline__ float identity() {
     return RED == FG_REDUCE_SUM ? 0.f : RED == FG_REDUCE_MAX ? -INFINITY : INFINITY;
 }
-// Whether candidate (m, at element em) replaces (acc, at element ea): the better value, or the same value at an
-// earlier element; the first value that is not a NaN always enters.
+// Max / min treat a NaN message as beating every number, so that it reaches the row's result the way it does through
+// a sum (what numpy's maximum / minimum reductions and argmax / argmin do): the running extreme of (acc, m).
+template <int RED> __device__ __forceinline__ float extreme(float acc, float m) {
+    // once acc is a NaN no comparison with it holds and it stays; a NaN m enters through m != m
+    return ((RED == FG_REDUCE_MAX ? m > acc : m < acc) || m != m) ? m : acc;
+}
+// Whether candidate (m, at element em) replaces (acc, at element ea): the better value (a NaN is better than any
+// number), or the same value (two NaNs count as the same) at an earlier element; the first value always enters.
 template <int RED> __device__ __forceinline__ bool replaces(float m, int em, float acc, int ea) {
-    const bool better = RED == FG_REDUCE_MAX ? m > acc : m < acc;
-    return em != INT_MAX && m == m && (ea == INT_MAX || better || (m == acc && em < ea));
+    const bool m_nan = m != m, acc_nan = acc != acc;
+    const bool better = m_nan ? !acc_nan : (!acc_nan && (RED == FG_REDUCE_MAX ? m > acc : m < acc));
+    const bool same = m_nan ? acc_nan : m == acc;
+    return em != INT_MAX && (ea == INT_MAX || better || (same && em < ea));
 }
 
 // LC / RC (V == 4 only): the operand's 4 features are consecutive (one 128-bit load), else one value 4 times.
@@ -229,7 +237,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
                         } else if (ARG) {
                             if (ok[k] && replaces<RED>(m[k][i], e, acc[i], at[i])) { acc[i] = m[k][i]; at[i] = e; }
                         } else if (ok[k]) {
-                            acc[i] = RED == FG_REDUCE_MAX ? fmaxf(acc[i], m[k][i]) : fminf(acc[i], m[k][i]);
+                            acc[i] = extreme<RED>(acc[i], m[k][i]);
                         }
                     }
                 }
@@ -243,7 +251,7 @@ __global__ __launch_bounds__(kBlock) void gspmm_bcast_kernel(const GenArgs a) {
                     else if (ARG) {
                         const int oa = __shfl_xor(at[i], off);
                         if (replaces<RED>(o, oa, acc[i], at[i])) { acc[i] = o; at[i] = oa; }
-                    } else acc[i] = RED == FG_REDUCE_MAX ? fmaxf(acc[i], o) : fminf(acc[i], o);
+                    } else acc[i] = extreme<RED>(acc[i], o);
                 }
             }
             if ((OWN ? mine : g == 0) && active) {
@@ -314,7 +322,7 @@ __global__ __launch_bounds__(256) void gspmm_bcast_fixup_kernel(const Fixup *fix
         else if (ARG) {
             const int am = partial_arg[from + (int64_t)(fx.slot0 + p) * F + f];
             if (am >= 0 && replaces<RED>(m, am, acc, at)) { acc = m; at = am; }
-        } else acc = RED == FG_REDUCE_MAX ? fmaxf(acc, m) : fminf(acc, m);
+        } else acc = extreme<RED>(acc, m);
     }
     if (row_scale) acc *= row_scale[fx.row];
     out[to + (int64_t)fx.row * F + f] = acc;
@@ -342,7 +350,7 @@ __global__ __launch_bounds__(256) void gspmm_bcast_combine_kernel(const float *b
             if (ARG) {
                 const int am = abuf[p * buf_stride + t];
                 if (am >= 0 && replaces<RED>(m, am, acc, at)) { acc = m; at = am; }
-            } else acc = RED == FG_REDUCE_MAX ? fmaxf(acc, m) : fminf(acc, m);
+            } else acc = extreme<RED>(acc, m);
         }
     }
     if (RED != FG_REDUCE_SUM && !any) acc = 0.f;

@@ -483,7 +483,8 @@ __global__ __launch_bounds__(kBlock) void spmm_items_wide_kernel(const SpmmArgs 
 // each row in turn and a lane without an element in the last batch keeps its running extreme.
 
 template <bool IS_MAX> __device__ __forceinline__ float ext_identity() { return IS_MAX ? -INFINITY : INFINITY; }
-template <bool IS_MAX> __device__ __forceinline__ float ext_op(float a, float b) { return IS_MAX ? fmaxf(a, b) : fminf(a, b); }
+// a NaN message beats every number (it reaches the result, as through a sum); once the running extreme is a NaN it stays
+template <bool IS_MAX> __device__ __forceinline__ float ext_op(float a, float b) { return ((IS_MAX ? b > a : b < a) || b != b) ? b : a; }
 template <bool IS_MAX> __device__ __forceinline__ void vext(float4 &a, const float4 &b) {
     a.x = ext_op<IS_MAX>(a.x, b.x); a.y = ext_op<IS_MAX>(a.y, b.y);
     a.z = ext_op<IS_MAX>(a.z, b.z); a.w = ext_op<IS_MAX>(a.w, b.w);
@@ -629,15 +630,17 @@ __global__ __launch_bounds__(256) void gspmm_extreme_fixup_kernel(const Fixup *f
 // and lane layout; the products are formed by the same multiplication, so the comparison is exact.
 // Pieces of split rows combine through atomicMin on arg (set to INT_MAX beforehand).
 
+// equal, or both NaN (a NaN extreme is matched by the first NaN message)
+__device__ __forceinline__ bool same_value(float m, float t) { return m == t || (m != m && t != t); }
 __device__ __forceinline__ int4 imin4(const int4 &a, const int4 &b) {
     return make_int4(min(a.x, b.x), min(a.y, b.y), min(a.z, b.z), min(a.w, b.w));
 }
 __device__ __forceinline__ int imin4(const int &a, const int &b) { return min(a, b); }
 __device__ __forceinline__ int4 imatch(const float4 &m, const float4 &t, int e, const int4 &cur) {
-    return make_int4(m.x == t.x ? min(cur.x, e) : cur.x, m.y == t.y ? min(cur.y, e) : cur.y,
-                     m.z == t.z ? min(cur.z, e) : cur.z, m.w == t.w ? min(cur.w, e) : cur.w);
+    return make_int4(same_value(m.x, t.x) ? min(cur.x, e) : cur.x, same_value(m.y, t.y) ? min(cur.y, e) : cur.y,
+                     same_value(m.z, t.z) ? min(cur.z, e) : cur.z, same_value(m.w, t.w) ? min(cur.w, e) : cur.w);
 }
-__device__ __forceinline__ int imatch(const float &m, const float &t, int e, const int &cur) { return m == t ? min(cur, e) : cur; }
+__device__ __forceinline__ int imatch(const float &m, const float &t, int e, const int &cur) { return same_value(m, t) ? min(cur, e) : cur; }
 __device__ __forceinline__ int4 ishfl_xor(const int4 &a, int off) {
     return make_int4(__shfl_xor(a.x, off), __shfl_xor(a.y, off), __shfl_xor(a.z, off), __shfl_xor(a.w, off));
 }

@@ -163,10 +163,10 @@ int orc_gspmm(int64_t n_dst, int F, int H, const int32_t *indptr, const int32_t 
             for (int f = 0; f < F; ++f) {
                 const float w = vals ? vals[(int64_t)k * H + f / D] : 1.0f;
                 const float m = w * xr[f];
+                /* max / min: a NaN message beats every number and stays (numpy's maximum / minimum reductions) */
                 if (reduce == 0) o[f] += m;
                 else if (k == b) o[f] = m;
-                else if (reduce == 1) o[f] = m > o[f] ? m : o[f];
-                else o[f] = m < o[f] ? m : o[f];
+                else if (o[f] == o[f] && ((reduce == 1 ? m > o[f] : m < o[f]) || m != m)) o[f] = m;
             }
         }
     }
@@ -194,7 +194,8 @@ int orc_gspmm_arg(int64_t n_dst, int F, int H, const int32_t *indptr, const int3
             for (int f = 0; f < F; ++f) {
                 const float w = vals ? vals[(int64_t)k * H + f / D] : 1.0f;
                 const float m = w * xr[f];
-                if (k == b || (reduce == 1 ? m > o[f] : m < o[f])) { o[f] = m; a[f] = k; }
+                /* the first NaN message, if there is one, is the selected element (numpy's argmax / argmin) */
+                if (k == b || (o[f] == o[f] && ((reduce == 1 ? m > o[f] : m < o[f]) || m != m))) { o[f] = m; a[f] = k; }
             }
         }
     }

@@ -227,7 +227,7 @@ def gspmm_bcast(indptr, indices, op, reduce, lhs, rhs, lhs_target="u", rhs_targe
         if b > a:
             seg = m2[a:b]
             out[v] = seg.max(0) if reduce == "max" else seg.min(0)
-            arg[v] = a + (seg == out[v]).argmax(0)
+            arg[v] = a + ((seg == out[v]) | (np.isnan(seg) & np.isnan(out[v]))).argmax(0)      # a NaN result: its first NaN message
     return out.reshape((n,) + feat), arg.reshape((n,) + feat)
 
 

@@ -152,3 +152,87 @@ def test_attention_nonfinite_values_do_not_leak(oracle, D, P):
     hit = _touching(adj, [222])
     assert np.isfinite(got[~hit]).all()
     assert np.array_equal(got[~hit], clean[~hit])
+
+
+@pytest.mark.parametrize("reduce", ["max", "min"])
+@pytest.mark.parametrize("P", [None, 3])
+@pytest.mark.parametrize("return_arg", [False, True])
+def test_extremes_propagate_nan(oracle, reduce, P, return_arg):
+    """max / min of messages: a NaN message becomes the row's result (as it would through a sum, and as numpy's
+    reductions do), the selected element is the row's first NaN message, a row of nothing but NaN messages gives NaN --
+    in rows that lane groups walk on their own, in rows the wavefront shares, in the pieces of a split row, with one
+    partition and with three, with and without the selected positions.  Rows that reference no NaN are bit-identical
+    to a run on clean features."""
+    import torch
+    from featgraph_amd.module import GSpMMhip, placeholder
+    rng = np.random.default_rng(5 + (P or 0))
+    adj = _short_row_graph(rng)
+    F = 32
+    nnz = adj.nnz
+    x = rng.standard_normal((adj.shape[1], F)).astype("float32")
+    e = (rng.random((nnz, 1)) + 0.5).astype("float32")
+    xb = x.copy()
+    xb[222] = np.nan                                   # referenced by three short rows (see _short_row_graph)
+    xb[1500, :7] = np.nan                              # some features only
+    # every source of one short row and of one medium row: rows whose messages are all NaN
+    lens = np.diff(adj.indptr)
+    r_short = int(np.flatnonzero((lens >= 1) & (lens <= 3))[5])
+    r_mid = int(np.flatnonzero((lens >= 20) & (lens < 100))[0])
+    for r in (r_short, r_mid):
+        xb[adj.indices[adj.indptr[r]:adj.indptr[r + 1]], 9] = np.nan
+    # the split row: a NaN among its last elements (another piece than the one holding its first elements)
+    xb[adj.indices[adj.indptr[701] - 3], 11] = np.nan
+    m = GSpMMhip(adj)
+    m.build([placeholder(x.shape), placeholder(e.shape)], {'msg': 'u_mul_e', 'reduce': reduce, 'return_arg': return_arg},
+            {'num_src_partitions': P})
+    assert m._active['P'] == (P or 1)
+    ed = torch.from_numpy(e).cuda()
+    clean = m.run([torch.from_numpy(x).cuda(), ed]).cpu().numpy().copy()
+    got = m.run([torch.from_numpy(xb).cuda(), ed]).cpu().numpy().copy()
+    want, want_arg = oracle.gspmm_bcast(adj.indptr, adj.indices, "mul", reduce, xb, e, "u", "e")
+    assert np.array_equal(got, want, equal_nan=True)
+    assert np.isnan(got[r_short, 9]) and np.isnan(got[r_mid, 9]) and np.isnan(got[700, 11])
+    touched = np.isnan(want).any(axis=1)
+    assert touched.sum() >= 5 and np.array_equal(got[~touched], clean[~touched])
+    if return_arg:
+        assert np.array_equal(m.arg_tvm.cpu().numpy(), want_arg)
+
+
+@pytest.mark.parametrize("reduce", ["max", "min"])
+def test_weighted_extremes_propagate_nan(oracle, reduce):
+    """The same through the C ABI's weighted max / min (fg_gspmm_f32 / fg_gspmm_arg_f32: one weight per edge)."""
+    import ctypes
+    import torch
+    from featgraph_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(8)
+    adj = _short_row_graph(rng)
+    F = 32
+    x = rng.standard_normal((adj.shape[1], F)).astype("float32")
+    x[222] = np.nan
+    x[1500, :7] = np.nan
+    x[adj.indices[adj.indptr[701] - 3], 11] = np.nan
+    lens = np.diff(adj.indptr)
+    r_mid = int(np.flatnonzero((lens >= 20) & (lens < 100))[0])
+    x[adj.indices[adj.indptr[r_mid]:adj.indptr[r_mid + 1]], 9] = np.nan
+    want, want_arg = oracle.gspmm_arg(adj.indptr, adj.indices, adj.data, x, reduce)
+    indptr = np.ascontiguousarray(adj.indptr, dtype=np.int32)
+    plan = ctypes.c_void_p()
+    _lib.check(L.fg_spmm_plan_create(_lib.host_ptr(indptr), adj.shape[0], adj.shape[1], 1, None, ctypes.byref(plan)))
+    try:
+        ip, ix, vl, xd = (torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (indptr, adj.indices, adj.data, x))
+        out = torch.full((adj.shape[0], F), 7.0, device="cuda")
+        arg = torch.full((adj.shape[0], F), -5, dtype=torch.int32, device="cuda")
+        p = _lib.dev_ptr
+        red = {"max": 1, "min": 2}[reduce]
+        _lib.check(L.fg_gspmm_arg_f32(plan, p(ip), p(ix), p(vl), p(xd), p(out), p(arg), F, 1, 0, red, 0, None))
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), want, equal_nan=True)
+        assert np.array_equal(arg.cpu().numpy(), want_arg)
+        out.fill_(7.0)
+        _lib.check(L.fg_gspmm_f32(plan, p(ip), p(ix), p(vl), p(xd), p(out), F, 1, 0, red, 0, None))
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), want, equal_nan=True)
+        assert np.isnan(want[r_mid, 9]) and np.isnan(want[700, 11])
+    finally:
+        L.fg_spmm_plan_destroy(plan)

@@ -458,3 +458,38 @@ def test_timing_copies_stay_within_tolerance_of_the_pinned_loops(oracle):
     empty = sp.csr_matrix((5, 9), dtype="float32")
     x = rng.standard_normal((9, 8)).astype("float32")
     assert (oracle.spmm_csr_x86(empty.indptr, empty.indices, empty.data, x, 2, 2, fast=True) == 0).all()
+
+
+def test_gspmm_extremes_propagate_nan(oracle):
+    """max / min aggregation treats a NaN message as numpy's maximum / minimum reductions and argmax / argmin do: it
+    becomes the row's result, and the selected element is the row's first NaN message -- in the C restatement and in
+    the numpy restatement of the broadcasting operator alike.  Rows of all-NaN messages give NaN, not an identity."""
+    rng = np.random.default_rng(22)
+    adj = _rand_csr(rng, 50, 40, 0.25).tolil()
+    adj[[3, 30], :] = 0
+    adj = adj.tocsr().astype("float32"); adj.eliminate_zeros(); adj.sort_indices()
+    adj.data = (rng.random(adj.nnz) + 0.5).astype("float32")
+    x = rng.standard_normal((40, 5)).astype("float32")
+    x[7] = np.nan                    # a whole source row
+    x[21, 2] = np.nan                # one feature of another
+    x[33] = np.inf
+    indptr, indices = adj.indptr, adj.indices
+    # a row whose messages are all NaN: every source it references is made NaN in column 4
+    r_all = int(np.argmax(np.diff(indptr) > 0))
+    x[indices[indptr[r_all]:indptr[r_all + 1]], 4] = np.nan
+    rows = np.flatnonzero(np.diff(indptr) > 0)
+    msgs = adj.data[:, None] * x[indices]
+    for reduce, ufunc, pick in (("max", np.maximum, np.argmax), ("min", np.minimum, np.argmin)):
+        want = np.zeros((50, 5), np.float32)
+        want[rows] = ufunc.reduceat(msgs, indptr[rows], axis=0)
+        out, arg = oracle.gspmm_arg(indptr, indices, adj.data, x, reduce)
+        assert np.array_equal(out, want, equal_nan=True)
+        assert np.array_equal(oracle.gspmm(indptr, indices, adj.data, x, reduce), want, equal_nan=True)
+        out_b, arg_b = oracle.gspmm_bcast(indptr, indices, "mul", reduce, x, adj.data.reshape(-1, 1), "u", "e")
+        assert np.array_equal(out_b, want, equal_nan=True)
+        for r in rows:
+            b, e = indptr[r], indptr[r + 1]
+            assert np.array_equal(arg[r], b + pick(msgs[b:e], axis=0))           # numpy: the first NaN wins
+            assert np.array_equal(arg_b[r], arg[r])
+        assert np.isnan(out[r_all, 4]) and arg[r_all, 4] == indptr[r_all]
+        assert np.isnan(want).any() and np.isfinite(want).any()
