@@ -163,6 +163,7 @@ class GraphAttentionhip(object):
         """[Q, K, V] -> self.out_tvm (the same tensor on every call); nothing is synchronised."""
         if self._placeholders is None:
             raise RuntimeError("call build() before run()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         self._launch(*input_tvm_ndarrays)
         return self.out_tvm
@@ -258,6 +259,7 @@ class GraphAttentionhip(object):
     def measure_average_time(self, input_tvm_ndarrays, num_runs):
         if self._placeholders is None:
             raise RuntimeError("call build() before measure_average_time()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         q, k, v = input_tvm_ndarrays
         return common.timed_mean_seconds(lambda: self._launch(q, k, v), num_runs)

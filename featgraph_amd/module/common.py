@@ -65,6 +65,16 @@ def check_inputs(tensors, placeholders, dev):
             raise ValueError("inputs must be contiguous (row-major)")
 
 
+def ensure_output(mod):
+    """A module that handed its output tensor out for good (featgraph_amd.autograd does: the gradient machinery keeps
+    the tensor, the module drops it) gets a new one of the built shape before its next direct run()."""
+    like = getattr(mod, '_fresh_like', None)
+    if getattr(mod, 'out_tvm', None) is None and like is not None:
+        mod.out_tvm = torch.empty(like[0], dtype=like[1], device=like[2])
+    if hasattr(mod, 'arg_tvm') and mod.arg_tvm is None and getattr(mod, '_return_arg', False) and mod.out_tvm is not None:
+        mod.arg_tvm = torch.full(mod.out_tvm.shape, -1, dtype=torch.int32, device=mod.out_tvm.device)
+
+
 def timed_mean_seconds(fn, num_runs):
     """Mean seconds of `num_runs` back-to-back launches between two events on the current
     stream, after one untimed call (the protocol of Module.time_evaluator(number=num_runs)

@@ -346,6 +346,7 @@ class GSpMMhip(VanillaSpMMhip):
         """[SrcFeat] or [SrcFeat, edge_weights]; returns self.out_tvm (overwritten in place)."""
         if self._func is None:
             raise RuntimeError("call build() before run()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         if self._bop is not None:
             self._launch_broadcast(input_tvm_ndarrays)
@@ -356,6 +357,7 @@ class GSpMMhip(VanillaSpMMhip):
     def measure_average_time(self, input_tvm_ndarrays, num_runs):
         if self._func is None:
             raise RuntimeError("call build() before measure_average_time()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         if self._bop is not None:
             return common.timed_mean_seconds(lambda: self._launch_broadcast(input_tvm_ndarrays), num_runs)

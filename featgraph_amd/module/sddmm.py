@@ -432,6 +432,7 @@ class SDDMMbase(object):
         stored (possibly partitioned) edge order; enqueued on torch's current stream."""
         if self._func is None:
             raise RuntimeError("call build() before run()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         self._launch(input_tvm_ndarrays[0], input_tvm_ndarrays[1])
         return self.out_tvm
@@ -440,6 +441,7 @@ class SDDMMbase(object):
         """Average run time in seconds over `num_runs` back-to-back launches."""
         if self._func is None:
             raise RuntimeError("call build() before measure_average_time()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         s, d = input_tvm_ndarrays
         return common.timed_mean_seconds(lambda: self._launch(s, d), num_runs)
@@ -598,6 +600,7 @@ class GSDDMMhip(VanillaSDDMMhip):
             input_tvm_ndarrays = list(input_tvm_ndarrays)[::-1]
         if self._bop is None:
             return super(GSDDMMhip, self).run(input_tvm_ndarrays)
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         self._launch(input_tvm_ndarrays[0], input_tvm_ndarrays[1] if len(input_tvm_ndarrays) > 1 else None)
         return self.out_tvm
@@ -609,6 +612,7 @@ class GSDDMMhip(VanillaSDDMMhip):
             input_tvm_ndarrays = list(input_tvm_ndarrays)[::-1]
         if self._bop is None:
             return super(GSDDMMhip, self).measure_average_time(input_tvm_ndarrays, num_runs)
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         a = input_tvm_ndarrays[0]
         b = input_tvm_ndarrays[1] if len(input_tvm_ndarrays) > 1 else None

@@ -79,6 +79,7 @@ class EdgeSoftmaxhip(object):
         """[Scores] -> self.out_tvm (the same tensor on every call); nothing is synchronised."""
         if self._placeholders is None:
             raise RuntimeError("call build() before run()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         self._forward(input_tvm_ndarrays[0], self.out_tvm)
         return self.out_tvm
@@ -90,7 +91,7 @@ class EdgeSoftmaxhip(object):
         common.check_inputs([softmax], self._placeholders, self._ctx)
         common.check_inputs([grad_softmax], self._placeholders, self._ctx)
         if self.grad_tvm is None:
-            self.grad_tvm = torch.zeros_like(self.out_tvm)
+            self.grad_tvm = torch.zeros_like(softmax)
         _lib.check(_lib.lib().fg_edge_softmax_backward_f32(self._plan, _lib.dev_ptr(self._indptr_dev),
                                                            _lib.dev_ptr(softmax), _lib.dev_ptr(grad_softmax),
                                                            _lib.dev_ptr(self.grad_tvm), self._heads,
@@ -100,6 +101,7 @@ class EdgeSoftmaxhip(object):
     def measure_average_time(self, input_tvm_ndarrays, num_runs):
         if self._placeholders is None:
             raise RuntimeError("call build() before measure_average_time()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         x = input_tvm_ndarrays[0]
         return common.timed_mean_seconds(lambda: self._forward(x, self.out_tvm), num_runs)
@@ -175,6 +177,7 @@ class EdgeSoftmaxSpMMhip(object):
         """[Scores, SrcFeat] -> self.out_tvm (the same tensor on every call); nothing is synchronised."""
         if self._placeholders is None:
             raise RuntimeError("call build() before run()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         self._launch(input_tvm_ndarrays[0], input_tvm_ndarrays[1])
         return self.out_tvm
@@ -182,6 +185,7 @@ class EdgeSoftmaxSpMMhip(object):
     def measure_average_time(self, input_tvm_ndarrays, num_runs):
         if self._placeholders is None:
             raise RuntimeError("call build() before measure_average_time()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         s, x = input_tvm_ndarrays
         return common.timed_mean_seconds(lambda: self._launch(s, x), num_runs)

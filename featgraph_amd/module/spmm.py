@@ -303,6 +303,7 @@ class SpMMbase(object):
         """
         if self._func is None:
             raise RuntimeError("call build() before run()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         self._launch(input_tvm_ndarrays[0])
         return self.out_tvm
@@ -311,6 +312,7 @@ class SpMMbase(object):
         """Average run time in seconds over `num_runs` back-to-back launches."""
         if self._func is None:
             raise RuntimeError("call build() before measure_average_time()")
+        common.ensure_output(self)
         common.check_inputs(input_tvm_ndarrays, self._placeholders, self._ctx)
         x = input_tvm_ndarrays[0]
         return common.timed_mean_seconds(lambda: self._launch(x), num_runs)

@@ -234,3 +234,31 @@ def test_generalised_sddmm_gradients(op, lt, l_shape, rt, r_shape):
     assert torch.allclose(out.double(), ref, rtol=1e-5, atol=1e-5)
     assert torch.allclose(lhs.grad.double(), l64.grad, rtol=1e-4, atol=1e-4)
     assert torch.allclose(rhs.grad.double(), r64.grad, rtol=1e-4, atol=1e-4)
+
+
+def test_modules_stay_usable_after_the_graph_handed_their_outputs_out():
+    """Graph's differentiable calls give the module's output tensor to autograd and the module drops it; a later direct
+    run() / measure_average_time() on the same cached module gets a new output tensor instead of a null pointer."""
+    import torch
+    from featgraph_amd.autograd import Graph
+    rng = np.random.default_rng(3)
+    adj = sp.random(300, 300, density=0.05, format="csr", random_state=rng).astype("float32")
+    adj.sort_indices()
+    g = Graph(adj)
+    x = torch.randn((300, 16), device="cuda", requires_grad=True)
+    w = torch.rand(adj.nnz, device="cuda")
+    y = g.spmm(x, w)
+    y.sum().backward()
+    s = g.sddmm(x.detach(), x.detach())
+    a = g.edge_softmax(s)
+    for key, mod in list(g._mods.items()):
+        if key[0] == 'spmm' and not key[1]:
+            assert mod.out_tvm is None
+            again = mod.run([x.detach(), w])
+            assert torch.equal(again, y.detach())
+            assert mod.measure_average_time([x.detach(), w], 2) > 0
+        if key[0] == 'sddmm':
+            assert torch.equal(mod.run([x.detach(), x.detach()]), s)
+        if key[0] == 'softmax':
+            assert torch.equal(mod.run([s]), a)
+            mod.backward(a, torch.ones_like(a))
