@@ -189,6 +189,15 @@ def test_default_tilings():
         assert F % t == 0 and p >= 1 and F // t >= 32
         p, t = tuning.choose_spmm(n, n, nnz, F)
         assert p >= 1 and (t == 0 or F % t == 0)
+    # a graph with locality (41 planted communities, ids community-contiguous or relabelled at random): the defaults,
+    # from the graph's own statistics, are the points that full sweeps on the GPU found within 2 % of the best
+    from featgraph_amd import synthetic
+    for name in ("communities-233k", "communities-233k-relabelled"):
+        ip, ix = synthetic.make_workload(name)
+        st = tuning.GraphStats.from_csr(ip, ix, n)
+        assert 112e6 < st.nnz < 117e6
+        assert tuning.choose_spmm(n, n, st.nnz, 512, st) == (8, 8) and tuning.choose_spmm(n, n, st.nnz, 128, st) == (8, 2)
+        assert tuning.choose_sddmm(n, n, st.nnz, 1, 512, st) == (8, 8) and tuning.choose_sddmm(n, n, st.nnz, 1, 128, st) == (16, 1)
     # hit-rate estimate: monotone in the capacity, 0 for an empty cache, compulsory misses only when all fits
     skew = tuning.GraphStats(1000, 1000, 100000, count_vals=[10, 1000], count_mult=[900, 91], deg_vals=[100], deg_mult=[1000])
     rates = [skew.hit_rate(k) for k in (1, 10, 91, 300, 991, 5000)]
@@ -305,3 +314,36 @@ def test_sizes_beyond_int32_are_refused():
     for shape in [(2 ** 31, 10, 5), (10, 2 ** 31 - 1, 5), (10, 10, 2 ** 31 - 1)]:
         with pytest.raises(ValueError, match="int32"):
             common.check_int32_sizes(*shape)
+
+
+def test_community_graph_generator():
+    """fg_synth_community_csr: bit-identical for a seed whatever the thread count, sorted duplicate-free rows with a
+    self-loop each, most of a row's sources inside its own community, and the relabelled variant the same kind of
+    graph (same size class, no community structure left in the id ranges)."""
+    from featgraph_amd import synthetic
+    spec = synthetic.WORKLOADS["communities-23k"]
+    ip, ix = synthetic.make_workload("communities-23k")
+    ip2, ix2 = synthetic.make_workload("communities-23k", num_threads=3)
+    assert np.array_equal(ip, ip2) and np.array_equal(ix, ix2)
+    n, C = spec["n"], spec["n_comm"]
+    assert ip.dtype == np.int32 and ix.dtype == np.int32 and ip[0] == 0 and ip[-1] == ix.shape[0]
+    rows = np.repeat(np.arange(n), np.diff(ip))
+    inner = np.ones(ix.shape[0], bool); inner[ip[1:-1]] = False
+    assert (np.diff(ix)[inner[1:]] > 0).all()                                   # sorted, no duplicates inside a row
+    assert (np.diff(ip) >= 1).all()
+    has_loop = np.zeros(n, bool); has_loop[rows[ix == rows]] = True
+    assert has_loop.all()
+    # contiguous ids: community c owns the id range [off[c], off[c + 1]) (ranks r with r % C == c)
+    off = np.concatenate([[0], np.cumsum(np.bincount(np.arange(n) % C, minlength=C))])
+    same = (np.searchsorted(off, rows, side='right') == np.searchsorted(off, ix, side='right'))
+    assert same.mean() > 0.7
+    relab = dict(spec, contiguous=False)
+    ip3, ix3 = synthetic.community_csr(relab["n"], relab["total_edges"], relab["exponent"], relab["max_degree"], C,
+                                       relab["p_in"], False, relab["seed"])
+    assert abs(int(ip3[-1]) - int(ip[-1])) < 0.02 * ip[-1]
+    rows3 = np.repeat(np.arange(n), np.diff(ip3))
+    same3 = (np.searchsorted(off, rows3, side='right') == np.searchsorted(off, ix3, side='right'))
+    assert same3.mean() < 0.3
+    # bad arguments are refused
+    from featgraph_amd import _lib
+    assert _lib.lib().fg_synth_community_csr(0, None, None, None, 1, None, None, None, None, 0.5, 1, 0, None, None) == -1
