@@ -167,7 +167,12 @@ def test_tiled_traversal(torch_cuda, oracle, feat_len, P, T, order):
 
 
 @pytest.mark.parametrize("H,D,P,T", [(8, 64, 4, 8), (4, 32, 2, 2), (8, 32, 3, 1), (2, 8, 2, 1), (4, 64, 1, 4),
-                                     (16, 16, 2, 4), (4, 256, 2, 4)])
+                                     (16, 16, 2, 4), (4, 256, 2, 4),
+                                     # one staged head per tile with head counts that are (12) and are not (5, 6) multiples of 4:
+                                     # the 128-bit and the one-thread-per-edge form of the last kernel, tiles launched 8 + 4, 4 + 1, 4 + 2
+                                     (12, 64, 2, 12), (5, 64, 2, 5), (6, 64, 3, 6), (8, 128, 2, 8),
+                                     # all heads in one 256-float tile (16 heads of 16 floats)
+                                     (16, 16, 3, 1)])
 def test_tiled_multihead(torch_cuda, oracle, H, D, P, T):
     """Whole heads per feature tile: results go straight to out[edge, head], or (one head per tile,
     four heads or more) through a per-tile staging array and a last kernel that writes each edge's heads."""
