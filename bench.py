@@ -204,7 +204,8 @@ def run_configs(torch, workload, indptr, indices, vals_d, spmm, sddmm, headline_
     reference's protocol (mean of 5 back-to-back runs after a warm-up, python/featgraph/module/spmm.py:179-186;
     check of the output, tests/test_module_sddmm.py:34-37) per entry.  cfg2: SpMM at the other feature lengths;
     cfg3: SDDMM at the other feature lengths (edges stored in CSR order, the library's choice of kernel) and at the
-    headline length with the kernel that walks the stored row / col arrays (`order='coo'`); cfg4: multi-head SDDMM;
+    headline length with the kernel that walks the stored row / col arrays (`order='coo'`, forced: the default takes the
+    tiled traversal there) and on the same edges stored in a random order (the default); cfg4: multi-head SDDMM;
     cfg5: SpMM then SDDMM on the 2.45M-node low-degree graph."""
     import numpy as np
     import scipy.sparse as sp
@@ -248,6 +249,21 @@ def run_configs(torch, workload, indptr, indices, vals_d, spmm, sddmm, headline_
         if F != headline_F:
             pair("cfg2/cfg3", workload, indptr, idx_d, rows_d, vals_d, spmm, sddmm, F)
     pair("cfg3", workload, indptr, idx_d, rows_d, vals_d, spmm, sddmm, headline_F, sddmm_only_order='coo')
+    # the same edges stored in a random order, at the library's default: sorted once at build(), walked by the tiled
+    # traversal, every result written back to its stored position
+    perm_d = torch.randperm(nnz, generator=torch.Generator().manual_seed(3)).cuda()
+    rows_s, cols_s = rows_d[perm_d], idx_d[perm_d]
+    shuffled = VanillaSDDMMhip(sp.coo_matrix((np.ones(nnz, np.float32), (rows_s.cpu().numpy().astype(np.int32),
+                                                                         cols_s.cpu().numpy().astype(np.int32))), shape=(n, n)))
+    F = headline_F
+    gen.manual_seed(2)
+    x = torch.randn((n, F), generator=gen, device="cuda")
+    y = torch.randn((n, F), generator=gen, device="cuda")
+    shuffled.build([placeholder((n, F)), placeholder((n, F))], {}, {})
+    t = shuffled.measure_average_time([x, y], 5)
+    entries.append(config_entry("cfg3", workload, "sddmm_shuffled_coo", "F=%d" % F, sddmm_tiling(shuffled), t, 2.0 * nnz * F,
+                                sddmm_bytes(n, nnz, F, 1, csr=False), chk.sddmm_failures(shuffled.run([x, y]), rows_s, cols_s, x, y)))
+    del shuffled, x, y, perm_d, rows_s, cols_s
     mh = MultiHeadSDDMMhip(sp.csr_matrix((np.ones(nnz, np.float32), indices, indptr), shape=(n, n)))
     mh.share_layouts(spmm)
     for H, D in ((4, 32), (4, 64), (8, 32), (8, 64)):
