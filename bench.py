@@ -184,6 +184,7 @@ VALU_PEAK_GFLOPS = 157300.0      # fp32 vector peak of the part
 
 
 def config_entry(config, workload, op, shape, tiling, seconds, flops, bytes_model, failures):
+    """`tiling`: source-column partitions x feature tiles, or "stored order" for the kernels that walk the edges as stored."""
     gflops = flops / seconds / 1e9
     return {"config": config, "workload": workload, "op": op, "shape": shape, "tiling": tiling,
             "ms_mean_of_5": round(seconds * 1e3, 4), "gflops": round(gflops, 1),
@@ -195,8 +196,8 @@ def config_entry(config, workload, op, shape, tiling, seconds, flops, bytes_mode
 
 def sddmm_tiling(m):
     if m._tiled:
-        return "%d partitions x %d tiles" % (m._tiled[0]['P'], m._tiled[1])
-    return "stored order (%s)" % ("sddmm_csr_kernel" if m._use_csr else "sddmm_coo_kernel")
+        return "%dx%d" % (m._tiled[0]['P'], m._tiled[1])
+    return "stored order"
 
 
 def run_configs(torch, workload, indptr, indices, vals_d, spmm, sddmm, headline_F, skip_low_degree=False):
@@ -231,7 +232,7 @@ def run_configs(torch, workload, indptr, indices, vals_d, spmm, sddmm, headline_
             spmm.build([placeholder((n, F))], {}, {})
             t = spmm.measure_average_time([x], 5)
             entries.append(config_entry(config.split("/")[0], name, "spmm", "F=%d" % F,
-                                        "%d partitions x %d tiles" % (spmm._active['P'], spmm._num_feat_partitions or 1),
+                                        "%dx%d" % (spmm._active['P'], spmm._num_feat_partitions or 1),
                                         t, 2.0 * nnz * F, spmm_bytes(n, n, nnz, F),
                                         chk.spmm_failures(spmm.run([x]), indptr, idx_d, vals_d, x)))
         sa = {} if sddmm_only_order is None else {'order': sddmm_only_order}
@@ -492,11 +493,20 @@ def main():
         del x_d, y_d
         torch.cuda.empty_cache()
         t0 = time.perf_counter()
-        line["configs"] = run_configs(torch, args.workload, indptr, indices, vals_d, spmm, sddmm, F)
-        line["configs_verified"] = sum(1 for e in line["configs"] if e["verified"])
+        entries = run_configs(torch, args.workload, indptr, indices, vals_d, spmm, sddmm, F)
+        # one row per configuration (the JSON line stays short; the same table goes to stderr in readable form)
+        cols = ["config", "workload", "op", "shape", "tiling", "ms_mean_of_5", "gflops", "compulsory_gb", "hbm_gbs",
+                "pct_hbm_roofline", "valu_frac", "verified"]
+        line["configs"] = {"columns": cols, "rows": [[e[c] for c in cols] for e in entries]}
+        line["configs_verified"] = sum(1 for e in entries if e["verified"])
+        line["configs_total"] = len(entries)
         line["configs_seconds"] = round(time.perf_counter() - t0, 1)
         failures = failures + ["%s %s %s: %s" % (e["workload"], e["op"], e["shape"], "; ".join(e["failures"]))
-                               for e in line["configs"] if not e["verified"]]
+                               for e in entries if not e["verified"]]
+        for e in entries:
+            print("%-5s %-15s %-19s %-9s %-38s %8.3f ms %7.0f GFLOP/s %6.2f %% of 8 TB/s  %s"
+                  % (e["config"], e["workload"], e["op"], e["shape"], e["tiling"], e["ms_mean_of_5"], e["gflops"],
+                     e["pct_hbm_roofline"], "verified" if e["verified"] else "FAILED"), file=sys.stderr)
     print(json.dumps(line))
     if failures:
         sys.exit("bench.py: output verification failed: " + "; ".join(failures))
