@@ -39,12 +39,25 @@ class Graph(object):
                                             tr.indptr.astype(np.int32)), shape=tr.shape)
         self._tr_pos_host = (tr.data - 1).astype(np.int64)      # transposed edge order -> CSR position
         self._mods = {}
+        # the first SpMM-like module of each orientation owns the device layouts (partitioned copies of the adjacency, plans,
+        # scratch); later ones of the same orientation use them too: every operator of a Graph runs on the caller's one
+        # stream, one after the other, so one scratch per orientation is enough
+        self._layout_owner = {}
+
+    def _gspmm_module(self, transposed):
+        m = GSpMMhip(self._tr if transposed else self._csr)
+        owner = self._layout_owner.get(transposed)
+        if owner is None:
+            self._layout_owner[transposed] = m
+        else:
+            m.share_layouts_with(owner)
+        return m
 
     def _spmm_mod(self, transposed, tail, w_heads):
         key = ('spmm', transposed, tail, w_heads)
         if key not in self._mods:
             adj = self._tr if transposed else self._csr
-            m = GSpMMhip(adj)
+            m = self._gspmm_module(transposed)
             w_shape = (self.nnz,) if w_heads == 0 else (self.nnz, w_heads)
             m.build([placeholder((adj.shape[1],) + tail), placeholder(w_shape)], {}, {})
             if transposed:
@@ -107,7 +120,7 @@ class Graph(object):
     def _aggregate_mod(self, feat_len, reduce):
         key = ('aggregate', feat_len, reduce)
         if key not in self._mods:
-            m = GSpMMhip(self._csr)
+            m = self._gspmm_module(False)
             args = {'reduce': reduce, 'msg': 'copy_u'}
             if reduce in ('max', 'min'):
                 args['return_arg'] = True
@@ -194,7 +207,7 @@ class Graph(object):
         arrays = [a.contiguous() for a in arrays]
         key = ('gspmm', msg, reduce, transposed, return_arg) + tuple(tuple(a.shape) for a in arrays)
         if key not in self._mods:
-            m = GSpMMhip(self._tr if transposed else self._csr)
+            m = self._gspmm_module(transposed)
             args = {'msg': msg, 'reduce': reduce, 'broadcast': True}      # numpy broadcasting, whatever the shapes
             if return_arg:
                 args['return_arg'] = True

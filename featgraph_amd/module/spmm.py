@@ -112,18 +112,38 @@ class SpMMbase(object):
                 pass
             lay['plan'] = None
 
+    def share_layouts_with(self, other):
+        """Uses the device layouts of `other` -- another SpMM-like module built on the same adjacency (same structure and
+        values) -- instead of making its own: every partitioned copy, plan, 16-bit id copy and scratch exists once for the
+        two (the scratch as large as the larger need).  To be called before build().  Their run() calls must follow each other
+        on one stream, as two calls on one module must.  Keeps `other` alive; `other` stops freeing layouts on re-builds."""
+        same = (self._num_rows, self._num_cols) == (other._num_rows, other._num_cols) \
+            and np.array_equal(self._adj_indptr, other._adj_indptr) and np.array_equal(self._adj_indices, other._adj_indices) \
+            and np.array_equal(self._adj_scipy_csr.data, other._adj_scipy_csr.data)
+        if not same:
+            raise ValueError("share_layouts_with needs a module built on the same adjacency")
+        if self._layouts:
+            raise RuntimeError("share_layouts_with must be called before the first build()")
+        owner = getattr(other, '_layout_owner', None) or other
+        owner._layout_sharers = getattr(owner, '_layout_sharers', 0) + 1
+        self._layout_owner = owner
+        self._layouts = owner._layouts
+
     def _release_unused_layouts(self):
         """Frees the partitioned copies (device arrays, plan, scratch) that the built configuration does not use; a
         later build() that wants one of them makes it again.  The constructor's own layout and the CSR arrays stay."""
+        if getattr(self, '_layout_owner', None) is not None or getattr(self, '_layout_sharers', 0):
+            return                  # the layouts serve several modules
         keep = {1, self._num_col_partitions, self._active['P']}
         for P in [P for P in self._layouts if P not in keep and not self._layouts[P].get('users')]:
             self._destroy_layout(self._layouts.pop(P))
 
     def device_bytes(self):
         """Device memory this module holds: {'graph': the adjacency's arrays in every layout kept, 'plans': work items,
-        scratch, tile-by-tile copy and 16-bit ids of their plans (fg_spmm_plan_bytes), 'buffers': output and padding}."""
+        scratch, tile-by-tile copy and 16-bit ids of their plans (fg_spmm_plan_bytes), 'buffers': output and padding};
+        layouts taken over from another module (share_layouts_with) are counted there."""
         graph = plans = 0
-        for lay in self._layouts.values():
+        for lay in ({} if getattr(self, '_layout_owner', None) is not None else self._layouts).values():
             graph += sum(t.numel() * t.element_size() for t in lay.values() if isinstance(t, torch.Tensor))
             plans += int(_lib.lib().fg_spmm_plan_bytes(lay['plan']))
         bufs = sum(t.numel() * t.element_size() for t in (self.out_tvm, getattr(self, '_x_pad', None), getattr(self, '_out_pad', None))
@@ -131,6 +151,10 @@ class SpMMbase(object):
         return {'graph': graph, 'plans': plans, 'buffers': bufs}
 
     def __del__(self):
+        owner = getattr(self, '_layout_owner', None)
+        if owner is not None:
+            owner._layout_sharers = max(0, getattr(owner, '_layout_sharers', 1) - 1)
+            return
         for lay in getattr(self, "_layouts", {}).values():
             self._destroy_layout(lay)
 

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 def _graph(rng, n_rows=400, n_cols=3000):
     a = sp.random(n_rows, n_cols, density=0.02, format="csr", random_state=rng).astype("float32").tolil()
     a[[0, 11], :] = 0
-    a[5, rng.choice(n_cols, size=2500, replace=False)] = 1.0          # longer than the split threshold
+    a[5, rng.choice(n_cols, size=min(2500, n_cols - 20), replace=False)] = 1.0     # longer than the split threshold where the matrix is wide enough
     a = a.tocsr().astype("float32"); a.eliminate_zeros(); a.sort_indices()
     a.data = (rng.random(a.nnz) + 0.1).astype("float32")
     return a
@@ -110,3 +110,49 @@ def test_shared_layouts_give_the_same_bits(oracle, H):
     p = rng.permutation(coo.nnz)
     with pytest.raises(ValueError):
         cls(sp.coo_matrix((coo.data[p], (coo.row[p], coo.col[p])), shape=coo.shape)).share_layouts(spmm)
+
+
+def test_graph_modules_share_one_set_of_layouts():
+    """featgraph_amd.autograd.Graph: the SpMM-like modules of one orientation (weighted sums of several shapes, per-head
+    weights, broadcasting messages, max aggregation) use one set of device layouts and plans, and the SDDMM modules take
+    theirs from the forward SpMM module; results as from modules of their own."""
+    import torch
+    from featgraph_amd.autograd import Graph
+    from featgraph_amd.module import GSpMMhip, placeholder
+    rng = np.random.default_rng(9)
+    adj = _graph(rng, 300, 300)
+    g = Graph(adj)
+    n, nnz = 300, adj.nnz
+    gen = torch.Generator(device="cuda"); gen.manual_seed(4)
+    x16 = torch.randn((n, 16), generator=gen, device="cuda", requires_grad=True)
+    x64 = torch.randn((n, 64), generator=gen, device="cuda", requires_grad=True)
+    xh = torch.randn((n, 4, 16), generator=gen, device="cuda", requires_grad=True)
+    w = torch.rand(nnz, generator=gen, device="cuda", requires_grad=True)
+    wh = torch.rand((nnz, 4), generator=gen, device="cuda", requires_grad=True)
+    outs = [g.spmm(x16, w), g.spmm(x64, w), g.spmm(xh, wh), g.aggregate(x16, 'max'), g.gspmm('u_add_e', x16, w.reshape(-1, 1), 'sum'),
+            g.sddmm(x64, x64)]
+    sum(o.square().sum() for o in outs).backward()
+    fwd = [m for k, m in g._mods.items() if isinstance(m, GSpMMhip) and m._adj_scipy_csr is g._csr]
+    bwd = [m for k, m in g._mods.items() if isinstance(m, GSpMMhip) and m._adj_scipy_csr is g._tr]
+    assert len(fwd) >= 4 and len(bwd) >= 2
+    for mods in (fwd, bwd):
+        owner = [m for m in mods if getattr(m, '_layout_owner', None) is None]
+        assert len(owner) == 1
+        assert all(m._layouts is owner[0]._layouts for m in mods)
+        assert sum(m.device_bytes()['plans'] > 0 for m in mods) == 1
+    # the same numbers as a module of its own gives
+    own = GSpMMhip(adj)
+    own.build([placeholder((n, 64)), placeholder((nnz,))], {}, {})
+    assert torch.equal(own.run([x64.detach(), w.detach()]), outs[1].detach())
+    # the gradient of the first weighted sum against torch autograd on the dense matrix
+    dense = torch.zeros((n, n), device="cuda", dtype=torch.float64)
+    coo = adj.tocoo()
+    rows, cols = torch.from_numpy(coo.row.astype(np.int64)).cuda(), torch.from_numpy(coo.col.astype(np.int64)).cuda()
+    x2 = x16.detach().double().requires_grad_()
+    w2 = w.detach().double().requires_grad_()
+    y = torch.zeros((n, 16), device="cuda", dtype=torch.float64).index_add(0, rows, w2[:, None] * x2[cols])
+    g2 = Graph(adj)
+    x3 = x16.detach().clone().requires_grad_(); w3 = w.detach().clone().requires_grad_()
+    g2.spmm(x3, w3).square().sum().backward()
+    y.square().sum().backward()
+    assert torch.allclose(x3.grad.double(), x2.grad, rtol=1e-4, atol=1e-4) and torch.allclose(w3.grad.double(), w2.grad, rtol=1e-4, atol=1e-4)
