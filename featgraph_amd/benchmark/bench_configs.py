@@ -6,7 +6,8 @@ Configurations: weighted CSR SpMM and SDDMM (CSR-ordered and shuffled COO edges)
 lengths 32..512 and multi-head SDDMM (H in {4, 8}, D in {32, 64}) on the 232,965-node power-law
 graph, plus the other two steps of an attention layer there (edge softmax and its gradient for
 H in {1, 4, 8}, per-head weighted SpMM for the same head shapes); SpMM followed by SDDMM at feature
-length 128 on the 2.45M-node low-degree graph; SpMM on the 10,000-node uniform graph.  One JSON line per measurement (mean of 5 launches after a warm-up).
+length 128 on the 2.45M-node low-degree graph; SpMM on the 10,000-node uniform graph.  One JSON line per measurement (mean of 5 launches after a warm-up);
+the SpMM / SDDMM lines carry `verified`: the output checks of featgraph_amd/benchmark/verify.py on the inputs that were timed.
 """
 import argparse
 import json
@@ -17,14 +18,17 @@ import torch
 
 from .. import synthetic
 from ..module import common
+from . import verify as chk
 from ..module import (VanillaSpMMhip, VanillaSDDMMhip, MultiHeadSDDMMhip, GSpMMhip, EdgeSoftmaxhip,
                       EdgeSoftmaxSpMMhip, GraphAttentionhip, placeholder)
 
 HBM_PEAK_GBS = 8000.0
 
 
-def _line(workload, op, knobs, seconds, nnz, feat_len, bytes_model):
+def _line(workload, op, knobs, seconds, nnz, feat_len, bytes_model, failures=None):
     out = dict(workload=workload, op=op, **knobs)
+    if failures is not None:            # the output of this configuration was checked (featgraph_amd/benchmark/verify.py)
+        out["verified"] = not failures
     out.update(ms=round(seconds * 1e3, 4), gflops=round(2.0 * nnz * feat_len / seconds / 1e9, 1),
                compulsory_gb=round(bytes_model / 1e9, 3), compulsory_gbs=round(bytes_model / seconds / 1e9, 1),
                pct_hbm_roofline=round(100.0 * bytes_model / seconds / 1e9 / HBM_PEAK_GBS, 3),
@@ -106,6 +110,9 @@ def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):
     gen.manual_seed(1)
     vals = torch.rand(nnz, generator=gen, device="cuda").cpu().numpy()
     adj = sp.csr_matrix((vals, indices, indptr), shape=(n, n))
+    vals_d = torch.from_numpy(vals).cuda()
+    idx_d = torch.from_numpy(indices).cuda().long()
+    rows_d = torch.repeat_interleave(torch.arange(n, device="cuda"), torch.from_numpy(np.diff(indptr)).cuda().long())
     spmm = VanillaSpMMhip(adj)
     sddmm = VanillaSDDMMhip(adj)
     for F in feat_lens:
@@ -115,12 +122,12 @@ def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):
         spmm.build([placeholder((n, F))], {}, {})
         t = spmm.measure_average_time([x], 5)
         _line(name, "spmm", {"feat_len": F, "partitions": spmm._active['P'], "tiles": spmm._num_feat_partitions},
-              t, nnz, F, 4 * (n + 1) + 8 * nnz + 8 * n * F)
+              t, nnz, F, 4 * (n + 1) + 8 * nnz + 8 * n * F, chk.spmm_failures(spmm.run([x]), indptr, idx_d, vals_d, x))
         sddmm.build([placeholder((n, F)), placeholder((n, F))], {}, {})
         t = sddmm.measure_average_time([x, y], 5)
         tiled = (sddmm._tiled[0]['P'], sddmm._tiled[1]) if sddmm._tiled else None
         _line(name, "sddmm_csr_order", {"feat_len": F, "tiled": tiled}, t, nnz, F,
-              4 * (n + 1) + 4 * nnz + 8 * n * F + 4 * nnz)
+              4 * (n + 1) + 4 * nnz + 8 * n * F + 4 * nnz, chk.sddmm_failures(sddmm.run([x, y]), rows_d, idx_d, x, y))
         del x, y
     for H, D in head_shapes:
         gen.manual_seed(2)
@@ -131,7 +138,7 @@ def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):
         t = mh.measure_average_time([x, y], 5)
         tiled = (mh._tiled[0]['P'], mh._tiled[1]) if mh._tiled else None
         _line(name, "sddmm_multihead", {"heads": H, "head_len": D, "tiled": tiled}, t, nnz, H * D,
-              4 * (n + 1) + 4 * nnz + 8 * n * H * D + 4 * nnz * H)
+              4 * (n + 1) + 4 * nnz + 8 * n * H * D + 4 * nnz * H, chk.sddmm_failures(mh.run([x, y]), rows_d, idx_d, x, y))
         del mh, x, y
     if softmax_heads:
         run_attention_steps(name, adj, softmax_heads, head_shapes)
@@ -139,6 +146,7 @@ def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):
         coo = adj.tocoo()
         perm = torch.randperm(nnz, generator=torch.Generator().manual_seed(3)).numpy()
         coo = sp.coo_matrix((coo.data[perm], (coo.row[perm], coo.col[perm])), shape=coo.shape)
+        perm_d = torch.from_numpy(perm).cuda()
         m = VanillaSDDMMhip(coo)
         for F in shuffled_coo:
             gen.manual_seed(2)
@@ -147,8 +155,8 @@ def run_workload(name, feat_lens, head_shapes, shuffled_coo, softmax_heads=()):
             for order in ("coo", "auto"):
                 m.build([placeholder((n, F)), placeholder((n, F))], {}, {'order': order})
                 t = m.measure_average_time([x, y], 5)
-                _line(name, "sddmm_shuffled_coo", {"feat_len": F, "order": order}, t, nnz, F,
-                      8 * nnz + 8 * n * F + 4 * nnz)
+                _line(name, "sddmm_shuffled_coo", {"feat_len": F, "order": order}, t, nnz, F, 8 * nnz + 8 * n * F + 4 * nnz,
+                      chk.sddmm_failures(m.run([x, y]), rows_d[perm_d], idx_d[perm_d], x, y))
             del x, y
 
 
